@@ -1,0 +1,189 @@
+/*
+ * turq.h — C ABI of libturq: GGUF block-quantized linear layers on MI355X (gfx950).
+ *
+ * This is the boundary a host engine binds (Rust `extern "C"`, ctypes, cgo ...).  Every entry
+ * point takes plain pointers and sizes, returns an integer status, and never aborts; the text of
+ * the last error is kept per context (and per thread when no context exists yet).
+ *
+ * Each declaration cites the reference interface it stands in for (paths are relative to the
+ * danylokravchenko/tur tree; "candle" means candle-core 0.10.2 as pinned by its Cargo.lock).
+ *
+ * Threading: a context is thread-compatible (calls on one context must be serialised by the
+ * caller, as the reference does by owning the model on one thread, src/server/worker.rs:69-100);
+ * different contexts may be used from different threads.  Weights are immutable after upload and
+ * reference counted, so clones of a layer share one device copy (LinearX is Clone,
+ * src/models/layers/linear.rs:8).
+ */
+#ifndef TURQ_H
+#define TURQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct turq_ctx turq_ctx;       /* device + stream + scratch, one per engine thread */
+typedef struct turq_weight turq_weight; /* one quantized [n, k] tensor resident in HBM */
+typedef struct turq_gguf turq_gguf;     /* an opened GGUF file (header parsed, tensors lazy) */
+
+/* status codes */
+enum {
+    TURQ_OK = 0,
+    TURQ_ERR_INVALID = 1,   /* null pointer, bad flag, bad argument */
+    TURQ_ERR_SHAPE = 2,     /* shape mismatch, k not a multiple of the block size, ld too small */
+    TURQ_ERR_DTYPE = 3,     /* ggml dtype or activation dtype not supported */
+    TURQ_ERR_HIP = 4,       /* a HIP runtime call failed (message holds hipGetErrorString) */
+    TURQ_ERR_OOM = 5,       /* host or device allocation failed */
+    TURQ_ERR_IO = 6,        /* file open/read/parse failure */
+    TURQ_ERR_NOT_FOUND = 7  /* tensor or metadata key absent */
+};
+
+/* ggml dtype ids as stored in GGUF tensor infos (candle GgmlDType) */
+enum {
+    TURQ_F32 = 0,
+    TURQ_F16 = 1,
+    TURQ_Q8_0 = 8,
+    TURQ_Q4_K = 12,
+    TURQ_Q5_K = 13,
+    TURQ_Q6_K = 14,
+    TURQ_BF16 = 30
+};
+
+/* element type of activation / output buffers */
+enum { TURQ_ACT_F32 = 0, TURQ_ACT_BF16 = 1, TURQ_ACT_F16 = 2 };
+
+/* weight layouts in HBM */
+enum {
+    TURQ_LAYOUT_NATIVE = 0, /* GGUF bytes as they are: rows of consecutive blocks */
+    TURQ_LAYOUT_TILED = 1   /* 16-row x 256-column tiles, lane-linear planes (see tur_amd/csrc/layout.h) */
+};
+
+/* where the pointers of a call live */
+enum { TURQ_MEM_HOST = 0, TURQ_MEM_DEVICE = 1 };
+
+/* matmul algorithm selection (TURQ_ALGO_AUTO picks by layout and m) */
+enum {
+    TURQ_ALGO_AUTO = 0,
+    TURQ_ALGO_SIMPLE = 1, /* one wave per output row, f32 FMA on dequantized values */
+    TURQ_ALGO_GEMV = 2,   /* MFMA skinny kernel for m <= 32, tiled layout */
+    TURQ_ALGO_GEMM = 3    /* LDS-tiled MFMA kernel for prefill chunks, tiled layout */
+};
+
+/* ---- library ---- */
+const char *turq_version(void);
+/* geometry of a ggml dtype: elements and bytes per block; 0 when the dtype is not supported */
+int turq_block_elems(int ggml_dtype);
+int turq_block_bytes(int ggml_dtype);
+/* bytes of an [n, k] tensor in GGUF = n * k / block_elems * block_bytes; 0 on invalid input.
+ * Replaces: the length computed inside candle `gguf_file::TensorInfo::read`. */
+size_t turq_weight_nbytes(int ggml_dtype, int64_t n, int64_t k);
+
+/* ---- context ---- */
+/* Replaces: the `Device` handed to `VarBuilderX::new` / `QVarBuilder::from_gguf`
+ * (src/weights/mod.rs:37-67, src/weights/gguf_varbuilder.rs:20-30; chosen at src/main.rs:188). */
+int turq_ctx_create(int device_ordinal, turq_ctx **out);
+void turq_ctx_destroy(turq_ctx *ctx);
+/* message of the most recent failing call on ctx (ctx may be NULL: last failure of this thread
+ * in a call that had no context).  Replaces: candle_core::Error -> TurError::CandleError
+ * (src/shared/errors.rs:5-6). */
+const char *turq_last_error(const turq_ctx *ctx);
+/* block until all work queued on the context's stream is done */
+int turq_sync(turq_ctx *ctx);
+/* the context's hipStream_t, for hosts that time or order their own work on it */
+void *turq_ctx_stream(turq_ctx *ctx);
+/* name and compute-unit count of the context's device */
+int turq_ctx_device_info(turq_ctx *ctx, char *name, size_t name_cap, int *compute_units);
+
+/* ---- device memory helpers for hosts without HIP bindings of their own ---- */
+int turq_dev_alloc(turq_ctx *ctx, size_t nbytes, void **out);
+int turq_dev_free(turq_ctx *ctx, void *ptr);
+/* synchronous copies (they wait for the context's stream first) */
+int turq_memcpy_h2d(turq_ctx *ctx, void *dst_dev, const void *src_host, size_t nbytes);
+int turq_memcpy_d2h(turq_ctx *ctx, void *dst_host, const void *src_dev, size_t nbytes);
+
+/* ---- weights ---- */
+/* Upload raw GGUF block bytes of a tensor of shape (n, k) (n output features, k input features,
+ * each row = k/block consecutive blocks).  `layout` picks how it is kept in HBM.
+ * Errors: unsupported dtype, k % block != 0, nbytes != turq_weight_nbytes(..).
+ * Replaces: candle `gguf_file::Content::tensor(reader, name, device)` -> `QTensor` as called by
+ * `QVarBuilder::get` (src/weights/gguf_varbuilder.rs:72-74) and `QMatMul::from_arc`
+ * (src/models/layers/linear.rs:69). */
+int turq_weight_upload(turq_ctx *ctx, int ggml_dtype, int64_t n, int64_t k, const void *host_bytes,
+                       size_t nbytes, int layout, turq_weight **out);
+/* Arc<QTensor> clone / drop */
+int turq_weight_retain(turq_weight *w);
+int turq_weight_release(turq_weight *w);
+/* QTensor::shape / dtype; any out pointer may be NULL */
+int turq_weight_info(const turq_weight *w, int *ggml_dtype, int64_t *n, int64_t *k, int *layout,
+                     size_t *device_bytes);
+/* Copy the tensor back to host in GGUF byte order whatever its HBM layout (round-trip check). */
+int turq_weight_export(turq_ctx *ctx, const turq_weight *w, void *host_bytes, size_t nbytes);
+
+/* Host-side layout transforms used by upload/export (no GPU needed): native GGUF bytes <-> tiled. */
+size_t turq_tiled_nbytes(int ggml_dtype, int64_t n, int64_t k);
+int turq_tile_host(int ggml_dtype, int64_t n, int64_t k, const void *native, void *tiled);
+int turq_untile_host(int ggml_dtype, int64_t n, int64_t k, const void *tiled, void *native);
+
+/* ---- dequantize ---- */
+/* out = f32 [n, k] row-major, bit-exact with candle's to_float.  `out_mem` says whether `out` is
+ * a host or a device pointer.
+ * Replaces: `QTensor::dequantize(device)` (call sites src/weights/mod.rs:150,161;
+ * src/models/layers/mod.rs:37; src/models/layers/norm.rs:84; src/models/layers/linear.rs:66). */
+int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem);
+
+/* ---- forward ---- */
+/* y[m, n] = x[m, k] * W^T  (+ bias[n] when bias != NULL).
+ *   x: m rows of k elements of `x_dtype`, row stride ldx elements (ldx >= k);
+ *   y: m rows of n elements of `y_dtype`, row stride ldy elements (ldy >= n);
+ *   bias: f32 [n] (in the same memory space as x and y) or NULL (the reference adds it with a separate broadcast_add,
+ *         src/models/layers/linear.rs:25-28);
+ *   mem: TURQ_MEM_DEVICE (x, y are device pointers; the call is asynchronous on the context's
+ *        stream) or TURQ_MEM_HOST (x, y are host pointers; staged through the context and
+ *        synchronous);
+ *   algo: TURQ_ALGO_*.
+ * Errors instead of panics for m < 0, ld too small, unsupported dtypes.  m == 0 is a no-op.
+ * Replaces: `LinearX::forward` -> `QMatMul::forward(&Tensor)` (src/models/layers/linear.rs:19-31)
+ * -> candle `CustomOp1::cpu_fwd` -> `k_quants::matmul`. */
+int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype, int64_t m,
+                 int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias, int mem, int algo);
+
+/* ---- activation quantisation (candle's VecDotType::from_float, bit-exact) ---- */
+/* x f32 [m, k] (row stride k) -> Q8_0 blocks (34 B per 32) / Q8_K blocks (292 B per 256).
+ * The GPU forward path does not use them (it keeps activations in f16); they are the device
+ * counterpart of candle `BlockQ8_0::from_float` / `BlockQ8K::from_float`, the first step of
+ * `k_quants::matmul`. */
+int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem);
+int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem);
+
+/* ---- GGUF files ---- */
+/* Parse the header (magic, version 1..3, metadata, tensor infos, alignment).
+ * Replaces: `QVarBuilder::from_gguf` -> candle `gguf_file::Content::read`
+ * (src/weights/gguf_varbuilder.rs:20-30). */
+int turq_gguf_open(const char *path, turq_gguf **out);
+void turq_gguf_close(turq_gguf *g);
+const char *turq_gguf_last_error(const turq_gguf *g);
+/* `all_keys` (gguf_varbuilder.rs:110-117) */
+int64_t turq_gguf_tensor_count(const turq_gguf *g);
+const char *turq_gguf_tensor_name(const turq_gguf *g, int64_t index);
+/* `contains_key` / `tensor_shape` (gguf_varbuilder.rs:100-108): dims come back outermost first
+ * ((n, k) for a matrix, i.e. GGUF order reversed as candle does).  TURQ_ERR_NOT_FOUND if absent. */
+int turq_gguf_tensor_info(const turq_gguf *g, const char *name, int *ggml_dtype, int *n_dims,
+                          int64_t dims[4], uint64_t *file_offset, size_t *nbytes);
+/* metadata lookups (Content::metadata): integer-like and string values */
+int turq_gguf_meta_u64(const turq_gguf *g, const char *key, uint64_t *out);
+int turq_gguf_meta_f64(const turq_gguf *g, const char *key, double *out);
+int turq_gguf_meta_str(const turq_gguf *g, const char *key, char *out, size_t cap);
+/* Read one tensor's raw bytes from the file (seek + read, nothing cached). */
+int turq_gguf_read_tensor(turq_gguf *g, const char *name, void *host_bytes, size_t nbytes);
+/* `QVarBuilder::get((n, k), name)` / `get_no_shape(name)` (gguf_varbuilder.rs:52-94): read the
+ * tensor and upload it.  expect_n/expect_k < 0 skip the shape check; a mismatch is TURQ_ERR_SHAPE
+ * ("shape mismatch for NAME, got .., expected .."). 1-D tensors load as (1, k). */
+int turq_gguf_load_weight(turq_ctx *ctx, turq_gguf *g, const char *name, int64_t expect_n,
+                          int64_t expect_k, int layout, turq_weight **out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TURQ_H */

@@ -1,0 +1,65 @@
+"""GPU parity at the full Qwen3-8B shapes the benchmark runs (decode GEMV, m = 1 and small batches).
+
+The oracle's dense matmul finishes these in seconds on the host cores, so the comparison is direct;
+the LM head (151936 x 4096) is checked on m = 1 only to keep the CPU time bounded.
+"""
+import numpy as np
+import pytest
+
+from oracle import capi as orc
+from tests.helpers import Gpu, rel_l2
+from tur_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    g = Gpu()
+    yield g
+    g.close()
+
+
+CASES = [
+    ("q8_0 gate 0.6B", Q8_0, 3072, 1024, [1]),
+    ("q4_k gate/up 8B", Q4_K, 12288, 4096, [1, 4, 16]),
+    ("q4_k down 8B", Q4_K, 4096, 12288, [1, 16]),
+    ("q4_k k_proj 8B", Q4_K, 1024, 4096, [1, 8, 32]),
+    ("q6_k v_proj 8B", Q6_K, 1024, 4096, [1, 8, 32]),
+    ("q6_k down 8B", Q6_K, 4096, 12288, [1, 32]),
+]
+
+
+@pytest.mark.parametrize("name,dt,n,k,ms", CASES, ids=[c[0] for c in CASES])
+def test_decode_shapes(gpu, name, dt, n, k, ms):
+    raw = synth.random_weight(dt, n, k, seed=n + k + dt)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    for m in ms:
+        x = synth.random_activation(m, k, seed=m)
+        y = gpu.qmatmul(w, x, n, k)
+        dense = orc.matmul_dequant(dt, x, raw, n, k)
+        assert rel_l2(y, dense) <= 1e-3
+        xb = synth.random_activation(m, k, seed=m + 1, bf16=True)
+        yb = gpu.qmatmul(w, xb, n, k, x_dtype=capi.ACT_BF16)
+        assert rel_l2(yb, orc.matmul_dequant(dt, xb, raw, n, k)) <= 2e-5
+        if m == ms[0]:
+            assert rel_l2(y, orc.qmatmul(dt, x, raw, n, k)) <= 1e-2
+    gpu.release(w)
+
+
+@pytest.mark.parametrize("dt", [Q6_K, Q5_K], ids=["q6_k", "q5_k"])
+def test_lm_head(gpu, dt):
+    n, k = 151936, 4096
+    raw = synth.random_weight(dt, n, k, seed=dt)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    x = synth.random_activation(1, k, seed=9, bf16=True)
+    y = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, k)) <= 2e-5
+    # m = 16: spot-check 4096 vocabulary rows spread over the matrix against the oracle
+    x16 = synth.random_activation(16, k, seed=10, bf16=True)
+    y16 = gpu.qmatmul(w, x16, n, k, x_dtype=capi.ACT_BF16)
+    rows = np.arange(0, n, n // 4096)[:4096]
+    sub = raw.reshape(n, -1)[rows].reshape(-1)
+    assert rel_l2(y16[:, rows], orc.matmul_dequant(dt, x16, sub, len(rows), k)) <= 2e-5
+    gpu.release(w)

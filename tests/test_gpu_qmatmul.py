@@ -1,0 +1,192 @@
+"""GPU parity of turq_qmatmul (the QMatMul::forward replacement), called through the C ABI.
+
+Bars (relative L2 over the whole output):
+  * <= 1e-3 against the f32 matmul on oracle-dequantized weights (f64-accumulated),
+  * <= 1e-2 against the restated candle CPU QMatMul (which quantises activations to Q8_K / Q8_0),
+and two sharper ones that catch indexing slips the loose bars could hide:
+  * the plain kernel (f32 FMA on dequantized values) must agree to 2e-5,
+  * the MFMA kernel must agree to 2e-5 once the oracle is given the same f16-rounded activations
+    (its weight side is exact integer arithmetic).
+"""
+import numpy as np
+import pytest
+
+from oracle import capi as orc
+from tests.helpers import Gpu, rel_l2
+from tur_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+ALL = [Q8_0, Q4_K, Q5_K, Q6_K]
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    g = Gpu()
+    yield g
+    g.close()
+
+
+def f16_round(x):
+    return x.astype(np.float16).astype(np.float32)
+
+
+def check_all_bars(y, dt, x, raw, n, k, f16_acts):
+    dense = orc.matmul_dequant(dt, x, raw, n, k)
+    assert rel_l2(y, dense) <= 1e-3
+    cpu = orc.qmatmul(dt, x, raw, n, k)
+    assert rel_l2(y, cpu) <= 1e-2
+    sharp = orc.matmul_dequant(dt, f16_round(x), raw, n, k) if f16_acts else dense
+    assert rel_l2(y, sharp) <= 2e-5, rel_l2(y, sharp)
+
+
+@pytest.mark.parametrize("dt", ALL)
+@pytest.mark.parametrize("m", [1, 5])
+def test_simple_kernel_native_layout(gpu, dt, m):
+    n, k = 77, 1024
+    raw = synth.random_weight(dt, n, k, seed=dt * 3 + m)
+    x = synth.random_activation(m, k, seed=m)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_NATIVE)
+    y = gpu.qmatmul(w, x, n, k, algo=capi.ALGO_SIMPLE)
+    gpu.release(w)
+    check_all_bars(y, dt, x, raw, n, k, f16_acts=False)
+
+
+@pytest.mark.parametrize("dt", ALL)
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8, 13, 16, 17, 32])
+def test_mfma_gemv_tiled_layout(gpu, dt, m):
+    n, k = 200, 2048           # ragged row tile (200 = 12 * 16 + 8), 8 column tiles
+    raw = synth.random_weight(dt, n, k, seed=dt * 5 + m)
+    x = synth.random_activation(m, k, seed=m + 50)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    y = gpu.qmatmul(w, x, n, k, algo=capi.ALGO_GEMV)
+    gpu.release(w)
+    check_all_bars(y, dt, x, raw, n, k, f16_acts=True)
+
+
+@pytest.mark.parametrize("dt", ALL)
+def test_mfma_more_rows_than_one_launch(gpu, dt):
+    n, k, m = 64, 512, 70       # m > 32 goes through the chunked / GEMM path
+    raw = synth.random_weight(dt, n, k, seed=dt)
+    x = synth.random_activation(m, k, seed=70)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    y = gpu.qmatmul(w, x, n, k)
+    gpu.release(w)
+    check_all_bars(y, dt, x, raw, n, k, f16_acts=True)
+
+
+@pytest.mark.parametrize("dt", ALL)
+def test_single_tile_shapes(gpu, dt):
+    # the smallest legal shapes: one block of columns, one row
+    k = 256
+    for n in (1, 16, 17):
+        raw = synth.random_weight(dt, n, k, seed=n)
+        x = synth.random_activation(2, k, seed=n + 1)
+        for layout, sharp in ((capi.LAYOUT_NATIVE, False), (capi.LAYOUT_TILED, True)):
+            w = gpu.upload(dt, n, k, raw, layout)
+            y = gpu.qmatmul(w, x, n, k)
+            gpu.release(w)
+            ref = orc.matmul_dequant(dt, f16_round(x) if sharp else x, raw, n, k)
+            assert rel_l2(y, ref) <= 2e-5
+
+
+def test_q8_0_ragged_k(gpu):
+    # Q8_0 needs k % 32 == 0 only: 96 columns fill 3 of the 8 blocks of a column tile
+    n, k = 48, 96 + 256
+    raw = synth.random_weight(Q8_0, n, k, seed=4)
+    x = synth.random_activation(3, k, seed=5)
+    w = gpu.upload(Q8_0, n, k, raw, capi.LAYOUT_TILED)
+    y = gpu.qmatmul(w, x, n, k)
+    gpu.release(w)
+    assert rel_l2(y, orc.matmul_dequant(Q8_0, f16_round(x), raw, n, k)) <= 2e-5
+
+
+@pytest.mark.parametrize("layout", [capi.LAYOUT_NATIVE, capi.LAYOUT_TILED])
+def test_activation_and_output_dtypes(gpu, layout):
+    n, k, m = 96, 1024, 4
+    raw = synth.random_weight(Q4_K, n, k, seed=21)
+    x = synth.random_activation(m, k, seed=22, bf16=True)     # bf16-representable values
+    w = gpu.upload(Q4_K, n, k, raw, layout)
+    dense = orc.matmul_dequant(Q4_K, x, raw, n, k)
+    # bf16 activations are exact in both kernels (bf16 -> f16 loses nothing for |x| in the f16 range)
+    y = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    assert rel_l2(y, dense) <= 2e-5
+    y = gpu.qmatmul(w, x.astype(np.float16).astype(np.float32), n, k, x_dtype=capi.ACT_F16)
+    assert rel_l2(y, orc.matmul_dequant(Q4_K, f16_round(x), raw, n, k)) <= 2e-5
+    # bf16 store: compare with the oracle rounded the same way (round to nearest even)
+    yb = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16)
+    want = synth.from_bf16_bits(synth.to_bf16_bits(dense)).reshape(m, n)
+    assert rel_l2(yb, want) <= 2e-3 and rel_l2(yb, dense) <= 4e-3
+    yh = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_F16)
+    assert rel_l2(yh, dense) <= 5e-4
+    gpu.release(w)
+
+
+@pytest.mark.parametrize("layout", [capi.LAYOUT_NATIVE, capi.LAYOUT_TILED])
+def test_bias_and_row_strides(gpu, layout):
+    n, k, m = 50, 512, 3
+    raw = synth.random_weight(Q6_K, n, k, seed=31)
+    x = synth.random_activation(m, k, seed=32, bf16=True)
+    bias = np.random.default_rng(33).standard_normal(n).astype(np.float32)
+    w = gpu.upload(Q6_K, n, k, raw, layout)
+    y = gpu.qmatmul(w, x, n, k, bias=bias, ldx=k + 24, ldy=n + 7)
+    gpu.release(w)
+    want = orc.matmul_dequant(Q6_K, x, raw, n, k) + bias[None, :]
+    assert rel_l2(y, want) <= 2e-5
+
+
+def test_linearity_and_zero_input(gpu):
+    # size-independent properties at a full Qwen3-8B row count: f(0) = 0, f(2x) = 2 f(x) exactly
+    # (scaling by 2 is exact in f16 and f32), f(x1 + x2) ~= f(x1) + f(x2)
+    n, k = 4096, 4096
+    raw = synth.random_weight(Q4_K, n, k, seed=41)
+    w = gpu.upload(Q4_K, n, k, raw, capi.LAYOUT_TILED)
+    x1 = synth.random_activation(1, k, seed=42, bf16=True)
+    x2 = synth.random_activation(1, k, seed=43, bf16=True)
+    y0 = gpu.qmatmul(w, np.zeros((1, k), np.float32), n, k)
+    assert np.all(y0 == 0)
+    y1 = gpu.qmatmul(w, x1, n, k)
+    assert np.array_equal(gpu.qmatmul(w, 2 * x1, n, k), 2 * y1)
+    y2 = gpu.qmatmul(w, x2, n, k)
+    y12 = gpu.qmatmul(w, x1 + x2, n, k)
+    assert rel_l2(y12, y1 + y2) <= 1e-3
+    gpu.release(w)
+
+
+def test_weight_clone_shares_device_copy(gpu):
+    # Arc<QTensor> semantics: retain / release, the weight stays usable until the last release
+    n, k = 32, 256
+    raw = synth.random_weight(Q4_K, n, k, seed=51)
+    x = synth.random_activation(1, k, seed=52)
+    w = gpu.upload(Q4_K, n, k, raw, capi.LAYOUT_TILED)
+    capi.check(gpu.L.turq_weight_retain(w))
+    gpu.release(w)
+    y = gpu.qmatmul(w, x, n, k)
+    gpu.release(w)
+    assert rel_l2(y, orc.matmul_dequant(Q4_K, f16_round(x), raw, n, k)) <= 2e-5
+
+
+def test_error_paths(gpu):
+    L, ctx = gpu.L, gpu.ctx
+    n, k = 32, 256
+    raw = synth.random_weight(Q4_K, n, k, seed=61)
+    import ctypes
+    w = ctypes.c_void_p()
+    # wrong byte count, k not a multiple of the block, unknown dtype
+    assert L.turq_weight_upload(ctx, Q4_K, n, k, capi.ptr(raw), raw.size - 1, 0, ctypes.byref(w)) == capi.ERR_SHAPE
+    assert "bytes" in capi.last_error(ctx)
+    assert L.turq_weight_upload(ctx, Q4_K, n, 100, capi.ptr(raw), raw.size, 0, ctypes.byref(w)) == capi.ERR_SHAPE
+    assert L.turq_weight_upload(ctx, 99, n, k, capi.ptr(raw), raw.size, 0, ctypes.byref(w)) == capi.ERR_DTYPE
+    w = gpu.upload(Q4_K, n, k, raw, capi.LAYOUT_TILED)
+    x = np.zeros((2, k), np.float32)
+    y = np.zeros((2, n), np.float32)
+    call = lambda **kw: L.turq_qmatmul(ctx, w, capi.ptr(x), kw.get("xt", 0), kw.get("m", 2), kw.get("ldx", k), capi.ptr(y),
+                                       kw.get("yt", 0), kw.get("ldy", n), None, kw.get("mem", 0), kw.get("algo", 0))
+    assert call(ldx=k - 1) == capi.ERR_SHAPE            # last dim != k
+    assert call(ldy=n - 1) == capi.ERR_SHAPE
+    assert call(m=-1) == capi.ERR_SHAPE
+    assert call(xt=7) == capi.ERR_DTYPE
+    assert call(algo=capi.ALGO_SIMPLE) == capi.ERR_INVALID   # plain kernel needs the native layout
+    assert call(m=0) == capi.OK                          # empty batch is a no-op
+    assert call() == capi.OK
+    gpu.release(w)

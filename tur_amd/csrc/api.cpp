@@ -1,0 +1,392 @@
+// C ABI of libturq: contexts, device memory helpers, weight upload/export, dequantize, forward.
+#include <memory>
+#include <new>
+#include <vector>
+
+#include "common.h"
+
+std::string &turq_thread_error() {
+    static thread_local std::string e;
+    return e;
+}
+
+int turq_ctx_reserve(turq_ctx *ctx, void **buf, size_t *cap, size_t need) {
+    if (need <= *cap) return TURQ_OK;
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));  // the old buffer may still be in use
+    if (*buf) {
+        TURQ_HIP(ctx, hipFree(*buf));
+        *buf = nullptr;
+        *cap = 0;
+    }
+    size_t want = need + need / 4 + 4096;
+    TURQ_HIP(ctx, hipMalloc(buf, want));
+    *cap = want;
+    return TURQ_OK;
+}
+
+namespace {
+
+struct DeviceGuard {  // make ctx's device current for the duration of a call
+    int prev = -1;
+    bool ok = true;
+    explicit DeviceGuard(int dev) {
+        if (hipGetDevice(&prev) != hipSuccess) prev = -1;
+        if (prev != dev) ok = hipSetDevice(dev) == hipSuccess;
+    }
+    ~DeviceGuard() {
+        int cur = -1;
+        if (prev >= 0 && hipGetDevice(&cur) == hipSuccess && cur != prev) (void)hipSetDevice(prev);
+    }
+};
+
+#define TURQ_ENTER(ctx)                                                                     \
+    if (!(ctx)) return turq_fail(nullptr, TURQ_ERR_INVALID, "%s: null context", __func__); \
+    DeviceGuard guard_((ctx)->device);                                                      \
+    if (!guard_.ok) return turq_fail((ctx), TURQ_ERR_HIP, "%s: hipSetDevice(%d) failed", __func__, (ctx)->device)
+
+}  // namespace
+
+extern "C" {
+
+const char *turq_version(void) { return "turq 0.1 (gfx950)"; }
+int turq_block_elems(int dt) { return turq_dt_block_elems(dt); }
+int turq_block_bytes(int dt) { return turq_dt_block_bytes(dt); }
+
+size_t turq_weight_nbytes(int dt, int64_t n, int64_t k) {
+    const int be = turq_dt_block_elems(dt);
+    if (be == 0 || n < 0 || k < 0 || k % be) return 0;
+    return (size_t)n * (size_t)(k / be) * (size_t)turq_dt_block_bytes(dt);
+}
+
+int turq_ctx_create(int device, turq_ctx **out) {
+    if (!out) return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_ctx_create: null out pointer");
+    *out = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess) return turq_fail(nullptr, TURQ_ERR_HIP, "hipGetDeviceCount failed: %s", hipGetErrorString(e));
+    if (device < 0 || device >= count)
+        return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_ctx_create: device %d out of range (%d visible)", device, count);
+    std::unique_ptr<turq_ctx> ctx(new (std::nothrow) turq_ctx);
+    if (!ctx) return turq_fail(nullptr, TURQ_ERR_OOM, "turq_ctx_create: out of host memory");
+    ctx->device = device;
+    DeviceGuard guard(device);
+    if (!guard.ok) return turq_fail(nullptr, TURQ_ERR_HIP, "turq_ctx_create: hipSetDevice(%d) failed", device);
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return turq_fail(nullptr, TURQ_ERR_HIP, "hipGetDeviceProperties failed: %s", hipGetErrorString(e));
+    ctx->compute_units = prop.multiProcessorCount;
+    snprintf(ctx->device_name, sizeof ctx->device_name, "%s (%s)", prop.name, prop.gcnArchName);
+    e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) return turq_fail(nullptr, TURQ_ERR_HIP, "hipStreamCreate failed: %s", hipGetErrorString(e));
+    *out = ctx.release();
+    return TURQ_OK;
+}
+
+void turq_ctx_destroy(turq_ctx *ctx) {
+    if (!ctx) return;
+    DeviceGuard guard(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->stage_x) (void)hipFree(ctx->stage_x);
+    if (ctx->stage_y) (void)hipFree(ctx->stage_y);
+    if (ctx->act_prep) (void)hipFree(ctx->act_prep);
+    if (ctx->stage_b) (void)hipFree(ctx->stage_b);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+}
+
+const char *turq_last_error(const turq_ctx *ctx) { return ctx ? ctx->err.c_str() : turq_thread_error().c_str(); }
+
+int turq_sync(turq_ctx *ctx) {
+    TURQ_ENTER(ctx);
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return TURQ_OK;
+}
+
+void *turq_ctx_stream(turq_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+int turq_ctx_device_info(turq_ctx *ctx, char *name, size_t cap, int *cus) {
+    if (!ctx) return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_ctx_device_info: null context");
+    if (name && cap) snprintf(name, cap, "%s", ctx->device_name);
+    if (cus) *cus = ctx->compute_units;
+    return TURQ_OK;
+}
+
+int turq_dev_alloc(turq_ctx *ctx, size_t nbytes, void **out) {
+    TURQ_ENTER(ctx);
+    if (!out) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_dev_alloc: null out pointer");
+    *out = nullptr;
+    if (nbytes == 0) return TURQ_OK;
+    TURQ_HIP(ctx, hipMalloc(out, nbytes));
+    return TURQ_OK;
+}
+
+int turq_dev_free(turq_ctx *ctx, void *ptr) {
+    TURQ_ENTER(ctx);
+    if (!ptr) return TURQ_OK;
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    TURQ_HIP(ctx, hipFree(ptr));
+    return TURQ_OK;
+}
+
+int turq_memcpy_h2d(turq_ctx *ctx, void *dst, const void *src, size_t nbytes) {
+    TURQ_ENTER(ctx);
+    if (nbytes == 0) return TURQ_OK;
+    if (!dst || !src) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_memcpy_h2d: null pointer");
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    TURQ_HIP(ctx, hipMemcpy(dst, src, nbytes, hipMemcpyHostToDevice));
+    return TURQ_OK;
+}
+
+int turq_memcpy_d2h(turq_ctx *ctx, void *dst, const void *src, size_t nbytes) {
+    TURQ_ENTER(ctx);
+    if (nbytes == 0) return TURQ_OK;
+    if (!dst || !src) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_memcpy_d2h: null pointer");
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    TURQ_HIP(ctx, hipMemcpy(dst, src, nbytes, hipMemcpyDeviceToHost));
+    return TURQ_OK;
+}
+
+// ---- weights ----
+
+int turq_weight_upload(turq_ctx *ctx, int dt, int64_t n, int64_t k, const void *host_bytes, size_t nbytes,
+                       int layout, turq_weight **out) {
+    TURQ_ENTER(ctx);
+    if (!out) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_weight_upload: null out pointer");
+    *out = nullptr;
+    const int be = turq_dt_block_elems(dt);
+    if (be == 0) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_weight_upload: unsupported ggml dtype %d", dt);
+    if (n < 0 || k < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_weight_upload: negative shape (%lld, %lld)", (long long)n, (long long)k);
+    if (k % be)
+        return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_weight_upload: k=%lld is not a multiple of the %s block size %d",
+                         (long long)k, turq_dt_name(dt), be);
+    const size_t expect = turq_weight_nbytes(dt, n, k);
+    if (nbytes != expect)
+        return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_weight_upload: got %zu bytes, a %s tensor of shape (%lld, %lld) has %zu",
+                         nbytes, turq_dt_name(dt), (long long)n, (long long)k, expect);
+    if (!host_bytes && nbytes) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_weight_upload: null data pointer");
+    if (layout != TURQ_LAYOUT_NATIVE && layout != TURQ_LAYOUT_TILED)
+        return turq_fail(ctx, TURQ_ERR_INVALID, "turq_weight_upload: unknown layout %d", layout);
+    if (layout == TURQ_LAYOUT_TILED && !turq_dt_is_quant(dt))
+        return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_weight_upload: the tiled layout holds quantized dtypes only, got %s", turq_dt_name(dt));
+
+    std::unique_ptr<turq_weight> w(new (std::nothrow) turq_weight);
+    if (!w) return turq_fail(ctx, TURQ_ERR_OOM, "turq_weight_upload: out of host memory");
+    w->device = ctx->device;
+    w->dtype = dt;
+    w->layout = layout;
+    w->n = n;
+    w->k = k;
+    w->native_bytes = nbytes;
+    const uint8_t *src = (const uint8_t *)host_bytes;
+    std::vector<uint8_t> tiled;
+    if (layout == TURQ_LAYOUT_TILED) {
+        w->dev_bytes = turq_tiled_nbytes(dt, n, k);
+        try {
+            tiled.resize(w->dev_bytes);
+        } catch (const std::bad_alloc &) {
+            return turq_fail(ctx, TURQ_ERR_OOM, "turq_weight_upload: out of host memory for the tiled copy (%zu bytes)", w->dev_bytes);
+        }
+        int rc = turq_tile_host(dt, n, k, host_bytes, tiled.data());
+        if (rc != TURQ_OK) return turq_fail(ctx, rc, "%s", turq_thread_error().c_str());
+        src = tiled.data();
+    } else {
+        w->dev_bytes = nbytes;
+    }
+    if (w->dev_bytes) {
+        // a few bytes of slack so that vector loads at the tail of the last row stay in bounds
+        TURQ_HIP(ctx, hipMalloc(&w->dev, w->dev_bytes + 64));
+        hipError_t e = hipMemcpy(w->dev, src, w->dev_bytes, hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = hipMemset((uint8_t *)w->dev + w->dev_bytes, 0, 64);
+        if (e != hipSuccess) {
+            (void)hipFree(w->dev);
+            return turq_fail(ctx, TURQ_ERR_HIP, "turq_weight_upload: copy to device failed: %s", hipGetErrorString(e));
+        }
+    }
+    *out = w.release();
+    return TURQ_OK;
+}
+
+int turq_weight_retain(turq_weight *w) {
+    if (!w) return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_weight_retain: null weight");
+    w->refs.fetch_add(1, std::memory_order_relaxed);
+    return TURQ_OK;
+}
+
+int turq_weight_release(turq_weight *w) {
+    if (!w) return TURQ_OK;
+    if (w->refs.fetch_sub(1, std::memory_order_acq_rel) == 1) {
+        if (w->dev) {
+            DeviceGuard guard(w->device);
+            (void)hipDeviceSynchronize();
+            (void)hipFree(w->dev);
+        }
+        delete w;
+    }
+    return TURQ_OK;
+}
+
+int turq_weight_info(const turq_weight *w, int *dt, int64_t *n, int64_t *k, int *layout, size_t *device_bytes) {
+    if (!w) return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_weight_info: null weight");
+    if (dt) *dt = w->dtype;
+    if (n) *n = w->n;
+    if (k) *k = w->k;
+    if (layout) *layout = w->layout;
+    if (device_bytes) *device_bytes = w->dev_bytes;
+    return TURQ_OK;
+}
+
+int turq_weight_export(turq_ctx *ctx, const turq_weight *w, void *host_bytes, size_t nbytes) {
+    TURQ_ENTER(ctx);
+    if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_weight_export: null weight");
+    if (nbytes != w->native_bytes)
+        return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_weight_export: buffer has %zu bytes, tensor has %zu", nbytes, w->native_bytes);
+    if (nbytes == 0) return TURQ_OK;
+    if (!host_bytes) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_weight_export: null buffer");
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (w->layout == TURQ_LAYOUT_NATIVE) {
+        TURQ_HIP(ctx, hipMemcpy(host_bytes, w->dev, nbytes, hipMemcpyDeviceToHost));
+        return TURQ_OK;
+    }
+    std::vector<uint8_t> tiled;
+    try {
+        tiled.resize(w->dev_bytes);
+    } catch (const std::bad_alloc &) {
+        return turq_fail(ctx, TURQ_ERR_OOM, "turq_weight_export: out of host memory");
+    }
+    TURQ_HIP(ctx, hipMemcpy(tiled.data(), w->dev, w->dev_bytes, hipMemcpyDeviceToHost));
+    int rc = turq_untile_host(w->dtype, w->n, w->k, tiled.data(), host_bytes);
+    if (rc != TURQ_OK) return turq_fail(ctx, rc, "%s", turq_thread_error().c_str());
+    return TURQ_OK;
+}
+
+// ---- dequantize ----
+
+int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem) {
+    TURQ_ENTER(ctx);
+    if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_dequantize: null weight");
+    if (w->device != ctx->device) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_dequantize: weight lives on device %d, context on %d", w->device, ctx->device);
+    const size_t nelem = (size_t)w->n * (size_t)w->k;
+    if (nelem == 0) return TURQ_OK;
+    if (!out) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_dequantize: null output");
+    if (!turq_dt_is_quant(w->dtype) && w->dtype != TURQ_F32 && w->dtype != TURQ_F16 && w->dtype != TURQ_BF16)
+        return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_dequantize: unsupported dtype %d", w->dtype);
+    if (out_mem == TURQ_MEM_DEVICE) {
+        TURQ_HIP(ctx, turq_launch_dequant(w->dtype, w->layout, w->dev, w->n, w->k, out, ctx->stream));
+        return TURQ_OK;
+    }
+    if (out_mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_dequantize: bad out_mem %d", out_mem);
+    int rc = turq_ctx_reserve(ctx, &ctx->stage_y, &ctx->stage_y_cap, nelem * sizeof(float));
+    if (rc != TURQ_OK) return rc;
+    TURQ_HIP(ctx, turq_launch_dequant(w->dtype, w->layout, w->dev, w->n, w->k, (float *)ctx->stage_y, ctx->stream));
+    TURQ_HIP(ctx, hipMemcpyAsync(out, ctx->stage_y, nelem * sizeof(float), hipMemcpyDeviceToHost, ctx->stream));
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return TURQ_OK;
+}
+
+// ---- forward ----
+
+static int qmatmul_device(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
+                          int yt, int64_t ldy, const float *bias, int algo) {
+    if (algo == TURQ_ALGO_AUTO) {
+        if (w->layout == TURQ_LAYOUT_NATIVE) algo = TURQ_ALGO_SIMPLE;
+        else algo = (m <= TURQ_GEMV_MAX_M) ? TURQ_ALGO_GEMV : TURQ_ALGO_GEMM;
+    }
+    switch (algo) {
+    case TURQ_ALGO_SIMPLE:
+        if (w->layout != TURQ_LAYOUT_NATIVE)
+            return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: TURQ_ALGO_SIMPLE needs a weight in the native layout");
+        TURQ_HIP(ctx, turq_launch_gemv_simple(w->dtype, w->dev, w->n, w->k, x, xt, m, ldx, y, yt, ldy, bias, ctx->stream));
+        return TURQ_OK;
+    case TURQ_ALGO_GEMV:
+    case TURQ_ALGO_GEMM:
+        if (w->layout != TURQ_LAYOUT_TILED)
+            return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: the MFMA kernels need a weight in the tiled layout");
+        return turq_qmatmul_mfma(ctx, w, x, xt, m, ldx, y, yt, ldy, bias, algo);
+    default:
+        return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: unknown algo %d", algo);
+    }
+}
+
+int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y, int yt,
+                 int64_t ldy, const float *bias, int mem, int algo) {
+    TURQ_ENTER(ctx);
+    if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: null weight");
+    if (w->device != ctx->device) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: weight lives on device %d, context on %d", w->device, ctx->device);
+    if (!turq_dt_is_quant(w->dtype))
+        return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: weight dtype %s is not block-quantized (dequantize it and use a dense matmul)", turq_dt_name(w->dtype));
+    const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
+    if (!xb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: unsupported activation dtype %d", xt);
+    if (!yb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: unsupported output dtype %d", yt);
+    if (m < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul: m=%lld is negative", (long long)m);
+    if (ldx < w->k) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul: ldx=%lld is smaller than k=%lld", (long long)ldx, (long long)w->k);
+    if (ldy < w->n) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul: ldy=%lld is smaller than n=%lld", (long long)ldy, (long long)w->n);
+    if (m == 0 || w->n == 0) return TURQ_OK;
+    if (!x || !y) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: null activation or output pointer");
+    if (w->k == 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul: k=0");
+
+    if (mem == TURQ_MEM_DEVICE) return qmatmul_device(ctx, w, x, xt, m, ldx, y, yt, ldy, bias, algo);
+    if (mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: bad mem %d", mem);
+
+    // host pointers: stage rows densely (ld = k / n on the device side), run, copy back
+    const size_t xrow = (size_t)w->k * xb, yrow = (size_t)w->n * yb;
+    int rc = turq_ctx_reserve(ctx, &ctx->stage_x, &ctx->stage_x_cap, xrow * (size_t)m);
+    if (rc != TURQ_OK) return rc;
+    rc = turq_ctx_reserve(ctx, &ctx->stage_y, &ctx->stage_y_cap, yrow * (size_t)m);
+    if (rc != TURQ_OK) return rc;
+    TURQ_HIP(ctx, hipMemcpy2DAsync(ctx->stage_x, xrow, x, (size_t)ldx * xb, xrow, (size_t)m, hipMemcpyHostToDevice, ctx->stream));
+    if (bias) {  // with host pointers the bias is a host array too
+        rc = turq_ctx_reserve(ctx, &ctx->stage_b, &ctx->stage_b_cap, (size_t)w->n * sizeof(float));
+        if (rc != TURQ_OK) return rc;
+        TURQ_HIP(ctx, hipMemcpyAsync(ctx->stage_b, bias, (size_t)w->n * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+        bias = (const float *)ctx->stage_b;
+    }
+    rc = qmatmul_device(ctx, w, ctx->stage_x, xt, m, w->k, ctx->stage_y, yt, w->n, bias, algo);
+    if (rc != TURQ_OK) return rc;
+    TURQ_HIP(ctx, hipMemcpy2DAsync(y, (size_t)ldy * yb, ctx->stage_y, yrow, yrow, (size_t)m, hipMemcpyDeviceToHost, ctx->stream));
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return TURQ_OK;
+}
+
+// ---- activation quantisation ----
+
+static int quantize_common(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem, bool q8k) {
+    const int be = q8k ? 256 : 32, bb = q8k ? 292 : 34;
+    if (m < 0 || k < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_quantize: negative shape");
+    if (k % be) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_quantize: k=%lld is not a multiple of %d", (long long)k, be);
+    const int64_t nblocks = m * (k / be);
+    if (nblocks == 0) return TURQ_OK;
+    if (!x || !out) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_quantize: null pointer");
+    const size_t in_bytes = (size_t)m * (size_t)k * 4, out_bytes = (size_t)nblocks * bb;
+    const float *dx = x;
+    void *dout = out;
+    if (mem == TURQ_MEM_HOST) {
+        int rc = turq_ctx_reserve(ctx, &ctx->stage_x, &ctx->stage_x_cap, in_bytes);
+        if (rc != TURQ_OK) return rc;
+        rc = turq_ctx_reserve(ctx, &ctx->stage_y, &ctx->stage_y_cap, out_bytes);
+        if (rc != TURQ_OK) return rc;
+        TURQ_HIP(ctx, hipMemcpyAsync(ctx->stage_x, x, in_bytes, hipMemcpyHostToDevice, ctx->stream));
+        dx = (const float *)ctx->stage_x;
+        dout = ctx->stage_y;
+    } else if (mem != TURQ_MEM_DEVICE) {
+        return turq_fail(ctx, TURQ_ERR_INVALID, "turq_quantize: bad mem %d", mem);
+    }
+    if (q8k) TURQ_HIP(ctx, turq_launch_quantize_q8_k(dx, nblocks, dout, ctx->stream));
+    else TURQ_HIP(ctx, turq_launch_quantize_q8_0(dx, nblocks, dout, ctx->stream));
+    if (mem == TURQ_MEM_HOST) {
+        TURQ_HIP(ctx, hipMemcpyAsync(out, dout, out_bytes, hipMemcpyDeviceToHost, ctx->stream));
+        TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    }
+    return TURQ_OK;
+}
+
+int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
+    TURQ_ENTER(ctx);
+    return quantize_common(ctx, x, m, k, out, mem, false);
+}
+
+int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
+    TURQ_ENTER(ctx);
+    return quantize_common(ctx, x, m, k, out, mem, true);
+}
+
+}  // extern "C"

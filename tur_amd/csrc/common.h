@@ -1,0 +1,124 @@
+// Internal definitions shared by the translation units of libturq (not part of the C ABI).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "../../include/turq.h"
+
+#define TURQ_QK_K 256
+#define TURQ_QK8_0 32
+
+// ---- dtype geometry (ggml block layouts) ----
+__host__ __device__ inline int turq_dt_block_elems(int dt) {
+    switch (dt) {
+    case TURQ_F32: case TURQ_F16: case TURQ_BF16: return 1;
+    case TURQ_Q8_0: return 32;
+    case TURQ_Q4_K: case TURQ_Q5_K: case TURQ_Q6_K: return 256;
+    default: return 0;
+    }
+}
+__host__ __device__ inline int turq_dt_block_bytes(int dt) {
+    switch (dt) {
+    case TURQ_F32: return 4;
+    case TURQ_F16: case TURQ_BF16: return 2;
+    case TURQ_Q8_0: return 34;
+    case TURQ_Q4_K: return 144;
+    case TURQ_Q5_K: return 176;
+    case TURQ_Q6_K: return 210;
+    default: return 0;
+    }
+}
+inline const char *turq_dt_name(int dt) {
+    switch (dt) {
+    case TURQ_F32: return "F32";
+    case TURQ_F16: return "F16";
+    case TURQ_BF16: return "BF16";
+    case TURQ_Q8_0: return "Q8_0";
+    case TURQ_Q4_K: return "Q4_K";
+    case TURQ_Q5_K: return "Q5_K";
+    case TURQ_Q6_K: return "Q6_K";
+    default: return "?";
+    }
+}
+inline bool turq_dt_is_quant(int dt) {
+    return dt == TURQ_Q8_0 || dt == TURQ_Q4_K || dt == TURQ_Q5_K || dt == TURQ_Q6_K;
+}
+inline int turq_act_bytes(int act) {
+    switch (act) {
+    case TURQ_ACT_F32: return 4;
+    case TURQ_ACT_BF16: case TURQ_ACT_F16: return 2;
+    default: return 0;
+    }
+}
+
+// ---- objects behind the opaque handles ----
+struct turq_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    int compute_units = 0;
+    char device_name[128] = {0};
+    std::string err;
+    // growable device scratch: host staging for TURQ_MEM_HOST calls and prepared activations
+    void *stage_x = nullptr;  size_t stage_x_cap = 0;
+    void *stage_y = nullptr;  size_t stage_y_cap = 0;
+    void *stage_b = nullptr;  size_t stage_b_cap = 0;
+    void *act_prep = nullptr; size_t act_prep_cap = 0;
+};
+
+struct turq_weight {
+    std::atomic<int> refs{1};
+    int device = 0;
+    int dtype = 0;
+    int layout = TURQ_LAYOUT_NATIVE;
+    int64_t n = 0, k = 0;
+    void *dev = nullptr;      // weight bytes in HBM (native or tiled)
+    size_t dev_bytes = 0;     // allocation size
+    size_t native_bytes = 0;  // n * k / blk * block_bytes
+};
+
+// ---- error plumbing ----
+std::string &turq_thread_error();  // last error of calls without a context
+
+inline int turq_fail(turq_ctx *ctx, int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (ctx) ctx->err = buf; else turq_thread_error() = buf;
+    return code;
+}
+
+#define TURQ_HIP(ctx, call)                                                                      \
+    do {                                                                                         \
+        hipError_t e_ = (call);                                                                  \
+        if (e_ != hipSuccess)                                                                    \
+            return turq_fail((ctx), e_ == hipErrorOutOfMemory ? TURQ_ERR_OOM : TURQ_ERR_HIP,     \
+                             "%s failed: %s", #call, hipGetErrorString(e_));                     \
+    } while (0)
+
+// grow-only scratch on the context's device
+int turq_ctx_reserve(turq_ctx *ctx, void **buf, size_t *cap, size_t need);
+
+// ---- kernel launchers implemented in the .hip translation units ----
+// All are asynchronous on `stream` and return hipGetLastError() of the launch.
+hipError_t turq_launch_dequant(int dtype, int layout, const void *w, int64_t n, int64_t k, float *out,
+                               hipStream_t stream);
+hipError_t turq_launch_quantize_q8_0(const float *x, int64_t nblocks, void *out, hipStream_t stream);
+hipError_t turq_launch_quantize_q8_k(const float *x, int64_t nblocks, void *out, hipStream_t stream);
+hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t k, const void *x, int x_dtype,
+                                   int64_t m, int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias,
+                                   hipStream_t stream);
+
+// largest m the skinny MFMA kernel takes; above it the LDS-tiled GEMM runs
+#define TURQ_GEMV_MAX_M 32
+// MFMA paths on the tiled layout (activation preparation + kernel launch), see mfma_dispatch.cpp
+int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
+                      int yt, int64_t ldy, const float *bias, int algo);

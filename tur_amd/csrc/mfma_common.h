@@ -1,0 +1,95 @@
+// Device helpers shared by the MFMA kernels: vector types, the "magic number" integer -> f16
+// unpack, and the layout of prepared activations.
+//
+// Integer -> f16 without a convert instruction.  OR-ing a small unsigned field into the mantissa of
+// a fixed f16 exponent gives base + field * ulp exactly:
+//   bits 0x6400 | v        = 1024 + v          (v < 1024, ulp 1)
+//   bits 0x6400 | (v << 4) = 1024 + 16 * v
+//   bits 0x5C00 | (v << 2) = 256 + v           (ulp 1/4)
+//   bits 0x4C00 | (v << 6) = 16 + v            (ulp 1/64)
+// One v_and_or_b32 therefore turns two fields of a packed dword (one per 16-bit half) into a packed
+// f16 pair, and one v_pk_fma_f16 with (scale, -base * scale) removes the base and applies an integer
+// block scale at the same time.  All products here are integers below 2048, so every value that
+// reaches the MFMA is exact; the only rounding on the weight side is none at all.
+//
+// Prepared activations ("A fragments").  The kernels use v_mfma_f32_16x16x32_f16 with the
+// activations as the A operand (16 rows of m) and the weights as the B operand (16 rows of n), so
+// lane (n, g) of the result holds y[m = 4g..4g+3][n].  For every 256-column tile b and MFMA step q
+// the activation fragment is stored lane-linear, 16 bytes (8 f16) per (g, r):
+//   chunk index = (((mt * ntc + b) * NQ + q) * 4 + g) * mpad + r          (mt = m / 16, r = m % 16)
+//   K-quants (NQ = 9): q < 8 holds x[m][256b + 64g + 8q + j];  q = 8 holds, for the four
+//     16-element groups of lane group g, the group sums of the f16-rounded activations split in
+//     two f16 (hi, lo): slots (hi0, lo0, hi1, lo1, hi2, lo2, hi3, lo3)
+//   Q8_0 (NQ = 8): q holds x[m][256b + 32q + 8g + j]
+// mpad is the m-tile height rounded up to 1, 2, 4, 8 or 16; rows beyond m are zero.
+#pragma once
+
+#include "common.h"
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+
+#define TURQ_NQ_KQUANT 9
+#define TURQ_NQ_Q8_0 8
+
+__host__ __device__ inline int turq_mpad(int64_t rows) {
+    return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : rows <= 8 ? 8 : 16;
+}
+__host__ __device__ inline int turq_nq(int dt) { return dt == TURQ_Q8_0 ? TURQ_NQ_Q8_0 : TURQ_NQ_KQUANT; }
+// bytes of the prepared-activation buffer for m rows against a weight of k columns
+__host__ __device__ inline size_t turq_act_prep_bytes(int dt, int64_t m, int64_t k) {
+    const int64_t mtiles = (m + 15) / 16;
+    const int mpad = mtiles > 1 ? 16 : turq_mpad(m);
+    return (size_t)mtiles * (size_t)((k + 255) / 256) * (size_t)turq_nq(dt) * 4u * (size_t)mpad * 16u;
+}
+
+#ifdef __HIPCC__
+__device__ inline half2v as_half2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
+__device__ inline uint32_t as_u32(half2v h) { return __builtin_bit_cast(uint32_t, h); }
+
+// (w & mask) | magic as a packed f16 pair: one v_and_or_b32
+__device__ inline half2v and_or_h2(uint32_t w, uint32_t mask, uint32_t magic) { return as_half2((w & mask) | magic); }
+
+// fused multiply-add on a packed pair (v_pk_fma_f16): must stay fused, the intermediate product
+// (base + v) * scale does not fit f16 on its own
+__device__ inline half2v pk_fma(half2v a, half2v b, half2v c) { return __builtin_elementwise_fma(a, b, c); }
+
+__device__ inline half2v splat2(_Float16 v) { return half2v{v, v}; }
+
+__device__ inline half8v make_half8(half2v a, half2v b, half2v c, half2v d) {
+    return half8v{a.x, a.y, b.x, b.y, c.x, c.y, d.x, d.y};
+}
+
+__device__ inline float4v mfma16x16x32(half8v a, half8v b, float4v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+__device__ inline uint32_t rotr32(uint32_t v, uint32_t s) { return __builtin_amdgcn_alignbit(v, v, s); }
+
+__device__ inline uint16_t turq_f2bf(float f) {  // round to nearest even, NaN kept quiet
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+template <int YT> __device__ inline void turq_store_out(void *y, int64_t i, float v) {
+    if (YT == TURQ_ACT_F32) ((float *)y)[i] = v;
+    else if (YT == TURQ_ACT_BF16) ((uint16_t *)y)[i] = turq_f2bf(v);
+    else {
+        const _Float16 h = (_Float16)v;
+        uint16_t b;
+        __builtin_memcpy(&b, &h, 2);
+        ((uint16_t *)y)[i] = b;
+    }
+}
+#endif
+
+// launchers (act_prep.hip, gemv_mfma.hip)
+hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
+                                hipStream_t stream);
+hipError_t turq_launch_gemv_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *frags, int64_t m,
+                                 void *y, int y_dtype, int64_t ldy, const float *bias, int waves_per_group,
+                                 hipStream_t stream);

@@ -1,0 +1,38 @@
+// Host side of the MFMA paths: prepare the activations, pick the launch shape, launch.
+#include <algorithm>
+
+#include "layout.h"
+#include "mfma_common.h"
+
+namespace {
+
+// Waves per workgroup (= how many ways a row tile's columns are split).  Enough waves to cover the
+// machine a few times over, never more than there are column tiles.
+int pick_waves(const turq_ctx *ctx, int64_t n, int64_t k) {
+    const int64_t row_tiles = turq_tile_rows(n);
+    const int64_t col_tiles = turq_tile_cols(k);
+    const int64_t want_waves = (int64_t)(ctx->compute_units > 0 ? ctx->compute_units : 256) * 12;
+    int64_t w = (want_waves + row_tiles - 1) / row_tiles;
+    w = std::max<int64_t>(1, std::min<int64_t>({w, col_tiles, 8}));
+    return (int)w;
+}
+
+}  // namespace
+
+int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
+                      int yt, int64_t ldy, const float *bias, int algo) {
+    (void)algo;
+    const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
+    const int nwaves = pick_waves(ctx, w->n, w->k);
+    for (int64_t m0 = 0; m0 < m; m0 += TURQ_GEMV_MAX_M) {
+        const int64_t mc = std::min<int64_t>(TURQ_GEMV_MAX_M, m - m0);
+        int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep_bytes(w->dtype, mc, w->k));
+        if (rc != TURQ_OK) return rc;
+        const uint8_t *xc = (const uint8_t *)x + (size_t)m0 * (size_t)ldx * xb;
+        uint8_t *yc = (uint8_t *)y + (size_t)m0 * (size_t)ldy * yb;
+        TURQ_HIP(ctx, turq_launch_act_prep(w->dtype, xc, xt, mc, w->k, ldx, ctx->act_prep, ctx->stream));
+        TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, mc, yc, yt, ldy, bias, nwaves,
+                                            ctx->stream));
+    }
+    return TURQ_OK;
+}
