@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the GGUF quantized-linear hot path on one MI355X.
+
+Default workload (the configuration the headline metric is quoted on): Q4_K decode GEMV at the
+Qwen3-8B MLP shapes — gate_proj and up_proj [12288 x 4096], down_proj [4096 x 12288] — at m = 1.
+One "step" is one decode pass over the MLPs of `--layers` decoder layers (default 36, the depth of
+Qwen3-8B): 3 * layers quantized matmuls, each on its OWN copy of the weights in HBM, so a step
+streams layers * 84.9 MB (3.06 GB by default) and nothing is served from the 256 MB Infinity
+Cache.  Inputs are resident in HBM when the clock starts; every matmul includes its activation
+preparation kernel.  The step is captured once into a HIP graph and replayed (one launch per step).
+
+Prints ONE JSON line.  `value` is whole-step algorithmic bytes (weights + activations + outputs)
+per second.  `roofline` prices the dominant kernel (the MFMA GEMV) alone: algorithmic bytes of one
+launch over its average duration, measured with HIP event pairs around every launch of it in a
+second, untimed pass of the same steps.  `cpu_baseline` times the oracle's restatement of candle's
+CPU QMatMul (quantise activations to Q8_K, integer dot products) on the host cores on one layer's
+three matmuls.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from tur_amd import capi, synth  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+WORKLOADS = {
+    # name: (description, [(label, ggml dtype, n, k), ...] per layer)
+    "q4k_mlp_8b": ("Q4_K GEMV, Qwen3-8B MLP (gate/up 12288x4096, down 4096x12288)", synth.CONFIGS["q4k_mlp_8b"]),
+    "q4km_layer_8b": ("Q4_K_M mixed decoder layer, Qwen3-8B (Q6_K v/down, Q4_K q/k/o/gate/up)", synth.CONFIGS["q4km_layer_8b"]),
+    "q8_0_gate_0p6b": ("Q8_0 GEMV, Qwen3-0.6B gate_proj 3072x1024", synth.CONFIGS["q8_0_gate_0p6b"]),
+    "lm_head_q6k_8b": ("LM head Q6_K 151936x4096", synth.CONFIGS["lm_head_q6k_8b"]),
+    "lm_head_q5k_8b": ("LM head Q5_K 151936x4096", synth.CONFIGS["lm_head_q5k_8b"]),
+}
+ACT = {"f32": (capi.ACT_F32, 4, np.float32), "bf16": (capi.ACT_BF16, 2, np.uint16)}
+
+
+def algorithmic_bytes(dt, n, k, m, xbytes, ybytes):
+    return synth.weight_nbytes(dt, n, k) + m * k * xbytes + m * n * ybytes
+
+
+class Bench:
+    def __init__(self, args):
+        self.args = args
+        self.L = capi.lib()
+        self.ctx = ctypes.c_void_p()
+        capi.check(self.L.turq_ctx_create(0, ctypes.byref(self.ctx)))
+        name = ctypes.create_string_buffer(128)
+        cus = ctypes.c_int()
+        capi.check(self.L.turq_ctx_device_info(self.ctx, name, 128, ctypes.byref(cus)), self.ctx)
+        self.device = name.value.decode()
+        self.cus = cus.value
+        self.desc, self.mats = WORKLOADS[args.workload]
+        self.m = args.m
+        self.xt, self.xbytes, self.xnp = ACT[args.act]
+        self.weights = []      # [layer][matrix] -> handle
+        self.host_raw = {}     # label -> raw bytes of the first layer (CPU baseline, checks)
+        self.calls = []        # (weight, x_dev, y_dev, n, k)
+        self._setup()
+
+    def dev_alloc(self, nbytes):
+        p = ctypes.c_void_p()
+        capi.check(self.L.turq_dev_alloc(self.ctx, nbytes, ctypes.byref(p)), self.ctx)
+        return p
+
+    def _setup(self):
+        L, ctx = self.L, self.ctx
+        layers = self.args.layers
+        per_layer = sum(synth.weight_nbytes(dt, n, k) for _, dt, n, k in self.mats)
+        if per_layer * layers > 200e9:
+            raise SystemExit("workload does not fit: lower --layers")
+        # one set of seeded weights; every layer gets its own device copy (distinct HBM addresses)
+        raws = []
+        for i, (label, dt, n, k) in enumerate(self.mats):
+            raw = synth.random_weight(dt, n, k, seed=1000 + i)
+            raws.append(raw)
+            self.host_raw[label] = raw
+        for _ in range(layers):
+            row = []
+            for (label, dt, n, k), raw in zip(self.mats, raws):
+                w = ctypes.c_void_p()
+                capi.check(L.turq_weight_upload(ctx, dt, n, k, capi.ptr(raw), raw.size, capi.LAYOUT_TILED, ctypes.byref(w)), ctx)
+                row.append(w)
+            self.weights.append(row)
+        # activations: one resident input per distinct k, one output buffer per matrix
+        self.x_host = {}
+        self.x_dev = {}
+        for _, _, n, k in self.mats:
+            if k not in self.x_dev:
+                x = synth.random_activation(self.m, k, seed=k, bf16=(self.args.act == "bf16"))
+                self.x_host[k] = x
+                send = synth.to_bf16_bits(x).reshape(self.m, k) if self.args.act == "bf16" else x
+                p = self.dev_alloc(send.nbytes)
+                capi.check(L.turq_memcpy_h2d(ctx, p, capi.ptr(send), send.nbytes), ctx)
+                self.x_dev[k] = p
+        self.y_dev = [self.dev_alloc(self.m * n * 4) for _, _, n, _ in self.mats]
+        for layer in self.weights:
+            for (label, dt, n, k), w, y in zip(self.mats, layer, self.y_dev):
+                self.calls.append((w, self.x_dev[k], y, n, k))
+        self.step_bytes = layers * sum(algorithmic_bytes(dt, n, k, self.m, self.xbytes, 4) for _, dt, n, k in self.mats)
+        self.step_flops = layers * sum(2 * self.m * n * k for _, _, n, k in self.mats)
+
+    def step_eager(self):
+        L, ctx, m, xt = self.L, self.ctx, self.m, self.xt
+        for w, x, y, n, k in self.calls:
+            rc = L.turq_qmatmul(ctx, w, x, xt, m, k, y, capi.ACT_F32, n, None, capi.MEM_DEVICE, capi.ALGO_AUTO)
+            if rc:
+                capi.check(rc, ctx)
+
+    def sync(self):
+        capi.check(self.L.turq_sync(self.ctx), self.ctx)
+
+    def verify(self):
+        """first layer's outputs against the oracle (small m only; it is a sanity gate, not the parity suite)"""
+        from oracle import capi as orc
+        self.step_eager()
+        self.sync()
+        worst = 0.0
+        for (label, dt, n, k), y in zip(self.mats, self.y_dev):
+            if n * k * self.m > 2e9:
+                continue
+            got = np.empty((self.m, n), np.float32)
+            capi.check(self.L.turq_memcpy_d2h(self.ctx, capi.ptr(got), y, got.nbytes), self.ctx)
+            want = orc.matmul_dequant(dt, self.x_host[k], self.host_raw[label], n, k)
+            rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+            worst = max(worst, rel)
+        if worst > 1e-3:
+            raise SystemExit(f"bench: output differs from the oracle (rel-L2 {worst:.3e} > 1e-3)")
+        return worst
+
+    def run(self):
+        a = self.args
+        L, ctx = self.L, self.ctx
+        rel = self.verify()
+        graph = None
+        if not a.eager:
+            capi.check(L.turq_graph_begin(ctx), ctx)
+            self.step_eager()
+            g = ctypes.c_void_p()
+            capi.check(L.turq_graph_end(ctx, ctypes.byref(g)), ctx)
+            graph = g
+        one = (lambda: capi.check(L.turq_graph_launch(ctx, graph), ctx)) if graph else self.step_eager
+        for _ in range(a.warmup):
+            one()
+        self.sync()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            one()
+        self.sync()
+        dt_s = time.perf_counter() - t0
+        ms_per_step = dt_s / a.steps * 1e3
+        gbps = self.step_bytes / (dt_s / a.steps) / 1e9
+
+        # dominant kernel alone: event pairs around every matmul kernel launch, same steps, untimed pass
+        capi.check(L.turq_profile_begin(ctx), ctx)
+        prof_steps = max(1, min(a.steps, 10))
+        for _ in range(prof_steps):
+            self.step_eager()
+        n_launch = ctypes.c_int64()
+        tot_ms = ctypes.c_double()
+        capi.check(L.turq_profile_end(ctx, ctypes.byref(n_launch), ctypes.byref(tot_ms)), ctx)
+        avg_us = tot_ms.value / max(1, n_launch.value) * 1e3
+        bytes_per_launch = self.step_bytes / len(self.calls)
+        achieved = bytes_per_launch / (avg_us * 1e-6) / 1e9
+        if graph:
+            L.turq_graph_destroy(graph)
+        roofline = {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+            "kernel": "gemv_mfma_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
+            "algorithmic_bytes_per_launch": int(bytes_per_launch),
+        }
+        out = {
+            "metric": "quantized GEMV HBM GB/s (Q4_K/Q6_K, Qwen3-8B shapes)",
+            "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+            "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": f"{a.workload}: {self.desc}", "m": self.m, "layers": a.layers,
+                       "activations": a.act, "launch": "eager" if a.eager else "hip-graph",
+                       "step_bytes": int(self.step_bytes), "device": self.device, "compute_units": self.cus,
+                       "max_rel_l2_vs_oracle": float(f"{rel:.3e}")},
+            "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
+            "roofline": roofline,
+            "cpu_baseline": self.cpu_baseline() if not a.no_cpu else None,
+        }
+        print(json.dumps(out), flush=True)
+
+    def calibrate_copy(self, nelem=64 * 1024 * 1024):
+        L, ctx = self.L, self.ctx
+        src = np.zeros(nelem, np.float32)
+        w = ctypes.c_void_p()
+        capi.check(L.turq_weight_upload(ctx, capi.F32, 1, nelem, capi.ptr(src), src.nbytes, capi.LAYOUT_NATIVE, ctypes.byref(w)), ctx)
+        dst = self.dev_alloc(src.nbytes)
+        for _ in range(3):
+            capi.check(L.turq_dequantize(ctx, w, dst, capi.MEM_DEVICE), ctx)
+        self.sync()
+        capi.check(L.turq_dev_free(ctx, dst), ctx)
+        capi.check(L.turq_weight_release(w))
+
+    def cpu_baseline(self):
+        """restated candle CPU QMatMul (quantise activations, integer vec_dot) on one layer's matmuls"""
+        from oracle import capi as orc
+        cores = min(os.cpu_count() or 1, 16)
+        layer_bytes = sum(algorithmic_bytes(dt, n, k, self.m, 4, 4) for _, dt, n, k in self.mats)
+        budget_s = 12.0
+        reps, t_used = 0, 0.0
+        while t_used < budget_s:
+            t0 = time.perf_counter()
+            for label, dt, n, k in self.mats:
+                orc.qmatmul(dt, self.x_host[k], self.host_raw[label], n, k, nthreads=cores)
+            t_used += time.perf_counter() - t0
+            reps += 1
+        return {"value": round(layer_bytes * reps / t_used / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": f"{reps} passes over one layer's matmuls ({len(self.mats)} calls, m={self.m}) in {t_used:.1f} s; "
+                          "restated candle CPU QMatMul (not candle itself), gcc -O3 scalar vec_dot, OpenMP over output columns"}
+
+    def close(self):
+        for layer in self.weights:
+            for w in layer:
+                self.L.turq_weight_release(w)
+        self.L.turq_ctx_destroy(self.ctx)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="q4k_mlp_8b", choices=sorted(WORKLOADS))
+    ap.add_argument("--m", type=int, default=1, help="activation rows (decode batch)")
+    ap.add_argument("--layers", type=int, default=None, help="distinct weight copies streamed per step")
+    ap.add_argument("--act", default="f32", choices=sorted(ACT))
+    ap.add_argument("--eager", action="store_true", help="launch every call from the host instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="before the workload, run a plain copy kernel of known size (dequantize of an F32 tensor: 256 MiB "
+                         "read + 256 MiB written) three times, as the yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.layers is None:
+        # enough distinct weight copies that a step streams well over the 256 MB Infinity Cache
+        per_layer = sum(synth.weight_nbytes(dt, n, k) for _, dt, n, k in WORKLOADS[args.workload][1])
+        args.layers = max(36 if per_layer < 200e6 else 2, -(-768_000_000 // per_layer))
+    b = Bench(args)
+    try:
+        if args.calibrate_copy:
+            b.calibrate_copy()
+        b.run()
+    finally:
+        b.close()
+
+
+if __name__ == "__main__":
+    main()

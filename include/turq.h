@@ -27,6 +27,7 @@ extern "C" {
 typedef struct turq_ctx turq_ctx;       /* device + stream + scratch, one per engine thread */
 typedef struct turq_weight turq_weight; /* one quantized [n, k] tensor resident in HBM */
 typedef struct turq_gguf turq_gguf;     /* an opened GGUF file (header parsed, tensors lazy) */
+typedef struct turq_graph turq_graph;   /* a captured sequence of forward calls (hipGraphExec) */
 
 /* status codes */
 enum {
@@ -156,6 +157,23 @@ int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype
  * `k_quants::matmul`. */
 int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem);
 int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem);
+
+/* ---- launch-overhead control and kernel timing (no counterpart in the reference, whose CPU path
+ * has no launches; a decode step here is hundreds of ~5 us kernels) ---- */
+/* Capture every TURQ_MEM_DEVICE forward call made on ctx between begin and end into a graph and
+ * replay it with one launch.  Run the same calls once eagerly first: scratch buffers must already
+ * have their final size, allocation is not allowed while capturing.  The captured calls keep
+ * referring to the same x / y / weight pointers. */
+int turq_graph_begin(turq_ctx *ctx);
+int turq_graph_end(turq_ctx *ctx, turq_graph **out);
+int turq_graph_launch(turq_ctx *ctx, turq_graph *g);
+void turq_graph_destroy(turq_graph *g);
+/* Between begin and end every MFMA matmul kernel (not the activation preparation) is launched
+ * with a pair of HIP events that the runtime stamps with the dispatch's own begin and end times;
+ * end waits for the stream and returns the number of timed launches and the sum of their
+ * execution times (launch gaps excluded). */
+int turq_profile_begin(turq_ctx *ctx);
+int turq_profile_end(turq_ctx *ctx, int64_t *launches, double *total_ms);
 
 /* ---- GGUF files ---- */
 /* Parse the header (magic, version 1..3, metadata, tensor infos, alignment).

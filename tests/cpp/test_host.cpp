@@ -1,0 +1,73 @@
+// Exercises the C++ host mirror (tur_amd/csrc/host/turq.hpp) against a GGUF file written by the
+// Python test that launches this program.  Usage: test_host FILE.gguf
+// Prints "name n k checksum" lines the Python side compares with the oracle; exits non-zero on error.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+#include "../../tur_amd/csrc/host/turq.hpp"
+
+static int fail(const char *what) {
+    std::fprintf(stderr, "FAIL: %s\n", what);
+    return 1;
+}
+
+int main(int argc, char **argv) {
+    if (argc < 2) return fail("usage: test_host FILE.gguf");
+    try {
+        turq::Device dev = turq::Device::new_hip(0);
+        turq::QVarBuilder vb = turq::QVarBuilder::from_gguf(argv[1], dev);
+        if (vb.all_keys().empty()) return fail("no tensors");
+        turq::QVarBuilder b0 = vb.pp("blk").pp(0);
+        if (b0.path("ffn_gate.weight") != "blk.0.ffn_gate.weight") return fail("path");
+        if (!b0.contains_key("ffn_gate.weight") || b0.contains_key("ffn_gate.bias")) return fail("contains_key");
+        auto shp = b0.tensor_shape("ffn_gate.weight");
+        if (!shp || shp->size() != 2) return fail("tensor_shape");
+        const int64_t n = (*shp)[0], k = (*shp)[1];
+        // shape mismatch must be an error with the reference's wording
+        bool threw = false;
+        try { b0.pp("ffn_gate").get({n + 1, k}, "weight"); } catch (const turq::Error &e) { threw = std::strstr(e.what(), "shape mismatch for weight") != nullptr; }
+        if (!threw) return fail("shape mismatch not reported");
+        threw = false;
+        try { b0.pp("nope").get({n, k}, "weight"); } catch (const turq::Error &e) { threw = e.code == TURQ_ERR_NOT_FOUND; }
+        if (!threw) return fail("missing tensor not reported");
+
+        turq::LinearX gate = turq::linear(k, n, b0.pp("ffn_gate"));
+        turq::LinearX biased = turq::linear(k, 96, b0.pp("biased"));
+        if (gate.bias() || !biased.bias() || biased.bias()->size() != 96) return fail("bias handling");
+        turq::LinearX copy = gate;  // Clone: shares the device weight
+
+        // x[i, j] = deterministic pattern the Python side reproduces
+        const int64_t m = 3;
+        std::vector<float> x((size_t)m * k);
+        for (int64_t i = 0; i < m; i++)
+            for (int64_t j = 0; j < k; j++) x[i * k + j] = std::sin(0.37f * (float)(i * k + j)) * 2.0f;
+        std::vector<float> y = copy.forward(x, m);
+        std::vector<float> yb = biased.forward(x, m);
+        if ((int64_t)y.size() != m * n || (int64_t)yb.size() != m * 96) return fail("output shape");
+        std::printf("gate %lld %lld\n", (long long)n, (long long)k);
+        for (float v : y) std::printf("%.9g\n", v);
+        std::printf("biased 96 %lld\n", (long long)k);
+        for (float v : yb) std::printf("%.9g\n", v);
+
+        // device-pointer forward (bf16 output) through QMatMul
+        turq::DeviceBuffer xd(dev, x.size() * 4), yd(dev, (size_t)m * n * 4);
+        xd.upload(x.data(), x.size() * 4);
+        copy.qmatmul().forward(xd.ptr(), TURQ_ACT_F32, m, k, yd.ptr(), TURQ_ACT_F32, n);
+        dev.synchronize();
+        std::vector<float> y2((size_t)m * n);
+        yd.download(y2.data(), y2.size() * 4);
+        for (size_t i = 0; i < y.size(); i++)
+            if (y[i] != y2[i]) return fail("host-pointer and device-pointer forward differ");
+
+        // dequantize of the norm weight (F32 tensor) is a copy
+        std::vector<float> norm = b0.pp("attn_norm").get({k}, "weight").dequantize();
+        std::printf("norm %zu %.9g %.9g\n", norm.size(), norm.front(), norm.back());
+        try { turq::QMatMul::from_arc(b0.pp("attn_norm").get({k}, "weight")); return fail("dense tensor accepted by QMatMul"); } catch (const turq::Error &) {}
+    } catch (const std::exception &e) {
+        std::fprintf(stderr, "FAIL: exception: %s\n", e.what());
+        return 1;
+    }
+    std::printf("OK\n");
+    return 0;
+}

@@ -1,0 +1,144 @@
+"""CPU-side checks of the C ABI: the library loads without a GPU, exports every symbol that
+include/turq.h declares, and the parts that need no device (geometry, GGUF reader, error plumbing)
+behave as the reference's interfaces do."""
+import ctypes
+import os
+import re
+import struct
+
+import numpy as np
+import pytest
+
+from tur_amd import capi, synth
+from tur_amd.gguf import write_gguf
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "turq.h")).read()
+    declared = set(re.findall(r"\b(turq_[a-z0-9_]+)\s*\(", header))
+    L = capi.lib()
+    missing = [s for s in sorted(declared) if not hasattr(L, s)]
+    assert not missing, missing
+    assert declared == set(capi.declared_symbols())      # the ctypes table binds exactly the header
+
+
+def test_geometry_entry_points():
+    L = capi.lib()
+    assert L.turq_version().startswith(b"turq")
+    assert [L.turq_block_bytes(d) for d in (Q8_0, Q4_K, Q5_K, Q6_K, 0, 1, 30, 99)] == [34, 144, 176, 210, 4, 2, 2, 0]
+    assert L.turq_weight_nbytes(Q4_K, 12288, 4096) == 28_311_552
+    assert L.turq_weight_nbytes(Q4_K, 4, 100) == 0                     # k not a multiple of 256
+    assert L.turq_tiled_nbytes(Q4_K, 12288, 4096) == 28_311_552        # the tiled layout adds nothing here
+    assert L.turq_tiled_nbytes(Q6_K, 17, 256) == 2 * 3360              # rows padded to 32
+
+
+def test_context_errors_are_reported_not_raised():
+    L = capi.lib()
+    ctx = ctypes.c_void_p()
+    assert L.turq_ctx_create(0, None) == capi.ERR_INVALID
+    assert "null" in capi.last_error(None)
+    assert L.turq_sync(None) == capi.ERR_INVALID
+    if not os.path.exists("/dev/kfd"):
+        rc = L.turq_ctx_create(0, ctypes.byref(ctx))
+        assert rc != capi.OK and capi.last_error(None)                 # no GPU: a clear error, no crash, no CPU fallback
+    assert L.turq_weight_release(None) == capi.OK
+    assert L.turq_weight_retain(None) == capi.ERR_INVALID
+
+
+@pytest.fixture()
+def gguf_file(tmp_path):
+    rng = np.random.default_rng(0)
+    tensors = [
+        ("blk.0.ffn_gate.weight", Q4_K, (48, 512), synth.random_weight(Q4_K, 48, 512, 1)),
+        ("blk.0.attn_v.weight", Q6_K, (32, 256), synth.random_weight(Q6_K, 32, 256, 2)),
+        ("blk.0.attn_q.weight", Q8_0, (16, 64), synth.random_weight(Q8_0, 16, 64, 3)),
+        ("blk.0.attn_q.bias", 0, (16,), rng.standard_normal(16).astype("<f4").view(np.uint8)),
+        ("output_norm.weight", 0, (512,), rng.standard_normal(512).astype("<f4").view(np.uint8)),
+        ("token_embd.weight", Q5_K, (20, 256), synth.random_weight(Q5_K, 20, 256, 4)),
+    ]
+    meta = {"general.architecture": "qwen3", "qwen3.block_count": 1, "qwen3.rope.freq_base": 1000000.0,
+            "tokenizer.ggml.tokens": ["a", "b", "c"], "general.file_type": 15}
+    p = tmp_path / "tiny.gguf"
+    write_gguf(str(p), tensors, meta)
+    return str(p), tensors, meta
+
+
+def test_gguf_reader(gguf_file):
+    path, tensors, meta = gguf_file
+    L = capi.lib()
+    g = ctypes.c_void_p()
+    capi.check(L.turq_gguf_open(path.encode(), ctypes.byref(g)))
+    assert L.turq_gguf_tensor_count(g) == len(tensors)
+    assert [L.turq_gguf_tensor_name(g, i).decode() for i in range(len(tensors))] == [t[0] for t in tensors]
+    for name, dt, shape, raw in tensors:
+        gdt, nd, nb, off = ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t(), ctypes.c_uint64()
+        dims = (ctypes.c_int64 * 4)()
+        capi.check(L.turq_gguf_tensor_info(g, name.encode(), ctypes.byref(gdt), ctypes.byref(nd), dims, ctypes.byref(off), ctypes.byref(nb)))
+        assert gdt.value == dt and tuple(dims[i] for i in range(nd.value)) == shape and nb.value == raw.size
+        assert off.value % 32 == 0                                      # data section aligned to general.alignment
+        buf = np.zeros(raw.size, np.uint8)
+        capi.check(L.turq_gguf_read_tensor(g, name.encode(), capi.ptr(buf), buf.size))
+        assert np.array_equal(buf, np.asarray(raw).view(np.uint8).reshape(-1))
+    # metadata
+    u, f = ctypes.c_uint64(), ctypes.c_double()
+    capi.check(L.turq_gguf_meta_u64(g, b"qwen3.block_count", ctypes.byref(u)))
+    assert u.value == 1
+    capi.check(L.turq_gguf_meta_f64(g, b"qwen3.rope.freq_base", ctypes.byref(f)))
+    assert f.value == 1000000.0
+    s = ctypes.create_string_buffer(64)
+    capi.check(L.turq_gguf_meta_str(g, b"general.architecture", s, 64))
+    assert s.value == b"qwen3"
+    capi.check(L.turq_gguf_meta_u64(g, b"tokenizer.ggml.tokens", ctypes.byref(u)))
+    assert u.value == 3                                                 # arrays report their length
+    assert L.turq_gguf_meta_u64(g, b"no.such.key", ctypes.byref(u)) == capi.ERR_NOT_FOUND
+    assert L.turq_gguf_meta_u64(g, b"general.architecture", ctypes.byref(u)) == capi.ERR_DTYPE
+    # lookups that miss
+    assert L.turq_gguf_tensor_info(g, b"blk.9.nope", None, None, None, None, None) == capi.ERR_NOT_FOUND
+    assert "cannot find tensor info" in L.turq_gguf_last_error(g).decode()
+    small = np.zeros(8, np.uint8)
+    assert L.turq_gguf_read_tensor(g, b"output_norm.weight", capi.ptr(small), small.size) == capi.ERR_SHAPE
+    L.turq_gguf_close(g)
+
+
+def test_gguf_reader_rejects_malformed_files(tmp_path):
+    L = capi.lib()
+    g = ctypes.c_void_p()
+    assert L.turq_gguf_open(str(tmp_path / "missing.gguf").encode(), ctypes.byref(g)) == capi.ERR_IO
+    bad = tmp_path / "bad.gguf"
+    bad.write_bytes(b"GGML" + b"\0" * 64)
+    assert L.turq_gguf_open(str(bad).encode(), ctypes.byref(g)) == capi.ERR_IO and "magic" in capi.last_error(None)
+    v9 = tmp_path / "v9.gguf"
+    v9.write_bytes(struct.pack("<IIQQ", 0x46554747, 9, 0, 0))
+    assert L.turq_gguf_open(str(v9).encode(), ctypes.byref(g)) == capi.ERR_IO and "version" in capi.last_error(None)
+    trunc = tmp_path / "trunc.gguf"
+    trunc.write_bytes(struct.pack("<IIQQ", 0x46554747, 3, 1, 0) + struct.pack("<Q", 5) + b"ab")
+    assert L.turq_gguf_open(str(trunc).encode(), ctypes.byref(g)) == capi.ERR_IO
+    # innermost dimension not divisible by the block size
+    ragged = tmp_path / "ragged.gguf"
+    name = b"w"
+    ragged.write_bytes(struct.pack("<IIQQ", 0x46554747, 3, 1, 0) + struct.pack("<Q", 1) + name + struct.pack("<I", 2) +
+                       struct.pack("<QQ", 100, 4) + struct.pack("<IQ", Q4_K, 0))
+    assert L.turq_gguf_open(str(ragged).encode(), ctypes.byref(g)) == capi.ERR_IO and "block size" in capi.last_error(None)
+
+
+def test_gguf_v2_and_alignment(tmp_path):
+    # version 2 header (same field widths as v3) and a non-default general.alignment
+    raw = synth.random_weight(Q8_0, 4, 32, 9)
+    p = tmp_path / "al.gguf"
+    write_gguf(str(p), [("a.weight", Q8_0, (4, 32), raw), ("b.weight", Q8_0, (4, 32), raw[::-1].copy())], {"k": 1}, alignment=64)
+    data = bytearray(p.read_bytes())
+    data[4:8] = struct.pack("<I", 2)
+    p.write_bytes(bytes(data))
+    L = capi.lib()
+    g = ctypes.c_void_p()
+    capi.check(L.turq_gguf_open(str(p).encode(), ctypes.byref(g)))
+    off = ctypes.c_uint64()
+    capi.check(L.turq_gguf_tensor_info(g, b"b.weight", None, None, None, ctypes.byref(off), None))
+    assert off.value % 64 == 0
+    buf = np.zeros(raw.size, np.uint8)
+    capi.check(L.turq_gguf_read_tensor(g, b"b.weight", capi.ptr(buf), buf.size))
+    assert np.array_equal(buf, raw[::-1])
+    L.turq_gguf_close(g)

@@ -1,0 +1,153 @@
+"""GPU tests of the host-side mirror (QVarBuilder / QMatMul / LinearX), written the way the reference
+tests its own layer (src/models/layers/linear.rs:117-316: shapes, batch shapes, bias, clone) and its
+integration tests check the quantized path (tests/qwen3_integration.rs: shape, finiteness,
+single-vs-batched consistency), with the numeric parity the reference's tests lack."""
+import numpy as np
+import pytest
+
+from oracle import capi as orc
+from tests.helpers import rel_l2
+from tur_amd import capi, qlinear, synth
+from tur_amd.gguf import write_gguf
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+HID, FFN, KV = 512, 1536, 256
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    """one synthetic decoder layer in the Q4_K_M mix + a biased projection + an F32 norm"""
+    rng = np.random.default_rng(5)
+    spec = [("blk.0.attn_q.weight", Q4_K, (HID, HID)), ("blk.0.attn_k.weight", Q4_K, (KV, HID)),
+            ("blk.0.attn_v.weight", Q6_K, (KV, HID)), ("blk.0.attn_output.weight", Q4_K, (HID, HID)),
+            ("blk.0.ffn_gate.weight", Q4_K, (FFN, HID)), ("blk.0.ffn_up.weight", Q4_K, (FFN, HID)),
+            ("blk.0.ffn_down.weight", Q6_K, (HID, FFN)), ("output.weight", Q8_0, (1000, HID)),
+            ("blk.0.biased.weight", Q5_K, (96, HID))]
+    tensors = [(name, dt, shape, synth.random_weight(dt, shape[0], shape[1], seed=i)) for i, (name, dt, shape) in enumerate(spec)]
+    bias = rng.standard_normal(96).astype("<f4")
+    norm = rng.standard_normal(HID).astype("<f4")
+    tensors += [("blk.0.biased.bias", 0, (96,), bias.view(np.uint8)), ("blk.0.attn_norm.weight", 0, (HID,), norm.view(np.uint8))]
+    path = tmp_path_factory.mktemp("gguf") / "layer.gguf"
+    write_gguf(str(path), tensors, {"general.architecture": "qwen3"})
+    dev = qlinear.Device.new_hip(0)
+    vb = qlinear.QVarBuilder.from_gguf(str(path), dev)
+    yield dev, vb, {t[0]: t for t in tensors}, bias, norm
+    dev.close()
+
+
+def test_varbuilder_lookups(model):
+    dev, vb, tensors, _, _ = model
+    assert sorted(vb.all_keys()) == sorted(tensors)
+    b0 = vb.pp("blk").pp(0)
+    assert b0.path("attn_q.weight") == "blk.0.attn_q.weight"
+    assert b0.contains_key("attn_q.weight") and not b0.contains_key("attn_q.bias")
+    assert b0.tensor_shape("ffn_down.weight") == [HID, FFN] and b0.tensor_shape("nope") is None
+    t = b0.pp("attn_k").get((KV, HID), "weight")
+    assert t.shape() == (KV, HID) and t.dtype() == Q4_K
+    with pytest.raises(capi.TurqError, match="shape mismatch for weight"):
+        b0.pp("attn_k").get((HID, HID), "weight")          # cached tensor, wrong shape
+    with pytest.raises(capi.TurqError, match="shape mismatch for weight"):
+        b0.pp("attn_v").get((HID, HID), "weight")          # fresh tensor, wrong shape
+    with pytest.raises(capi.TurqError, match="cannot find tensor info"):
+        b0.pp("attn_x").get((HID, HID), "weight")
+    assert b0.get_no_shape("attn_norm.weight").shape() == (HID,)
+
+
+def test_norm_weight_dequantizes_like_the_reference(model):
+    dev, vb, _, _, norm = model
+    got = vb.pp("blk").pp(0).pp("attn_norm").get(HID, "weight").dequantize(dev)
+    assert got.shape == (HID,) and np.array_equal(got, norm)
+
+
+@pytest.mark.parametrize("name,out_dim,in_dim", [("attn_q", HID, HID), ("attn_k", KV, HID), ("attn_v", KV, HID),
+                                                 ("attn_output", HID, HID), ("ffn_gate", FFN, HID), ("ffn_up", FFN, HID),
+                                                 ("ffn_down", HID, FFN)])
+def test_decoder_layer_linears(model, name, out_dim, in_dim):
+    dev, vb, tensors, _, _ = model
+    layer = qlinear.linear(in_dim, out_dim, vb.pp("blk").pp(0).pp(name))
+    assert repr(layer) == "LinearX::Quantized" and layer.bias is None
+    _, dt, _, raw = tensors[f"blk.0.{name}.weight"]
+    rng = np.random.default_rng(0)
+    for shape in ((1, 1, in_dim), (2, 5, in_dim), (1, 40, in_dim)):      # [batch, seq, hidden] as the models call it
+        x = rng.standard_normal(shape).astype(np.float32)
+        y = layer.forward(x)
+        assert y.shape == shape[:-1] + (out_dim,) and np.all(np.isfinite(y))
+        want = orc.matmul_dequant(dt, x.reshape(-1, in_dim), raw, out_dim, in_dim).reshape(y.shape)
+        assert rel_l2(y, want) <= 1e-3
+    # single vs batched: row 0 of a batch equals the same row alone (the reference allows 1e-2 here)
+    xb = rng.standard_normal((3, 1, in_dim)).astype(np.float32)
+    yb = layer.forward(xb)
+    y0 = layer.forward(xb[0:1])
+    assert np.max(np.abs(yb[0] - y0[0])) <= 1e-3 * np.max(np.abs(y0))
+
+
+def test_bias_is_dequantized_at_load_and_added(model):
+    dev, vb, tensors, bias, _ = model
+    layer = qlinear.linear(HID, 96, vb.pp("blk").pp(0).pp("biased"))
+    assert layer.bias is not None and np.array_equal(layer.bias, bias)
+    x = np.zeros((1, 2, HID), np.float32)
+    assert np.array_equal(layer.forward(x), np.broadcast_to(bias, (1, 2, 96)))      # zero input -> bias
+    x = np.random.default_rng(1).standard_normal((1, 3, HID)).astype(np.float32)
+    _, dt, _, raw = tensors["blk.0.biased.weight"]
+    want = orc.matmul_dequant(dt, x.reshape(-1, HID), raw, 96, HID).reshape(1, 3, 96) + bias
+    assert rel_l2(layer.forward(x), want) <= 1e-3
+
+
+def test_lm_head_and_clone(model):
+    dev, vb, tensors, _, _ = model
+    head = qlinear.linear(HID, 1000, vb.pp("output"))
+    clone = qlinear.LinearX(qlinear.QMatMul.from_arc(head.qmatmul.qtensor.clone()), None)
+    head.qmatmul.qtensor.release()                                     # the clone keeps the device copy alive
+    x = np.random.default_rng(2).standard_normal((1, 1, HID)).astype(np.float32)
+    y = clone.forward(x)
+    _, dt, _, raw = tensors["output.weight"]
+    assert y.shape == (1, 1, 1000)
+    assert rel_l2(y, orc.matmul_dequant(dt, x.reshape(1, HID), raw, 1000, HID).reshape(1, 1, 1000)) <= 1e-3
+
+
+def test_forward_argument_errors(model):
+    dev, vb, _, _, _ = model
+    layer = qlinear.linear(HID, KV, vb.pp("blk").pp(0).pp("attn_k"))
+    with pytest.raises(capi.TurqError):
+        layer.forward(np.zeros(HID, np.float32))                        # rank < 2
+    with pytest.raises(capi.TurqError):
+        layer.forward(np.zeros((1, HID + 1), np.float32))               # last dim != k
+    with pytest.raises(capi.TurqError):
+        layer.forward(np.zeros((2, 4, HID), np.float32)[:, ::2, :])     # not contiguous
+    with pytest.raises(capi.TurqError):
+        layer.forward(np.zeros((1, HID), np.float64))                   # unsupported dtype
+    with pytest.raises(capi.TurqError):
+        qlinear.QMatMul.from_arc(vb.pp("blk").pp(0).pp("attn_norm").get(HID, "weight"))   # dense tensor
+    assert layer.forward(np.zeros((0, HID), np.float32)).shape == (0, KV)   # empty batch
+
+
+def test_cpp_host_mirror(model, tmp_path):
+    """the C++ header mirror (tur_amd/csrc/host/turq.hpp) run as a program against the same kind of file"""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "test_host")
+    if not os.path.exists(exe):
+        pytest.fail("tests/cpp/test_host is not built (run __graft_entry__.build())")
+    rng = np.random.default_rng(11)
+    n, k = 160, 512
+    gate = synth.random_weight(Q4_K, n, k, seed=1)
+    biased = synth.random_weight(Q6_K, 96, k, seed=2)
+    bias = rng.standard_normal(96).astype("<f4")
+    norm = rng.standard_normal(k).astype("<f4")
+    path = tmp_path / "cpp.gguf"
+    write_gguf(str(path), [("blk.0.ffn_gate.weight", Q4_K, (n, k), gate), ("blk.0.biased.weight", Q6_K, (96, k), biased),
+                           ("blk.0.biased.bias", 0, (96,), bias.view(np.uint8)), ("blk.0.attn_norm.weight", 0, (k,), norm.view(np.uint8))])
+    res = subprocess.run([exe, str(path)], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr
+    lines = res.stdout.split("\n")
+    assert lines[-2] == "OK"
+    m = 3
+    x = (np.sin(np.float32(0.37) * np.arange(m * k, dtype=np.float32)) * np.float32(2.0)).astype(np.float32).reshape(m, k)
+    i = lines.index(f"gate {n} {k}")
+    y = np.array([float(v) for v in lines[i + 1:i + 1 + m * n]], np.float32).reshape(m, n)
+    j = lines.index(f"biased 96 {k}")
+    yb = np.array([float(v) for v in lines[j + 1:j + 1 + m * 96]], np.float32).reshape(m, 96)
+    assert rel_l2(y, orc.matmul_dequant(Q4_K, x, gate, n, k)) <= 1e-3
+    assert rel_l2(yb, orc.matmul_dequant(Q6_K, x, biased, 96, k) + bias) <= 1e-3
+    assert lines[-3].startswith(f"norm {k} ")

@@ -45,6 +45,12 @@ _SIGS = {
     "turq_qmatmul": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int, c_int]),
     "turq_quantize_q8_0": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
     "turq_quantize_q8_k": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
+    "turq_graph_begin": (c_int, [c_void_p]),
+    "turq_graph_end": (c_int, [c_void_p, POINTER(c_void_p)]),
+    "turq_graph_launch": (c_int, [c_void_p, c_void_p]),
+    "turq_graph_destroy": (None, [c_void_p]),
+    "turq_profile_begin": (c_int, [c_void_p]),
+    "turq_profile_end": (c_int, [c_void_p, POINTER(c_int64), POINTER(c_double)]),
     "turq_gguf_open": (c_int, [c_char_p, POINTER(c_void_p)]),
     "turq_gguf_close": (None, [c_void_p]),
     "turq_gguf_last_error": (c_char_p, [c_void_p]),

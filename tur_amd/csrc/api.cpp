@@ -12,6 +12,8 @@ std::string &turq_thread_error() {
 
 int turq_ctx_reserve(turq_ctx *ctx, void **buf, size_t *cap, size_t need) {
     if (need <= *cap) return TURQ_OK;
+    if (ctx->capturing)
+        return turq_fail(ctx, TURQ_ERR_INVALID, "a scratch buffer would have to grow (%zu > %zu bytes) while a graph is being captured: run the same calls once before turq_graph_begin", need, *cap);
     TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));  // the old buffer may still be in use
     if (*buf) {
         TURQ_HIP(ctx, hipFree(*buf));
@@ -22,6 +24,24 @@ int turq_ctx_reserve(turq_ctx *ctx, void **buf, size_t *cap, size_t need) {
     TURQ_HIP(ctx, hipMalloc(buf, want));
     *cap = want;
     return TURQ_OK;
+}
+
+hipError_t turq_prof_next(turq_ctx *ctx, hipEvent_t *start, hipEvent_t *stop) {
+    *start = nullptr;
+    *stop = nullptr;
+    if (!ctx->profiling) return hipSuccess;
+    if (ctx->prof_used == ctx->prof_events.size()) {
+        hipEvent_t a = nullptr, b = nullptr;
+        hipError_t e = hipEventCreate(&a);
+        if (e != hipSuccess) return e;
+        e = hipEventCreate(&b);
+        if (e != hipSuccess) { (void)hipEventDestroy(a); return e; }
+        ctx->prof_events.emplace_back(a, b);
+    }
+    *start = ctx->prof_events[ctx->prof_used].first;
+    *stop = ctx->prof_events[ctx->prof_used].second;
+    ctx->prof_used++;
+    return hipSuccess;
 }
 
 namespace {
@@ -90,6 +110,7 @@ void turq_ctx_destroy(turq_ctx *ctx) {
     if (ctx->stage_y) (void)hipFree(ctx->stage_y);
     if (ctx->act_prep) (void)hipFree(ctx->act_prep);
     if (ctx->stage_b) (void)hipFree(ctx->stage_b);
+    for (auto &p : ctx->prof_events) { (void)hipEventDestroy(p.first); (void)hipEventDestroy(p.second); }
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -344,6 +365,83 @@ int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int
     if (rc != TURQ_OK) return rc;
     TURQ_HIP(ctx, hipMemcpy2DAsync(y, (size_t)ldy * yb, ctx->stage_y, yrow, yrow, (size_t)m, hipMemcpyDeviceToHost, ctx->stream));
     TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return TURQ_OK;
+}
+
+// ---- graphs and kernel timing ----
+
+int turq_graph_begin(turq_ctx *ctx) {
+    TURQ_ENTER(ctx);
+    if (ctx->capturing) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_begin: a capture is already running");
+    if (ctx->profiling) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_begin: kernel timing is on; events cannot be captured");
+    TURQ_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return TURQ_OK;
+}
+
+int turq_graph_end(turq_ctx *ctx, turq_graph **out) {
+    TURQ_ENTER(ctx);
+    if (!out) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_end: null out pointer");
+    *out = nullptr;
+    if (!ctx->capturing) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_end: no capture is running");
+    ctx->capturing = false;
+    std::unique_ptr<turq_graph> g(new (std::nothrow) turq_graph);
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    if (e != hipSuccess || !g) {
+        if (graph) (void)hipGraphDestroy(graph);
+        return turq_fail(ctx, g ? TURQ_ERR_HIP : TURQ_ERR_OOM, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
+    }
+    g->graph = graph;
+    g->device = ctx->device;
+    e = hipGraphInstantiate(&g->exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(graph);
+        return turq_fail(ctx, TURQ_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    *out = g.release();
+    return TURQ_OK;
+}
+
+int turq_graph_launch(turq_ctx *ctx, turq_graph *g) {
+    TURQ_ENTER(ctx);
+    if (!g || !g->exec) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_launch: null graph");
+    if (g->device != ctx->device) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_launch: graph was captured on device %d", g->device);
+    TURQ_HIP(ctx, hipGraphLaunch(g->exec, ctx->stream));
+    return TURQ_OK;
+}
+
+void turq_graph_destroy(turq_graph *g) {
+    if (!g) return;
+    DeviceGuard guard(g->device);
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
+}
+
+int turq_profile_begin(turq_ctx *ctx) {
+    TURQ_ENTER(ctx);
+    if (ctx->capturing) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_profile_begin: a graph capture is running");
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    ctx->profiling = true;
+    ctx->prof_used = 0;
+    return TURQ_OK;
+}
+
+int turq_profile_end(turq_ctx *ctx, int64_t *launches, double *total_ms) {
+    TURQ_ENTER(ctx);
+    if (!ctx->profiling) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_profile_end: timing was not started");
+    ctx->profiling = false;
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    double sum = 0.0;
+    for (size_t i = 0; i < ctx->prof_used; i++) {
+        float ms = 0.0f;
+        TURQ_HIP(ctx, hipEventElapsedTime(&ms, ctx->prof_events[i].first, ctx->prof_events[i].second));
+        sum += ms;
+    }
+    if (launches) *launches = (int64_t)ctx->prof_used;
+    if (total_ms) *total_ms = sum;
+    ctx->prof_used = 0;
     return TURQ_OK;
 }
 

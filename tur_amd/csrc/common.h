@@ -9,6 +9,8 @@
 #include <cstdio>
 #include <cstring>
 #include <string>
+#include <utility>
+#include <vector>
 
 #include "../../include/turq.h"
 
@@ -70,7 +72,23 @@ struct turq_ctx {
     void *stage_y = nullptr;  size_t stage_y_cap = 0;
     void *stage_b = nullptr;  size_t stage_b_cap = 0;
     void *act_prep = nullptr; size_t act_prep_cap = 0;
+    // kernel timing (turq_profile_*): event pairs recorded around matmul kernels
+    bool profiling = false;
+    bool capturing = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_events;
+    size_t prof_used = 0;
 };
+
+struct turq_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int device = 0;
+};
+
+// Kernel timing: hands out the next event pair (both null unless turq_profile_begin is active).
+// The launcher passes them to hipExtLaunchKernelGGL, which stamps them with the dispatch's own
+// begin / end times, i.e. the kernel's execution time without launch gaps.
+hipError_t turq_prof_next(turq_ctx *ctx, hipEvent_t *start, hipEvent_t *stop);
 
 struct turq_weight {
     std::atomic<int> refs{1};

@@ -10,6 +10,8 @@
 //
 // HBM traffic per launch = the weight once (+ activations and outputs, tiny): the kernel is bound
 // by HBM bandwidth, the VALU unpack (about 2 to 3 instructions per weight byte) rides along.
+#include <hip/hip_ext.h>
+
 #include "layout.h"
 #include "mfma_common.h"
 
@@ -27,11 +29,74 @@ __device__ inline float h2f_bits(uint32_t bits16) {
     return (float)h;
 }
 
-// activation fragment of step q for this lane (zero for rows beyond the prepared height)
-__device__ inline half8v load_afrag(const half8v *__restrict__ tile_frags, int q, int g, int r, int mpad) {
-    half8v z = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (r < mpad) z = tile_frags[(q * 4 + g) * mpad + r];
-    return z;
+// ---- weight registers of one tile (everything a lane loads from HBM for it) ----
+__device__ inline void turq_store_any(void *y, int yt, int64_t i, float v) {
+    if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, i, v);
+    else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, i, v);
+    else turq_store_out<TURQ_ACT_F16>(y, i, v);
+}
+
+template <int DT> struct WRegs;
+template <> struct WRegs<TURQ_Q4_K> { uint4v qa, qb, hd; };
+template <> struct WRegs<TURQ_Q5_K> { uint4v qa, qb, hd; uint2v hh; };
+template <> struct WRegs<TURQ_Q6_K> { uint4v qla, qlb, qh; uint32_t scw; uint32_t d16; };
+template <> struct WRegs<TURQ_Q8_0> { uint4v p[4]; uint4v dd; };
+
+template <int DT> __device__ inline WRegs<DT> load_tile(const uint8_t *__restrict__ tile, int lane);
+template <> __device__ inline WRegs<TURQ_Q4_K> load_tile<TURQ_Q4_K>(const uint8_t *__restrict__ tile, int lane) {
+    using F = TiledFmt<TURQ_Q4_K>;
+    WRegs<TURQ_Q4_K> w;
+    w.qa = *(const uint4v *)(tile + F::kQA + 16 * lane);
+    w.qb = *(const uint4v *)(tile + F::kQB + 16 * lane);
+    w.hd = *(const uint4v *)(tile + F::kHDR + 16 * (lane & 15));
+    return w;
+}
+template <> __device__ inline WRegs<TURQ_Q5_K> load_tile<TURQ_Q5_K>(const uint8_t *__restrict__ tile, int lane) {
+    using F = TiledFmt<TURQ_Q5_K>;
+    WRegs<TURQ_Q5_K> w;
+    w.qa = *(const uint4v *)(tile + F::kQA + 16 * lane);
+    w.qb = *(const uint4v *)(tile + F::kQB + 16 * lane);
+    w.hh = *(const uint2v *)(tile + F::kQH + 8 * lane);
+    w.hd = *(const uint4v *)(tile + F::kHDR + 16 * (lane & 15));
+    return w;
+}
+template <> __device__ inline WRegs<TURQ_Q6_K> load_tile<TURQ_Q6_K>(const uint8_t *__restrict__ tile, int lane) {
+    using F = TiledFmt<TURQ_Q6_K>;
+    WRegs<TURQ_Q6_K> w;
+    w.qla = *(const uint4v *)(tile + F::kQLA + 16 * lane);
+    w.qlb = *(const uint4v *)(tile + F::kQLB + 16 * lane);
+    w.qh = *(const uint4v *)(tile + F::kQH + 16 * lane);
+    w.scw = *(const uint32_t *)(tile + F::kSC + 4 * lane);
+    w.d16 = *(const uint16_t *)(tile + F::kD + 2 * (lane & 15));
+    return w;
+}
+template <> __device__ inline WRegs<TURQ_Q8_0> load_tile<TURQ_Q8_0>(const uint8_t *__restrict__ tile, int lane) {
+    using F = TiledFmt<TURQ_Q8_0>;
+    WRegs<TURQ_Q8_0> w;
+#pragma unroll
+    for (int i = 0; i < 4; i++) w.p[i] = *(const uint4v *)(tile + 1024 * i + 16 * lane);
+    w.dd = *(const uint4v *)(tile + F::kD + 16 * (lane & 15));
+    return w;
+}
+
+// ---- activation fragments of one tile: NQ steps for each of MT m-tiles ----
+// Rows of the A operand beyond the prepared height are never stored (every output row depends on
+// its own A row only), so lanes of those rows simply re-read a valid row instead of zeros.
+template <int DT, int MT> struct AFrags {
+    static constexpr int NQ = DT == TURQ_Q8_0 ? TURQ_NQ_Q8_0 : TURQ_NQ_KQUANT;
+    half8v a[MT][NQ];
+};
+
+template <int DT, int MT>
+__device__ inline AFrags<DT, MT> load_frags_global(const half8v *__restrict__ tile_frags, int64_t mt_stride, int mpad,
+                                                   int lane) {
+    AFrags<DT, MT> f;
+    const int g = lane >> 4, r = (lane & 15) & (mpad - 1);
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int q = 0; q < AFrags<DT, MT>::NQ; q++) f.a[mt][q] = tile_frags[mt * mt_stride + (q * 4 + g) * mpad + r];
+    return f;
 }
 
 // The 6-bit scales and mins of the two sub-blocks a lane owns, as packed f16 constants.
@@ -71,77 +136,70 @@ template <bool HIGH>
 __device__ inline half8v k45_operand(uint32_t w, half2v s, half2v s16, half2v c1, half2v c2, uint32_t h0, uint32_t h1,
                                      int u0) {
     const uint32_t w8 = w >> 8;
-    uint32_t t0 = (w & 0x000F000Fu) | kMagic1024;
-    uint32_t t1 = (w & 0x00F000F0u) | kMagic1024;
-    uint32_t t2 = (w8 & 0x000F000Fu) | kMagic1024;
-    uint32_t t3 = (w8 & 0x00F000F0u) | kMagic1024;
+    uint32_t t0 = and_or_u32(w, 0x000F000Fu, kMagic1024);
+    uint32_t t1 = and_or_u32(w, 0x00F000F0u, kMagic1024);
+    uint32_t t2 = and_or_u32(w8, 0x000F000Fu, kMagic1024);
+    uint32_t t3 = and_or_u32(w8, 0x00F000F0u, kMagic1024);
     if (HIGH) {  // fifth bit: +16 on top of the nibble (bit 4 / 20, or bit 8 / 24 for the x16 form)
-        t0 |= rotr32(h0, (uint32_t)u0) & 0x00100010u;
-        t1 |= rotr32(h1, (uint32_t)u0) & 0x01000100u;
-        t2 |= rotr32(h0, (uint32_t)(u0 + 1)) & 0x00100010u;
-        t3 |= rotr32(h1, (uint32_t)(u0 + 1)) & 0x01000100u;
+        t0 = and_or_u32(rotr32(h0, (uint32_t)u0), 0x00100010u, t0);
+        t1 = and_or_u32(rotr32(h1, (uint32_t)u0), 0x01000100u, t1);
+        t2 = and_or_u32(rotr32(h0, (uint32_t)(u0 + 1)), 0x00100010u, t2);
+        t3 = and_or_u32(rotr32(h1, (uint32_t)(u0 + 1)), 0x01000100u, t3);
     }
     return make_half8(pk_fma(as_half2(t0), s, c1), pk_fma(as_half2(t1), s16, c2), pk_fma(as_half2(t2), s, c1),
                       pk_fma(as_half2(t3), s16, c2));
 }
 
-template <int DT, int MT> struct TileOp;
+// ---- per-format tile arithmetic: acc[mt] += (this tile's contribution) ----
+// NV = how many of a lane's four result rows get the f32 scale applied.  Always instantiated with 4:
+// with NV < 4 (skipping rows that are never stored) the unused MFMA result registers become free,
+// the register allocator reuses them for VALU temporaries a few cycles after the MFMA issues, and
+// on MI355X the Q8_0 kernel then returned garbage (a write-after-write on the MFMA destination:
+// the MFMA's late result write clobbers the temporary).  Consuming all four rows keeps the
+// destination registers live until the MFMA has retired.
+template <int DT, int MT, int NV> struct TileOp;
 
-// ---- Q4_K and Q5_K ----
-template <int DT, int MT> struct TileOpK45 {
-    using F = TiledFmt<DT>;
+template <int DT, int MT, int NV> struct TileOpK45 {
     static constexpr bool HIGH = DT == TURQ_Q5_K;
-    __device__ static void run(const uint8_t *__restrict__ tile, const half8v *__restrict__ fr, int64_t mt_stride,
-                               int mpad, int lane, float4v *acc) {
-        const int r = lane & 15, g = lane >> 4;
-        const uint4v qa = *(const uint4v *)(tile + F::kQA + 16 * lane);
-        const uint4v qb = *(const uint4v *)(tile + F::kQB + 16 * lane);
-        const uint4v hd = *(const uint4v *)(tile + F::kHDR + 16 * r);
-        uint2v hh = {0, 0};
-        if constexpr (HIGH) hh = *(const uint2v *)(tile + TiledFmt<TURQ_Q5_K>::kQH + 8 * lane);
-        const K4Consts c = k4_consts(hd, g);
-        const uint32_t wq[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+    __device__ static void run(const WRegs<DT> &w, const AFrags<DT, MT> &f, int lane, float4v *acc) {
+        const int g = lane >> 4;
+        uint32_t h0 = 0, h1 = 0;
+        if constexpr (HIGH) { h0 = w.hh.x; h1 = w.hh.y; }
+        const K4Consts c = k4_consts(w.hd, g);
+        const uint32_t wq[8] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w, w.qb.x, w.qb.y, w.qb.z, w.qb.w};
         float4v tmp[MT];
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) tmp[mt] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const half8v bop = i < 4 ? k45_operand<HIGH>(wq[i], c.s_lo, c.s16_lo, c.c1_lo, c.c2_lo, hh.x, hh.y, 2 * i)
-                                     : k45_operand<HIGH>(wq[i], c.s_hi, c.s16_hi, c.c1_hi, c.c2_hi, hh.x, hh.y, 2 * i);
+            const half8v bop = i < 4 ? k45_operand<HIGH>(wq[i], c.s_lo, c.s16_lo, c.c1_lo, c.c2_lo, h0, h1, 2 * i)
+                                     : k45_operand<HIGH>(wq[i], c.s_hi, c.s16_hi, c.c1_hi, c.c2_hi, h0, h1, 2 * i);
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-                tmp[mt] = mfma16x16x32(load_afrag(fr + mt * mt_stride, i, g, r, mpad), bop, tmp[mt]);
+            for (int mt = 0; mt < MT; mt++) tmp[mt] = mfma16x16x32(f.a[mt][i], bop, tmp[mt]);
         }
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
-            const float4v tmin =
-                mfma16x16x32(load_afrag(fr + mt * mt_stride, 8, g, r, mpad), c.bmin, float4v{0.f, 0.f, 0.f, 0.f});
-            acc[mt] += c.d * tmp[mt] - c.dmin * tmin;
+            const float4v tmin = mfma16x16x32(f.a[mt][8], c.bmin, float4v{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+            for (int i = 0; i < NV; i++) acc[mt][i] += c.d * tmp[mt][i] - c.dmin * tmin[i];
         }
     }
 };
-template <int MT> struct TileOp<TURQ_Q4_K, MT> : TileOpK45<TURQ_Q4_K, MT> {};
-template <int MT> struct TileOp<TURQ_Q5_K, MT> : TileOpK45<TURQ_Q5_K, MT> {};
+template <int MT, int NV> struct TileOp<TURQ_Q4_K, MT, NV> : TileOpK45<TURQ_Q4_K, MT, NV> {};
+template <int MT, int NV> struct TileOp<TURQ_Q5_K, MT, NV> : TileOpK45<TURQ_Q5_K, MT, NV> {};
 
-// ---- Q6_K ----
-template <int MT> struct TileOp<TURQ_Q6_K, MT> {
-    using F = TiledFmt<TURQ_Q6_K>;
-    __device__ static void run(const uint8_t *__restrict__ tile, const half8v *__restrict__ fr, int64_t mt_stride,
-                               int mpad, int lane, float4v *acc) {
-        const int r = lane & 15, g = lane >> 4;
-        const uint4v qla = *(const uint4v *)(tile + F::kQLA + 16 * lane);
-        const uint4v qlb = *(const uint4v *)(tile + F::kQLB + 16 * lane);
-        const uint4v qh = *(const uint4v *)(tile + F::kQH + 16 * lane);
-        const uint32_t scw = *(const uint32_t *)(tile + F::kSC + 4 * lane);
-        const float d = h2f_bits(*(const uint16_t *)(tile + F::kD + 2 * r));
-        const uint32_t wl[8] = {qla.x, qla.y, qla.z, qla.w, qlb.x, qlb.y, qlb.z, qlb.w};
-        const uint32_t wh[4] = {qh.x, qh.y, qh.z, qh.w};
+template <int MT, int NV> struct TileOp<TURQ_Q6_K, MT, NV> {
+    __device__ static void run(const WRegs<TURQ_Q6_K> &w, const AFrags<TURQ_Q6_K, MT> &f, int lane, float4v *acc) {
+        (void)lane;
+        const float d = h2f_bits(w.d16);
+        const uint32_t wl[8] = {w.qla.x, w.qla.y, w.qla.z, w.qla.w, w.qlb.x, w.qlb.y, w.qlb.z, w.qlb.w};
+        const uint32_t wh[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
         float4v tmp[MT];
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) tmp[mt] = float4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int sg = 0; sg < 4; sg++) {  // scale group sg covers steps 2sg, 2sg+1
-            const _Float16 sc = (_Float16)(float)(int)(int8_t)(scw >> (8 * sg));
+            const _Float16 sc = (_Float16)(float)(int)(int8_t)(w.scw >> (8 * sg));
             const half2v s1 = splat2(sc);
             const half2v c256 = s1 * splat2((_Float16)-256.0f);
             const half2v c16 = s1 * splat2((_Float16)-16.0f);
@@ -152,10 +210,10 @@ template <int MT> struct TileOp<TURQ_Q6_K, MT> {
             for (int ii = 0; ii < 2; ii++) {
                 const int i = 2 * sg + ii;
                 // low nibbles: n * sc
-                const uint32_t w = wl[i];
-                const uint32_t w8 = rotr32(w, 8);
-                const half8v b1 = make_half8(pk_fma(and_or_h2(w, 0x003C003Cu, kMagic256), s1, c256),
-                                             pk_fma(and_or_h2(w, 0x03C003C0u, kMagic16), s1, c16),
+                const uint32_t wv = wl[i];
+                const uint32_t w8 = rotr32(wv, 8);
+                const half8v b1 = make_half8(pk_fma(and_or_h2(wv, 0x003C003Cu, kMagic256), s1, c256),
+                                             pk_fma(and_or_h2(wv, 0x03C003C0u, kMagic16), s1, c16),
                                              pk_fma(and_or_h2(w8, 0x003C003Cu, kMagic256), s1, c256),
                                              pk_fma(and_or_h2(w8, 0x03C003C0u, kMagic16), s1, c16));
                 // high two bits: 16 * (h - 2) * sc   (the "- 32" of the 6-bit value lives here)
@@ -167,33 +225,27 @@ template <int MT> struct TileOp<TURQ_Q6_K, MT> {
                                              pk_fma(and_or_h2(hB, 0x03000300u, kMagic4), s16, c96));
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) {
-                    const half8v a = load_afrag(fr + mt * mt_stride, i, g, r, mpad);
-                    tmp[mt] = mfma16x16x32(a, b1, tmp[mt]);
-                    tmp[mt] = mfma16x16x32(a, b2, tmp[mt]);
+                    tmp[mt] = mfma16x16x32(f.a[mt][i], b1, tmp[mt]);
+                    tmp[mt] = mfma16x16x32(f.a[mt][i], b2, tmp[mt]);
                 }
             }
         }
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) acc[mt] += d * tmp[mt];
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int i = 0; i < NV; i++) acc[mt][i] += d * tmp[mt][i];
     }
 };
 
-// ---- Q8_0 ----
-template <int MT> struct TileOp<TURQ_Q8_0, MT> {
-    using F = TiledFmt<TURQ_Q8_0>;
-    __device__ static void run(const uint8_t *__restrict__ tile, const half8v *__restrict__ fr, int64_t mt_stride,
-                               int mpad, int lane, float4v *acc) {
-        const int r = lane & 15, g = lane >> 4;
-        uint4v p[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++) p[i] = *(const uint4v *)(tile + 1024 * i + 16 * lane);
-        const uint4v dd = *(const uint4v *)(tile + F::kD + 16 * r);
-        const uint32_t dw[4] = {dd.x, dd.y, dd.z, dd.w};
+template <int MT, int NV> struct TileOp<TURQ_Q8_0, MT, NV> {
+    __device__ static void run(const WRegs<TURQ_Q8_0> &w, const AFrags<TURQ_Q8_0, MT> &f, int lane, float4v *acc) {
+        (void)lane;
+        const uint32_t dw[4] = {w.dd.x, w.dd.y, w.dd.z, w.dd.w};
         const half2v k1152 = splat2((_Float16)-1152.0f);  // 1024 + the 128 the bytes were offset by
 #pragma unroll
         for (int q = 0; q < 8; q++) {
-            const uint32_t w0 = (q & 1) ? p[q >> 1].z : p[q >> 1].x;
-            const uint32_t w1 = (q & 1) ? p[q >> 1].w : p[q >> 1].y;
+            const uint32_t w0 = (q & 1) ? w.p[q >> 1].z : w.p[q >> 1].x;
+            const uint32_t w1 = (q & 1) ? w.p[q >> 1].w : w.p[q >> 1].y;
             const half8v bop = make_half8(and_or_h2(w0, 0x00FF00FFu, kMagic1024) + k1152,
                                           and_or_h2(w0 >> 8, 0x00FF00FFu, kMagic1024) + k1152,
                                           and_or_h2(w1, 0x00FF00FFu, kMagic1024) + k1152,
@@ -201,47 +253,195 @@ template <int MT> struct TileOp<TURQ_Q8_0, MT> {
             const float d = h2f_bits((q & 1) ? (dw[q >> 1] >> 16) : (dw[q >> 1] & 0xFFFFu));
 #pragma unroll
             for (int mt = 0; mt < MT; mt++) {
-                const float4v t = mfma16x16x32(load_afrag(fr + mt * mt_stride, q, g, r, mpad), bop,
-                                               float4v{0.f, 0.f, 0.f, 0.f});
-                acc[mt] += d * t;
+                const float4v t = mfma16x16x32(f.a[mt][q], bop, float4v{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                for (int i = 0; i < NV; i++) acc[mt][i] += d * t[i];
             }
         }
     }
 };
 
-template <int DT, int MT, int YT>
-__global__ void __launch_bounds__(512) gemv_mfma_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t ntc,
-                                                         const half8v *__restrict__ frags, int64_t m, int mpad,
-                                                         void *__restrict__ y, int64_t ldy,
-                                                         const float *__restrict__ bias) {
-    extern __shared__ float4v red[];  // [wave][mt][lane]
+// ---- fused activation preparation (small m): the wave converts its own slice of x ----
+// Raw activations of one tile for one lane: 4 consecutive columns of each of MP rows.
+template <int XT, int MP> struct XRegs { float v[MP][4]; };
+
+template <int XT, int MP>
+__device__ inline XRegs<XT, MP> load_x(const void *__restrict__ x, int64_t ldx, int64_t m, int64_t k, int64_t b,
+                                       int lane) {
+    XRegs<XT, MP> xr;
+    const int64_t col = b * 256 + 4 * lane;
+#pragma unroll
+    for (int rr = 0; rr < MP; rr++) {
+        const bool ok = rr < m && col < k;  // k is a multiple of 32, so 4 columns are in or out together
+        const int64_t off = ok ? rr * ldx + col : 0;
+        if (XT == TURQ_ACT_F32) {
+            const float4 t = *(const float4 *)((const float *)x + off);
+            xr.v[rr][0] = t.x; xr.v[rr][1] = t.y; xr.v[rr][2] = t.z; xr.v[rr][3] = t.w;
+        } else {
+            const uint2 t = *(const uint2 *)((const uint16_t *)x + off);
+            const uint32_t u[2] = {t.x, t.y};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t bits = (u[j >> 1] >> (16 * (j & 1))) & 0xFFFFu;
+                xr.v[rr][j] = XT == TURQ_ACT_BF16 ? __uint_as_float(bits << 16) : h2f_bits(bits);
+            }
+        }
+        if (!ok) { xr.v[rr][0] = 0.f; xr.v[rr][1] = 0.f; xr.v[rr][2] = 0.f; xr.v[rr][3] = 0.f; }
+    }
+    return xr;
+}
+
+// Write the wave's slice to its LDS region as f16 (+ group sums), then read the fragments back.
+// Region layout: MP rows of 256 f16 (512 B each), then MP rows of 16 (hi, lo) sum pairs (64 B each).
+template <int DT, int XT, int MP>
+__device__ inline AFrags<DT, 1> stage_frags_lds(const XRegs<XT, MP> &xr, uint8_t *region, int lane) {
+    constexpr bool KQ = DT != TURQ_Q8_0;
+    const int g = lane >> 4, r = (lane & 15) & (MP - 1);
+#pragma unroll
+    for (int rr = 0; rr < MP; rr++) {
+        const half2v h01 = {(_Float16)xr.v[rr][0], (_Float16)xr.v[rr][1]};
+        const half2v h23 = {(_Float16)xr.v[rr][2], (_Float16)xr.v[rr][3]};
+        *(uint2v *)(region + rr * 512 + 8 * lane) = uint2v{as_u32(h01), as_u32(h23)};
+        if (KQ) {  // sum of the 16 f16-rounded values of a group = 4 lanes
+            float s = ((float)h01.x + (float)h01.y) + ((float)h23.x + (float)h23.y);
+            s += __shfl_xor(s, 1, 64);
+            s += __shfl_xor(s, 2, 64);
+            const _Float16 hi = (_Float16)s;
+            const _Float16 lo = (_Float16)(s - (float)hi);
+            if ((lane & 3) == 0) *(uint32_t *)(region + MP * 512 + rr * 64 + lane) = as_u32(half2v{hi, lo});
+        }
+    }
+    // same-wave LDS traffic is processed in order; the fences keep the compiler from reordering
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    AFrags<DT, 1> f;
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const int col = KQ ? 64 * g + 8 * q : 32 * q + 8 * g;
+        f.a[0][q] = *(const half8v *)(region + r * 512 + 2 * col);
+    }
+    if constexpr (KQ) f.a[0][8] = *(const half8v *)(region + MP * 512 + r * 64 + 16 * g);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    return f;
+}
+
+// ---- the kernel ----
+// FUSED: activations come raw from x (m <= MP <= 4) and are prepared per wave through LDS;
+// otherwise they come from the fragment buffer written by the activation preparation kernel.
+// P = tiles whose loads a wave keeps in flight together.
+// MAXT = largest workgroup the instantiation is launched with (bounds the registers per lane).
+template <int DT, int MT, int XT, bool FUSED, int MP, int P, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_mfma_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
+                                                          const void *__restrict__ xin, int64_t ldx, int64_t m,
+                                                          int mpad, void *__restrict__ y, int yt, int64_t ldy,
+                                                          const float *__restrict__ bias) {
+    extern __shared__ uint8_t smem[];
     constexpr int NQ = DT == TURQ_Q8_0 ? TURQ_NQ_Q8_0 : TURQ_NQ_KQUANT;
     constexpr int TB = TiledFmt<DT>::kTileBytes;
+    constexpr int REGION = FUSED ? MP * (512 + 64) : 0;
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // wave-uniform: scalar address math
     const int nwaves = blockDim.x >> 6;
     const int64_t rt = blockIdx.x;
+    const int64_t ntc = turq_tile_cols(k);
     const int64_t tile_chunks = (int64_t)NQ * 4 * mpad;  // 16-byte chunks of one (mt, b) fragment set
     const int64_t mt_stride = ntc * tile_chunks;
+    float4v *red = (float4v *)(smem + (size_t)nwaves * REGION);
+    uint8_t *region = smem + (size_t)wave * REGION;
     float4v acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[mt] = float4v{0.f, 0.f, 0.f, 0.f};
     const uint8_t *wrow = w + rt * ntc * TB;
-    for (int64_t b = wave; b < ntc; b += nwaves)
-        TileOp<DT, MT>::run(wrow + b * TB, frags + b * tile_chunks, mt_stride, mpad, lane, acc);
+    for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
+        WRegs<DT> wr[P];
+        XRegs<XT, MP> xr[P];
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            const int64_t b = b0 + (int64_t)p * nwaves;
+            const int64_t bc = b < ntc ? b : b0;  // keep the address in bounds; the result is not used
+            wr[p] = load_tile<DT>(wrow + bc * TB, lane);
+            if constexpr (FUSED) xr[p] = load_x<XT, MP>(xin, ldx, m, k, bc, lane);
+        }
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            const int64_t b = b0 + (int64_t)p * nwaves;
+            if (b < ntc) {  // uniform per wave
+                if constexpr (FUSED) {
+                    const AFrags<DT, 1> f = stage_frags_lds<DT, XT, MP>(xr[p], region, lane);
+                    TileOp<DT, 1, 4>::run(wr[p], f, lane, acc);
+                } else {
+                    const AFrags<DT, MT> f =
+                        load_frags_global<DT, MT>((const half8v *)xin + b * tile_chunks, mt_stride, mpad, lane);
+                    TileOp<DT, MT, 4>::run(wr[p], f, lane, acc);
+                }
+            }
+        }
+    }
 
+    const int nn = lane & 15, g = lane >> 4;
+    const int64_t col = rt * 16 + nn;
+    if constexpr (FUSED) {
+        // only rows 0..MP-1 exist: lanes 0..15 hold them in components 0..MP-1.
+        // partial sums go to LDS as ps[row][n][wave]; wave 0 adds them up four waves per lane.
+        float *ps = (float *)red;
+        if (nwaves > 1) {
+            if (lane < 16)
+#pragma unroll
+                for (int i = 0; i < MP; i++) ps[(i * 16 + nn) * 16 + wave] = acc[0][i];
+            __syncthreads();
+            if (wave != 0) return;
+            const int n4 = lane >> 2, w4 = (lane & 3) * 4;  // lane sums waves w4..w4+3 of column n4
+#pragma unroll
+            for (int i = 0; i < MP; i++) {
+                float s = 0.f;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (w4 + j < nwaves) s += ps[(i * 16 + n4) * 16 + w4 + j];
+                s += __shfl_xor(s, 1, 64);
+                s += __shfl_xor(s, 2, 64);
+                acc[0][i] = s;  // every lane of the quad holds column n4's total
+            }
+            const int64_t c4 = rt * 16 + n4;
+            if ((lane & 3) == 0 && c4 < n) {
+                const float bv = bias ? bias[c4] : 0.0f;
+#pragma unroll
+                for (int i = 0; i < MP; i++)
+                    if (i < m) turq_store_any(y, yt, (int64_t)i * ldy + c4, acc[0][i] + bv);
+            }
+            return;
+        }
+        if (lane < 16 && col < n) {
+            const float bv = bias ? bias[col] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < MP; i++)
+                if (i < m) turq_store_any(y, yt, (int64_t)i * ldy + col, acc[0][i] + bv);
+        }
+        return;
+    }
     if (nwaves > 1) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) red[(wave * MT + mt) * 64 + lane] = acc[mt];
         __syncthreads();
         if (wave != 0) return;
-        for (int wv = 1; wv < nwaves; wv++)
+        float4v extra[MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) extra[mt] = float4v{0.f, 0.f, 0.f, 0.f};
+        int wv = 1;
+        for (; wv + 1 < nwaves; wv += 2)  // two independent chains so the LDS reads overlap
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+                acc[mt] += red[(wv * MT + mt) * 64 + lane];
+                extra[mt] += red[((wv + 1) * MT + mt) * 64 + lane];
+            }
+        if (wv < nwaves)
 #pragma unroll
             for (int mt = 0; mt < MT; mt++) acc[mt] += red[(wv * MT + mt) * 64 + lane];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[mt] += extra[mt];
     }
     // lane (nn, g) holds y[16 mt + 4 g + i][16 rt + nn], i = 0..3
-    const int nn = lane & 15, g = lane >> 4;
-    const int64_t col = rt * 16 + nn;
     if (col >= n) return;
     const float bv = bias ? bias[col] : 0.0f;
 #pragma unroll
@@ -249,49 +449,88 @@ __global__ void __launch_bounds__(512) gemv_mfma_kernel(const uint8_t *__restric
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int64_t row = 16 * mt + 4 * g + i;
-            if (row < m) turq_store_out<YT>(y, row * ldy + col, acc[mt][i] + bv);
+            if (row < m) turq_store_any(y, yt, row * ldy + col, acc[mt][i] + bv);
         }
 }
 
-template <int DT, int MT>
-hipError_t launch2(int yt, const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y, int64_t ldy,
-                   const float *bias, int nwaves, hipStream_t s) {
-    const int64_t ntc = turq_tile_cols(k);
-    const int mpad = MT > 1 ? 16 : turq_mpad(m);
-    const unsigned grid = (unsigned)turq_tile_rows(n);
-    const size_t lds = nwaves > 1 ? (size_t)nwaves * MT * 64 * sizeof(float4v) : 0;
-    const dim3 block((unsigned)(64 * nwaves));
-#define TURQ_GO(YT)                                                                                            \
-    gemv_mfma_kernel<DT, MT, YT><<<grid, block, lds, s>>>((const uint8_t *)w, n, ntc, (const half8v *)frags, m, \
-                                                           mpad, y, ldy, bias)
-    switch (yt) {
-    case TURQ_ACT_F32: TURQ_GO(TURQ_ACT_F32); break;
-    case TURQ_ACT_BF16: TURQ_GO(TURQ_ACT_BF16); break;
-    case TURQ_ACT_F16: TURQ_GO(TURQ_ACT_F16); break;
-    default: return hipErrorInvalidValue;
+struct GemvArgs {
+    const void *w; int64_t n, k; const void *xin; int64_t ldx, m; void *y; int yt; int64_t ldy; const float *bias;
+    int nwaves; hipStream_t s;
+    hipEvent_t ev_start, ev_stop;  // kernel timing: the dispatch's own begin / end timestamps (or null)
+};
+
+template <int DT, int MT, int XT, bool FUSED, int MP, int P, int MAXT>
+hipError_t launch_final(const GemvArgs &a) {
+    const int mpad = FUSED ? MP : (MT > 1 ? 16 : turq_mpad(a.m));
+    const unsigned grid = (unsigned)turq_tile_rows(a.n);
+    const size_t region = FUSED ? (size_t)MP * (512 + 64) : 0;
+    // reduction buffer: full 16x16 tiles per wave, or (fused) MP rows x 16 columns x 16 wave slots
+    const size_t red = FUSED ? (size_t)MP * 16 * 16 * sizeof(float) : (size_t)a.nwaves * MT * 64 * sizeof(float4v);
+    const size_t lds = (size_t)a.nwaves * region + (a.nwaves > 1 ? red : 0);
+    if (a.ev_start) {
+        hipExtLaunchKernelGGL((gemv_mfma_kernel<DT, MT, XT, FUSED, MP, P, MAXT>), dim3(grid), dim3((unsigned)(64 * a.nwaves)),
+                              (unsigned)lds, a.s, a.ev_start, a.ev_stop, 0, (const uint8_t *)a.w, a.n, a.k, a.xin, a.ldx, a.m,
+                              mpad, a.y, a.yt, a.ldy, a.bias);
+        return hipGetLastError();
     }
-#undef TURQ_GO
+    gemv_mfma_kernel<DT, MT, XT, FUSED, MP, P, MAXT><<<grid, dim3((unsigned)(64 * a.nwaves)), lds, a.s>>>(
+        (const uint8_t *)a.w, a.n, a.k, a.xin, a.ldx, a.m, mpad, a.y, a.yt, a.ldy, a.bias);
     return hipGetLastError();
 }
 
+// Prefetch depth by workgroup size: small groups (<= 4 waves) may use up to 512 registers per lane
+// and keep four tiles in flight; 16-wave groups are held to 128 registers and keep at most two.
+template <int DT, int MT, int XT, bool FUSED, int MP>
+hipError_t launch_p(const GemvArgs &a) {
+    const int64_t per_wave = (turq_tile_cols(a.k) + a.nwaves - 1) / a.nwaves;
+    if (a.nwaves <= 4) {
+        if (per_wave <= 1) return launch_final<DT, MT, XT, FUSED, MP, 1, 256>(a);
+        if (per_wave <= 2) return launch_final<DT, MT, XT, FUSED, MP, 2, 256>(a);
+        return launch_final<DT, MT, XT, FUSED, MP, 4, 256>(a);
+    }
+    if (per_wave <= 1 || MT > 1) return launch_final<DT, MT, XT, FUSED, MP, 1, 1024>(a);
+    return launch_final<DT, MT, XT, FUSED, MP, 2, 1024>(a);
+}
+
+template <int DT, int XT>
+hipError_t launch_fused(const GemvArgs &a) {
+    if (a.m <= 1) return launch_p<DT, 1, XT, true, 1>(a);
+    if (a.m <= 2) return launch_p<DT, 1, XT, true, 2>(a);
+    return launch_p<DT, 1, XT, true, 4>(a);
+}
+
 template <int DT>
-hipError_t launch1(int yt, const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y, int64_t ldy,
-                   const float *bias, int nwaves, hipStream_t s) {
-    if (m <= 16) return launch2<DT, 1>(yt, w, n, k, frags, m, y, ldy, bias, nwaves, s);
-    return launch2<DT, 2>(yt, w, n, k, frags, m, y, ldy, bias, nwaves, s);
+hipError_t launch_x(int xt, bool fused, const GemvArgs &a) {
+    if (!fused) {
+        if (a.m <= 16) return launch_p<DT, 1, TURQ_ACT_F16, false, 1>(a);
+        return launch_p<DT, 2, TURQ_ACT_F16, false, 1>(a);
+    }
+    switch (xt) {
+    case TURQ_ACT_F32: return launch_fused<DT, TURQ_ACT_F32>(a);
+    case TURQ_ACT_BF16: return launch_fused<DT, TURQ_ACT_BF16>(a);
+    case TURQ_ACT_F16: return launch_fused<DT, TURQ_ACT_F16>(a);
+    default: return hipErrorInvalidValue;
+    }
 }
 
 }  // namespace
 
-hipError_t turq_launch_gemv_mfma(int dtype, const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
-                                 int y_dtype, int64_t ldy, const float *bias, int nwaves, hipStream_t stream) {
+// `xin` is the prepared fragment buffer (fused == false; ldx and x_dtype unused) or the raw
+// activations (fused == true, m <= TURQ_GEMV_FUSED_MAX_M).
+hipError_t turq_launch_gemv_mfma(int dtype, const void *w, int64_t n, int64_t k, const void *xin, int x_dtype,
+                                 int64_t ldx, int64_t m, bool fused, void *y, int y_dtype, int64_t ldy,
+                                 const float *bias, int nwaves, hipStream_t stream, hipEvent_t ev_start,
+                                 hipEvent_t ev_stop) {
     if (n == 0 || m == 0) return hipSuccess;
-    if (m > TURQ_GEMV_MAX_M || nwaves < 1 || nwaves > 8) return hipErrorInvalidValue;
+    if (m > TURQ_GEMV_MAX_M || nwaves < 1 || nwaves > 16) return hipErrorInvalidValue;
+    if (fused && m > TURQ_GEMV_FUSED_MAX_M) return hipErrorInvalidValue;
+    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    const GemvArgs a{w, n, k, xin, ldx, m, y, y_dtype, ldy, bias, nwaves, stream, ev_start, ev_stop};
     switch (dtype) {
-    case TURQ_Q4_K: return launch1<TURQ_Q4_K>(y_dtype, w, n, k, frags, m, y, ldy, bias, nwaves, stream);
-    case TURQ_Q5_K: return launch1<TURQ_Q5_K>(y_dtype, w, n, k, frags, m, y, ldy, bias, nwaves, stream);
-    case TURQ_Q6_K: return launch1<TURQ_Q6_K>(y_dtype, w, n, k, frags, m, y, ldy, bias, nwaves, stream);
-    case TURQ_Q8_0: return launch1<TURQ_Q8_0>(y_dtype, w, n, k, frags, m, y, ldy, bias, nwaves, stream);
+    case TURQ_Q4_K: return launch_x<TURQ_Q4_K>(x_dtype, fused, a);
+    case TURQ_Q5_K: return launch_x<TURQ_Q5_K>(x_dtype, fused, a);
+    case TURQ_Q6_K: return launch_x<TURQ_Q6_K>(x_dtype, fused, a);
+    case TURQ_Q8_0: return launch_x<TURQ_Q8_0>(x_dtype, fused, a);
     default: return hipErrorInvalidValue;
     }
 }

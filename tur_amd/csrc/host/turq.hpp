@@ -1,0 +1,237 @@
+// C++ host-side mirror of the reference's quantized-linear interface over the libturq C ABI.
+//
+// The reference is Rust; its toolchain is not part of this build, so the host side above the C ABI
+// is given in C++ with the reference's names, argument meaning and error behaviour:
+//   turq::Device        the candle `Device` passed to `QVarBuilder::from_gguf`
+//   turq::QTensor       `Arc<QTensor>` (shared, reference counted device copy; shape, dtype, dequantize)
+//   turq::QMatMul       `QMatMul::from_arc` / `forward`
+//   turq::LinearX       src/models/layers/linear.rs:8-31 (Quantized arm: matmul, then the bias)
+//   turq::QVarBuilder   src/weights/gguf_varbuilder.rs (from_gguf, pp, get, get_no_shape, contains_key,
+//                       tensor_shape, all_keys, one-entry last-tensor cache)
+//   turq::linear()      src/models/layers/linear.rs:50-70 (GGUF arm)
+// Failures throw turq::Error (the reference returns candle_core::Error through Result).
+// Tensors here are device pointers (turq::DeviceBuffer) or host vectors; nothing computes on the CPU.
+#pragma once
+
+#include <cstdint>
+#include <memory>
+#include <mutex>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "../../../include/turq.h"
+
+namespace turq {
+
+struct Error : std::runtime_error {
+    int code;
+    Error(int c, const std::string &m) : std::runtime_error(m), code(c) {}
+};
+
+class Device {
+public:
+    explicit Device(int ordinal = 0) {
+        turq_ctx *c = nullptr;
+        int rc = turq_ctx_create(ordinal, &c);
+        if (rc != TURQ_OK) throw Error(rc, turq_last_error(nullptr));
+        ctx_ = std::shared_ptr<turq_ctx>(c, turq_ctx_destroy);
+    }
+    static Device new_hip(int ordinal) { return Device(ordinal); }
+    turq_ctx *ctx() const { return ctx_.get(); }
+    void check(int rc) const { if (rc != TURQ_OK) throw Error(rc, turq_last_error(ctx_.get())); }
+    void synchronize() const { check(turq_sync(ctx_.get())); }
+
+private:
+    std::shared_ptr<turq_ctx> ctx_;
+};
+
+// RAII device allocation for callers without HIP bindings of their own
+class DeviceBuffer {
+public:
+    DeviceBuffer(const Device &d, size_t nbytes) : dev_(d), nbytes_(nbytes) { dev_.check(turq_dev_alloc(dev_.ctx(), nbytes, &p_)); }
+    ~DeviceBuffer() { if (p_) turq_dev_free(dev_.ctx(), p_); }
+    DeviceBuffer(const DeviceBuffer &) = delete;
+    DeviceBuffer &operator=(const DeviceBuffer &) = delete;
+    void *ptr() const { return p_; }
+    size_t nbytes() const { return nbytes_; }
+    void upload(const void *src, size_t n) { dev_.check(turq_memcpy_h2d(dev_.ctx(), p_, src, n)); }
+    void download(void *dst, size_t n) const { dev_.check(turq_memcpy_d2h(dev_.ctx(), dst, p_, n)); }
+
+private:
+    Device dev_;
+    void *p_ = nullptr;
+    size_t nbytes_ = 0;
+};
+
+class QTensor {
+public:
+    QTensor(const Device &d, turq_weight *w, bool one_dim) : dev_(d), w_(w, turq_weight_release), one_dim_(one_dim) {
+        d.check(turq_weight_info(w, &dtype_, &n_, &k_, &layout_, &device_bytes_));
+    }
+    // raw GGUF block bytes of a tensor of shape (n, k)
+    static QTensor from_blocks(const Device &d, int ggml_dtype, int64_t n, int64_t k, const void *bytes, size_t nbytes,
+                               int layout = TURQ_LAYOUT_TILED) {
+        turq_weight *w = nullptr;
+        d.check(turq_weight_upload(d.ctx(), ggml_dtype, n, k, bytes, nbytes, layout, &w));
+        return QTensor(d, w, false);
+    }
+    std::vector<int64_t> shape() const { return one_dim_ ? std::vector<int64_t>{k_} : std::vector<int64_t>{n_, k_}; }
+    int dtype() const { return dtype_; }
+    int64_t rows() const { return n_; }
+    int64_t cols() const { return k_; }
+    turq_weight *handle() const { return w_.get(); }
+    const Device &device() const { return dev_; }
+    // `QTensor::dequantize(device)`: f32 values, bit-exact with candle's to_float
+    std::vector<float> dequantize() const {
+        std::vector<float> out((size_t)n_ * (size_t)k_);
+        dev_.check(turq_dequantize(dev_.ctx(), w_.get(), out.data(), TURQ_MEM_HOST));
+        return out;
+    }
+    void dequantize_to(DeviceBuffer &out) const { dev_.check(turq_dequantize(dev_.ctx(), w_.get(), (float *)out.ptr(), TURQ_MEM_DEVICE)); }
+
+private:
+    Device dev_;
+    std::shared_ptr<turq_weight> w_;  // copies share the device weight, like Arc<QTensor>
+    bool one_dim_;
+    int dtype_ = 0, layout_ = 0;
+    int64_t n_ = 0, k_ = 0;
+    size_t device_bytes_ = 0;
+};
+
+class QMatMul {
+public:
+    static QMatMul from_arc(const QTensor &t) {
+        const int dt = t.dtype();
+        if (dt != TURQ_Q8_0 && dt != TURQ_Q4_K && dt != TURQ_Q5_K && dt != TURQ_Q6_K)
+            throw Error(TURQ_ERR_DTYPE, "QMatMul needs a block-quantized tensor");
+        return QMatMul(t);
+    }
+    // host tensors: xs is [m, k] row-major f32, returns [m, n]
+    std::vector<float> forward(const std::vector<float> &xs, int64_t m, const float *bias = nullptr) const {
+        if (m < 0 || (int64_t)xs.size() != m * t_.cols()) throw Error(TURQ_ERR_SHAPE, "shape mismatch in matmul: input is not [m, k]");
+        std::vector<float> y((size_t)m * (size_t)t_.rows());
+        t_.device().check(turq_qmatmul(t_.device().ctx(), t_.handle(), xs.data(), TURQ_ACT_F32, m, t_.cols(), y.data(), TURQ_ACT_F32,
+                                       t_.rows(), bias, TURQ_MEM_HOST, TURQ_ALGO_AUTO));
+        return y;
+    }
+    // device tensors: asynchronous on the device's stream
+    void forward(const void *x_dev, int x_dtype, int64_t m, int64_t ldx, void *y_dev, int y_dtype, int64_t ldy,
+                 const float *bias_dev = nullptr) const {
+        t_.device().check(turq_qmatmul(t_.device().ctx(), t_.handle(), x_dev, x_dtype, m, ldx, y_dev, y_dtype, ldy, bias_dev,
+                                       TURQ_MEM_DEVICE, TURQ_ALGO_AUTO));
+    }
+    const QTensor &qtensor() const { return t_; }
+
+private:
+    explicit QMatMul(const QTensor &t) : t_(t) {}
+    QTensor t_;
+};
+
+// LinearX::Quantized { qmatmul, bias }: forward = qmatmul.forward(x), then broadcast_add(bias)
+class LinearX {
+public:
+    LinearX(QMatMul q, std::optional<std::vector<float>> bias) : q_(std::move(q)), bias_(std::move(bias)) {}
+    std::vector<float> forward(const std::vector<float> &x, int64_t m) const {
+        return q_.forward(x, m, bias_ ? bias_->data() : nullptr);
+    }
+    const QMatMul &qmatmul() const { return q_; }
+    const std::optional<std::vector<float>> &bias() const { return bias_; }
+    static const char *name() { return "LinearX::Quantized"; }
+
+private:
+    QMatMul q_;
+    std::optional<std::vector<float>> bias_;
+};
+
+class QVarBuilder {
+public:
+    static QVarBuilder from_gguf(const std::string &path, const Device &d, int layout = TURQ_LAYOUT_TILED) {
+        turq_gguf *g = nullptr;
+        int rc = turq_gguf_open(path.c_str(), &g);
+        if (rc != TURQ_OK) throw Error(rc, turq_gguf_last_error(nullptr));
+        QVarBuilder vb(d, layout);
+        vb.g_ = std::shared_ptr<turq_gguf>(g, turq_gguf_close);
+        vb.cache_ = std::make_shared<Cache>();
+        return vb;
+    }
+    QVarBuilder pp(const std::string &s) const {
+        QVarBuilder vb(*this);
+        vb.path_.push_back(s);
+        return vb;
+    }
+    QVarBuilder pp(int64_t i) const { return pp(std::to_string(i)); }
+    std::string path(const std::string &tensor_name) const {
+        std::string p;
+        for (const auto &s : path_) p += s + ".";
+        return p + tensor_name;
+    }
+    const Device &device() const { return dev_; }
+    bool contains_key(const std::string &key) const {
+        return turq_gguf_tensor_info(g_.get(), path(key).c_str(), nullptr, nullptr, nullptr, nullptr, nullptr) == TURQ_OK;
+    }
+    std::optional<std::vector<int64_t>> tensor_shape(const std::string &key) const {
+        int nd = 0;
+        int64_t dims[4];
+        if (turq_gguf_tensor_info(g_.get(), path(key).c_str(), nullptr, &nd, dims, nullptr, nullptr) != TURQ_OK) return std::nullopt;
+        return std::vector<int64_t>(dims, dims + nd);
+    }
+    std::vector<std::string> all_keys() const {
+        std::vector<std::string> keys;
+        for (int64_t i = 0; i < turq_gguf_tensor_count(g_.get()); i++) keys.emplace_back(turq_gguf_tensor_name(g_.get(), i));
+        return keys;
+    }
+    // get((n, k), name) / get((k), name): shape-checked, served from the one-entry cache when the name repeats
+    QTensor get(const std::vector<int64_t> &shape, const std::string &name) const {
+        const std::string full = path(name);
+        std::lock_guard<std::mutex> lock(cache_->mu);
+        if (!cache_->tensor || cache_->name != full) {
+            cache_->tensor = std::make_shared<QTensor>(load(full));
+            cache_->name = full;
+        }
+        if (cache_->tensor->shape() != shape) throw Error(TURQ_ERR_SHAPE, "shape mismatch for " + name + ", got " + fmt(cache_->tensor->shape()) + ", expected " + fmt(shape));
+        return *cache_->tensor;
+    }
+    QTensor get_no_shape(const std::string &name) const { return load(path(name)); }
+
+private:
+    struct Cache { std::mutex mu; std::string name; std::shared_ptr<QTensor> tensor; };
+    QVarBuilder(const Device &d, int layout) : dev_(d), layout_(layout) {}
+    static std::string fmt(const std::vector<int64_t> &s) {
+        std::string r = "[";
+        for (size_t i = 0; i < s.size(); i++) r += (i ? ", " : "") + std::to_string(s[i]);
+        return r + "]";
+    }
+    QTensor load(const std::string &full) const {
+        int dt = 0, nd = 0;
+        if (turq_gguf_tensor_info(g_.get(), full.c_str(), &dt, &nd, nullptr, nullptr, nullptr) != TURQ_OK)
+            throw Error(TURQ_ERR_NOT_FOUND, turq_gguf_last_error(g_.get()));
+        const bool quant = dt == TURQ_Q8_0 || dt == TURQ_Q4_K || dt == TURQ_Q5_K || dt == TURQ_Q6_K;
+        turq_weight *w = nullptr;
+        dev_.check(turq_gguf_load_weight(dev_.ctx(), g_.get(), full.c_str(), -1, -1, quant ? layout_ : TURQ_LAYOUT_NATIVE, &w));
+        return QTensor(dev_, w, nd == 1);
+    }
+    Device dev_;
+    int layout_;
+    std::shared_ptr<turq_gguf> g_;
+    std::shared_ptr<Cache> cache_;
+    std::vector<std::string> path_;
+};
+
+// GGUF arm of layers::linear: the weight stays quantized, an optional bias is dequantized at load (`.ok()`)
+inline LinearX linear(int64_t in_dim, int64_t out_dim, const QVarBuilder &vb) {
+    QTensor qweight = vb.get({out_dim, in_dim}, "weight");
+    std::optional<std::vector<float>> bias;
+    if (vb.contains_key("bias")) {
+        try {
+            bias = vb.get({out_dim}, "bias").dequantize();
+        } catch (const Error &) {
+            bias.reset();
+        }
+    }
+    return LinearX(QMatMul::from_arc(qweight), std::move(bias));
+}
+
+}  // namespace turq

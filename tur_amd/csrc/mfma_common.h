@@ -34,6 +34,8 @@ typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
 #define TURQ_NQ_KQUANT 9
 #define TURQ_NQ_Q8_0 8
+// up to this many rows the GEMV kernel prepares the activations itself (no separate launch)
+#define TURQ_GEMV_FUSED_MAX_M 4
 
 __host__ __device__ inline int turq_mpad(int64_t rows) {
     return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : rows <= 8 ? 8 : 16;
@@ -50,8 +52,15 @@ __host__ __device__ inline size_t turq_act_prep_bytes(int dt, int64_t m, int64_t
 __device__ inline half2v as_half2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
 __device__ inline uint32_t as_u32(half2v h) { return __builtin_bit_cast(uint32_t, h); }
 
-// (w & mask) | magic as a packed f16 pair: one v_and_or_b32
-__device__ inline half2v and_or_h2(uint32_t w, uint32_t mask, uint32_t magic) { return as_half2((w & mask) | magic); }
+// (w & mask) | magic in ONE instruction.  v_and_or_b32 is a VOP3 encoding, which on this ISA takes no
+// literal operands; left to itself the compiler prefers v_and_b32 + v_or_b32 with literals.  Here the
+// (wave-uniform) mask is forced into a scalar register and the magic into a vector register.
+__device__ inline uint32_t and_or_u32(uint32_t w, uint32_t mask, uint32_t magic) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "s"(mask), "v"(magic));
+    return r;
+}
+__device__ inline half2v and_or_h2(uint32_t w, uint32_t mask, uint32_t magic) { return as_half2(and_or_u32(w, mask, magic)); }
 
 // fused multiply-add on a packed pair (v_pk_fma_f16): must stay fused, the intermediate product
 // (base + v) * scale does not fit f16 on its own
@@ -90,6 +99,7 @@ template <int YT> __device__ inline void turq_store_out(void *y, int64_t i, floa
 // launchers (act_prep.hip, gemv_mfma.hip)
 hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
                                 hipStream_t stream);
-hipError_t turq_launch_gemv_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *frags, int64_t m,
-                                 void *y, int y_dtype, int64_t ldy, const float *bias, int waves_per_group,
-                                 hipStream_t stream);
+hipError_t turq_launch_gemv_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *xin, int x_dtype,
+                                 int64_t ldx, int64_t m, bool fused, void *y, int y_dtype, int64_t ldy,
+                                 const float *bias, int waves_per_group, hipStream_t stream, hipEvent_t ev_start,
+                                 hipEvent_t ev_stop);

@@ -1,5 +1,6 @@
 // Host side of the MFMA paths: prepare the activations, pick the launch shape, launch.
 #include <algorithm>
+#include <cstdlib>
 
 #include "layout.h"
 #include "mfma_common.h"
@@ -9,11 +10,13 @@ namespace {
 // Waves per workgroup (= how many ways a row tile's columns are split).  Enough waves to cover the
 // machine a few times over, never more than there are column tiles.
 int pick_waves(const turq_ctx *ctx, int64_t n, int64_t k) {
+    static const int forced = [] { const char *e = getenv("TURQ_GEMV_WAVES"); return e ? atoi(e) : 0; }();
+    if (forced >= 1 && forced <= 16) return (int)std::min<int64_t>(forced, turq_tile_cols(k));
     const int64_t row_tiles = turq_tile_rows(n);
     const int64_t col_tiles = turq_tile_cols(k);
     const int64_t want_waves = (int64_t)(ctx->compute_units > 0 ? ctx->compute_units : 256) * 12;
     int64_t w = (want_waves + row_tiles - 1) / row_tiles;
-    w = std::max<int64_t>(1, std::min<int64_t>({w, col_tiles, 8}));
+    w = std::max<int64_t>(1, std::min<int64_t>({w, col_tiles, 16}));
     return (int)w;
 }
 
@@ -26,13 +29,23 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
     const int nwaves = pick_waves(ctx, w->n, w->k);
     for (int64_t m0 = 0; m0 < m; m0 += TURQ_GEMV_MAX_M) {
         const int64_t mc = std::min<int64_t>(TURQ_GEMV_MAX_M, m - m0);
-        int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep_bytes(w->dtype, mc, w->k));
-        if (rc != TURQ_OK) return rc;
         const uint8_t *xc = (const uint8_t *)x + (size_t)m0 * (size_t)ldx * xb;
         uint8_t *yc = (uint8_t *)y + (size_t)m0 * (size_t)ldy * yb;
+        static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
+        hipEvent_t ev0 = nullptr, ev1 = nullptr;
+        TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+        // raw activation rows must be 16-byte (f32) / 8-byte (16-bit) aligned for the fused loads
+        const bool aligned = ((uintptr_t)xc % 16 == 0) && ((size_t)ldx * xb) % 16 == 0;
+        if (mc <= TURQ_GEMV_FUSED_MAX_M && aligned && !no_fuse) {
+            TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, xc, xt, ldx, mc, true, yc, yt, ldy, bias,
+                                                nwaves, ctx->stream, ev0, ev1));
+            continue;
+        }
+        int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep_bytes(w->dtype, mc, w->k));
+        if (rc != TURQ_OK) return rc;
         TURQ_HIP(ctx, turq_launch_act_prep(w->dtype, xc, xt, mc, w->k, ldx, ctx->act_prep, ctx->stream));
-        TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, mc, yc, yt, ldy, bias, nwaves,
-                                            ctx->stream));
+        TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, TURQ_ACT_F16, 0, mc, false, yc, yt,
+                                            ldy, bias, nwaves, ctx->stream, ev0, ev1));
     }
     return TURQ_OK;
 }

@@ -1,0 +1,245 @@
+"""Host-side mirror of the reference's quantized-linear interface, on top of the C ABI.
+
+Same names, argument meaning and error behaviour as the reference so that tests read like its own:
+
+* ``Device``          — the ``candle_core::Device`` handed to ``QVarBuilder::from_gguf`` (a libturq context);
+* ``QTensor``         — ``candle_core::quantized::QTensor``: raw blocks on the device, ``shape()``, ``dtype()``,
+                        ``dequantize()``; clones share one device copy (``Arc<QTensor>``);
+* ``QMatMul``         — ``QMatMul::from_arc(qtensor)`` + ``forward(x)``;
+* ``LinearX``         — ``src/models/layers/linear.rs:8-31``: ``Quantized{qmatmul, bias}``, ``forward`` adds the bias;
+* ``QVarBuilder``     — ``src/weights/gguf_varbuilder.rs``: ``from_gguf``, ``pp``, ``get``, ``get_no_shape``,
+                        ``contains_key``, ``tensor_shape``, ``all_keys``, with the one-entry last-tensor cache;
+* ``linear(in_dim, out_dim, vb)`` — ``src/models/layers/linear.rs:50-70`` (GGUF arm).
+
+Activations and results are NumPy arrays on the host here (this mirror is for tests and scripting; an engine
+binds the C ABI directly and keeps its tensors on the device).
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import capi, synth
+from .capi import TurqError
+
+
+class Device:
+    """One GPU context (device ordinal + stream + scratch)."""
+
+    def __init__(self, ordinal: int = 0):
+        self.L = capi.lib()
+        h = ctypes.c_void_p()
+        capi.check(self.L.turq_ctx_create(ordinal, ctypes.byref(h)))
+        self.ctx = h
+        self.ordinal = ordinal
+
+    @staticmethod
+    def new_hip(ordinal: int = 0) -> "Device":
+        return Device(ordinal)
+
+    def synchronize(self) -> None:
+        capi.check(self.L.turq_sync(self.ctx), self.ctx)
+
+    def close(self) -> None:
+        if self.ctx:
+            self.L.turq_ctx_destroy(self.ctx)
+            self.ctx = None
+
+
+class QTensor:
+    """Quantized (or dense F32/F16/BF16) GGUF tensor resident in HBM."""
+
+    def __init__(self, device: Device, handle, owns: bool = True):
+        self.device = device
+        self.handle = handle
+        self._owns = owns
+        dt, n, k, layout, nbytes = ctypes.c_int(), ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int(), ctypes.c_size_t()
+        capi.check(device.L.turq_weight_info(handle, ctypes.byref(dt), ctypes.byref(n), ctypes.byref(k), ctypes.byref(layout),
+                                             ctypes.byref(nbytes)))
+        self._dtype, self._n, self._k, self._layout, self._nbytes = dt.value, n.value, k.value, layout.value, nbytes.value
+        self._one_dim = False
+
+    @classmethod
+    def new(cls, device: Device, ggml_dtype: int, shape: Sequence[int], raw, layout: int = capi.LAYOUT_TILED) -> "QTensor":
+        """raw GGUF block bytes of a tensor of ``shape`` = (n, k) or (k,)"""
+        raw = np.ascontiguousarray(raw).view(np.uint8).reshape(-1)
+        n, k = (1, shape[0]) if len(shape) == 1 else (shape[0], shape[1])
+        if not (ggml_dtype in (capi.Q8_0, capi.Q4_K, capi.Q5_K, capi.Q6_K)):
+            layout = capi.LAYOUT_NATIVE
+        h = ctypes.c_void_p()
+        capi.check(device.L.turq_weight_upload(device.ctx, ggml_dtype, n, k, capi.ptr(raw), raw.size, layout, ctypes.byref(h)),
+                   device.ctx)
+        t = cls(device, h)
+        t._one_dim = len(shape) == 1
+        return t
+
+    def shape(self) -> Tuple[int, ...]:
+        return (self._k,) if self._one_dim else (self._n, self._k)
+
+    def dtype(self) -> int:
+        return self._dtype
+
+    def clone(self) -> "QTensor":
+        capi.check(self.device.L.turq_weight_retain(self.handle))
+        t = QTensor(self.device, self.handle)
+        t._one_dim = self._one_dim
+        return t
+
+    def dequantize(self, device: Optional[Device] = None) -> np.ndarray:
+        """f32 array of ``shape()`` — bit-exact with candle's ``QTensor::dequantize``"""
+        dev = device or self.device
+        out = np.empty(self._n * self._k, np.float32)
+        capi.check(dev.L.turq_dequantize(dev.ctx, self.handle, capi.ptr(out), capi.MEM_HOST), dev.ctx)
+        return out.reshape(self.shape())
+
+    def release(self) -> None:
+        if self._owns and self.handle:
+            self.device.L.turq_weight_release(self.handle)
+            self.handle = None
+
+    def __del__(self):  # Arc drop
+        try:
+            self.release()
+        except Exception:
+            pass
+
+
+class QMatMul:
+    """``QMatMul::from_arc`` + ``forward``: y = x @ W.T for x of shape [..., k]."""
+
+    def __init__(self, qtensor: QTensor):
+        if qtensor.dtype() not in (capi.Q8_0, capi.Q4_K, capi.Q5_K, capi.Q6_K):
+            raise TurqError(capi.ERR_DTYPE, "QMatMul needs a block-quantized tensor; dequantize F32/F16/BF16 tensors")
+        self.qtensor = qtensor
+
+    @classmethod
+    def from_arc(cls, qtensor: QTensor) -> "QMatMul":
+        return cls(qtensor)
+
+    def forward(self, xs: np.ndarray, bias: Optional[np.ndarray] = None, algo: int = capi.ALGO_AUTO) -> np.ndarray:
+        q = self.qtensor
+        n, k = q._n, q._k
+        xs = np.asarray(xs)
+        if xs.ndim < 2:
+            raise TurqError(capi.ERR_SHAPE, f"QMatMul::forward needs rank >= 2, got shape {xs.shape}")
+        if xs.shape[-1] != k:
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch in matmul: last dim {xs.shape[-1]} != {k}")
+        if xs.dtype == np.float32:
+            xt = capi.ACT_F32
+        elif xs.dtype == np.float16:
+            xt = capi.ACT_F16
+        else:
+            raise TurqError(capi.ERR_DTYPE, f"unsupported activation dtype {xs.dtype}")
+        if not xs.flags["C_CONTIGUOUS"]:
+            raise TurqError(capi.ERR_INVALID, "QMatMul::forward needs a contiguous input")
+        lead = xs.shape[:-1]
+        m = int(np.prod(lead)) if lead else 1
+        y = np.empty((m, n), np.float32)
+        b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+        dev = q.device
+        capi.check(dev.L.turq_qmatmul(dev.ctx, q.handle, capi.ptr(xs), xt, m, k, capi.ptr(y), capi.ACT_F32, n, capi.ptr(b),
+                                      capi.MEM_HOST, algo), dev.ctx)
+        return y.reshape(lead + (n,))
+
+
+class LinearX:
+    """``LinearX::Quantized { qmatmul, bias }`` (src/models/layers/linear.rs:8-31)."""
+
+    def __init__(self, qmatmul: QMatMul, bias: Optional[np.ndarray] = None):
+        self.qmatmul = qmatmul
+        self.bias = bias
+
+    def forward(self, x: np.ndarray) -> np.ndarray:
+        return self.qmatmul.forward(x, bias=self.bias)
+
+    def __repr__(self) -> str:
+        return "LinearX::Quantized"
+
+
+class QVarBuilder:
+    """``src/weights/gguf_varbuilder.rs``: GGUF header parsed once, tensors read lazily."""
+
+    def __init__(self, device: Device, gguf, path: List[str], cache: list, layout: int):
+        self._device = device
+        self._g = gguf
+        self._path = path
+        self._cache = cache          # shared one-entry [name, tensor] cache
+        self._layout = layout
+
+    @classmethod
+    def from_gguf(cls, p: str, device: Device, layout: int = capi.LAYOUT_TILED) -> "QVarBuilder":
+        g = ctypes.c_void_p()
+        capi.check(device.L.turq_gguf_open(str(p).encode(), ctypes.byref(g)))
+        return cls(device, g, [], [None, None], layout)
+
+    def pp(self, s) -> "QVarBuilder":
+        return QVarBuilder(self._device, self._g, self._path + [str(s)], self._cache, self._layout)
+
+    def path(self, tensor_name: str) -> str:
+        return tensor_name if not self._path else ".".join(self._path) + "." + tensor_name
+
+    def device(self) -> Device:
+        return self._device
+
+    def _load(self, full: str, shape) -> QTensor:
+        L, dev = self._device.L, self._device
+        dt, nd, nb = ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t()
+        dims = (ctypes.c_int64 * 4)()
+        off = ctypes.c_uint64()
+        capi.check(L.turq_gguf_tensor_info(self._g, full.encode(), ctypes.byref(dt), ctypes.byref(nd), dims, ctypes.byref(off),
+                                           ctypes.byref(nb)))
+        got = tuple(dims[i] for i in range(nd.value))
+        layout = self._layout if dt.value in (capi.Q8_0, capi.Q4_K, capi.Q5_K, capi.Q6_K) else capi.LAYOUT_NATIVE
+        h = ctypes.c_void_p()
+        capi.check(L.turq_gguf_load_weight(dev.ctx, self._g, full.encode(), -1, -1, layout, ctypes.byref(h)), dev.ctx)
+        t = QTensor(dev, h)
+        t._one_dim = nd.value == 1
+        return t
+
+    def get(self, s, name: str) -> QTensor:
+        shape = (s,) if isinstance(s, int) else tuple(s)
+        full = self.path(name)
+        if self._cache[0] == full:
+            t = self._cache[1]
+        else:
+            t = self._load(full, shape)
+            self._cache[0], self._cache[1] = full, t
+        if t.shape() != shape:
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch for {name}, got {list(t.shape())}, expected {list(shape)}")
+        return t.clone()
+
+    def get_no_shape(self, name: str) -> QTensor:
+        return self._load(self.path(name), None)
+
+    def contains_key(self, key: str) -> bool:
+        return self._device.L.turq_gguf_tensor_info(self._g, self.path(key).encode(), None, None, None, None, None) == capi.OK
+
+    def tensor_shape(self, key: str):
+        nd = ctypes.c_int()
+        dims = (ctypes.c_int64 * 4)()
+        rc = self._device.L.turq_gguf_tensor_info(self._g, self.path(key).encode(), None, ctypes.byref(nd), dims, None, None)
+        return None if rc != capi.OK else [dims[i] for i in range(nd.value)]
+
+    def all_keys(self) -> List[str]:
+        L = self._device.L
+        return [L.turq_gguf_tensor_name(self._g, i).decode() for i in range(L.turq_gguf_tensor_count(self._g))]
+
+    def metadata_u64(self, key: str) -> int:
+        v = ctypes.c_uint64()
+        capi.check(self._device.L.turq_gguf_meta_u64(self._g, key.encode(), ctypes.byref(v)))
+        return v.value
+
+
+def linear(in_dim: int, out_dim: int, vb: QVarBuilder) -> LinearX:
+    """GGUF arm of ``layers::linear`` (src/models/layers/linear.rs:59-70): weight stays quantized, an optional
+    bias tensor is dequantized at load."""
+    qweight = vb.get((out_dim, in_dim), "weight")
+    bias = None
+    if vb.contains_key("bias"):
+        try:
+            bias = vb.get(out_dim, "bias").dequantize(vb.device()).reshape(-1)
+        except TurqError:
+            bias = None     # the reference looks the bias up with `.ok()`
+    return LinearX(QMatMul.from_arc(qweight), bias)
