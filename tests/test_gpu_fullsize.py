@@ -63,3 +63,20 @@ def test_lm_head(gpu, dt):
     sub = raw.reshape(n, -1)[rows].reshape(-1)
     assert rel_l2(y16[:, rows], orc.matmul_dequant(dt, x16, sub, len(rows), k)) <= 2e-5
     gpu.release(w)
+
+
+@pytest.mark.parametrize("m", [512, 2048])
+def test_prefill_up_proj(gpu, m):
+    # BASELINE config 4: Q4_K up_proj 12288 x 4096, bf16 activations [m, 4096]; the oracle checks every 16th
+    # weight row (768 rows spread over all workgroups) to keep the CPU time bounded
+    n, k = 12288, 4096
+    raw = synth.random_weight(Q4_K, n, k, seed=44)
+    w = gpu.upload(Q4_K, n, k, raw, capi.LAYOUT_TILED)
+    x = synth.random_activation(m, k, seed=m, bf16=True)
+    y = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    gpu.release(w)
+    rows = np.arange(5, n, 16)
+    sub = raw.reshape(n, -1)[rows].reshape(-1)
+    want = orc.matmul_dequant(Q4_K, x, sub, len(rows), k)
+    assert np.all(np.isfinite(y))
+    assert rel_l2(y[:, rows], want) <= 1e-3

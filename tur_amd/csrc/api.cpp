@@ -1,4 +1,5 @@
 // C ABI of libturq: contexts, device memory helpers, weight upload/export, dequantize, forward.
+#include <cmath>
 #include <memory>
 #include <new>
 #include <vector>
@@ -45,6 +46,23 @@ hipError_t turq_prof_next(turq_ctx *ctx, hipEvent_t *start, hipEvent_t *stop) {
 }
 
 namespace {
+
+float half_bits_to_float(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu, bits;
+    if (exp == 0) {
+        if (man == 0) bits = sign;
+        else {
+            int e = -1;
+            do { man <<= 1; e++; } while (!(man & 0x400u));
+            bits = sign | ((uint32_t)(112 - e) << 23) | ((man & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) bits = sign | 0x7F800000u | (man << 13);
+    else bits = sign | ((exp + 112u) << 23) | (man << 13);
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
 
 struct DeviceGuard {  // make ctx's device current for the duration of a call
     int prev = -1;
@@ -199,6 +217,16 @@ int turq_weight_upload(turq_ctx *ctx, int dt, int64_t n, int64_t k, const void *
     w->k = k;
     w->native_bytes = nbytes;
     const uint8_t *src = (const uint8_t *)host_bytes;
+    if (dt == TURQ_Q4_K) {  // bound on d * sc (6-bit scale <= 63), see turq_weight::max_scale
+        float mx = 0.0f;
+        const int64_t nblk = n * (k / 256);
+        for (int64_t i = 0; i < nblk; i++) {
+            const uint8_t *b = src + i * 144;
+            const float d = std::fabs(half_bits_to_float((uint16_t)(b[0] | (b[1] << 8))));
+            if (d > mx || d != d) mx = d;
+        }
+        w->max_scale = mx * 63.0f;
+    }
     std::vector<uint8_t> tiled;
     if (layout == TURQ_LAYOUT_TILED) {
         w->dev_bytes = turq_tiled_nbytes(dt, n, k);

@@ -99,6 +99,9 @@ struct turq_weight {
     void *dev = nullptr;      // weight bytes in HBM (native or tiled)
     size_t dev_bytes = 0;     // allocation size
     size_t native_bytes = 0;  // n * k / blk * block_bytes
+    // largest |d| * (largest block scale) over the tensor: the prefill GEMM folds d into f16 constants
+    // scaled by 1024 and is only used while that cannot overflow f16
+    float max_scale = 0.0f;
 };
 
 // ---- error plumbing ----

@@ -103,3 +103,6 @@ hipError_t turq_launch_gemv_mfma(int dtype, const void *w_tiled, int64_t n, int6
                                  int64_t ldx, int64_t m, bool fused, void *y, int y_dtype, int64_t ldy,
                                  const float *bias, int waves_per_group, hipStream_t stream, hipEvent_t ev_start,
                                  hipEvent_t ev_stop);
+hipError_t turq_launch_gemm_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
+                                 int y_dtype, int64_t ldy, const float *bias, hipStream_t stream, hipEvent_t ev_start,
+                                 hipEvent_t ev_stop);

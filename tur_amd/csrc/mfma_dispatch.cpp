@@ -24,8 +24,20 @@ int pick_waves(const turq_ctx *ctx, int64_t n, int64_t k) {
 
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
                       int yt, int64_t ldy, const float *bias, int algo) {
-    (void)algo;
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
+    // prefill chunks: LDS-tiled MFMA GEMM (Q4_K; needs d * sc * 1024 to stay inside f16)
+    const bool gemm_ok = w->dtype == TURQ_Q4_K && w->max_scale * 1024.0f < 60000.0f;
+    if (algo == TURQ_ALGO_GEMM && !gemm_ok && m > TURQ_GEMV_MAX_M)
+        algo = TURQ_ALGO_GEMV;  // formats without a GEMM kernel yet: walk m in chunks through the skinny kernel
+    if (m > TURQ_GEMV_MAX_M && algo == TURQ_ALGO_GEMM) {
+        int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep_bytes(w->dtype, m, w->k));
+        if (rc != TURQ_OK) return rc;
+        hipEvent_t ev0 = nullptr, ev1 = nullptr;
+        TURQ_HIP(ctx, turq_launch_act_prep(w->dtype, x, xt, m, w->k, ldx, ctx->act_prep, ctx->stream));
+        TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+        TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, ctx->stream, ev0, ev1));
+        return TURQ_OK;
+    }
     const int nwaves = pick_waves(ctx, w->n, w->k);
     for (int64_t m0 = 0; m0 < m; m0 += TURQ_GEMV_MAX_M) {
         const int64_t mc = std::min<int64_t>(TURQ_GEMV_MAX_M, m - m0);
