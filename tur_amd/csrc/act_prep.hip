@@ -73,6 +73,49 @@ hipError_t launch(int dtype, const void *x, int64_t m, int64_t k, int64_t ldx, v
     return hipGetLastError();
 }
 
+// ---- fragments for the prefill GEMM (v_mfma_f32_32x32x16_f16) ----
+// 32-row m-tiles; per 256-column tile b there are 16 operand steps plus one group-sum step.  Lane
+// (r, g32) = r + 32 * g32 of step q holds x[32 mt + r][256 b + 128 g32 + 8 q + j], j = 0..7; step 16
+// holds for the four 32-column sub-blocks of the lane's 128 columns the sums of the f16-rounded
+// activations as (hi, lo) f16 pairs.  chunk index = ((mt * ntc + b) * 17 + q) * 64 + lane.
+template <int XT>
+__global__ void __launch_bounds__(256) act_prep32_kernel(const void *__restrict__ x, int64_t m, int64_t k, int64_t ldx,
+                                                         int64_t ntc, int64_t nchunks, half8v *__restrict__ frags) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= nchunks) return;
+    const int lane = (int)(t & 63);
+    const int64_t blk = t >> 6;            // (mt * ntc + b) * 17 + q
+    const int q = (int)(blk % 17);
+    const int64_t tb = blk / 17;
+    const int64_t b = tb % ntc, mt = tb / ntc;
+    const int r = lane & 31, g32 = lane >> 5;
+    const int64_t row = mt * 32 + r;
+    const bool row_ok = row < m;
+    half8v h;
+    if (q < 16) {
+        const int64_t col0 = b * 256 + 128 * g32 + 8 * q;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int64_t c = col0 + j;
+            h[j] = (_Float16)((row_ok && c < k) ? ld_act<XT>(x, row * ldx + c) : 0.0f);
+        }
+    } else {
+#pragma unroll
+        for (int sb = 0; sb < 4; sb++) {
+            const int64_t col0 = b * 256 + 128 * g32 + 32 * sb;
+            float sum = 0.0f;
+            for (int j = 0; j < 32; j++) {
+                const int64_t c = col0 + j;
+                sum += (float)(_Float16)((row_ok && c < k) ? ld_act<XT>(x, row * ldx + c) : 0.0f);
+            }
+            const _Float16 hi = (_Float16)sum;
+            h[2 * sb] = hi;
+            h[2 * sb + 1] = (_Float16)(sum - (float)hi);
+        }
+    }
+    frags[t] = h;
+}
+
 }  // namespace
 
 hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
@@ -84,4 +127,18 @@ hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m
     case TURQ_ACT_F16: return launch<TURQ_ACT_F16>(dtype, x, m, k, ldx, frags, stream);
     default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t turq_launch_act_prep32(const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags, hipStream_t stream) {
+    if (m == 0 || k == 0) return hipSuccess;
+    const int64_t ntc = (k + 255) / 256;
+    const int64_t nchunks = ((m + 31) / 32) * ntc * 17 * 64;
+    const unsigned grid = (unsigned)((nchunks + 255) / 256);
+    switch (x_dtype) {
+    case TURQ_ACT_F32: act_prep32_kernel<TURQ_ACT_F32><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, nchunks, (half8v *)frags); break;
+    case TURQ_ACT_BF16: act_prep32_kernel<TURQ_ACT_BF16><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, nchunks, (half8v *)frags); break;
+    case TURQ_ACT_F16: act_prep32_kernel<TURQ_ACT_F16><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, nchunks, (half8v *)frags); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
 }

@@ -96,7 +96,13 @@ template <int YT> __device__ inline void turq_store_out(void *y, int64_t i, floa
 }
 #endif
 
+// bytes of the prefill GEMM's fragment buffer (32-row m-tiles, 17 steps of 1 KiB per column tile)
+__host__ __device__ inline size_t turq_act_prep32_bytes(int64_t m, int64_t k) {
+    return (size_t)((m + 31) / 32) * (size_t)((k + 255) / 256) * 17u * 1024u;
+}
+
 // launchers (act_prep.hip, gemv_mfma.hip)
+hipError_t turq_launch_act_prep32(const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags, hipStream_t stream);
 hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
                                 hipStream_t stream);
 hipError_t turq_launch_gemv_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *xin, int x_dtype,

@@ -30,10 +30,10 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
     if (algo == TURQ_ALGO_GEMM && !gemm_ok && m > TURQ_GEMV_MAX_M)
         algo = TURQ_ALGO_GEMV;  // formats without a GEMM kernel yet: walk m in chunks through the skinny kernel
     if (m > TURQ_GEMV_MAX_M && algo == TURQ_ALGO_GEMM) {
-        int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep_bytes(w->dtype, m, w->k));
+        int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep32_bytes(m, w->k));
         if (rc != TURQ_OK) return rc;
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
-        TURQ_HIP(ctx, turq_launch_act_prep(w->dtype, x, xt, m, w->k, ldx, ctx->act_prep, ctx->stream));
+        TURQ_HIP(ctx, turq_launch_act_prep32(x, xt, m, w->k, ldx, ctx->act_prep, ctx->stream));
         TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
         TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, ctx->stream, ev0, ev1));
         return TURQ_OK;
