@@ -3,18 +3,36 @@
 //
 // MFMA shape.  v_mfma_f32_32x32x16_f16: on MI355X it sustains about 2.1 PFLOP/s in a register-only
 // loop, the 16x16x32 form only about 1.4, so the GEMM uses 32x32 tiles (the skinny kernel keeps
-// 16x16x32 because its limit is HBM, not the matrix pipe).
+// 16x16x32 because its limit is HBM, not the matrix pipe).  Vector ALU work of the same SIMD is NOT
+// hidden under the MFMAs (about 2 cycles per VALU instruction on top of the 32 of an MFMA, also with
+// two waves per SIMD), so the loop is written to spend as few other instructions as it can.
 //
-// Tiling.  Workgroup tile 256 (m) x 96 (n), 4 waves stacked along m; wave tile 64 x 96 = 2 x 3 MFMA
-// tiles (96 accumulator registers).  Activations arrive prepared in 32-row A-fragment order
-// (act_prep32_kernel) and are copied global -> LDS by global_load_lds_dwordx4 (no registers, no
-// ds_write), 64 columns (4 operand steps) per stage, three stage buffers, loads issued two stages
-// ahead, one barrier per stage.  Weights do NOT go through LDS: each wave loads the packed bytes of
-// its six row tiles straight into registers and unpacks them with the and_or / pk_fma arithmetic of
-// the skinny kernel; one unpacked B operand (32 rows x 16 columns) feeds two MFMAs.
+// Tiling.  Workgroup tile 128 (m) x 192 (n), 4 waves as 2 x 2, wave tile 64 x 96 = 2 x 3 MFMA tiles
+// (96 accumulator registers).  The activations are the expensive operand here (2 bytes per element
+// against 0.56 for the weights), hence the wide n.
+//
+// Everything reaches the LDS by global_load_lds_dwordx4 (no registers, no ds_write):
+//   * activations, prepared in 32-row A-fragment order (act_prep32_kernel), 64 columns (4 operand
+//     steps) of the workgroup's 4 m-tiles per stage = 16 KiB, ring of 4 stages; stage s + 4 is issued
+//     as soon as every wave is done with stage s;
+//   * the packed weight tiles of the workgroup's 12 row tiles, 27 KiB per super-block, ring of 3,
+//     issued two super-blocks ahead in four groups, because they come from HBM and loads of one wave
+//     retire in order: a late weight load delays every younger activation load of that wave;
+//   * the activation sub-block sums of the 4 m-tiles, 4 KiB per super-block, ring of 2.
+// Every wave issues the same number of copies at every stage boundary (4 + 2, + 1 sums block at the
+// first of a super-block; past the end they repeat the last super-block into buffers nobody reads),
+// so the "at most N copies outstanding" waits are compile-time constants.  There is one barrier per
+// stage; it sits before the last operand step of the previous stage, so that the first LDS reads of
+// the new stage run under those MFMAs.
+//
+// LDS reads and the copies are written as asm with hand-placed waits: the compiler counts an LDS-DMA
+// copy both as a memory and as an LDS event and from then on waits for lgkmcnt(0) at every LDS use,
+// and __syncthreads() would drain the copies that are meant to stay in flight.
+//
 //   B operand of 32 rows = two 16-row tiles: lane l = n32 + 32 * g32 reads row r = n32 % 16 of tile
 //   n32 / 16 and takes the tile's lane slots 2 * g32 and 2 * g32 + 1 (columns 128 * g32 .. +127 of
 //   the super-block), 16 operand steps of 8 columns each; the activation fragments use the same order.
+//   Stage ks of a super-block is the lane's sub-block ks: one 16-byte LDS read per 32-row tile.
 //
 // Block scales.  The skinny kernel keeps the weights as exact integers and applies d / dmin in f32 on
 // each tile result; with 96 accumulators that would need a second accumulator set.  Here the f16
@@ -23,10 +41,18 @@
 // the activation sub-block sums with B = -f16(dmin * m).  Against the f32 matmul on dequantized
 // weights this costs about 3e-4 relative L2 (bar: 1e-3).  The dispatcher only uses this kernel while
 // 1024 * d * sc stays inside f16.
+//
+// Results leave through the LDS (free after the main loop): each wave transposes its 64 x 96 tile so
+// that a lane stores 16 contiguous bytes and a row segment is 192 (bf16, f16) or 384 (f32) bytes.
 #include <hip/hip_ext.h>
+
+#include <type_traits>
+#include <utility>
 
 #include "layout.h"
 #include "mfma_common.h"
+
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is named as a clobber on purpose
 
 namespace {
 
@@ -34,11 +60,31 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kMagic1024 = 0x64006400u;  // 1024.0: a nibble in mantissa bits 0..3 reads as 1024 + n
 constexpr uint32_t kMagic64 = 0x54005400u;    // 64.0:   a nibble in mantissa bits 4..7 reads as 64 + n
-constexpr int BM = 256, BN = 96;              // workgroup tile
+constexpr int WGM = 2, WGN = 2;               // waves of a workgroup along m and n
 constexpr int WM = 2, WN = 3;                 // 32x32 MFMA tiles per wave: 64 x 96
-constexpr int STAGE_STEPS = 4;                // operand steps (16 columns each) per LDS stage
-constexpr int STAGE_BYTES = STAGE_STEPS * (BM / 32) * 1024;  // 32 KiB
-constexpr int NBUF = 3;
+constexpr int BM = WGM * WM * 32, BN = WGN * WN * 32;  // 128 x 192
+constexpr int MT = BM / 32;                   // m-tiles per workgroup; wave w copies m-tile w
+constexpr int NT16 = BN / 16;                 // 16-row weight tiles per workgroup
+constexpr int TB = TiledFmt<TURQ_Q4_K>::kTileBytes;  // 2304: [QA 1024][QB 1024][HDR 256]
+constexpr int A_STAGE = MT * 4 * 1024;        // [m-tile][step] blocks of 1 KiB
+constexpr int NA = 4;                         // stage ring; 4 stages per super-block, so stage ks lives in buffer ks
+constexpr int W_BYTES = NT16 * TB;            // 27648 = 27 copies of 1 KiB
+constexpr int W_CHUNKS = W_BYTES / 1024;
+constexpr int NW = 3;
+constexpr int S_BYTES = MT * 1024;
+constexpr int NS = 2;
+constexpr int A_OFF = 0, W_OFF = NA * A_STAGE, S_OFF = W_OFF + NW * W_BYTES;
+constexpr int LDS_BYTES = S_OFF + NS * S_BYTES;  // 156672
+constexpr int OUT_PITCH = 104;                // floats per staged result row: rows r and r + 4 land 32 banks apart
+static_assert(MT == 4 && WGM * WGN == 4 && WM == 2 && WN == 3, "the copy and read schedules below are written for this shape");
+static_assert(W_BYTES % 1024 == 0 && W_CHUNKS <= 32, "weight copies: two per wave and group");
+static_assert(4 * 64 * OUT_PITCH * 4 <= LDS_BYTES, "result staging fits");
+
+template <int... I, typename F> __device__ inline void static_for_impl(std::integer_sequence<int, I...>, F &&f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): loop indices usable as template arguments
+template <int N, typename F> __device__ inline void static_for(F &&f) { static_for_impl(std::make_integer_sequence<int, N>{}, f); }
 
 __device__ inline _Float16 h_from_bits(uint32_t bits16) {
     const uint16_t u = (uint16_t)bits16;
@@ -55,38 +101,31 @@ __device__ inline float16v mfma32x32x16(half8v a, half8v b, float16v c) {
 template <int N> __device__ inline void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
+// wait until at most N of this wave's LDS reads are outstanding
+template <int N> __device__ inline void wait_lds() { asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory"); }
+// a value read by lds_read128 may be used only after a wait; passing it through an (empty) volatile
+// statement placed after that wait keeps its users from being scheduled ahead of the wait
+template <typename T> __device__ inline void pin(T &v) { asm volatile("" : "+v"(v)); }
 
-// LDS reads of the activation fragments are written as asm with hand-placed waits: the compiler counts an
-// LDS-DMA copy as both a memory and an LDS event and from then on waits for lgkmcnt(0) at every LDS use, which
-// would serialise each read with the MFMAs that follow it.
-template <int OFF> __device__ inline half8v lds_read128(uint32_t addr) {
-    half8v v;
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
-    return v;
-}
-// wait until at most N LDS reads are outstanding; the two fragments pass through the statement so that their
-// users cannot be scheduled ahead of it
-template <int N> __device__ inline void lds_wait_pin(half8v &a0, half8v &a1) {
-    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(a0), "+v"(a1) : "n"(N));
+template <int OFF, typename T> __device__ inline void lds_read128(T &dst, uint32_t addr) {
+    static_assert(sizeof(T) == 16 && OFF >= 0 && OFF < 65536, "one ds_read_b128");
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
 
-// packed bytes of one 32-row group for one super-block: two lane slots of a tile + that row's header
-struct BRegs { uint4v qa[2], qb[2], hd; };
-
-__device__ inline BRegs b_load(const uint8_t *__restrict__ tile, int r, int g32) {
-    using F = TiledFmt<TURQ_Q4_K>;
-    BRegs t;
-#pragma unroll
-    for (int s = 0; s < 2; s++) {
-        const int slot = r + 16 * (2 * g32 + s);
-        t.qa[s] = *(const uint4v *)(tile + F::kQA + 16 * slot);
-        t.qb[s] = *(const uint4v *)(tile + F::kQB + 16 * slot);
-    }
-    t.hd = *(const uint4v *)(tile + F::kHDR + 16 * r);
-    return t;
+// 64 lanes x 16 bytes, global -> LDS.  The instruction offset applies to both sides: lane l copies
+// sbase[voff_l + IMM .. + 15] to LDS byte lds_addr + IMM + 16 * l.
+template <int IMM> __device__ inline void dma_set(uint32_t voff, const uint8_t *sbase, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+                 :
+                 : "v"(voff), "s"(sbase), "s"(lds_addr), "n"(IMM)
+                 : "memory", "m0");
+}
+// same LDS base (m0) as the preceding dma_set of this wave
+template <int IMM> __device__ inline void dma_more(uint32_t voff, const uint8_t *sbase) {
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
 }
 
-// constants of the lane's four sub-blocks u = 2 * slot + half (sub-block 4 * g32 + u of the super-block)
+// constants of the lane's four sub-blocks u (sub-block 4 * g32 + u of the super-block)
 struct BConsts {
     half2v s[4], c1[4], c2[4];  // d*sc, -1024*d*sc, -64*d*sc (both halves equal)
     half8v bmin;                // -(dmin*m_u) twice each, against the (hi, lo) sums fragment
@@ -129,15 +168,33 @@ __device__ inline half8v q4_operand(uint32_t w, half2v s, half2v c1, half2v c2) 
                       pk_fma(and_or_h2(w8, 0x000F000Fu, kMagic1024), s, c1), pk_fma(and_or_h2(w8, 0x00F000F0u, kMagic64), s, c2));
 }
 
+// 64-bit address arithmetic may run on the vector ALU even when every input is uniform; the copies take
+// their base address in scalar registers
+__device__ inline const uint8_t *uniform_ptr(const uint8_t *p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint8_t *)(((uint64_t)hi << 32) | lo);
+}
+
+template <int I> __device__ inline uint32_t word_of(uint4v v) { return I == 0 ? v.x : I == 1 ? v.y : I == 2 ? v.z : v.w; }
+
+__device__ inline uint32_t pack_bf16x2(float a, float b) { return (uint32_t)turq_f2bf(a) | ((uint32_t)turq_f2bf(b) << 16); }
+__device__ inline uint32_t pack_f16x2(float a, float b) {
+    const half2v h{(_Float16)a, (_Float16)b};
+    return as_u32(h);
+}
+
 // frags: 32-row fragments, 1 KiB block index (mt * ntc + b) * 17 + q
+// vec_out: rows of y can be written as aligned 16-byte pieces
 __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
                                                        const uint8_t *__restrict__ frags, int64_t m, void *__restrict__ y,
                                                        int yt, int64_t ldy, const float *__restrict__ bias, int nblocks_n,
-                                                       int nblocks_m) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // NBUF stages of 32 KiB
+                                                       int nblocks_m, int vec_out) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
     const int n32 = lane & 31, g32 = lane >> 5;
     const int r16 = n32 & 15, tsel = n32 >> 4;
     // Workgroups of one XCD (blockIdx % 8) get consecutive logical ids and the m-blocks of one n-block are
@@ -146,19 +203,66 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
     int lid = blockIdx.x;
     if ((nwg & 7) == 0) lid = (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3);
     const int nb = lid / nblocks_m, mb = lid - nb * nblocks_m;
-    const int64_t ntc = turq_tile_cols(k);
+    const int ntc = (int)turq_tile_cols(k);
     const int64_t mtiles = (m + 31) / 32;
-    const int64_t nrt = turq_tile_rows(n);
-    constexpr int TB = TiledFmt<TURQ_Q4_K>::kTileBytes;
+    const int nrt = (int)turq_tile_rows(n);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    const uint32_t lane_off = 16u * (uint32_t)lane;
 
-    // the 16-row tile this lane reads for each of the wave's three 32-row groups (clamped at the end)
-    const uint8_t *wrow[WN];
+    // ---- copy schedule (all wave-uniform except the per-lane weight offsets) ----
+    // activations: this wave's m-tile; one past the end re-reads the last valid tile (never stored)
+    int64_t my_mt = (int64_t)mb * MT + wave;
+    my_mt = my_mt < mtiles ? my_mt : mtiles - 1;
+    const uint8_t *a_src = uniform_ptr(frags + ((size_t)(my_mt * ntc * 17) << 10));
+    const uint32_t a_dst = lds_base + A_OFF + (uint32_t)wave * 4096u;  // + ks * A_STAGE (+ step * 1024 by the offset)
+    const uint32_t s_dst = lds_base + S_OFF + (uint32_t)wave * 1024u;  // + (b & 1) * S_BYTES
+    // weights: copy c of a super-block covers bytes [1024 c, 1024 c + 1024) of the 12 concatenated tiles;
+    // group g = 0..3 holds copies 4g + wave and 16 + 4g + wave (the latter clamped to the last one)
+    const int tile0 = nb * NT16;
+    const uint8_t *w_src = uniform_ptr(w + (size_t)tile0 * ntc * TB);  // + b * TB
+    uint32_t w_voff[4][2];
+    uint32_t w_dst[4][2];
 #pragma unroll
-    for (int j = 0; j < WN; j++) {
-        int64_t rt = (int64_t)nb * (BN / 16) + 2 * j + tsel;
-        rt = rt < nrt ? rt : nrt - 1;
-        wrow[j] = w + rt * ntc * TB;
-    }
+    for (int g = 0; g < 4; g++)
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            int c = i == 0 ? 4 * g + wave : 16 + 4 * g + wave;
+            c = c < W_CHUNKS ? c : W_CHUNKS - 1;
+            const uint32_t o = (uint32_t)c * 1024u + lane_off;
+            const uint32_t t = o / (uint32_t)TB;
+            const uint32_t within = o - t * (uint32_t)TB;
+            int tg = tile0 + (int)t;
+            tg = tg < nrt ? tg : nrt - 1;  // row tiles past the end re-read the last one (never stored)
+            w_voff[g][i] = (uint32_t)(tg - tile0) * (uint32_t)ntc * (uint32_t)TB + within;
+            w_dst[g][i] = lds_base + W_OFF + (uint32_t)c * 1024u;  // + ring offset
+        }
+    // ring offsets of the weight buffers of super-blocks b, b + 1, b + 2
+    uint32_t wr0 = 0, wr1 = W_BYTES, wr2 = 2 * W_BYTES;
+
+    auto issue_a = [&](int bb, int ks) {  // stage (bb, ks) -> stage buffer ks
+        const uint8_t *src = a_src + ((size_t)(bb * 17 + 4 * ks) << 10);
+        dma_set<0>(lane_off, src, a_dst + (uint32_t)ks * A_STAGE);
+        dma_more<1024>(lane_off, src);
+        dma_more<2048>(lane_off, src);
+        dma_more<3072>(lane_off, src);
+    };
+    auto issue_w = [&](int bb, int g, uint32_t ring) {  // group g of super-block bb
+        const uint8_t *src = w_src + (size_t)bb * TB;
+        dma_set<0>(w_voff[g][0], src, w_dst[g][0] + ring);
+        dma_set<0>(w_voff[g][1], src, w_dst[g][1] + ring);
+    };
+    auto issue_s = [&](int bb) {
+        dma_set<0>(lane_off, a_src + ((size_t)(bb * 17 + 16) << 10), s_dst + (uint32_t)(bb & 1) * S_BYTES);
+    };
+
+    // ---- LDS read addresses ----
+    // activations: stage ks, m-tile 2 wm + i, step st at A_OFF + ks * A_STAGE + ((2 wm + i) * 4 + st) * 1024
+    const uint32_t a_rd = lds_base + A_OFF + (uint32_t)wm * (WM * 4096u) + lane_off;
+    const uint32_t s_rd = lds_base + S_OFF + (uint32_t)wm * (WM * 1024u) + lane_off;
+    // weights: 32-row tile j of this wave = 16-row tiles 6 wn + 2 j + tsel; stage ks reads lane slot
+    // r16 + 16 * (2 g32 + (ks >> 1)) of plane QA (ks even) or QB (ks odd)
+    const uint32_t w_rd = lds_base + W_OFF + (uint32_t)(6 * wn + tsel) * TB + 16u * (uint32_t)(r16 + 32 * g32);
+    const uint32_t h_rd = lds_base + W_OFF + (uint32_t)(6 * wn + tsel) * TB + 2048u + 16u * (uint32_t)r16;
 
     float16v acc[WM][WN];
 #pragma unroll
@@ -168,155 +272,197 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    // Stage s = 5 * b + ks.  ks < 4: operand steps 4ks .. 4ks+3 of super-block b for the 8 m-tiles of the
-    // workgroup (32 blocks of 1 KiB; wave w copies step 4ks + w for all 8 m-tiles); ks == 4: the sums step
-    // (8 blocks, wave w copies m-tiles 2w, 2w+1).  All index arithmetic is 32-bit and wave-uniform.
-    const int nstages = (int)ntc * 5;
-    const int ntc_i = (int)ntc;
-    // 1 KiB block index of (m-tile c of this workgroup, super-block 0, step 0); tiles past the end re-read the
-    // last valid one (their rows are never stored) so that every wave always issues the same number of loads,
-    // which the vmcnt bookkeeping below relies on
-    int mt_blk[8];
+    // ---- prologue: super-block 0 complete, weights of 1 and the first group of 2 on their way ----
+    const int last = ntc - 1;
 #pragma unroll
-    for (int c = 0; c < 8; c++) {
-        int64_t mtg = (int64_t)mb * (BM / 32) + c;
-        mtg = mtg < mtiles ? mtg : mtiles - 1;
-        mt_blk[c] = (int)(mtg * ntc * 17);
-    }
-    const uint32_t lane_off = 16u * (uint32_t)lane;
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
-    auto issue_one = [&](int blk1k, int dst_off) {
-        const uint8_t *src = frags + ((size_t)blk1k << 10);  // wave-uniform
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + lane_off),
-                                         (__attribute__((address_space(3))) void *)(lds + dst_off), 16, 0, 0);
-    };
-    // issue stage (b, ks) into buffer `buf`
-    auto stage_issue = [&](int b, int ks, int buf) {
-        const int base = buf * STAGE_BYTES;
-        if (ks < 4) {
-            const int q = 4 * ks + wave;
+    for (int ks = 0; ks < 4; ks++) issue_a(0, ks);
 #pragma unroll
-            for (int c = 0; c < 8; c++) issue_one(mt_blk[c] + b * 17 + q, base + ((wave * 8 + c) << 10));
-        } else {
+    for (int g = 0; g < 4; g++) issue_w(0, g, wr0);
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const int mt = 2 * wave + c;
-                int blk = 0;
-#pragma unroll
-                for (int t = 0; t < 8; t++) blk = (t == mt) ? mt_blk[t] : blk;  // uniform select, no dynamic indexing
-                issue_one(blk + b * 17 + 16, base + (mt << 10));
-            }
-        }
-    };
+    for (int g = 0; g < 4; g++) issue_w(1 < last ? 1 : last, g, wr1);
+    issue_w(2 < last ? 2 : last, 0, wr2);
+    issue_s(0);
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 
-    BRegs wt[WN], wnext[WN];
+    half8v af[2][WM];  // [step parity][m-tile]
+    half8v sf[WM];
+    uint4v wq[2][WN];  // [stage parity][n-tile]: the four operand words of the stage
+    uint4v hd[WN];
     BConsts cs[WN], cs_next[WN];
+    static_for<WN>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+        lds_read128<j * 2 * TB>(hd[j], h_rd);
+        lds_read128<j * 2 * TB>(wq[0][j], w_rd);
+    });
+    lds_read128<0>(af[0][0], a_rd);
+    lds_read128<4096>(af[0][1], a_rd);
+    wait_lds<0>();
 #pragma unroll
-    for (int j = 0; j < WN; j++) wt[j] = b_load(wrow[j], r16, g32);
-#pragma unroll
-    for (int j = 0; j < WN; j++) cs[j] = b_consts(wt[j].hd, g32);
-    stage_issue(0, 0, 0);
-    stage_issue(0, 1, 1);
-    int buf = 0;          // buffer of the stage being computed
-    int ib = 0, iks = 2;  // (super-block, ks) of the next stage to issue, i.e. stage s + 2
-    int ibuf = 2;
+    for (int j = 0; j < WN; j++) {
+        pin(hd[j]);
+        cs[j] = b_consts(hd[j], g32);
+    }
 
-    for (int b = 0; b < ntc_i; b++) {
+    for (int b = 0; b < ntc; b++) {
+        const uint32_t w_cur = w_rd + wr0, w_nxt = w_rd + wr1, h_nxt = h_rd + wr1;
+        const uint32_t s_cur = s_rd + (uint32_t)(b & 1) * S_BYTES;
+        const int b1 = b + 1 < last ? b + 1 : last, b2 = b + 2 < last ? b + 2 : last, b3 = b + 3 < last ? b + 3 : last;
+        static_for<4>([&](auto KS) {  // the four stages of the super-block: ks selects registers, buffers and offsets
+            constexpr int ks = decltype(KS)::value;
+            constexpr int cur = ks & 1, nxt = cur ^ 1;
+            // entering: wq[cur], af[0] (step 0) and, for ks == 3, hd are in flight
+            static_for<4>([&](auto ST) {
+                constexpr int st = decltype(ST)::value;
+                constexpr int pa = st & 1;
+                if constexpr (st < 3) {
+                    // next step's activation fragments come in while this step computes
+                    lds_read128<ks * A_STAGE + (st + 1) * 1024>(af[pa ^ 1][0], a_rd);
+                    lds_read128<ks * A_STAGE + 4096 + (st + 1) * 1024>(af[pa ^ 1][1], a_rd);
+                    wait_lds<2>();  // everything but the two reads just issued
+                    pin(af[pa][0]);
+                    pin(af[pa][1]);
+                    if constexpr (st == 0) {
 #pragma unroll
-        for (int ks = 0; ks < 5; ks++) {  // fully unrolled: ks selects registers at compile time
-            // Stage s was issued two stages ago.  Loads retire in order, so "at most as many outstanding as the
-            // newest stage issued" means stage s (and the weight loads before it) have landed.
-            // (Past the last stage the issue below repeats the last super-block into a buffer nobody reads any
-            // more, which keeps these counts the same for every stage and the loop free of branches.)
-            if (ks == 3) wait_vmcnt<2>(); else wait_vmcnt<8>();   // the sums stage has 2 loads per wave
-            // plain s_barrier: __syncthreads() would also drain the loads that are meant to stay in flight
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-            // now stage s is visible to all waves and nobody reads buffer (s + 2) % 3 any more
-            static_assert(WM == 2, "fragment double buffering below is written for two m-tiles per wave");
-            const uint32_t abase = lds_base + (uint32_t)(buf * STAGE_BYTES + (wave * WM << 10)) + lane_off;
-            half8v af[2][WM];  // [step parity][m-tile]
-            af[0][0] = lds_read128<0>(abase);
-            af[0][1] = lds_read128<1024>(abase);
-            if (ks == 2) {
-                // the next super-block's weights were issued before stage s + 1's copies, so the wait of the
-                // previous stage has covered them
+                        for (int j = 0; j < WN; j++) pin(wq[cur][j]);
+                        if constexpr (ks == 3) {
 #pragma unroll
-                for (int j = 0; j < WN; j++) cs_next[j] = b_consts(wnext[j].hd, g32);
-            }
-            if (ks == 0) {
-                const int bn = b + 1 < ntc_i ? b + 1 : b;  // last super-block: harmless re-read
-#pragma unroll
-                for (int j = 0; j < WN; j++) wnext[j] = b_load(wrow[j] + (int64_t)bn * TB, r16, g32);
-            }
-            stage_issue(ib < ntc_i ? ib : ntc_i - 1, iks, ibuf);
-            iks = iks == 4 ? 0 : iks + 1;
-            ib += iks == 0 ? 1 : 0;
-            ibuf = ibuf == NBUF - 1 ? 0 : ibuf + 1;
-            if (ks < 4) {
-#pragma unroll
-                for (int st = 0; st < STAGE_STEPS; st++) {
-                    const int cur = st & 1, nxt = cur ^ 1;
-                    if (st + 1 < STAGE_STEPS) {  // next step's activation fragments come in while this step computes
-                        const uint32_t an = abase + (uint32_t)((st + 1) * (BM / 32) << 10);
-                        af[nxt][0] = lds_read128<0>(an);
-                        af[nxt][1] = lds_read128<1024>(an);
-                        lds_wait_pin<2>(af[cur][0], af[cur][1]);
-                    } else {
-                        lds_wait_pin<0>(af[cur][0], af[cur][1]);
+                            for (int j = 0; j < WN; j++) {
+                                pin(hd[j]);
+                                cs_next[j] = b_consts(hd[j], g32);
+                            }
+                        }
                     }
-                    const int q = 4 * ks + st;            // operand step 0..15: slot q >> 3, dword q & 7
-                    const int slot = q >> 3, dw = q & 7;
-                    const int u = 2 * slot + (dw >> 2);   // sub-block index among the lane's four
-                    half8v bop[WN];
-#pragma unroll
-                    for (int j = 0; j < WN; j++) {
-                        const uint4v src = dw < 4 ? wt[j].qa[slot] : wt[j].qb[slot];
-                        const uint32_t wd = (dw & 3) == 0 ? src.x : (dw & 3) == 1 ? src.y : (dw & 3) == 2 ? src.z : src.w;
-                        bop[j] = q4_operand(wd, cs[j].s[u], cs[j].c1[u], cs[j].c2[u]);
+                } else {
+                    // ---- stage boundary, before the last step: the next stage becomes readable ----
+                    wait_lds<0>();  // step 3's fragments are in registers: this wave is done with the stage's LDS
+                    pin(af[1][0]);
+                    pin(af[1][1]);
+                    // The next stage's copies were issued three boundaries ago; younger than them are that
+                    // boundary's weight (and sums) copies and everything of the two boundaries since.
+                    if constexpr (ks == 0) wait_vmcnt<14>(); else wait_vmcnt<15>();
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    // now stage buffer ks is free: stage (b + 1, ks) goes there
+                    issue_a(b1, ks);
+                    if constexpr (ks == 3) issue_w(b3, 0, wr0); else issue_w(b2, ks + 1, wr2);
+                    if constexpr (ks == 0) issue_s(b1);
+                    // first reads of the next stage, hidden under step 3's MFMAs
+                    if constexpr (ks == 3) {
+                        lds_read128<0>(sf[0], s_cur);
+                        lds_read128<1024>(sf[1], s_cur);
                     }
-#pragma unroll
-                    for (int i = 0; i < WM; i++)
-#pragma unroll
-                        for (int j = 0; j < WN; j++) acc[i][j] = mfma32x32x16(af[cur][i], bop[j], acc[i][j]);
+                    constexpr int nks = (ks + 1) & 3;  // next stage: plane QA / QB and lane slot half
+                    constexpr int woff = (nks & 1) * 1024 + (nks >> 1) * 256;
+                    const uint32_t w_from = ks == 3 ? w_nxt : w_cur;
+                    lds_read128<0 * 2 * TB + woff>(wq[nxt][0], w_from);
+                    lds_read128<1 * 2 * TB + woff>(wq[nxt][1], w_from);
+                    lds_read128<2 * 2 * TB + woff>(wq[nxt][2], w_from);
+                    if constexpr (ks == 2) {
+                        lds_read128<0 * 2 * TB>(hd[0], h_nxt);
+                        lds_read128<1 * 2 * TB>(hd[1], h_nxt);
+                        lds_read128<2 * 2 * TB>(hd[2], h_nxt);
+                    }
+                    lds_read128<nks * A_STAGE>(af[0][0], a_rd);
+                    lds_read128<nks * A_STAGE + 4096>(af[0][1], a_rd);
                 }
-            } else {
-                // "- dmin * m" term against the sub-block sums; then the prefetched weights take over
-                lds_wait_pin<0>(af[0][0], af[0][1]);
+                // operand step 4 ks + st: word st of the stage, sub-block u = ks of the lane's four
+                half8v bop[WN];
+#pragma unroll
+                for (int j = 0; j < WN; j++) bop[j] = q4_operand(word_of<st>(wq[cur][j]), cs[j].s[ks], cs[j].c1[ks], cs[j].c2[ks]);
 #pragma unroll
                 for (int i = 0; i < WM; i++)
 #pragma unroll
-                    for (int j = 0; j < WN; j++) acc[i][j] = mfma32x32x16(af[0][i], cs[j].bmin, acc[i][j]);
+                    for (int j = 0; j < WN; j++) acc[i][j] = mfma32x32x16(af[pa][i], bop[j], acc[i][j]);
+            });
+            if constexpr (ks == 3) {
+                // "- dmin * m" term against the sub-block sums; then the next super-block's constants take over
+                wait_lds<5>();  // all but the three weight and two fragment reads of the next stage
+                pin(sf[0]);
+                pin(sf[1]);
 #pragma unroll
-                for (int j = 0; j < WN; j++) {
-                    wt[j] = wnext[j];
-                    cs[j] = cs_next[j];
-                }
+                for (int i = 0; i < WM; i++)
+#pragma unroll
+                    for (int j = 0; j < WN; j++) acc[i][j] = mfma32x32x16(sf[i], cs[j].bmin, acc[i][j]);
+#pragma unroll
+                for (int j = 0; j < WN; j++) cs[j] = cs_next[j];
             }
-            buf = buf == NBUF - 1 ? 0 : buf + 1;
-        }
+        });
+        const uint32_t t = wr0;
+        wr0 = wr1;
+        wr1 = wr2;
+        wr2 = t;
     }
-    wait_vmcnt<0>();  // the two trailing dummy stages must not outlive the workgroup's LDS
+    wait_lds<0>();
+    wait_vmcnt<0>();  // the trailing copies must neither outlive the workgroup's LDS nor land in the staged results
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 
+    // ---- results ----
     // 32x32 result: lane (n32, g32), register e holds row 8 * (e / 4) + 4 * g32 + e % 4 of column n32
+    const int64_t row0 = (int64_t)mb * BM + wm * (WM * 32);
+    const int64_t col0 = (int64_t)nb * BN + wn * (WN * 32);
+    if (vec_out) {
+        float *stage = (float *)lds + (size_t)wave * (64 * OUT_PITCH);
 #pragma unroll
-    for (int j = 0; j < WN; j++) {
-        const int64_t col = (int64_t)nb * BN + 32 * j + n32;
-        if (col >= n) continue;
-        const float bv = bias ? bias[col] : 0.0f;
+        for (int j = 0; j < WN; j++) {
+            const int64_t col = col0 + 32 * j + n32;
+            const float bv = (bias && col < n) ? bias[col] : 0.0f;
 #pragma unroll
-        for (int i = 0; i < WM; i++)
+            for (int i = 0; i < WM; i++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int64_t row = (int64_t)mb * BM + (wave * WM + i) * 32 + 8 * (e >> 2) + 4 * g32 + (e & 3);
-                if (row < m) {
-                    const float v = acc[i][j][e] + bv;
-                    if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, row * ldy + col, v);
-                    else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, row * ldy + col, v);
-                    else turq_store_out<TURQ_ACT_F16>(y, row * ldy + col, v);
-                }
+                for (int e = 0; e < 16; e++)
+                    stage[(32 * i + 8 * (e >> 2) + 4 * g32 + (e & 3)) * OUT_PITCH + 32 * j + n32] = acc[i][j][e] + bv;
+        }
+        // each wave reads back only what it wrote itself; LDS operations of one wave complete in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (yt == TURQ_ACT_F32) {
+            constexpr int CPR = WN * 32 / 4;  // 16-byte pieces per row
+#pragma unroll 4
+            for (int it = 0; it < CPR; it++) {
+                const int c = it * 64 + lane;
+                const int r = c / CPR, cc = c - r * CPR;
+                const float4v v = *(const float4v *)(stage + r * OUT_PITCH + 4 * cc);
+                if (row0 + r < m && col0 + 4 * cc < n) *(float4v *)((float *)y + (row0 + r) * ldy + col0 + 4 * cc) = v;
             }
+        } else {
+            constexpr int CPR = WN * 32 / 8;
+#pragma unroll 4
+            for (int it = 0; it < CPR; it++) {
+                const int c = it * 64 + lane;
+                const int r = c / CPR, cc = c - r * CPR;
+                const float4v v0 = *(const float4v *)(stage + r * OUT_PITCH + 8 * cc);
+                const float4v v1 = *(const float4v *)(stage + r * OUT_PITCH + 8 * cc + 4);
+                uint4v o;
+                if (yt == TURQ_ACT_BF16)
+                    o = uint4v{pack_bf16x2(v0.x, v0.y), pack_bf16x2(v0.z, v0.w), pack_bf16x2(v1.x, v1.y), pack_bf16x2(v1.z, v1.w)};
+                else
+                    o = uint4v{pack_f16x2(v0.x, v0.y), pack_f16x2(v0.z, v0.w), pack_f16x2(v1.x, v1.y), pack_f16x2(v1.z, v1.w)};
+                if (row0 + r < m && col0 + 8 * cc < n) *(uint4v *)((uint16_t *)y + (row0 + r) * ldy + col0 + 8 * cc) = o;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < WN; j++) {
+            const int64_t col = col0 + 32 * j + n32;
+            if (col >= n) continue;
+            const float bv = bias ? bias[col] : 0.0f;
+#pragma unroll
+            for (int i = 0; i < WM; i++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int64_t row = row0 + 32 * i + 8 * (e >> 2) + 4 * g32 + (e & 3);
+                    if (row < m) {
+                        const float v = acc[i][j][e] + bv;
+                        if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, row * ldy + col, v);
+                        else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, row * ldy + col, v);
+                        else turq_store_out<TURQ_ACT_F16>(y, row * ldy + col, v);
+                    }
+                }
+        }
     }
 }
 
@@ -327,19 +473,22 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
                                  int y_dtype, int64_t ldy, const float *bias, hipStream_t stream, hipEvent_t ev_start,
                                  hipEvent_t ev_stop) {
     if (n == 0 || m == 0) return hipSuccess;
-    if (dtype != TURQ_Q4_K) return hipErrorInvalidValue;
-    static const hipError_t attr = hipFuncSetAttribute((const void *)gemm_q4k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                       NBUF * STAGE_BYTES);
+    if (dtype != TURQ_Q4_K || k <= 0 || k % 256 != 0) return hipErrorInvalidValue;
+    // per-lane weight offsets are 32-bit
+    if ((uint64_t)NT16 * (uint64_t)(k / 256) * TB >= (1ull << 32)) return hipErrorInvalidValue;
+    static const hipError_t attr =
+        hipFuncSetAttribute((const void *)gemm_q4k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (attr != hipSuccess) return attr;
     const int nbn = (int)((n + BN - 1) / BN), nbm = (int)((m + BM - 1) / BM);
     const dim3 grid((unsigned)(nbn * nbm)), block(256);
-    const unsigned lds_bytes = NBUF * STAGE_BYTES;
+    const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
+    const int vec_out = ((uintptr_t)y % 16 == 0 && ((uint64_t)ldy * es) % 16 == 0 && n % 8 == 0) ? 1 : 0;
     if (ev_start) {
-        hipExtLaunchKernelGGL(gemm_q4k_kernel, grid, block, lds_bytes, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
-                              (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm);
+        hipExtLaunchKernelGGL(gemm_q4k_kernel, grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
+                              (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out);
     } else {
-        gemm_q4k_kernel<<<grid, block, lds_bytes, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype, ldy,
-                                                            bias, nbn, nbm);
+        gemm_q4k_kernel<<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype, ldy,
+                                                            bias, nbn, nbm, vec_out);
     }
     return hipGetLastError();
 }
