@@ -78,42 +78,72 @@ hipError_t launch(int dtype, const void *x, int64_t m, int64_t k, int64_t ldx, v
 // (r, g32) = r + 32 * g32 of step q holds x[32 mt + r][256 b + 128 g32 + 8 q + j], j = 0..7; step 16
 // holds for the four 32-column sub-blocks of the lane's 128 columns the sums of the f16-rounded
 // activations as (hi, lo) f16 pairs.  chunk index = ((mt * ntc + b) * 17 + q) * 64 + lane.
+// One workgroup per (m-tile, column tile): 32 rows x 256 columns come in along the rows (a thread reads 8
+// neighbouring columns, 32 threads one row), are rounded to f16 and transposed through the LDS into fragment
+// order, and leave as one contiguous 17 KiB piece.
 template <int XT>
 __global__ void __launch_bounds__(256) act_prep32_kernel(const void *__restrict__ x, int64_t m, int64_t k, int64_t ldx,
-                                                         int64_t ntc, int64_t nchunks, half8v *__restrict__ frags) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= nchunks) return;
-    const int lane = (int)(t & 63);
-    const int64_t blk = t >> 6;            // (mt * ntc + b) * 17 + q
-    const int q = (int)(blk % 17);
-    const int64_t tb = blk / 17;
+                                                         int64_t ntc, half8v *__restrict__ frags) {
+    __shared__ half8v out[17 * 64];
+    __shared__ float part[32][33];  // per row: sums of its 32 pieces of 8 columns
+    const int tid = threadIdx.x;
+    const int64_t tb = blockIdx.x;  // mt * ntc + b
     const int64_t b = tb % ntc, mt = tb / ntc;
-    const int r = lane & 31, g32 = lane >> 5;
-    const int64_t row = mt * 32 + r;
-    const bool row_ok = row < m;
-    half8v h;
-    if (q < 16) {
-        const int64_t col0 = b * 256 + 128 * g32 + 8 * q;
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int c = it * 256 + tid;
+        const int r = c >> 5, cc = c & 31;  // row of the tile, piece of 8 columns
+        const int64_t row = mt * 32 + r, col0 = b * 256 + 8 * cc;
+        float v[8];
+        const char *src = (const char *)x + (row * ldx + col0) * (XT == TURQ_ACT_F32 ? 4 : 2);
+        if (row < m && col0 + 8 <= k && ((uintptr_t)src & 15) == 0) {
+            if (XT == TURQ_ACT_F32) {
+                const float4v lo = ((const float4v *)src)[0], hi = ((const float4v *)src)[1];
+                v[0] = lo.x, v[1] = lo.y, v[2] = lo.z, v[3] = lo.w, v[4] = hi.x, v[5] = hi.y, v[6] = hi.z, v[7] = hi.w;
+            } else {
+                const uint4v u = *(const uint4v *)src;
+                const uint32_t wd[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (XT == TURQ_ACT_BF16) {
+                        v[2 * j] = __uint_as_float(wd[j] << 16);
+                        v[2 * j + 1] = __uint_as_float(wd[j] & 0xFFFF0000u);
+                    } else {
+                        const half2v hh = as_half2(wd[j]);
+                        v[2 * j] = (float)hh.x;
+                        v[2 * j + 1] = (float)hh.y;
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = (row < m && col0 + j < k) ? ld_act<XT>(x, row * ldx + col0 + j) : 0.0f;
+        }
+        half8v h;
+        float sum = 0.0f;
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const int64_t c = col0 + j;
-            h[j] = (_Float16)((row_ok && c < k) ? ld_act<XT>(x, row * ldx + c) : 0.0f);
+            h[j] = (_Float16)v[j];
+            sum += (float)h[j];
         }
-    } else {
-#pragma unroll
-        for (int sb = 0; sb < 4; sb++) {
-            const int64_t col0 = b * 256 + 128 * g32 + 32 * sb;
-            float sum = 0.0f;
-            for (int j = 0; j < 32; j++) {
-                const int64_t c = col0 + j;
-                sum += (float)(_Float16)((row_ok && c < k) ? ld_act<XT>(x, row * ldx + c) : 0.0f);
-            }
-            const _Float16 hi = (_Float16)sum;
-            h[2 * sb] = hi;
-            h[2 * sb + 1] = (_Float16)(sum - (float)hi);
-        }
+        const int g32 = cc >> 4, q = cc & 15;
+        out[q * 64 + r + 32 * g32] = h;
+        part[r][cc] = sum;
     }
-    frags[t] = h;
+    __syncthreads();
+    {
+        // thread (r, g32, sb): sum of the 32 columns of sub-block sb of the lane's 128, as (hi, lo)
+        const int r = tid & 31, g32 = (tid >> 5) & 1, sb = tid >> 6;
+        const float *p = &part[r][16 * g32 + 4 * sb];
+        const float sum = (p[0] + p[1]) + (p[2] + p[3]);
+        const _Float16 hi = (_Float16)sum;
+        const _Float16 lo = (_Float16)(sum - (float)hi);
+        half2v *dst = (half2v *)&out[16 * 64 + r + 32 * g32];
+        dst[sb] = half2v{hi, lo};
+    }
+    __syncthreads();
+    half8v *dst = frags + tb * (17 * 64);
+    for (int c = tid; c < 17 * 64; c += 256) dst[c] = out[c];
 }
 
 }  // namespace
@@ -132,12 +162,11 @@ hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m
 hipError_t turq_launch_act_prep32(const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags, hipStream_t stream) {
     if (m == 0 || k == 0) return hipSuccess;
     const int64_t ntc = (k + 255) / 256;
-    const int64_t nchunks = ((m + 31) / 32) * ntc * 17 * 64;
-    const unsigned grid = (unsigned)((nchunks + 255) / 256);
+    const unsigned grid = (unsigned)(((m + 31) / 32) * ntc);
     switch (x_dtype) {
-    case TURQ_ACT_F32: act_prep32_kernel<TURQ_ACT_F32><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, nchunks, (half8v *)frags); break;
-    case TURQ_ACT_BF16: act_prep32_kernel<TURQ_ACT_BF16><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, nchunks, (half8v *)frags); break;
-    case TURQ_ACT_F16: act_prep32_kernel<TURQ_ACT_F16><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, nchunks, (half8v *)frags); break;
+    case TURQ_ACT_F32: act_prep32_kernel<TURQ_ACT_F32><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, (half8v *)frags); break;
+    case TURQ_ACT_BF16: act_prep32_kernel<TURQ_ACT_BF16><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, (half8v *)frags); break;
+    case TURQ_ACT_F16: act_prep32_kernel<TURQ_ACT_F16><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, (half8v *)frags); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
