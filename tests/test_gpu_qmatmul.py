@@ -213,6 +213,10 @@ def test_prefill_gemm_q4k(gpu, n, k, m):
     yb = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16, bias=bias, ldx=k + 8, ldy=n + 3)
     want = synth.from_bf16_bits(synth.to_bf16_bits(dense + bias)).reshape(m, n)
     assert rel_l2(yb, want) <= 3e-3 and rel_l2(yb, dense + bias) <= 4e-3
+    # row strides that keep 16-byte alignment leave through the wide stores (when n is a multiple of 8), f16 and bf16
+    for yd, bar in ((capi.ACT_F16, 1.2e-3), (capi.ACT_BF16, 4e-3)):
+        ya = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=yd, bias=bias, ldy=n + (-n) % 8 + 8)
+        assert rel_l2(ya, dense + bias) <= bar
     # f32 activations take the same path (rounded to f16 on the way in)
     xf = synth.random_activation(m, k, seed=m + 1)
     yf = gpu.qmatmul(w, xf, n, k)
