@@ -115,11 +115,32 @@ class Bench:
         for layer in self.weights:
             for (label, dt, n, k), w, y in zip(self.mats, layer, self.y_dev):
                 self.calls.append((w, self.x_dev[k], y, n, k))
+        # neighbouring matrices that take the same input (gate/up, q/k/v) go through turq_qmatmul_multi, as the
+        # reference calls them back to back on one tensor (src/models/qwen3.rs:161-167, 272-274)
+        self.groups = []       # (count, weight array, x, y array, ldy array, k)
+        for layer in self.weights:
+            i = 0
+            while i < len(self.mats):
+                j = i + 1
+                while j < len(self.mats) and self.mats[j][3] == self.mats[i][3]:
+                    j += 1
+                cnt = j - i
+                warr = (ctypes.c_void_p * cnt)(*[w.value for w in layer[i:j]])
+                yarr = (ctypes.c_void_p * cnt)(*[y.value for y in self.y_dev[i:j]])
+                ldys = (ctypes.c_int64 * cnt)(*[mt[2] for mt in self.mats[i:j]])
+                self.groups.append((cnt, warr, self.x_dev[self.mats[i][3]], yarr, ldys, self.mats[i][3]))
+                i = j
         self.step_bytes = layers * sum(algorithmic_bytes(dt, n, k, self.m, self.xbytes, self.ybytes) for _, dt, n, k in self.mats)
         self.step_flops = layers * sum(2 * self.m * n * k for _, _, n, k in self.mats)
 
     def step_eager(self):
         L, ctx, m, xt = self.L, self.ctx, self.m, self.xt
+        if not self.args.single_calls:
+            for cnt, warr, x, yarr, ldys, k in self.groups:
+                rc = L.turq_qmatmul_multi(ctx, cnt, warr, x, xt, m, k, yarr, self.yt, ldys, None, capi.MEM_DEVICE, capi.ALGO_AUTO)
+                if rc:
+                    capi.check(rc, ctx)
+            return
         for w, x, y, n, k in self.calls:
             rc = L.turq_qmatmul(ctx, w, x, xt, m, k, y, self.yt, n, None, capi.MEM_DEVICE, capi.ALGO_AUTO)
             if rc:
@@ -182,13 +203,14 @@ class Bench:
         tot_ms = ctypes.c_double()
         capi.check(L.turq_profile_end(ctx, ctypes.byref(n_launch), ctypes.byref(tot_ms)), ctx)
         avg_us = tot_ms.value / max(1, n_launch.value) * 1e3
-        bytes_per_launch = self.step_bytes / len(self.calls)
+        # all timed launches are the matmul kernel (one per matrix, or one per group of matrices with a common input)
+        bytes_per_launch = self.step_bytes * prof_steps / max(1, n_launch.value)
         achieved = bytes_per_launch / (avg_us * 1e-6) / 1e9
         if graph:
             L.turq_graph_destroy(graph)
         gemm = self.m > 32
         if gemm:
-            flops_per_launch = self.step_flops / len(self.calls)
+            flops_per_launch = self.step_flops * prof_steps / max(1, n_launch.value)
             tfl = flops_per_launch / (avg_us * 1e-6) / 1e12
             roofline = {
                 "bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -201,7 +223,7 @@ class Bench:
             roofline = {
                 "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC.get((a.workload, self.m, a.act)),
-                "kernel": "gemv_mfma_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
+                "kernel": "gemv_mfma_kernel" if a.single_calls or self.m > 4 else "gemv_multi_kernel / gemv_mfma_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "algorithmic_bytes_per_launch": int(bytes_per_launch),
             }
             metric, value, unit = "quantized GEMV HBM GB/s (Q4_K/Q6_K, Qwen3-8B shapes)", gbps, "GB/s"
@@ -212,6 +234,7 @@ class Bench:
             "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": f"{a.workload}: {self.desc}", "m": self.m, "layers": a.layers,
                        "activations": a.act, "outputs": a.out, "launch": "eager" if a.eager else "hip-graph",
+                       "calls": "turq_qmatmul" if a.single_calls else "turq_qmatmul_multi",
                        "step_bytes": int(self.step_bytes), "device": self.device, "compute_units": self.cus,
                        "max_rel_l2_vs_oracle": float(f"{rel:.3e}")},
             "whole_step_gbps": round(gbps, 1), "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
@@ -273,6 +296,8 @@ def main():
     ap.add_argument("--out", default="f32", choices=sorted(OUT), help="output element type")
     ap.add_argument("--eager", action="store_true", help="launch every call from the host instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--single-calls", action="store_true",
+                    help="one turq_qmatmul per matrix instead of turq_qmatmul_multi per group of matrices with a common input")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the workload, run a plain copy kernel of known size (dequantize of an F32 tensor: 256 MiB "
                          "read + 256 MiB written) three times, as the yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")

@@ -150,6 +150,16 @@ int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem
 int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype, int64_t m,
                  int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias, int mem, int algo);
 
+/* The same product for `count` weights that take the same activations: ys[i][m, n_i] = x[m, k] * W_i^T (+ biases[i]).
+ * All weights must share k.  With device pointers, tiled weights, m <= 4 and 16-byte aligned activation rows,
+ * neighbouring weights of one format go out as ONE kernel launch; every other case is exactly the
+ * turq_qmatmul calls one after the other (including their errors).  `biases` may be NULL, and so may its entries.
+ * Replaces: the back-to-back `forward` calls on one input in the reference's decoder layer - q_proj / k_proj /
+ * v_proj (src/models/qwen3.rs:272-274) and gate_proj / up_proj (src/models/qwen3.rs:161-167). */
+int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int x_dtype, int64_t m,
+                       int64_t ldx, void *const *ys, int y_dtype, const int64_t *ldys, const float *const *biases, int mem,
+                       int algo);
+
 /* ---- activation quantisation (candle's VecDotType::from_float, bit-exact) ---- */
 /* x f32 [m, k] (row stride k) -> Q8_0 blocks (34 B per 32) / Q8_K blocks (292 B per 256).
  * The GPU forward path does not use them (it keeps activations in f16); they are the device

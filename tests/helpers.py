@@ -65,6 +65,54 @@ class Gpu:
             y = synth.from_bf16_bits(y).reshape(m, ldy)
         return np.asarray(y, np.float32)[:, :n]
 
+    def qmatmul_multi(self, ws, x, ns, k, x_dtype=capi.ACT_F32, biases=None, mem=capi.MEM_DEVICE):
+        """several weights against the same activations through turq_qmatmul_multi; f32 outputs.
+        With mem = MEM_DEVICE the activations, biases and outputs live in device buffers."""
+        L, ctx = self.L, self.ctx
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
+        m = x.shape[0]
+        xsend = synth.to_bf16_bits(x).reshape(m, k) if x_dtype == capi.ACT_BF16 else x
+        count = len(ws)
+        outs = [np.zeros((m, n), np.float32) for n in ns]
+        bias_host = [None if biases is None or b is None else np.ascontiguousarray(b, np.float32) for b in (biases or [None] * count)]
+        freed = []
+
+        def dev(nbytes):
+            p = ctypes.c_void_p()
+            capi.check(L.turq_dev_alloc(ctx, max(nbytes, 16), ctypes.byref(p)), ctx)
+            freed.append(p)
+            return p
+
+        if mem == capi.MEM_DEVICE:
+            xd = dev(xsend.nbytes)
+            capi.check(L.turq_memcpy_h2d(ctx, xd, capi.ptr(xsend), xsend.nbytes), ctx)
+            yd = [dev(o.nbytes) for o in outs]
+            bd = []
+            for b in bias_host:
+                if b is None:
+                    bd.append(None)
+                else:
+                    p = dev(b.nbytes)
+                    capi.check(L.turq_memcpy_h2d(ctx, p, capi.ptr(b), b.nbytes), ctx)
+                    bd.append(p)
+            xp, yp, bp = xd, [p.value for p in yd], [None if p is None else p.value for p in bd]
+        else:
+            xp, yp = capi.ptr(xsend), [o.ctypes.data for o in outs]
+            bp = [None if b is None else b.ctypes.data for b in bias_host]
+        warr = (ctypes.c_void_p * count)(*[w.value for w in ws])
+        yarr = (ctypes.c_void_p * count)(*yp)
+        barr = (ctypes.c_void_p * count)(*bp)
+        ldys = (ctypes.c_int64 * count)(*ns)
+        rc = L.turq_qmatmul_multi(ctx, count, warr, xp, x_dtype, m, k, yarr, capi.ACT_F32, ldys,
+                                  barr if biases is not None else None, mem, capi.ALGO_AUTO)
+        capi.check(rc, ctx)
+        if mem == capi.MEM_DEVICE:
+            for o, p in zip(outs, yd):
+                capi.check(L.turq_memcpy_d2h(ctx, capi.ptr(o), p, o.nbytes), ctx)
+        for p in freed:
+            capi.check(L.turq_dev_free(ctx, p), ctx)
+        return outs
+
     def quantize(self, x, kind):
         x = np.ascontiguousarray(x, np.float32)
         m, k = x.shape

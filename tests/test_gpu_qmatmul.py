@@ -8,6 +8,8 @@ and two sharper ones that catch indexing slips the loose bars could hide:
   * the MFMA kernel must agree to 2e-5 once the oracle is given the same f16-rounded activations
     (its weight side is exact integer arithmetic).
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -236,3 +238,51 @@ def test_prefill_gemm_large_scales_fall_back(gpu):
     gpu.release(w)
     assert np.all(np.isfinite(y))
     assert rel_l2(y, orc.matmul_dequant(Q4_K, x, raw, n, k)) <= 2e-5
+
+
+# ---------------------------------------------------------------------------------------------
+# several weights against the same activations (q/k/v, gate/up): one launch per run of equal formats
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dts", [(Q4_K, Q4_K), (Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0), (Q4_K, Q4_K, Q6_K), (Q5_K, Q4_K, Q4_K, Q4_K, Q4_K, Q4_K)])
+@pytest.mark.parametrize("m", [1, 3])
+def test_multi_weight_launch(gpu, dts, m):
+    k = 1024
+    ns = [64, 100, 272, 16, 48, 528][: len(dts)]
+    raws = [synth.random_weight(dt, n, k, seed=10 * i + n) for i, (dt, n) in enumerate(zip(dts, ns))]
+    ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
+    x = synth.random_activation(m, k, seed=m, bf16=True)
+    biases = [None if i == 1 else np.random.default_rng(i).standard_normal(n).astype(np.float32) for i, n in enumerate(ns)]
+    for x_dtype in (capi.ACT_F32, capi.ACT_BF16):
+        ys = gpu.qmatmul_multi(ws, x, ns, k, x_dtype=x_dtype, biases=biases)
+        for dt, n, raw, w, y, b in zip(dts, ns, raws, ws, ys, biases):
+            want = orc.matmul_dequant(dt, x, raw, n, k) + (0 if b is None else b)
+            assert rel_l2(y, want) <= 2e-5, (dt, n)
+            single = gpu.qmatmul(w, x, n, k, x_dtype=x_dtype, bias=b)
+            assert rel_l2(y, single) <= 1e-6, (dt, n)     # same kernel body; only the split over waves may differ
+    for w in ws:
+        gpu.release(w)
+
+
+def test_multi_weight_falls_back_to_single_calls(gpu):
+    # more than four rows, or host pointers: the same as the calls one after the other
+    k, ns, dts = 512, [48, 80], (Q4_K, Q4_K)
+    raws = [synth.random_weight(dt, n, k, seed=n) for dt, n in zip(dts, ns)]
+    ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
+    for m, mem in ((8, capi.MEM_DEVICE), (2, capi.MEM_HOST), (40, capi.MEM_DEVICE)):
+        x = synth.random_activation(m, k, seed=m)
+        ys = gpu.qmatmul_multi(ws, x, ns, k, mem=mem)
+        for dt, n, raw, y in zip(dts, ns, raws, ys):
+            # 40 rows take the prefill GEMM with its f16-folded scales, the others the exact skinny kernel
+            assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, k)) <= (1e-3 if m > 32 else 2e-5)
+    # an argument a single call refuses is refused here too
+    L, ctx = gpu.L, gpu.ctx
+    warr = (ctypes.c_void_p * 2)(ws[0].value, None)
+    yarr = (ctypes.c_void_p * 2)(None, None)
+    ldys = (ctypes.c_int64 * 2)(*ns)
+    assert L.turq_qmatmul_multi(ctx, 2, warr, None, capi.ACT_F32, 1, k, yarr, capi.ACT_F32, ldys, None, capi.MEM_DEVICE,
+                                capi.ALGO_AUTO) == capi.ERR_INVALID
+    assert L.turq_qmatmul_multi(ctx, 0, None, None, capi.ACT_F32, 1, k, None, capi.ACT_F32, None, None, capi.MEM_DEVICE,
+                                capi.ALGO_AUTO) == capi.OK
+    for w in ws:
+        gpu.release(w)
+

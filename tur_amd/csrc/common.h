@@ -140,6 +140,10 @@ hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t 
 
 // largest m the skinny MFMA kernel takes; above it the LDS-tiled GEMM runs
 #define TURQ_GEMV_MAX_M 32
+// up to this many rows the skinny kernel prepares the activations itself (no separate launch)
+#define TURQ_GEMV_FUSED_MAX_M 4
 // MFMA paths on the tiled layout (activation preparation + kernel launch), see mfma_dispatch.cpp
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
                       int yt, int64_t ldy, const float *bias, int algo);
+int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m,
+                            int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias);

@@ -332,11 +332,11 @@ __device__ inline AFrags<DT, 1> stage_frags_lds(const XRegs<XT, MP> &xr, uint8_t
 // otherwise they come from the fragment buffer written by the activation preparation kernel.
 // P = tiles whose loads a wave keeps in flight together.
 // MAXT = largest workgroup the instantiation is launched with (bounds the registers per lane).
-template <int DT, int MT, int XT, bool FUSED, int MP, int P, int MAXT>
-__global__ void __launch_bounds__(MAXT) gemv_mfma_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
-                                                          const void *__restrict__ xin, int64_t ldx, int64_t m,
-                                                          int mpad, void *__restrict__ y, int yt, int64_t ldy,
-                                                          const float *__restrict__ bias) {
+// the work of one workgroup: row tile rt of one weight
+template <int DT, int MT, int XT, bool FUSED, int MP, int P>
+__device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ w, int64_t n, int64_t k, const void *__restrict__ xin,
+                                          int64_t ldx, int64_t m, int mpad, void *__restrict__ y, int yt, int64_t ldy,
+                                          const float *__restrict__ bias, int64_t rt) {
     extern __shared__ uint8_t smem[];
     constexpr int NQ = DT == TURQ_Q8_0 ? TURQ_NQ_Q8_0 : TURQ_NQ_KQUANT;
     constexpr int TB = TiledFmt<DT>::kTileBytes;
@@ -344,7 +344,6 @@ __global__ void __launch_bounds__(MAXT) gemv_mfma_kernel(const uint8_t *__restri
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // wave-uniform: scalar address math
     const int nwaves = blockDim.x >> 6;
-    const int64_t rt = blockIdx.x;
     const int64_t ntc = turq_tile_cols(k);
     const int64_t tile_chunks = (int64_t)NQ * 4 * mpad;  // 16-byte chunks of one (mt, b) fragment set
     const int64_t mt_stride = ntc * tile_chunks;
@@ -453,6 +452,45 @@ __global__ void __launch_bounds__(MAXT) gemv_mfma_kernel(const uint8_t *__restri
         }
 }
 
+template <int DT, int MT, int XT, bool FUSED, int MP, int P, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_mfma_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
+                                                          const void *__restrict__ xin, int64_t ldx, int64_t m,
+                                                          int mpad, void *__restrict__ y, int yt, int64_t ldy,
+                                                          const float *__restrict__ bias) {
+    gemv_body<DT, MT, XT, FUSED, MP, P>(w, n, k, xin, ldx, m, mpad, y, yt, ldy, bias, (int64_t)blockIdx.x);
+}
+
+// Several weights of one format and one k against the same activations in one launch (gate and up, or q and k,
+// of a decoder layer): workgroups [first[i], first[i + 1]) work on weight i.  One launch instead of several
+// spares the small matrices their start-up and tail, which at decode sizes is a third of a launch.
+constexpr int kMaxMulti = 4;
+struct MultiArgs {
+    const uint8_t *w[kMaxMulti];
+    void *y[kMaxMulti];
+    const float *bias[kMaxMulti];
+    int64_t n[kMaxMulti], ldy[kMaxMulti];
+    int first[kMaxMulti];
+    int count;
+};
+
+template <int DT, int XT, int MP, int P, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_multi_kernel(MultiArgs a, int64_t k, const void *__restrict__ x, int64_t ldx,
+                                                           int64_t m, int yt) {
+    // wave-uniform selection without indexing the argument block dynamically
+    const int blk = (int)blockIdx.x;
+    const uint8_t *w = a.w[0];
+    void *y = a.y[0];
+    const float *bias = a.bias[0];
+    int64_t n = a.n[0], ldy = a.ldy[0];
+    int first = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxMulti; i++)
+        if (i < a.count && blk >= a.first[i]) {
+            w = a.w[i], y = a.y[i], bias = a.bias[i], n = a.n[i], ldy = a.ldy[i], first = a.first[i];
+        }
+    gemv_body<DT, 1, XT, true, MP, P>(w, n, k, x, ldx, m, MP, y, yt, ldy, bias, (int64_t)(blk - first));
+}
+
 struct GemvArgs {
     const void *w; int64_t n, k; const void *xin; int64_t ldx, m; void *y; int yt; int64_t ldy; const float *bias;
     int nwaves; hipStream_t s;
@@ -513,7 +551,84 @@ hipError_t launch_x(int xt, bool fused, const GemvArgs &a) {
     }
 }
 
+template <int DT, int XT, int MP, int P, int MAXT>
+hipError_t launch_multi_final(const MultiArgs &ma, int total_blocks, int64_t k, const void *x, int64_t ldx, int64_t m, int yt,
+                              int nwaves, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    const size_t region = (size_t)MP * (512 + 64);
+    const size_t red = (size_t)MP * 16 * 16 * sizeof(float);
+    const size_t lds = (size_t)nwaves * region + (nwaves > 1 ? red : 0);
+    if (ev0) {
+        hipExtLaunchKernelGGL((gemv_multi_kernel<DT, XT, MP, P, MAXT>), dim3((unsigned)total_blocks), dim3((unsigned)(64 * nwaves)),
+                              (unsigned)lds, s, ev0, ev1, 0, ma, k, x, ldx, m, yt);
+        return hipGetLastError();
+    }
+    gemv_multi_kernel<DT, XT, MP, P, MAXT><<<(unsigned)total_blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(ma, k, x, ldx, m, yt);
+    return hipGetLastError();
+}
+
+template <int DT, int XT, int MP>
+hipError_t launch_multi_p(const MultiArgs &ma, int total_blocks, int64_t k, const void *x, int64_t ldx, int64_t m, int yt,
+                          int nwaves, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
+    if (nwaves <= 4) {
+        if (per_wave <= 1) return launch_multi_final<DT, XT, MP, 1, 256>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+        if (per_wave <= 2) return launch_multi_final<DT, XT, MP, 2, 256>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+        return launch_multi_final<DT, XT, MP, 4, 256>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+    }
+    if (per_wave <= 1) return launch_multi_final<DT, XT, MP, 1, 1024>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+    return launch_multi_final<DT, XT, MP, 2, 1024>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+}
+
+template <int DT, int XT>
+hipError_t launch_multi_m(const MultiArgs &ma, int total_blocks, int64_t k, const void *x, int64_t ldx, int64_t m, int yt,
+                          int nwaves, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    if (m <= 1) return launch_multi_p<DT, XT, 1>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+    if (m <= 2) return launch_multi_p<DT, XT, 2>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+    return launch_multi_p<DT, XT, 4>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+}
+
+template <int DT>
+hipError_t launch_multi_x(int xt, const MultiArgs &ma, int total_blocks, int64_t k, const void *x, int64_t ldx, int64_t m,
+                          int yt, int nwaves, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    switch (xt) {
+    case TURQ_ACT_F32: return launch_multi_m<DT, TURQ_ACT_F32>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+    case TURQ_ACT_BF16: return launch_multi_m<DT, TURQ_ACT_BF16>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+    case TURQ_ACT_F16: return launch_multi_m<DT, TURQ_ACT_F16>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 }  // namespace
+
+// count (2..4) weights of one format and one k, raw activations (m <= TURQ_GEMV_FUSED_MAX_M, rows 16-byte aligned)
+hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w, const int64_t *n, int64_t k, const void *x,
+                                  int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
+                                  const float *const *bias, int nwaves, hipStream_t stream, hipEvent_t ev_start,
+                                  hipEvent_t ev_stop) {
+    if (count < 1 || count > kMaxMulti || m < 1 || m > TURQ_GEMV_FUSED_MAX_M || nwaves < 1 || nwaves > 16) return hipErrorInvalidValue;
+    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    MultiArgs ma{};
+    int64_t blocks = 0;
+    for (int i = 0; i < count; i++) {
+        ma.w[i] = (const uint8_t *)w[i];
+        ma.y[i] = y[i];
+        ma.bias[i] = bias ? bias[i] : nullptr;
+        ma.n[i] = n[i];
+        ma.ldy[i] = ldy[i];
+        ma.first[i] = (int)blocks;
+        blocks += turq_tile_rows(n[i]);
+    }
+    ma.count = count;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    switch (dtype) {
+    case TURQ_Q4_K: return launch_multi_x<TURQ_Q4_K>(x_dtype, ma, (int)blocks, k, x, ldx, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q5_K: return launch_multi_x<TURQ_Q5_K>(x_dtype, ma, (int)blocks, k, x, ldx, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q6_K: return launch_multi_x<TURQ_Q6_K>(x_dtype, ma, (int)blocks, k, x, ldx, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q8_0: return launch_multi_x<TURQ_Q8_0>(x_dtype, ma, (int)blocks, k, x, ldx, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+    default: return hipErrorInvalidValue;
+    }
+}
 
 // `xin` is the prepared fragment buffer (fused == false; ldx and x_dtype unused) or the raw
 // activations (fused == true, m <= TURQ_GEMV_FUSED_MAX_M).

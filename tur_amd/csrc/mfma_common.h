@@ -34,8 +34,6 @@ typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
 
 #define TURQ_NQ_KQUANT 9
 #define TURQ_NQ_Q8_0 8
-// up to this many rows the GEMV kernel prepares the activations itself (no separate launch)
-#define TURQ_GEMV_FUSED_MAX_M 4
 
 __host__ __device__ inline int turq_mpad(int64_t rows) {
     return rows <= 1 ? 1 : rows <= 2 ? 2 : rows <= 4 ? 4 : rows <= 8 ? 8 : 16;
@@ -109,6 +107,10 @@ hipError_t turq_launch_gemv_mfma(int dtype, const void *w_tiled, int64_t n, int6
                                  int64_t ldx, int64_t m, bool fused, void *y, int y_dtype, int64_t ldy,
                                  const float *bias, int waves_per_group, hipStream_t stream, hipEvent_t ev_start,
                                  hipEvent_t ev_stop);
+hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w_tiled, const int64_t *n, int64_t k, const void *x,
+                                  int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
+                                  const float *const *bias, int waves_per_group, hipStream_t stream, hipEvent_t ev_start,
+                                  hipEvent_t ev_stop);
 hipError_t turq_launch_gemm_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
                                  int y_dtype, int64_t ldy, const float *bias, hipStream_t stream, hipEvent_t ev_start,
                                  hipEvent_t ev_stop);
