@@ -2,19 +2,22 @@
 """Benchmark of the GGUF quantized-linear hot path on one MI355X.
 
 Default workload (the configuration the headline metric is quoted on): Q4_K decode GEMV at the
-Qwen3-8B MLP shapes — gate_proj and up_proj [12288 x 4096], down_proj [4096 x 12288] — at m = 1.
+Qwen3-8B MLP shapes - gate_proj and up_proj [12288 x 4096], down_proj [4096 x 12288] - at m = 1.
 One "step" is one decode pass over the MLPs of `--layers` decoder layers (default 36, the depth of
 Qwen3-8B): 3 * layers quantized matmuls, each on its OWN copy of the weights in HBM, so a step
 streams layers * 84.9 MB (3.06 GB by default) and nothing is served from the 256 MB Infinity
-Cache.  Inputs are resident in HBM when the clock starts; every matmul includes its activation
-preparation kernel.  The step is captured once into a HIP graph and replayed (one launch per step).
+Cache.  Inputs are resident in HBM when the clock starts.  Matrices that take the same input (gate
+and up; q, k and v) are issued through turq_qmatmul_multi, as the reference calls them back to back
+on one tensor: for up to four activation rows that is one kernel launch per run of equal formats
+(`--single-calls` issues one turq_qmatmul per matrix instead).  The step is captured once into a HIP
+graph and replayed (one graph launch per step).
 
 Prints ONE JSON line.  `value` is whole-step algorithmic bytes (weights + activations + outputs)
-per second.  `roofline` prices the dominant kernel (the MFMA GEMV) alone: algorithmic bytes of one
-launch over its average duration, measured with HIP event pairs around every launch of it in a
-second, untimed pass of the same steps.  `cpu_baseline` times the oracle's restatement of candle's
-CPU QMatMul (quantise activations to Q8_K, integer dot products) on the host cores on one layer's
-three matmuls.
+per second (TFLOP/s for the prefill workload).  `roofline` prices the matmul kernels alone:
+algorithmic bytes (or flops) of the step over the sum of the kernel durations, i.e. per average
+launch, measured with HIP events stamped with every kernel's own begin and end in a second, untimed
+pass of the same steps.  `cpu_baseline` times the oracle's restatement of candle's CPU QMatMul
+(quantise activations to Q8_K, integer dot products) on the host cores on one layer's matmuls.
 """
 from __future__ import annotations
 
@@ -34,9 +37,15 @@ from tur_amd import capi, synth  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
 MFMA_F16_PEAK_TFLOPS = 2500.0   # dense f16 / bf16 MFMA, vendor figure
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by the same
-# counters on a copy kernel of known size (profiles/gemv_mfma_q4k_mlp_8b_m1.md); keyed by (workload, m, activations)
-TRAFFIC = {("q4k_mlp_8b", 1, "f32"): 28_680_000}
+# HBM bytes per launch of the timed kernels (average over the launches of a step) from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE, scaled by the same counters on a copy kernel of known size (summaries under profiles/); keyed by
+# (workload, m, activations, one call per matrix?)
+TRAFFIC = {
+    ("q4k_mlp_8b", 1, "f32", False): 42_894_850,    # gate + up in one launch 56 986 200, down 28 803 500
+    ("q4k_mlp_8b", 1, "f32", True): 28_680_000,
+    ("q4k_prefill_up_8b", 512, "bf16", False): 76_816_300,   # every XCD's L2 fetches the activation fragments once
+    ("q4k_prefill_up_8b", 512, "bf16", True): 76_816_300,
+}
 
 WORKLOADS = {
     # name: (description, [(label, ggml dtype, n, k), ...] per layer)
@@ -214,7 +223,7 @@ class Bench:
             tfl = flops_per_launch / (avg_us * 1e-6) / 1e12
             roofline = {
                 "bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(tfl / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                "frac": round(tfl / MFMA_F16_PEAK_TFLOPS, 4), "traffic": TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls))),
                 "kernel": "gemm_q4k_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "flops_per_launch": int(flops_per_launch),
             }
@@ -222,7 +231,7 @@ class Bench:
         else:
             roofline = {
                 "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC.get((a.workload, self.m, a.act)),
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls))),
                 "kernel": "gemv_mfma_kernel" if a.single_calls or self.m > 4 else "gemv_multi_kernel / gemv_mfma_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "algorithmic_bytes_per_launch": int(bytes_per_launch),
             }
