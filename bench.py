@@ -224,7 +224,7 @@ class Bench:
             roofline = {
                 "bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(tfl / MFMA_F16_PEAK_TFLOPS, 4), "traffic": TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls))),
-                "kernel": "gemm_q4k_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
+                "kernel": "gemm_kq_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "flops_per_launch": int(flops_per_launch),
             }
             metric, value, unit = "quantized prefill GEMM TFLOP/s (Q4_K, Qwen3-8B up_proj)", self.step_flops / (dt_s / a.steps) / 1e12, "TFLOP/s"

@@ -68,14 +68,14 @@ def test_mfma_gemv_tiled_layout(gpu, dt, m):
 
 @pytest.mark.parametrize("dt", ALL)
 def test_mfma_more_rows_than_one_launch(gpu, dt):
-    n, k, m = 64, 512, 70       # m > 32: the GEMM kernel (Q4_K) or chunks of 32 through the skinny kernel
+    n, k, m = 64, 512, 70       # m > 32: the GEMM kernel (K-quants) or chunks of 32 through the skinny kernel (Q8_0)
     raw = synth.random_weight(dt, n, k, seed=dt)
     x = synth.random_activation(m, k, seed=70)
     w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
     y = gpu.qmatmul(w, x, n, k)
     gpu.release(w)
     # the GEMM folds the f16 super-block scale into its f16 weights: about 3e-4 instead of exact integers
-    check_all_bars(y, dt, x, raw, n, k, f16_acts=True, sharp_bar=4e-4 if dt == Q4_K else 2e-5)
+    check_all_bars(y, dt, x, raw, n, k, f16_acts=True, sharp_bar=2e-5 if dt == Q8_0 else 4e-4)
 
 
 @pytest.mark.parametrize("dt", ALL)
@@ -196,19 +196,21 @@ def test_error_paths(gpu):
 
 
 # ---------------------------------------------------------------------------------------------
-# prefill GEMM (m > 32, Q4_K): weights carry the f16 super-block scale inside the kernel, so the
+# prefill GEMM (m > 32, K-quants): weights carry the f16 product d * sc inside the kernel, so the
 # sharp bar is looser than the GEMV's; the 1e-3 bar against the f32 matmul on dequantized weights holds
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("n,k,m", [(96, 256, 33), (200, 1024, 300), (512, 2048, 512), (100, 512, 700)])
-def test_prefill_gemm_q4k(gpu, n, k, m):
-    raw = synth.random_weight(Q4_K, n, k, seed=n + m)
+@pytest.mark.parametrize("dt", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("n,k,m", [(96, 256, 33), (200, 1024, 300), (512, 2048, 512), (100, 512, 700), (16, 768, 129)])
+def test_prefill_gemm(gpu, dt, n, k, m):
+    raw = synth.random_weight(dt, n, k, seed=n + m)
     x = synth.random_activation(m, k, seed=m, bf16=True)
-    w = gpu.upload(Q4_K, n, k, raw, capi.LAYOUT_TILED)
-    dense = orc.matmul_dequant(Q4_K, x, raw, n, k)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    dense = orc.matmul_dequant(dt, x, raw, n, k)
     y = gpu.qmatmul(w, x, n, k, algo=capi.ALGO_GEMM, x_dtype=capi.ACT_BF16)
     assert rel_l2(y, dense) <= 1e-3
     assert rel_l2(y, dense) <= 4e-4, rel_l2(y, dense)           # what the folded f16 scales are expected to cost
     yg = gpu.qmatmul(w, x, n, k, algo=capi.ALGO_GEMV, x_dtype=capi.ACT_BF16)   # same call through the chunked skinny kernel
+    assert rel_l2(yg, dense) <= 2e-5                            # (which keeps the weights as exact integers)
     assert rel_l2(y, yg) <= 5e-4
     # bf16 store, compared with the oracle rounded the same way; bias rides along
     bias = np.random.default_rng(1).standard_normal(n).astype(np.float32)
@@ -222,22 +224,25 @@ def test_prefill_gemm_q4k(gpu, n, k, m):
     # f32 activations take the same path (rounded to f16 on the way in)
     xf = synth.random_activation(m, k, seed=m + 1)
     yf = gpu.qmatmul(w, xf, n, k)
-    assert rel_l2(yf, orc.matmul_dequant(Q4_K, xf, raw, n, k)) <= 1e-3
+    assert rel_l2(yf, orc.matmul_dequant(dt, xf, raw, n, k)) <= 1e-3
     gpu.release(w)
 
 
-def test_prefill_gemm_large_scales_fall_back(gpu):
-    # d * sc * 1024 would overflow f16 inside the GEMM: the dispatcher must take the exact skinny kernel instead
+@pytest.mark.parametrize("dt", [Q4_K, Q5_K, Q6_K])
+def test_prefill_gemm_large_scales_fall_back(gpu, dt):
+    # (base + q) * d * sc would overflow f16 inside the GEMM: the dispatcher must take the exact skinny kernel instead
     n, k, m = 64, 512, 80
-    raw = synth.random_weight(Q4_K, n, k, seed=3).reshape(-1, 144)
-    raw[:, 0:2] = np.array([3.0], np.float16).view(np.uint8)     # d = 3 -> d * 63 * 1024 > 65504
+    bs = {Q4_K: 144, Q5_K: 176, Q6_K: 210}[dt]
+    raw = synth.random_weight(dt, n, k, seed=3).reshape(-1, bs)
+    d_at = 208 if dt == Q6_K else 0
+    raw[:, d_at:d_at + 2] = np.array([3.0], np.float16).view(np.uint8)     # d = 3 -> 1024 * 63 * d, 256 * 128 * d > 65504
     raw = raw.reshape(-1)
     x = synth.random_activation(m, k, seed=4, bf16=True)
-    w = gpu.upload(Q4_K, n, k, raw, capi.LAYOUT_TILED)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
     y = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
     gpu.release(w)
     assert np.all(np.isfinite(y))
-    assert rel_l2(y, orc.matmul_dequant(Q4_K, x, raw, n, k)) <= 2e-5
+    assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, k)) <= 2e-5
 
 
 # ---------------------------------------------------------------------------------------------

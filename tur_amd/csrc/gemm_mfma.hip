@@ -42,6 +42,12 @@
 // weights this costs about 3e-4 relative L2 (bar: 1e-3).  The dispatcher only uses this kernel while
 // 1024 * d * sc stays inside f16.
 //
+// Formats.  Q4_K as above (wave tile 2 x 3, workgroup 128 x 192).  Q5_K adds the fifth bit from the tile's
+// high-bit plane with one rotate and one v_and_or_b32 per packed register; Q6_K builds the whole 6-bit value in
+// the mantissa of 256.0 (low nibble at bits 2..5, high field rotated onto bits 6..7) and needs no sums term.  Their
+// tiles are larger (2816 / 3360 bytes), so their workgroup is 128 x 128 (wave tile 2 x 2) to keep three
+// super-blocks of weights in the LDS.  Q8_0 has no GEMM yet.
+//
 // Results leave through the LDS (free after the main loop): each wave transposes its 64 x 96 tile so
 // that a lane stores 16 contiguous bytes and a row segment is 192 (bf16, f16) or 384 (f32) bytes.
 #include <hip/hip_ext.h>
@@ -60,25 +66,31 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 
 constexpr uint32_t kMagic1024 = 0x64006400u;  // 1024.0: a nibble in mantissa bits 0..3 reads as 1024 + n
 constexpr uint32_t kMagic64 = 0x54005400u;    // 64.0:   a nibble in mantissa bits 4..7 reads as 64 + n
+constexpr uint32_t kMagic256 = 0x5C005C00u;   // 256.0:  a 6-bit value in mantissa bits 2..7 reads as 256 + q
 constexpr int WGM = 2, WGN = 2;               // waves of a workgroup along m and n
-constexpr int WM = 2, WN = 3;                 // 32x32 MFMA tiles per wave: 64 x 96
-constexpr int BM = WGM * WM * 32, BN = WGN * WN * 32;  // 128 x 192
+constexpr int WM = 2;                         // 32x32 MFMA tiles per wave along m
+constexpr int BM = WGM * WM * 32;             // 128
 constexpr int MT = BM / 32;                   // m-tiles per workgroup; wave w copies m-tile w
-constexpr int NT16 = BN / 16;                 // 16-row weight tiles per workgroup
-constexpr int TB = TiledFmt<TURQ_Q4_K>::kTileBytes;  // 2304: [QA 1024][QB 1024][HDR 256]
 constexpr int A_STAGE = MT * 4 * 1024;        // [m-tile][step] blocks of 1 KiB
 constexpr int NA = 4;                         // stage ring; 4 stages per super-block, so stage ks lives in buffer ks
-constexpr int W_BYTES = NT16 * TB;            // 27648 = 27 copies of 1 KiB
-constexpr int W_CHUNKS = W_BYTES / 1024;
-constexpr int NW = 3;
+constexpr int NW = 3;                         // weight ring (super-blocks)
 constexpr int S_BYTES = MT * 1024;
 constexpr int NS = 2;
-constexpr int A_OFF = 0, W_OFF = NA * A_STAGE, S_OFF = W_OFF + NW * W_BYTES;
-constexpr int LDS_BYTES = S_OFF + NS * S_BYTES;  // 156672
-constexpr int OUT_PITCH = 104;                // floats per staged result row: rows r and r + 4 land 32 banks apart
-static_assert(MT == 4 && WGM * WGN == 4 && WM == 2 && WN == 3, "the copy and read schedules below are written for this shape");
-static_assert(W_BYTES % 1024 == 0 && W_CHUNKS <= 32, "weight copies: two per wave and group");
-static_assert(4 * 64 * OUT_PITCH * 4 <= LDS_BYTES, "result staging fits");
+static_assert(MT == 4 && WGM * WGN == 4 && WM == 2, "the copy and read schedules below are written for this shape");
+
+// geometry that depends on the format: WN = 32x32 tiles per wave along n
+template <int DT, int WN_> struct Geo {
+    static constexpr int WN = WN_;
+    static constexpr int BN = WGN * WN * 32;
+    static constexpr int NT16 = BN / 16;                           // 16-row weight tiles per workgroup
+    static constexpr int TB = TiledFmt<DT>::kTileBytes;
+    static constexpr int W_BYTES = NT16 * TB;
+    static constexpr int W_CHUNKS = (W_BYTES + 1023) / 1024;       // copies of 1 KiB; the last may be partial
+    static constexpr int W_STRIDE = W_CHUNKS * 1024;               // ring stride: a partial last copy lands in padding
+    static constexpr int A_OFF = 0, W_OFF = NA * A_STAGE, S_OFF = W_OFF + NW * W_STRIDE;
+    static constexpr int OUT_PITCH = WN * 32 + 8;                  // floats per staged result row: rows r and r + 4 land 32 banks apart
+    static_assert(W_CHUNKS <= 32, "weight copies: two per wave and group");
+};
 
 template <int... I, typename F> __device__ inline void static_for_impl(std::integer_sequence<int, I...>, F &&f) {
     (f(std::integral_constant<int, I>{}), ...);
@@ -112,6 +124,16 @@ template <int OFF, typename T> __device__ inline void lds_read128(T &dst, uint32
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
 }
 
+template <int OFF> __device__ inline void lds_read64(uint2v &dst, uint32_t addr) {
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF> __device__ inline void lds_read32(uint32_t &dst, uint32_t addr) {
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF> __device__ inline void lds_read16(uint32_t &dst, uint32_t addr) {
+    asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+
 // 64 lanes x 16 bytes, global -> LDS.  The instruction offset applies to both sides: lane l copies
 // sbase[voff_l + IMM .. + 15] to LDS byte lds_addr + IMM + 16 * l.
 template <int IMM> __device__ inline void dma_set(uint32_t voff, const uint8_t *sbase, uint32_t lds_addr) {
@@ -123,49 +145,6 @@ template <int IMM> __device__ inline void dma_set(uint32_t voff, const uint8_t *
 // same LDS base (m0) as the preceding dma_set of this wave
 template <int IMM> __device__ inline void dma_more(uint32_t voff, const uint8_t *sbase) {
     asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
-}
-
-// constants of the lane's four sub-blocks u (sub-block 4 * g32 + u of the super-block)
-struct BConsts {
-    half2v s[4], c1[4], c2[4];  // d*sc, -1024*d*sc, -64*d*sc (both halves equal)
-    half8v bmin;                // -(dmin*m_u) twice each, against the (hi, lo) sums fragment
-};
-
-__device__ inline BConsts b_consts(uint4v hd, int g32) {
-    // 24-bit groups of lane slots 2*g32 and 2*g32+1 inside the 96-bit field hd.y, hd.z, hd.w
-    // (both candidates are computed and selected: a divergent branch would cost more than the two shifts)
-    const uint32_t g0a = hd.y, g0b = __builtin_amdgcn_alignbit(hd.w, hd.z, 16);
-    const uint32_t g1a = __builtin_amdgcn_alignbit(hd.z, hd.y, 24), g1b = hd.w >> 8;
-    const uint32_t msk = (uint32_t)-g32;  // all ones for the upper lane half
-    const uint32_t G0 = (g0a & ~msk) | (g0b & msk);
-    const uint32_t G1 = (g1a & ~msk) | (g1b & msk);
-    const half2v k1024 = splat2((_Float16)1024.0f);
-    const half2v dd = splat2(h_from_bits(hd.x & 0xFFFFu));
-    const half2v dm = splat2((_Float16)(-(float)h_from_bits(hd.x >> 16)));
-    BConsts c;
-    half2v mn[2];
-#pragma unroll
-    for (int s = 0; s < 2; s++) {
-        const uint32_t G = s ? G1 : G0;
-        const half2v sc = as_half2((G & 0x3Fu) | ((G << 4) & 0x003F0000u) | kMagic1024) - k1024;
-        mn[s] = (as_half2(((G >> 6) & 0x3Fu) | ((G >> 2) & 0x003F0000u) | kMagic1024) - k1024) * dm;
-        const half2v dsc = sc * dd;  // (d*sc of half 0, d*sc of half 1), rounded to f16
-        c.s[2 * s] = splat2(dsc.x);
-        c.s[2 * s + 1] = splat2(dsc.y);
-    }
-#pragma unroll
-    for (int u = 0; u < 4; u++) {
-        c.c1[u] = c.s[u] * splat2((_Float16)-1024.0f);
-        c.c2[u] = c.s[u] * splat2((_Float16)-64.0f);
-    }
-    c.bmin = half8v{mn[0].x, mn[0].x, mn[0].y, mn[0].y, mn[1].x, mn[1].x, mn[1].y, mn[1].y};
-    return c;
-}
-
-__device__ inline half8v q4_operand(uint32_t w, half2v s, half2v c1, half2v c2) {
-    const uint32_t w8 = w >> 8;
-    return make_half8(pk_fma(and_or_h2(w, 0x000F000Fu, kMagic1024), s, c1), pk_fma(and_or_h2(w, 0x00F000F0u, kMagic64), s, c2),
-                      pk_fma(and_or_h2(w8, 0x000F000Fu, kMagic1024), s, c1), pk_fma(and_or_h2(w8, 0x00F000F0u, kMagic64), s, c2));
 }
 
 // 64-bit address arithmetic may run on the vector ALU even when every input is uniform; the copies take
@@ -184,12 +163,189 @@ __device__ inline uint32_t pack_f16x2(float a, float b) {
     return as_u32(h);
 }
 
+// ---- per-format pieces -------------------------------------------------------------------------------------
+// A lane (n32, g32) of a 32-row B tile works on row r16 = n32 % 16 of 16-row tile n32 / 16 and on that tile's lane
+// slots 2 g32 and 2 g32 + 1 (64 columns each).  Stage ks of a super-block covers the 32 columns of half (ks & 1) of
+// slot 2 g32 + (ks >> 1): operand steps i = 4 (ks & 1) + st, st = 0..3, of that slot.
+//   Stage   what a lane reads from the LDS for one stage and one 32-row tile (NSTG reads)
+//   Hdr     what it reads once per super-block (NHDR reads)
+//   Consts  packed-f16 constants derived from Hdr
+//   `tile` is the LDS address of the lane's 16-row tile in the weight ring entry.
+template <int DT> struct GFmt;
+
+struct K4Consts {
+    half2v s[4], s16[4], c1[4], c2[4];  // per sub-block u = ks: d*sc, d*sc/16, -1024*d*sc, -64*d*sc (both halves equal)
+    half8v bmin;                        // -(dmin*m_u) twice each, against the (hi, lo) sums fragment
+};
+
+// constants of the lane's four sub-blocks u (sub-block 4 * g32 + u of the super-block) from a Q4_K / Q5_K header row
+__device__ inline K4Consts k4_consts(uint4v hd, int g32) {
+    // 24-bit groups of lane slots 2*g32 and 2*g32+1 inside the 96-bit field hd.y, hd.z, hd.w
+    // (both candidates are computed and selected: a divergent branch would cost more than the two shifts)
+    const uint32_t g0a = hd.y, g0b = __builtin_amdgcn_alignbit(hd.w, hd.z, 16);
+    const uint32_t g1a = __builtin_amdgcn_alignbit(hd.z, hd.y, 24), g1b = hd.w >> 8;
+    const uint32_t msk = (uint32_t)-g32;  // all ones for the upper lane half
+    const uint32_t G0 = (g0a & ~msk) | (g0b & msk);
+    const uint32_t G1 = (g1a & ~msk) | (g1b & msk);
+    const half2v k1024 = splat2((_Float16)1024.0f);
+    const half2v dd = splat2(h_from_bits(hd.x & 0xFFFFu));
+    const half2v dm = splat2((_Float16)(-(float)h_from_bits(hd.x >> 16)));
+    K4Consts c;
+    half2v mn[2];
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+        const uint32_t G = s ? G1 : G0;
+        const half2v sc = as_half2((G & 0x3Fu) | ((G << 4) & 0x003F0000u) | kMagic1024) - k1024;
+        mn[s] = (as_half2(((G >> 6) & 0x3Fu) | ((G >> 2) & 0x003F0000u) | kMagic1024) - k1024) * dm;
+        const half2v dsc = sc * dd;  // (d*sc of half 0, d*sc of half 1), rounded to f16
+        c.s[2 * s] = splat2(dsc.x);
+        c.s[2 * s + 1] = splat2(dsc.y);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        c.s16[u] = c.s[u] * splat2((_Float16)0.0625f);
+        c.c1[u] = c.s[u] * splat2((_Float16)-1024.0f);
+        c.c2[u] = c.s[u] * splat2((_Float16)-64.0f);
+    }
+    c.bmin = half8v{mn[0].x, mn[0].x, mn[0].y, mn[0].y, mn[1].x, mn[1].x, mn[1].y, mn[1].y};
+    return c;
+}
+
+template <> struct GFmt<TURQ_Q4_K> {
+    using F = TiledFmt<TURQ_Q4_K>;
+    static constexpr int WN = 3, NSTG = 1, NHDR = 1;
+    static constexpr bool SUMS = true;
+    struct Stage { uint4v q; };
+    struct Hdr { uint4v hd; };
+    using Consts = K4Consts;
+    struct Addr { uint32_t q, h; };
+    __device__ static Addr addr(uint32_t tile, int r16, int g32) {
+        return Addr{tile + 16u * (uint32_t)(r16 + 32 * g32), tile + (uint32_t)F::kHDR + 16u * (uint32_t)r16};
+    }
+    // OFF = byte offset of the n-tile inside the ring entry (compile time)
+    template <int KS, int OFF> __device__ static void read_stage(Stage &st, const Addr &a, uint32_t ring) {
+        lds_read128<OFF + (KS & 1) * 1024 + (KS >> 1) * 256>(st.q, a.q + ring);
+    }
+    template <int OFF> __device__ static void read_hdr(Hdr &h, const Addr &a, uint32_t ring) { lds_read128<OFF>(h.hd, a.h + ring); }
+    __device__ static void pin_stage(Stage &st) { pin(st.q); }
+    __device__ static void pin_hdr(Hdr &h) { pin(h.hd); }
+    __device__ static Consts consts(const Hdr &h, int g32) { return k4_consts(h.hd, g32); }
+    __device__ static half8v bmin(const Consts &c) { return c.bmin; }
+    template <int KS, int ST> __device__ static half8v operand(const Stage &st, const Consts &c) {
+        const uint32_t w = word_of<ST>(st.q), w8 = w >> 8;
+        return make_half8(pk_fma(and_or_h2(w, 0x000F000Fu, kMagic1024), c.s[KS], c.c1[KS]), pk_fma(and_or_h2(w, 0x00F000F0u, kMagic64), c.s[KS], c.c2[KS]),
+                          pk_fma(and_or_h2(w8, 0x000F000Fu, kMagic1024), c.s[KS], c.c1[KS]),
+                          pk_fma(and_or_h2(w8, 0x00F000F0u, kMagic64), c.s[KS], c.c2[KS]));
+    }
+};
+
+template <> struct GFmt<TURQ_Q5_K> {
+    using F = TiledFmt<TURQ_Q5_K>;
+    static constexpr int WN = 2, NSTG = 2, NHDR = 1;
+    static constexpr bool SUMS = true;
+    struct Stage { uint4v q; uint2v hh; };
+    struct Hdr { uint4v hd; };
+    using Consts = K4Consts;
+    struct Addr { uint32_t q, hh, h; };
+    __device__ static Addr addr(uint32_t tile, int r16, int g32) {
+        return Addr{tile + 16u * (uint32_t)(r16 + 32 * g32), tile + (uint32_t)F::kQH + 8u * (uint32_t)(r16 + 32 * g32),
+                    tile + (uint32_t)F::kHDR + 16u * (uint32_t)r16};
+    }
+    template <int KS, int OFF> __device__ static void read_stage(Stage &st, const Addr &a, uint32_t ring) {
+        lds_read128<OFF + (KS & 1) * 1024 + (KS >> 1) * 256>(st.q, a.q + ring);
+        lds_read64<OFF + (KS >> 1) * 128>(st.hh, a.hh + ring);  // the two high-bit dwords of the lane slot
+    }
+    template <int OFF> __device__ static void read_hdr(Hdr &h, const Addr &a, uint32_t ring) { lds_read128<OFF>(h.hd, a.h + ring); }
+    __device__ static void pin_stage(Stage &st) { pin(st.q); pin(st.hh); }
+    __device__ static void pin_hdr(Hdr &h) { pin(h.hd); }
+    __device__ static Consts consts(const Hdr &h, int g32) { return k4_consts(h.hd, g32); }
+    __device__ static half8v bmin(const Consts &c) { return c.bmin; }
+    template <int KS, int ST> __device__ static half8v operand(const Stage &st, const Consts &c) {
+        // step i of the slot; with v = 4 i + t the packed register t, u = v >> 1: its two high bits sit in H0 (even t) at
+        // bits (4 + u, 20 + u) or in H1 (odd t) at bits (8 + u, 24 + u): a rotate right by u puts them on bit 4 / 20
+        // (+16 on a nibble at bits 0..3) or bit 8 / 24 (+16 on a nibble at bits 4..7 read with 16 units per step)
+        constexpr uint32_t u0 = 2 * (4 * (KS & 1) + ST);
+        const uint32_t w = word_of<ST>(st.q), w8 = w >> 8;
+        uint32_t t0 = and_or_u32(w, 0x000F000Fu, kMagic1024);
+        uint32_t t1 = and_or_u32(w, 0x00F000F0u, kMagic1024);
+        uint32_t t2 = and_or_u32(w8, 0x000F000Fu, kMagic1024);
+        uint32_t t3 = and_or_u32(w8, 0x00F000F0u, kMagic1024);
+        t0 = and_or_u32(rotr32(st.hh.x, u0), 0x00100010u, t0);
+        t1 = and_or_u32(rotr32(st.hh.y, u0), 0x01000100u, t1);
+        t2 = and_or_u32(rotr32(st.hh.x, u0 + 1), 0x00100010u, t2);
+        t3 = and_or_u32(rotr32(st.hh.y, u0 + 1), 0x01000100u, t3);
+        return make_half8(pk_fma(as_half2(t0), c.s[KS], c.c1[KS]), pk_fma(as_half2(t1), c.s16[KS], c.c2[KS]),
+                          pk_fma(as_half2(t2), c.s[KS], c.c1[KS]), pk_fma(as_half2(t3), c.s16[KS], c.c2[KS]));
+    }
+};
+
+template <> struct GFmt<TURQ_Q6_K> {
+    using F = TiledFmt<TURQ_Q6_K>;
+    static constexpr int WN = 2, NSTG = 2, NHDR = 3;
+    static constexpr bool SUMS = false;
+    struct Stage { uint4v ql, qh; };
+    struct Hdr { uint32_t sc0, sc1, d16; };  // the four int8 scales of lane slots 2 g32 and 2 g32 + 1; the row's d
+    struct Consts { half2v s[8]; };          // per 16-column group of the lane's 128 columns: d*sc, rounded to f16
+    struct Addr { uint32_t q, qh, sc, d; };
+    __device__ static Addr addr(uint32_t tile, int r16, int g32) {
+        const uint32_t slot = (uint32_t)(r16 + 32 * g32);
+        return Addr{tile + 16u * slot, tile + (uint32_t)F::kQH + 16u * slot, tile + (uint32_t)F::kSC + 4u * slot,
+                    tile + (uint32_t)F::kD + 2u * (uint32_t)r16};
+    }
+    template <int KS, int OFF> __device__ static void read_stage(Stage &st, const Addr &a, uint32_t ring) {
+        lds_read128<OFF + (KS & 1) * 1024 + (KS >> 1) * 256>(st.ql, a.q + ring);
+        lds_read128<OFF + (KS >> 1) * 256>(st.qh, a.qh + ring);  // all 64 high fields of the lane slot
+    }
+    template <int OFF> __device__ static void read_hdr(Hdr &h, const Addr &a, uint32_t ring) {
+        lds_read32<OFF>(h.sc0, a.sc + ring);
+        lds_read32<OFF + 64>(h.sc1, a.sc + ring);
+        lds_read16<OFF>(h.d16, a.d + ring);
+    }
+    __device__ static void pin_stage(Stage &st) { pin(st.ql); pin(st.qh); }
+    __device__ static void pin_hdr(Hdr &h) { pin(h.sc0); pin(h.sc1); pin(h.d16); }
+    __device__ static Consts consts(const Hdr &h, int) {
+        const float d = (float)h_from_bits(h.d16);
+        Consts c;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int sc = (int)(int8_t)((i < 4 ? h.sc0 : h.sc1) >> (8 * (i & 3)));
+            const _Float16 s = (_Float16)(d * (float)sc);
+            c.s[i] = splat2(s);
+        }
+        return c;
+    }
+    __device__ static half8v bmin(const Consts &c) { return half8v{}; }
+    template <int KS, int ST> __device__ static half8v operand(const Stage &st, const Consts &c) {
+        // step i = 4 (KS & 1) + ST of the slot: low nibbles of register t at bits 2 + 4 t (and + 16), high fields at bits
+        // 6 + 8 (i & 1) + 2 t (and + 16) of high dword i >> 1; scale group i >> 1 of the slot
+        constexpr int i = 4 * (KS & 1) + ST;
+        constexpr int grp = 4 * (KS >> 1) + (i >> 1);
+        const uint32_t wl = word_of<ST>(st.ql);
+        const uint32_t wh = word_of<(i >> 1)>(st.qh);
+        half2v r[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const uint32_t lo = and_or_u32(t == 0 ? wl : rotr32(wl, 4 * t), 0x003C003Cu, kMagic256);
+            const uint32_t hi_src = (8 * (i & 1) + 2 * t) == 0 ? wh : rotr32(wh, (uint32_t)(8 * (i & 1) + 2 * t));
+            // (256 + q) - 288 = q - 32 exactly, then one rounding in the product; a fused form would need the constant
+            // -288 * d * sc, which f16 cannot hold exactly (288 is not a power of two)
+            r[t] = (as_half2(and_or_u32(hi_src, 0x00C000C0u, lo)) - splat2((_Float16)288.0f)) * c.s[grp];
+        }
+        return make_half8(r[0], r[1], r[2], r[3]);
+    }
+};
+
 // frags: 32-row fragments, 1 KiB block index (mt * ntc + b) * 17 + q
 // vec_out: rows of y can be written as aligned 16-byte pieces
-__global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
-                                                       const uint8_t *__restrict__ frags, int64_t m, void *__restrict__ y,
-                                                       int yt, int64_t ldy, const float *__restrict__ bias, int nblocks_n,
-                                                       int nblocks_m, int vec_out) {
+template <int DT>
+__global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
+                                                      const uint8_t *__restrict__ frags, int64_t m, void *__restrict__ y,
+                                                      int yt, int64_t ldy, const float *__restrict__ bias, int nblocks_n,
+                                                      int nblocks_m, int vec_out) {
+    using Fm = GFmt<DT>;
+    using G = Geo<DT, Fm::WN>;
+    constexpr int WN = Fm::WN, TB = G::TB;
+    constexpr bool SUMS = Fm::SUMS;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -214,11 +370,12 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
     int64_t my_mt = (int64_t)mb * MT + wave;
     my_mt = my_mt < mtiles ? my_mt : mtiles - 1;
     const uint8_t *a_src = uniform_ptr(frags + ((size_t)(my_mt * ntc * 17) << 10));
-    const uint32_t a_dst = lds_base + A_OFF + (uint32_t)wave * 4096u;  // + ks * A_STAGE (+ step * 1024 by the offset)
-    const uint32_t s_dst = lds_base + S_OFF + (uint32_t)wave * 1024u;  // + (b & 1) * S_BYTES
-    // weights: copy c of a super-block covers bytes [1024 c, 1024 c + 1024) of the 12 concatenated tiles;
-    // group g = 0..3 holds copies 4g + wave and 16 + 4g + wave (the latter clamped to the last one)
-    const int tile0 = nb * NT16;
+    const uint32_t a_dst = lds_base + G::A_OFF + (uint32_t)wave * 4096u;  // + ks * A_STAGE (+ step * 1024 by the offset)
+    const uint32_t s_dst = lds_base + G::S_OFF + (uint32_t)wave * 1024u;  // + (b & 1) * S_BYTES
+    // weights: copy c of a super-block covers bytes [1024 c, 1024 c + 1024) of the concatenated tiles of the workgroup;
+    // group g = 0..3 holds copies 4g + wave and 16 + 4g + wave (clamped to the last copy; lanes past the end of the
+    // tiles re-read the last 16 bytes into the padding of the ring entry)
+    const int tile0 = nb * G::NT16;
     const uint8_t *w_src = uniform_ptr(w + (size_t)tile0 * ntc * TB);  // + b * TB
     uint32_t w_voff[4][2];
     uint32_t w_dst[4][2];
@@ -227,17 +384,18 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             int c = i == 0 ? 4 * g + wave : 16 + 4 * g + wave;
-            c = c < W_CHUNKS ? c : W_CHUNKS - 1;
-            const uint32_t o = (uint32_t)c * 1024u + lane_off;
+            c = c < G::W_CHUNKS ? c : G::W_CHUNKS - 1;
+            uint32_t o = (uint32_t)c * 1024u + lane_off;
+            o = o < (uint32_t)G::W_BYTES ? o : (uint32_t)G::W_BYTES - 16u;
             const uint32_t t = o / (uint32_t)TB;
             const uint32_t within = o - t * (uint32_t)TB;
             int tg = tile0 + (int)t;
             tg = tg < nrt ? tg : nrt - 1;  // row tiles past the end re-read the last one (never stored)
             w_voff[g][i] = (uint32_t)(tg - tile0) * (uint32_t)ntc * (uint32_t)TB + within;
-            w_dst[g][i] = lds_base + W_OFF + (uint32_t)c * 1024u;  // + ring offset
+            w_dst[g][i] = lds_base + G::W_OFF + (uint32_t)c * 1024u;  // + ring offset
         }
     // ring offsets of the weight buffers of super-blocks b, b + 1, b + 2
-    uint32_t wr0 = 0, wr1 = W_BYTES, wr2 = 2 * W_BYTES;
+    uint32_t wr0 = 0, wr1 = G::W_STRIDE, wr2 = 2 * G::W_STRIDE;
 
     auto issue_a = [&](int bb, int ks) {  // stage (bb, ks) -> stage buffer ks
         const uint8_t *src = a_src + ((size_t)(bb * 17 + 4 * ks) << 10);
@@ -252,17 +410,15 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
         dma_set<0>(w_voff[g][1], src, w_dst[g][1] + ring);
     };
     auto issue_s = [&](int bb) {
-        dma_set<0>(lane_off, a_src + ((size_t)(bb * 17 + 16) << 10), s_dst + (uint32_t)(bb & 1) * S_BYTES);
+        if constexpr (SUMS) dma_set<0>(lane_off, a_src + ((size_t)(bb * 17 + 16) << 10), s_dst + (uint32_t)(bb & 1) * S_BYTES);
     };
 
     // ---- LDS read addresses ----
     // activations: stage ks, m-tile 2 wm + i, step st at A_OFF + ks * A_STAGE + ((2 wm + i) * 4 + st) * 1024
-    const uint32_t a_rd = lds_base + A_OFF + (uint32_t)wm * (WM * 4096u) + lane_off;
-    const uint32_t s_rd = lds_base + S_OFF + (uint32_t)wm * (WM * 1024u) + lane_off;
-    // weights: 32-row tile j of this wave = 16-row tiles 6 wn + 2 j + tsel; stage ks reads lane slot
-    // r16 + 16 * (2 g32 + (ks >> 1)) of plane QA (ks even) or QB (ks odd)
-    const uint32_t w_rd = lds_base + W_OFF + (uint32_t)(6 * wn + tsel) * TB + 16u * (uint32_t)(r16 + 32 * g32);
-    const uint32_t h_rd = lds_base + W_OFF + (uint32_t)(6 * wn + tsel) * TB + 2048u + 16u * (uint32_t)r16;
+    const uint32_t a_rd = lds_base + G::A_OFF + (uint32_t)wm * (WM * 4096u) + lane_off;
+    const uint32_t s_rd = lds_base + G::S_OFF + (uint32_t)wm * (WM * 1024u) + lane_off;
+    // weights: 32-row tile j of this wave = 16-row tiles 2 WN wn + 2 j + tsel of the ring entry
+    const typename Fm::Addr w_rd = Fm::addr(lds_base + G::W_OFF + (uint32_t)(2 * WN * wn + tsel) * TB, r16, g32);
 
     float16v acc[WM][WN];
 #pragma unroll
@@ -288,25 +444,24 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
 
     half8v af[2][WM];  // [step parity][m-tile]
     half8v sf[WM];
-    uint4v wq[2][WN];  // [stage parity][n-tile]: the four operand words of the stage
-    uint4v hd[WN];
-    BConsts cs[WN], cs_next[WN];
+    typename Fm::Stage wq[2][WN];  // [stage parity][n-tile]: the packed weights of the stage
+    typename Fm::Hdr hd[WN];
+    typename Fm::Consts cs[WN], cs_next[WN];
     static_for<WN>([&](auto J) {
         constexpr int j = decltype(J)::value;
-        lds_read128<j * 2 * TB>(hd[j], h_rd);
-        lds_read128<j * 2 * TB>(wq[0][j], w_rd);
+        Fm::template read_hdr<j * 2 * TB>(hd[j], w_rd, wr0);
+        Fm::template read_stage<0, j * 2 * TB>(wq[0][j], w_rd, wr0);
     });
     lds_read128<0>(af[0][0], a_rd);
     lds_read128<4096>(af[0][1], a_rd);
     wait_lds<0>();
 #pragma unroll
     for (int j = 0; j < WN; j++) {
-        pin(hd[j]);
-        cs[j] = b_consts(hd[j], g32);
+        Fm::pin_hdr(hd[j]);
+        cs[j] = Fm::consts(hd[j], g32);
     }
 
     for (int b = 0; b < ntc; b++) {
-        const uint32_t w_cur = w_rd + wr0, w_nxt = w_rd + wr1, h_nxt = h_rd + wr1;
         const uint32_t s_cur = s_rd + (uint32_t)(b & 1) * S_BYTES;
         const int b1 = b + 1 < last ? b + 1 : last, b2 = b + 2 < last ? b + 2 : last, b3 = b + 3 < last ? b + 3 : last;
         static_for<4>([&](auto KS) {  // the four stages of the super-block: ks selects registers, buffers and offsets
@@ -325,12 +480,12 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
                     pin(af[pa][1]);
                     if constexpr (st == 0) {
 #pragma unroll
-                        for (int j = 0; j < WN; j++) pin(wq[cur][j]);
+                        for (int j = 0; j < WN; j++) Fm::pin_stage(wq[cur][j]);
                         if constexpr (ks == 3) {
 #pragma unroll
                             for (int j = 0; j < WN; j++) {
-                                pin(hd[j]);
-                                cs_next[j] = b_consts(hd[j], g32);
+                                Fm::pin_hdr(hd[j]);
+                                cs_next[j] = Fm::consts(hd[j], g32);
                             }
                         }
                     }
@@ -341,7 +496,7 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
                     pin(af[1][1]);
                     // The next stage's copies were issued three boundaries ago; younger than them are that
                     // boundary's weight (and sums) copies and everything of the two boundaries since.
-                    if constexpr (ks == 0) wait_vmcnt<14>(); else wait_vmcnt<15>();
+                    if constexpr (ks == 0 || !SUMS) wait_vmcnt<14>(); else wait_vmcnt<15>();
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
                     // now stage buffer ks is free: stage (b + 1, ks) goes there
@@ -349,42 +504,46 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
                     if constexpr (ks == 3) issue_w(b3, 0, wr0); else issue_w(b2, ks + 1, wr2);
                     if constexpr (ks == 0) issue_s(b1);
                     // first reads of the next stage, hidden under step 3's MFMAs
-                    if constexpr (ks == 3) {
+                    if constexpr (ks == 3 && SUMS) {
                         lds_read128<0>(sf[0], s_cur);
                         lds_read128<1024>(sf[1], s_cur);
                     }
-                    constexpr int nks = (ks + 1) & 3;  // next stage: plane QA / QB and lane slot half
-                    constexpr int woff = (nks & 1) * 1024 + (nks >> 1) * 256;
-                    const uint32_t w_from = ks == 3 ? w_nxt : w_cur;
-                    lds_read128<0 * 2 * TB + woff>(wq[nxt][0], w_from);
-                    lds_read128<1 * 2 * TB + woff>(wq[nxt][1], w_from);
-                    lds_read128<2 * 2 * TB + woff>(wq[nxt][2], w_from);
+                    constexpr int nks = (ks + 1) & 3;
+                    const uint32_t ring_from = ks == 3 ? wr1 : wr0;
+                    static_for<WN>([&](auto J) {
+                        constexpr int j = decltype(J)::value;
+                        Fm::template read_stage<nks, j * 2 * TB>(wq[nxt][j], w_rd, ring_from);
+                    });
                     if constexpr (ks == 2) {
-                        lds_read128<0 * 2 * TB>(hd[0], h_nxt);
-                        lds_read128<1 * 2 * TB>(hd[1], h_nxt);
-                        lds_read128<2 * 2 * TB>(hd[2], h_nxt);
+                        static_for<WN>([&](auto J) {
+                            constexpr int j = decltype(J)::value;
+                            Fm::template read_hdr<j * 2 * TB>(hd[j], w_rd, wr1);
+                        });
                     }
                     lds_read128<nks * A_STAGE>(af[0][0], a_rd);
                     lds_read128<nks * A_STAGE + 4096>(af[0][1], a_rd);
                 }
-                // operand step 4 ks + st: word st of the stage, sub-block u = ks of the lane's four
+                // operand step 4 ks + st of the lane's 128 columns
                 half8v bop[WN];
 #pragma unroll
-                for (int j = 0; j < WN; j++) bop[j] = q4_operand(word_of<st>(wq[cur][j]), cs[j].s[ks], cs[j].c1[ks], cs[j].c2[ks]);
+                for (int j = 0; j < WN; j++) bop[j] = Fm::template operand<ks, st>(wq[cur][j], cs[j]);
 #pragma unroll
                 for (int i = 0; i < WM; i++)
 #pragma unroll
                     for (int j = 0; j < WN; j++) acc[i][j] = mfma32x32x16(af[pa][i], bop[j], acc[i][j]);
             });
             if constexpr (ks == 3) {
-                // "- dmin * m" term against the sub-block sums; then the next super-block's constants take over
-                wait_lds<5>();  // all but the three weight and two fragment reads of the next stage
-                pin(sf[0]);
-                pin(sf[1]);
+                if constexpr (SUMS) {
+                    // "- dmin * m" term against the sub-block sums
+                    wait_lds<WN * Fm::NSTG + 2>();  // all but the weight and fragment reads of the next stage
+                    pin(sf[0]);
+                    pin(sf[1]);
 #pragma unroll
-                for (int i = 0; i < WM; i++)
+                    for (int i = 0; i < WM; i++)
 #pragma unroll
-                    for (int j = 0; j < WN; j++) acc[i][j] = mfma32x32x16(sf[i], cs[j].bmin, acc[i][j]);
+                        for (int j = 0; j < WN; j++) acc[i][j] = mfma32x32x16(sf[i], Fm::bmin(cs[j]), acc[i][j]);
+                }
+                // the next super-block's constants take over
 #pragma unroll
                 for (int j = 0; j < WN; j++) cs[j] = cs_next[j];
             }
@@ -401,8 +560,9 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
 
     // ---- results ----
     // 32x32 result: lane (n32, g32), register e holds row 8 * (e / 4) + 4 * g32 + e % 4 of column n32
+    constexpr int OUT_PITCH = G::OUT_PITCH;
     const int64_t row0 = (int64_t)mb * BM + wm * (WM * 32);
-    const int64_t col0 = (int64_t)nb * BN + wn * (WN * 32);
+    const int64_t col0 = (int64_t)nb * G::BN + wn * (WN * 32);
     if (vec_out) {
         float *stage = (float *)lds + (size_t)wave * (64 * OUT_PITCH);
 #pragma unroll
@@ -466,6 +626,31 @@ __global__ void __launch_bounds__(256) gemm_q4k_kernel(const uint8_t *__restrict
     }
 }
 
+template <int DT>
+hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y, int y_dtype, int64_t ldy,
+                       const float *bias, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+    using G = Geo<DT, GFmt<DT>::WN>;
+    constexpr int LDS_BYTES = G::S_OFF + (GFmt<DT>::SUMS ? NS * S_BYTES : 0);
+    static_assert(LDS_BYTES <= 160 * 1024 && 4 * 64 * G::OUT_PITCH * 4 <= LDS_BYTES, "LDS of one workgroup; result staging fits");
+    // per-lane weight offsets are 32-bit
+    if ((uint64_t)G::NT16 * (uint64_t)(k / 256) * G::TB >= (1ull << 32)) return hipErrorInvalidValue;
+    static const hipError_t attr =
+        hipFuncSetAttribute((const void *)gemm_kq_kernel<DT>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (attr != hipSuccess) return attr;
+    const int nbn = (int)((n + G::BN - 1) / G::BN), nbm = (int)((m + BM - 1) / BM);
+    const dim3 grid((unsigned)(nbn * nbm)), block(256);
+    const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
+    const int vec_out = ((uintptr_t)y % 16 == 0 && ((uint64_t)ldy * es) % 16 == 0 && n % 8 == 0) ? 1 : 0;
+    if (ev_start) {
+        hipExtLaunchKernelGGL(gemm_kq_kernel<DT>, grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
+                              (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out);
+    } else {
+        gemm_kq_kernel<DT><<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype, ldy,
+                                                               bias, nbn, nbm, vec_out);
+    }
+    return hipGetLastError();
+}
+
 }  // namespace
 
 // frags: activations prepared by turq_launch_act_prep32 for all m rows
@@ -473,22 +658,11 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
                                  int y_dtype, int64_t ldy, const float *bias, hipStream_t stream, hipEvent_t ev_start,
                                  hipEvent_t ev_stop) {
     if (n == 0 || m == 0) return hipSuccess;
-    if (dtype != TURQ_Q4_K || k <= 0 || k % 256 != 0) return hipErrorInvalidValue;
-    // per-lane weight offsets are 32-bit
-    if ((uint64_t)NT16 * (uint64_t)(k / 256) * TB >= (1ull << 32)) return hipErrorInvalidValue;
-    static const hipError_t attr =
-        hipFuncSetAttribute((const void *)gemm_q4k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    if (attr != hipSuccess) return attr;
-    const int nbn = (int)((n + BN - 1) / BN), nbm = (int)((m + BM - 1) / BM);
-    const dim3 grid((unsigned)(nbn * nbm)), block(256);
-    const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
-    const int vec_out = ((uintptr_t)y % 16 == 0 && ((uint64_t)ldy * es) % 16 == 0 && n % 8 == 0) ? 1 : 0;
-    if (ev_start) {
-        hipExtLaunchKernelGGL(gemm_q4k_kernel, grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
-                              (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out);
-    } else {
-        gemm_q4k_kernel<<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype, ldy,
-                                                            bias, nbn, nbm, vec_out);
+    if (k <= 0 || k % 256 != 0) return hipErrorInvalidValue;
+    switch (dtype) {
+    case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
+    case TURQ_Q5_K: return launch_gemm<TURQ_Q5_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
+    case TURQ_Q6_K: return launch_gemm<TURQ_Q6_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
+    default: return hipErrorInvalidValue;
     }
-    return hipGetLastError();
 }

@@ -25,8 +25,11 @@ int pick_waves(const turq_ctx *ctx, int64_t n, int64_t k) {
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
                       int yt, int64_t ldy, const float *bias, int algo) {
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
-    // prefill chunks: LDS-tiled MFMA GEMM (Q4_K; needs d * sc * 1024 to stay inside f16)
-    const bool gemm_ok = w->dtype == TURQ_Q4_K && w->max_scale * 1024.0f < 60000.0f;
+    // prefill chunks: LDS-tiled MFMA GEMM (K-quants; the largest packed-f16 value (base + q) * d * sc of the unpack
+    // must stay inside f16: base 1024 for the nibbles of Q4_K / Q5_K, 256 for the 6-bit values of Q6_K)
+    const float top = w->dtype == TURQ_Q4_K ? 1039.0f : w->dtype == TURQ_Q5_K ? 1055.0f : 319.0f;
+    const bool gemm_ok = (w->dtype == TURQ_Q4_K || w->dtype == TURQ_Q5_K || w->dtype == TURQ_Q6_K) && w->k % 256 == 0 &&
+                         w->max_scale * top < 60000.0f;
     if (algo == TURQ_ALGO_GEMM && !gemm_ok && m > TURQ_GEMV_MAX_M)
         algo = TURQ_ALGO_GEMV;  // formats without a GEMM kernel yet: walk m in chunks through the skinny kernel
     if (m > TURQ_GEMV_MAX_M && algo == TURQ_ALGO_GEMM) {
