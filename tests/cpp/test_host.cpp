@@ -60,6 +60,26 @@ int main(int argc, char **argv) {
         for (size_t i = 0; i < y.size(); i++)
             if (y[i] != y2[i]) return fail("host-pointer and device-pointer forward differ");
 
+        // two projections of the same device tensor in one call: equal to the single calls
+        {
+            turq::DeviceBuffer ya(dev, (size_t)m * n * 4), yc(dev, (size_t)m * 96 * 4);
+            turq::QMatMul::forward_multi({&copy.qmatmul(), &biased.qmatmul()}, xd.ptr(), TURQ_ACT_F32, m, k, {ya.ptr(), yc.ptr()},
+                                         TURQ_ACT_F32);
+            dev.synchronize();
+            std::vector<float> y3((size_t)m * n), y4((size_t)m * 96);
+            ya.download(y3.data(), y3.size() * 4);
+            yc.download(y4.data(), y4.size() * 4);
+            for (size_t i = 0; i < y.size(); i++)
+                if (std::fabs(y3[i] - y[i]) > 1e-4f * (1.0f + std::fabs(y[i]))) return fail("forward_multi differs from forward (first layer)");
+            turq::DeviceBuffer ys(dev, (size_t)m * 96 * 4);
+            biased.qmatmul().forward(xd.ptr(), TURQ_ACT_F32, m, k, ys.ptr(), TURQ_ACT_F32, 96);
+            dev.synchronize();
+            std::vector<float> y5((size_t)m * 96);
+            ys.download(y5.data(), y5.size() * 4);
+            for (size_t i = 0; i < y5.size(); i++)
+                if (std::fabs(y4[i] - y5[i]) > 1e-4f * (1.0f + std::fabs(y5[i]))) return fail("forward_multi differs from forward (second layer)");
+        }
+
         // dequantize of the norm weight (F32 tensor) is a copy
         std::vector<float> norm = b0.pp("attn_norm").get({k}, "weight").dequantize();
         std::printf("norm %zu %.9g %.9g\n", norm.size(), norm.front(), norm.back());

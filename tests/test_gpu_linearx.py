@@ -82,6 +82,20 @@ def test_decoder_layer_linears(model, name, out_dim, in_dim):
     assert np.max(np.abs(yb[0] - y0[0])) <= 1e-3 * np.max(np.abs(y0))
 
 
+def test_qkv_projections_in_one_call(model):
+    # the reference applies q_proj, k_proj and v_proj to the same hidden state back to back (qwen3.rs:272-274)
+    dev, vb, tensors, _, _ = model
+    names = [("attn_q", HID), ("attn_k", KV), ("attn_v", KV)]
+    layers = [qlinear.linear(HID, out, vb.pp("blk").pp(0).pp(nm)) for nm, out in names]
+    x = np.random.default_rng(5).standard_normal((1, 2, HID)).astype(np.float32)
+    ys = qlinear.QMatMul.forward_multi([l.qmatmul for l in layers], x)
+    for (nm, out), layer, y in zip(names, layers, ys):
+        assert y.shape == (1, 2, out)
+        assert np.array_equal(y, layer.forward(x))          # host tensors: literally the single calls
+    with pytest.raises(capi.TurqError):
+        qlinear.QMatMul.forward_multi([l.qmatmul for l in layers], x[..., :-1].copy())
+
+
 def test_bias_is_dequantized_at_load_and_added(model):
     dev, vb, tensors, bias, _ = model
     layer = qlinear.linear(HID, 96, vb.pp("blk").pp(0).pp("biased"))

@@ -123,6 +123,22 @@ public:
         t_.device().check(turq_qmatmul(t_.device().ctx(), t_.handle(), x_dev, x_dtype, m, ldx, y_dev, y_dtype, ldy, bias_dev,
                                        TURQ_MEM_DEVICE, TURQ_ALGO_AUTO));
     }
+    // Several projections of one device tensor (q / k / v, gate / up: src/models/qwen3.rs:161-167, 272-274), ys[i] is
+    // [m, n_i] with row stride n_i: one kernel launch per run of equal formats for m <= 4, the single calls otherwise.
+    static void forward_multi(const std::vector<const QMatMul *> &layers, const void *x_dev, int x_dtype, int64_t m, int64_t ldx,
+                              const std::vector<void *> &ys_dev, int y_dtype) {
+        if (layers.empty()) return;
+        if (layers.size() != ys_dev.size()) throw Error(TURQ_ERR_SHAPE, "forward_multi: one output per layer");
+        std::vector<const turq_weight *> w;
+        std::vector<int64_t> ldy;
+        for (const QMatMul *l : layers) {
+            w.push_back(l->t_.handle());
+            ldy.push_back(l->t_.rows());
+        }
+        const Device &d = layers[0]->t_.device();
+        d.check(turq_qmatmul_multi(d.ctx(), (int)w.size(), w.data(), x_dev, x_dtype, m, ldx, ys_dev.data(), y_dtype, ldy.data(), nullptr,
+                                   TURQ_MEM_DEVICE, TURQ_ALGO_AUTO));
+    }
     const QTensor &qtensor() const { return t_; }
 
 private:

@@ -143,6 +143,35 @@ class QMatMul:
                                       capi.MEM_HOST, algo), dev.ctx)
         return y.reshape(lead + (n,))
 
+    @staticmethod
+    def forward_multi(layers: "list[QMatMul]", xs: np.ndarray, biases: "Optional[list]" = None) -> "list[np.ndarray]":
+        """Several projections of one tensor (q / k / v, gate / up: src/models/qwen3.rs:161-167, 272-274) through
+        ``turq_qmatmul_multi``.  With host arrays, as here, that is the single calls one after the other; with
+        device-resident activations and up to four rows it is one kernel launch per run of equal formats."""
+        import ctypes
+
+        if not layers:
+            return []
+        xs = np.asarray(xs)
+        k = layers[0].qtensor._k
+        if xs.ndim < 2 or xs.shape[-1] != k or any(l.qtensor._k != k for l in layers):
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch in matmul: input {xs.shape}, layers need last dim {k}")
+        if xs.dtype != np.float32 or not xs.flags["C_CONTIGUOUS"]:
+            raise TurqError(capi.ERR_INVALID, "forward_multi needs a contiguous f32 input")
+        lead = xs.shape[:-1]
+        m = int(np.prod(lead)) if lead else 1
+        cnt = len(layers)
+        ys = [np.empty((m, l.qtensor._n), np.float32) for l in layers]
+        bs = [None if biases is None or b is None else np.ascontiguousarray(b, np.float32) for b in (biases or [None] * cnt)]
+        warr = (ctypes.c_void_p * cnt)(*[l.qtensor.handle.value for l in layers])
+        yarr = (ctypes.c_void_p * cnt)(*[y.ctypes.data for y in ys])
+        barr = (ctypes.c_void_p * cnt)(*[None if b is None else b.ctypes.data for b in bs])
+        ldys = (ctypes.c_int64 * cnt)(*[l.qtensor._n for l in layers])
+        dev = layers[0].qtensor.device
+        capi.check(dev.L.turq_qmatmul_multi(dev.ctx, cnt, warr, capi.ptr(xs), capi.ACT_F32, m, k, yarr, capi.ACT_F32, ldys,
+                                            barr if biases is not None else None, capi.MEM_HOST, capi.ALGO_AUTO), dev.ctx)
+        return [y.reshape(lead + (y.shape[1],)) for y in ys]
+
 
 class LinearX:
     """``LinearX::Quantized { qmatmul, bias }`` (src/models/layers/linear.rs:8-31)."""
