@@ -249,7 +249,7 @@ def test_prefill_gemm_large_scales_fall_back(gpu, dt):
 # several weights against the same activations (q/k/v, gate/up): one launch per run of equal formats
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dts", [(Q4_K, Q4_K), (Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0), (Q4_K, Q4_K, Q6_K), (Q5_K, Q4_K, Q4_K, Q4_K, Q4_K, Q4_K)])
-@pytest.mark.parametrize("m", [1, 3])
+@pytest.mark.parametrize("m", [1, 3, 8, 20, 32])
 def test_multi_weight_launch(gpu, dts, m):
     k = 1024
     ns = [64, 100, 272, 16, 48, 528][: len(dts)]
@@ -269,7 +269,7 @@ def test_multi_weight_launch(gpu, dts, m):
 
 
 def test_multi_weight_falls_back_to_single_calls(gpu):
-    # more than four rows, or host pointers: the same as the calls one after the other
+    # more than 32 rows, or host pointers: the same as the calls one after the other
     k, ns, dts = 512, [48, 80], (Q4_K, Q4_K)
     raws = [synth.random_weight(dt, n, k, seed=n) for dt, n in zip(dts, ns)]
     ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]

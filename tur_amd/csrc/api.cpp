@@ -405,14 +405,15 @@ int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weigh
     if (count == 0) return TURQ_OK;
     if (!weights || !ys || !ldys) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_multi: null weight, output or stride array");
     bool one_launch = mem == TURQ_MEM_DEVICE && (algo == TURQ_ALGO_AUTO || algo == TURQ_ALGO_GEMV) && count > 1 && m >= 1 &&
-                      m <= TURQ_GEMV_FUSED_MAX_M && x != nullptr;
+                      m <= TURQ_GEMV_MAX_M && x != nullptr;
     for (int i = 0; i < count && one_launch; i++) {
         const turq_weight *w = weights[i];
         one_launch = w && ys[i] && w->device == ctx->device && turq_dt_is_quant(w->dtype) && w->layout == TURQ_LAYOUT_TILED &&
                      w->k == weights[0]->k && w->k > 0 && w->n > 0 && ldys[i] >= w->n;
     }
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
-    one_launch = one_launch && xb && yb && ldx >= weights[0]->k && (uintptr_t)x % 16 == 0 && ((size_t)ldx * xb) % 16 == 0;
+    one_launch = one_launch && xb && yb && ldx >= weights[0]->k &&
+                 (m > TURQ_GEMV_FUSED_MAX_M || ((uintptr_t)x % 16 == 0 && ((size_t)ldx * xb) % 16 == 0));
     if (!one_launch) {
         // anything else is the same as the calls one after the other (which also report what is wrong with an argument)
         for (int i = 0; i < count; i++) {

@@ -491,6 +491,24 @@ __global__ void __launch_bounds__(MAXT) gemv_multi_kernel(MultiArgs a, int64_t k
     gemv_body<DT, 1, XT, true, MP, P>(w, n, k, x, ldx, m, MP, y, yt, ldy, bias, (int64_t)(blk - first));
 }
 
+// the same for 5 <= m <= 32: activation fragments prepared once by act_prep_kernel and shared by all the weights
+template <int DT, int MT, int P, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_multi_frag_kernel(MultiArgs a, int64_t k, const void *__restrict__ frags, int64_t m,
+                                                                int mpad, int yt) {
+    const int blk = (int)blockIdx.x;
+    const uint8_t *w = a.w[0];
+    void *y = a.y[0];
+    const float *bias = a.bias[0];
+    int64_t n = a.n[0], ldy = a.ldy[0];
+    int first = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxMulti; i++)
+        if (i < a.count && blk >= a.first[i]) {
+            w = a.w[i], y = a.y[i], bias = a.bias[i], n = a.n[i], ldy = a.ldy[i], first = a.first[i];
+        }
+    gemv_body<DT, MT, TURQ_ACT_F16, false, 1, P>(w, n, k, frags, 0, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
+}
+
 struct GemvArgs {
     const void *w; int64_t n, k; const void *xin; int64_t ldx, m; void *y; int yt; int64_t ldy; const float *bias;
     int nwaves; hipStream_t s;
@@ -587,6 +605,40 @@ hipError_t launch_multi_m(const MultiArgs &ma, int total_blocks, int64_t k, cons
     return launch_multi_p<DT, XT, 4>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
 }
 
+template <int DT, int MT, int P, int MAXT>
+hipError_t launch_multi_frag_final(const MultiArgs &ma, int total_blocks, int64_t k, const void *frags, int64_t m, int yt, int nwaves,
+                                   hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    const int mpad = MT > 1 ? 16 : turq_mpad(m);
+    const size_t lds = nwaves > 1 ? (size_t)nwaves * MT * 64 * sizeof(float4v) : 0;
+    if (ev0) {
+        hipExtLaunchKernelGGL((gemv_multi_frag_kernel<DT, MT, P, MAXT>), dim3((unsigned)total_blocks), dim3((unsigned)(64 * nwaves)),
+                              (unsigned)lds, s, ev0, ev1, 0, ma, k, frags, m, mpad, yt);
+        return hipGetLastError();
+    }
+    gemv_multi_frag_kernel<DT, MT, P, MAXT><<<(unsigned)total_blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(ma, k, frags, m, mpad, yt);
+    return hipGetLastError();
+}
+
+template <int DT, int MT>
+hipError_t launch_multi_frag_p(const MultiArgs &ma, int total_blocks, int64_t k, const void *frags, int64_t m, int yt, int nwaves,
+                               hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
+    if (nwaves <= 4) {
+        if (per_wave <= 1) return launch_multi_frag_final<DT, MT, 1, 256>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+        if (per_wave <= 2) return launch_multi_frag_final<DT, MT, 2, 256>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+        return launch_multi_frag_final<DT, MT, 4, 256>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+    }
+    if (per_wave <= 1 || MT > 1) return launch_multi_frag_final<DT, MT, 1, 1024>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+    return launch_multi_frag_final<DT, MT, 2, 1024>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+}
+
+template <int DT>
+hipError_t launch_multi_frag(const MultiArgs &ma, int total_blocks, int64_t k, const void *frags, int64_t m, int yt, int nwaves,
+                             hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    if (m <= 16) return launch_multi_frag_p<DT, 1>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+    return launch_multi_frag_p<DT, 2>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+}
+
 template <int DT>
 hipError_t launch_multi_x(int xt, const MultiArgs &ma, int total_blocks, int64_t k, const void *x, int64_t ldx, int64_t m,
                           int yt, int nwaves, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
@@ -600,12 +652,14 @@ hipError_t launch_multi_x(int xt, const MultiArgs &ma, int total_blocks, int64_t
 
 }  // namespace
 
-// count (2..4) weights of one format and one k, raw activations (m <= TURQ_GEMV_FUSED_MAX_M, rows 16-byte aligned)
+// count (2..4) weights of one format and one k.  fused: `x` are the raw activations (m <= TURQ_GEMV_FUSED_MAX_M, rows 16-byte
+// aligned); otherwise `x` is the fragment buffer prepared for this format (m <= TURQ_GEMV_MAX_M; x_dtype and ldx unused).
 hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w, const int64_t *n, int64_t k, const void *x,
-                                  int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
+                                  int x_dtype, int64_t ldx, int64_t m, bool fused, void *const *y, int y_dtype, const int64_t *ldy,
                                   const float *const *bias, int nwaves, hipStream_t stream, hipEvent_t ev_start,
                                   hipEvent_t ev_stop) {
-    if (count < 1 || count > kMaxMulti || m < 1 || m > TURQ_GEMV_FUSED_MAX_M || nwaves < 1 || nwaves > 16) return hipErrorInvalidValue;
+    if (count < 1 || count > kMaxMulti || m < 1 || m > (fused ? TURQ_GEMV_FUSED_MAX_M : TURQ_GEMV_MAX_M) || nwaves < 1 || nwaves > 16)
+        return hipErrorInvalidValue;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
     MultiArgs ma{};
     int64_t blocks = 0;
@@ -621,6 +675,15 @@ hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w, co
     ma.count = count;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    if (!fused) {
+        switch (dtype) {
+        case TURQ_Q4_K: return launch_multi_frag<TURQ_Q4_K>(ma, (int)blocks, k, x, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+        case TURQ_Q5_K: return launch_multi_frag<TURQ_Q5_K>(ma, (int)blocks, k, x, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+        case TURQ_Q6_K: return launch_multi_frag<TURQ_Q6_K>(ma, (int)blocks, k, x, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+        case TURQ_Q8_0: return launch_multi_frag<TURQ_Q8_0>(ma, (int)blocks, k, x, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+        default: return hipErrorInvalidValue;
+        }
+    }
     switch (dtype) {
     case TURQ_Q4_K: return launch_multi_x<TURQ_Q4_K>(x_dtype, ma, (int)blocks, k, x, ldx, m, y_dtype, nwaves, stream, ev_start, ev_stop);
     case TURQ_Q5_K: return launch_multi_x<TURQ_Q5_K>(x_dtype, ma, (int)blocks, k, x, ldx, m, y_dtype, nwaves, stream, ev_start, ev_stop);

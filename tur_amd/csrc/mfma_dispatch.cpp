@@ -66,34 +66,40 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
 }
 
 // Runs of neighbouring weights with the same format go out as one launch of the skinny kernel; the caller has
-// checked that all weights are tiled, share k and the device, that m <= TURQ_GEMV_FUSED_MAX_M and that the
-// activation rows are 16-byte aligned.
+// checked that all weights are tiled, share k and the device, that m <= TURQ_GEMV_MAX_M and, for
+// m <= TURQ_GEMV_FUSED_MAX_M, that the activation rows are 16-byte aligned.  Above that row count the activation
+// fragments are prepared once per fragment order (K-quants / Q8_0) and shared by all the weights.
 int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m,
                             int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias) {
+    const bool fused = m <= TURQ_GEMV_FUSED_MAX_M;
+    int prepared = 0;  // fragment order currently in ctx->act_prep: 0 none, 1 K-quants, 2 Q8_0
     int i = 0;
     while (i < count) {
         int j = i + 1;
         while (j < count && j - i < 4 && w[j]->dtype == w[i]->dtype) j++;
-        if (j - i == 1) {
-            int rc = turq_qmatmul_mfma(ctx, w[i], x, xt, m, ldx, y[i], yt, ldy[i], bias ? bias[i] : nullptr, TURQ_ALGO_GEMV);
-            if (rc != TURQ_OK) return rc;
-        } else {
-            const void *wp[4];
-            int64_t nn[4];
-            int64_t rows = 0;
-            for (int t = i; t < j; t++) {
-                wp[t - i] = w[t]->dev;
-                nn[t - i] = w[t]->n;
-                rows += w[t]->n;
+        if (!fused) {
+            const int order = w[i]->dtype == TURQ_Q8_0 ? 2 : 1;
+            if (prepared != order) {
+                int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep_bytes(w[i]->dtype, m, w[i]->k));
+                if (rc != TURQ_OK) return rc;
+                TURQ_HIP(ctx, turq_launch_act_prep(w[i]->dtype, x, xt, m, w[i]->k, ldx, ctx->act_prep, ctx->stream));
+                prepared = order;
             }
-            const int nwaves = pick_waves(ctx, rows, w[i]->k);
-            hipEvent_t ev0 = nullptr, ev1 = nullptr;
-            TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
-            TURQ_HIP(ctx, turq_launch_gemv_multi(w[i]->dtype, j - i, wp, nn, w[i]->k, x, xt, ldx, m, y + i, yt, ldy + i,
-                                                 bias ? bias + i : nullptr, nwaves, ctx->stream, ev0, ev1));
         }
+        const void *wp[4];
+        int64_t nn[4];
+        int64_t rows = 0;
+        for (int t = i; t < j; t++) {
+            wp[t - i] = w[t]->dev;
+            nn[t - i] = w[t]->n;
+            rows += w[t]->n;
+        }
+        const int nwaves = pick_waves(ctx, rows, w[i]->k);
+        hipEvent_t ev0 = nullptr, ev1 = nullptr;
+        TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+        TURQ_HIP(ctx, turq_launch_gemv_multi(w[i]->dtype, j - i, wp, nn, w[i]->k, fused ? x : ctx->act_prep, xt, ldx, m, fused, y + i, yt,
+                                             ldy + i, bias ? bias + i : nullptr, nwaves, ctx->stream, ev0, ev1));
         i = j;
     }
     return TURQ_OK;
 }
-
