@@ -15,47 +15,74 @@ template <int XT> __device__ inline float ld_act(const void *x, int64_t i) {
     return (float)h;
 }
 
-// One thread per (m-tile, column tile b, lane group g, row r): 64 activations of one row.
+// One workgroup of 256 threads per (m-tile, column tile b): thread (r, pc) converts the 16 columns 16 pc .. 16 pc + 15 of
+// row r (consecutive threads read consecutive columns), which are two 16-byte fragment pieces and, for the K-quants,
+// exactly one of the 16-element groups whose sum the kernels need.
 template <int XT, bool KQ>
 __global__ void __launch_bounds__(256) act_prep_kernel(const void *__restrict__ x, int64_t m, int64_t k, int64_t ldx,
-                                                       int64_t ntc, int mpad, int64_t nthreads,
-                                                       half8v *__restrict__ frags) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= nthreads) return;
+                                                       int64_t ntc, int mpad, half8v *__restrict__ frags) {
     constexpr int NQ = KQ ? TURQ_NQ_KQUANT : TURQ_NQ_Q8_0;
-    const int r = (int)(t % mpad);
-    const int g = (int)((t / mpad) & 3);
-    const int64_t tb = t / (4 * (int64_t)mpad);  // = mt * ntc + b
-    const int64_t b = tb % ntc;
-    const int64_t mt = tb / ntc;
-    const int64_t row = mt * 16 + r;
-    const bool row_ok = row < m;
-    float gsum[4] = {0.f, 0.f, 0.f, 0.f};
+    const int r = (int)threadIdx.x >> 4, pc = (int)threadIdx.x & 15;
+    if (r >= mpad) return;
+    const int64_t tb = blockIdx.x;  // mt * ntc + b
+    const int64_t b = tb % ntc, mt = tb / ntc;
+    const int64_t row = mt * 16 + r, col0 = b * 256 + 16 * pc;
+    float v[16];
+    const char *src = (const char *)x + (row * ldx + col0) * (XT == TURQ_ACT_F32 ? 4 : 2);
+    if (row < m && col0 + 16 <= k && ((uintptr_t)src & 15) == 0) {
+        if (XT == TURQ_ACT_F32) {
 #pragma unroll
-    for (int q = 0; q < 8; q++) {
-        // K-quants: lane group g owns columns 64g..64g+63, step q its 8q..8q+7
-        // Q8_0:     step q is block q (32 columns), lane group g owns 8g..8g+7 of it
-        const int64_t col0 = b * 256 + (KQ ? 64 * g + 8 * q : 32 * q + 8 * g);
-        half8v h;
+            for (int i = 0; i < 4; i++) {
+                const float4v t = ((const float4v *)src)[i];
+                v[4 * i] = t.x, v[4 * i + 1] = t.y, v[4 * i + 2] = t.z, v[4 * i + 3] = t.w;
+            }
+        } else {
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int64_t c = col0 + j;
-            const float v = (row_ok && c < k) ? ld_act<XT>(x, row * ldx + c) : 0.0f;
-            h[j] = (_Float16)v;
-            if (KQ) gsum[q >> 1] += (float)h[j];
+            for (int i = 0; i < 2; i++) {
+                const uint4v u = ((const uint4v *)src)[i];
+                const uint32_t wd[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if (XT == TURQ_ACT_BF16) {
+                        v[8 * i + 2 * j] = __uint_as_float(wd[j] << 16);
+                        v[8 * i + 2 * j + 1] = __uint_as_float(wd[j] & 0xFFFF0000u);
+                    } else {
+                        const half2v hh = as_half2(wd[j]);
+                        v[8 * i + 2 * j] = (float)hh.x;
+                        v[8 * i + 2 * j + 1] = (float)hh.y;
+                    }
+                }
+            }
         }
-        frags[((tb * NQ + q) * 4 + g) * mpad + r] = h;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = (row < m && col0 + j < k) ? ld_act<XT>(x, row * ldx + col0 + j) : 0.0f;
     }
-    if (KQ) {
-        half8v s;
+    half8v h0, h1;
+    float sum = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const _Float16 hi = (_Float16)gsum[i];
-            const _Float16 lo = (_Float16)(gsum[i] - (float)hi);
-            s[2 * i] = hi;
-            s[2 * i + 1] = lo;
-        }
-        frags[((tb * NQ + 8) * 4 + g) * mpad + r] = s;
+    for (int j = 0; j < 8; j++) {
+        h0[j] = (_Float16)v[j];
+        h1[j] = (_Float16)v[8 + j];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; j++) sum += (float)h0[j];
+#pragma unroll
+    for (int j = 0; j < 8; j++) sum += (float)h1[j];
+    half8v *tile = frags + tb * (NQ * 4 * mpad);
+    if (KQ) {
+        // lane group g owns columns 64g..64g+63, step q its 8q..8q+7
+        const int g = pc >> 2, q0 = 2 * (pc & 3);
+        tile[(q0 * 4 + g) * mpad + r] = h0;
+        tile[((q0 + 1) * 4 + g) * mpad + r] = h1;
+        const _Float16 hi = (_Float16)sum;
+        const _Float16 lo = (_Float16)(sum - (float)hi);
+        ((half2v *)&tile[(8 * 4 + g) * mpad + r])[pc & 3] = half2v{hi, lo};
+    } else {
+        // step q is block q (32 columns), lane group g owns 8g..8g+7 of it
+        const int q = pc >> 1, g0 = 2 * (pc & 1);
+        tile[(q * 4 + g0) * mpad + r] = h0;
+        tile[(q * 4 + g0 + 1) * mpad + r] = h1;
     }
 }
 
@@ -64,12 +91,11 @@ hipError_t launch(int dtype, const void *x, int64_t m, int64_t k, int64_t ldx, v
     const int64_t mtiles = (m + 15) / 16;
     const int mpad = mtiles > 1 ? 16 : turq_mpad(m);
     const int64_t ntc = (k + 255) / 256;
-    const int64_t nthreads = mtiles * ntc * 4 * mpad;
-    const unsigned grid = (unsigned)((nthreads + 255) / 256);
+    const unsigned grid = (unsigned)(mtiles * ntc);
     if (dtype == TURQ_Q8_0)
-        act_prep_kernel<XT, false><<<grid, 256, 0, s>>>(x, m, k, ldx, ntc, mpad, nthreads, (half8v *)frags);
+        act_prep_kernel<XT, false><<<grid, 256, 0, s>>>(x, m, k, ldx, ntc, mpad, (half8v *)frags);
     else
-        act_prep_kernel<XT, true><<<grid, 256, 0, s>>>(x, m, k, ldx, ntc, mpad, nthreads, (half8v *)frags);
+        act_prep_kernel<XT, true><<<grid, 256, 0, s>>>(x, m, k, ldx, ntc, mpad, (half8v *)frags);
     return hipGetLastError();
 }
 
