@@ -43,8 +43,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # dense f16 / bf16 MFMA, vendor figure
 TRAFFIC = {
     ("q4k_mlp_8b", 1, "f32", False): 42_894_850,    # gate + up in one launch 56 986 200, down 28 803 500
     ("q4k_mlp_8b", 1, "f32", True): 28_680_000,
-    ("q4k_prefill_up_8b", 512, "bf16", False): 76_816_300,   # every XCD's L2 fetches the activation fragments once
-    ("q4k_prefill_up_8b", 512, "bf16", True): 76_816_300,
+    ("q4k_prefill_up_8b", 512, "bf16", False): 76_827_600,   # every XCD's L2 fetches the activation fragments once
+    ("q4k_prefill_up_8b", 512, "bf16", True): 76_827_600,
 }
 
 WORKLOADS = {
