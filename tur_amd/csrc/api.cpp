@@ -412,8 +412,7 @@ int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weigh
                      w->k == weights[0]->k && w->k > 0 && w->n > 0 && ldys[i] >= w->n;
     }
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
-    one_launch = one_launch && xb && yb && ldx >= weights[0]->k &&
-                 (m > TURQ_GEMV_FUSED_MAX_M || ((uintptr_t)x % 16 == 0 && ((size_t)ldx * xb) % 16 == 0));
+    one_launch = one_launch && xb && yb && ldx >= weights[0]->k;
     if (!one_launch) {
         // anything else is the same as the calls one after the other (which also report what is wrong with an argument)
         for (int i = 0; i < count; i++) {

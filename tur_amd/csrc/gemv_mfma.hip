@@ -491,8 +491,82 @@ __global__ void __launch_bounds__(MAXT) gemv_multi_kernel(MultiArgs a, int64_t k
     gemv_body<DT, 1, XT, true, MP, P>(w, n, k, x, ldx, m, MP, y, yt, ldy, bias, (int64_t)(blk - first));
 }
 
+// Prepared fragments, R row tiles per workgroup: a wave applies the fragments of a column tile, once fetched, to R weight
+// tiles, which divides the fragment traffic through L2 (9 - 18 KiB per column tile against 2 - 4 KiB per weight tile) by R.
+template <int DT, int MT, int P, int R>
+__device__ __forceinline__ void gemv_frag_body(const uint8_t *__restrict__ w, int64_t n, int64_t k, const void *__restrict__ frags,
+                                               int64_t m, int mpad, void *__restrict__ y, int yt, int64_t ldy,
+                                               const float *__restrict__ bias, int64_t rtg) {
+    extern __shared__ uint8_t smem[];
+    constexpr int NQ = DT == TURQ_Q8_0 ? TURQ_NQ_Q8_0 : TURQ_NQ_KQUANT;
+    constexpr int TB = TiledFmt<DT>::kTileBytes;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nwaves = blockDim.x >> 6;
+    const int64_t ntc = turq_tile_cols(k), nrt = turq_tile_rows(n);
+    const int64_t rt0 = rtg * R;
+    const int64_t tile_chunks = (int64_t)NQ * 4 * mpad;
+    const int64_t mt_stride = ntc * tile_chunks;
+    float4v *red = (float4v *)smem;
+    float4v acc[R][MT];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[r][mt] = float4v{0.f, 0.f, 0.f, 0.f};
+    const uint8_t *wrow[R];  // row tiles past the end re-read the last one; their results are not stored
+#pragma unroll
+    for (int r = 0; r < R; r++) wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+    for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
+        WRegs<DT> wr[P][R];
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            const int64_t b = b0 + (int64_t)p * nwaves;
+            const int64_t bc = b < ntc ? b : b0;
+#pragma unroll
+            for (int r = 0; r < R; r++) wr[p][r] = load_tile<DT>(wrow[r] + bc * TB, lane);
+        }
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            const int64_t b = b0 + (int64_t)p * nwaves;
+            if (b < ntc) {  // uniform per wave
+                const AFrags<DT, MT> f = load_frags_global<DT, MT>((const half8v *)frags + b * tile_chunks, mt_stride, mpad, lane);
+#pragma unroll
+                for (int r = 0; r < R; r++) TileOp<DT, MT, 4>::run(wr[p][r], f, lane, acc[r]);
+            }
+        }
+    }
+    if (nwaves > 1) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) red[((wave * R + r) * MT + mt) * 64 + lane] = acc[r][mt];
+        __syncthreads();
+        if (wave != 0) return;
+        for (int wv = 1; wv < nwaves; wv++)
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) acc[r][mt] += red[((wv * R + r) * MT + mt) * 64 + lane];
+    }
+    // lane (nn, g) holds y[16 mt + 4 g + i][16 (rt0 + r) + nn], i = 0..3
+    const int nn = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int64_t col = (rt0 + r) * 16 + nn;
+        if (rt0 + r >= nrt || col >= n) continue;
+        const float bv = bias ? bias[col] : 0.0f;
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int64_t row = 16 * mt + 4 * g + i;
+                if (row < m) turq_store_any(y, yt, row * ldy + col, acc[r][mt][i] + bv);
+            }
+    }
+}
+
 // the same for 5 <= m <= 32: activation fragments prepared once by act_prep_kernel and shared by all the weights
-template <int DT, int MT, int P, int MAXT>
+template <int DT, int MT, int P, int MAXT, int R>
 __global__ void __launch_bounds__(MAXT) gemv_multi_frag_kernel(MultiArgs a, int64_t k, const void *__restrict__ frags, int64_t m,
                                                                 int mpad, int yt) {
     const int blk = (int)blockIdx.x;
@@ -506,7 +580,8 @@ __global__ void __launch_bounds__(MAXT) gemv_multi_frag_kernel(MultiArgs a, int6
         if (i < a.count && blk >= a.first[i]) {
             w = a.w[i], y = a.y[i], bias = a.bias[i], n = a.n[i], ldy = a.ldy[i], first = a.first[i];
         }
-    gemv_body<DT, MT, TURQ_ACT_F16, false, 1, P>(w, n, k, frags, 0, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
+    if constexpr (R == 1) gemv_body<DT, MT, TURQ_ACT_F16, false, 1, P>(w, n, k, frags, 0, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
+    else gemv_frag_body<DT, MT, P, R>(w, n, k, frags, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
 }
 
 struct GemvArgs {
@@ -605,38 +680,42 @@ hipError_t launch_multi_m(const MultiArgs &ma, int total_blocks, int64_t k, cons
     return launch_multi_p<DT, XT, 4>(ma, total_blocks, k, x, ldx, m, yt, nwaves, s, ev0, ev1);
 }
 
-template <int DT, int MT, int P, int MAXT>
+template <int DT, int MT, int P, int MAXT, int R>
 hipError_t launch_multi_frag_final(const MultiArgs &ma, int total_blocks, int64_t k, const void *frags, int64_t m, int yt, int nwaves,
                                    hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
     const int mpad = MT > 1 ? 16 : turq_mpad(m);
-    const size_t lds = nwaves > 1 ? (size_t)nwaves * MT * 64 * sizeof(float4v) : 0;
+    const size_t lds = nwaves > 1 ? (size_t)nwaves * R * MT * 64 * sizeof(float4v) : 0;
     if (ev0) {
-        hipExtLaunchKernelGGL((gemv_multi_frag_kernel<DT, MT, P, MAXT>), dim3((unsigned)total_blocks), dim3((unsigned)(64 * nwaves)),
+        hipExtLaunchKernelGGL((gemv_multi_frag_kernel<DT, MT, P, MAXT, R>), dim3((unsigned)total_blocks), dim3((unsigned)(64 * nwaves)),
                               (unsigned)lds, s, ev0, ev1, 0, ma, k, frags, m, mpad, yt);
         return hipGetLastError();
     }
-    gemv_multi_frag_kernel<DT, MT, P, MAXT><<<(unsigned)total_blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(ma, k, frags, m, mpad, yt);
+    gemv_multi_frag_kernel<DT, MT, P, MAXT, R><<<(unsigned)total_blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(ma, k, frags, m, mpad, yt);
     return hipGetLastError();
 }
 
 template <int DT, int MT>
 hipError_t launch_multi_frag_p(const MultiArgs &ma, int total_blocks, int64_t k, const void *frags, int64_t m, int yt, int nwaves,
-                               hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+                               int rtiles, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
     const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
-    if (nwaves <= 4) {
-        if (per_wave <= 1) return launch_multi_frag_final<DT, MT, 1, 256>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
-        if (per_wave <= 2) return launch_multi_frag_final<DT, MT, 2, 256>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
-        return launch_multi_frag_final<DT, MT, 4, 256>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+    if (rtiles == 2) {  // two row tiles per workgroup, at most four waves: four weight tiles in flight per wave where there are that many
+        if (per_wave <= 1) return launch_multi_frag_final<DT, MT, 1, 256, 2>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+        return launch_multi_frag_final<DT, MT, 2, 256, 2>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
     }
-    if (per_wave <= 1 || MT > 1) return launch_multi_frag_final<DT, MT, 1, 1024>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
-    return launch_multi_frag_final<DT, MT, 2, 1024>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+    if (nwaves <= 4) {
+        if (per_wave <= 1) return launch_multi_frag_final<DT, MT, 1, 256, 1>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+        if (per_wave <= 2) return launch_multi_frag_final<DT, MT, 2, 256, 1>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+        return launch_multi_frag_final<DT, MT, 4, 256, 1>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+    }
+    if (per_wave <= 1 || MT > 1) return launch_multi_frag_final<DT, MT, 1, 1024, 1>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+    return launch_multi_frag_final<DT, MT, 2, 1024, 1>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
 }
 
 template <int DT>
 hipError_t launch_multi_frag(const MultiArgs &ma, int total_blocks, int64_t k, const void *frags, int64_t m, int yt, int nwaves,
-                             hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
-    if (m <= 16) return launch_multi_frag_p<DT, 1>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
-    return launch_multi_frag_p<DT, 2>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+                             int rtiles, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    if (m <= 16) return launch_multi_frag_p<DT, 1>(ma, total_blocks, k, frags, m, yt, nwaves, rtiles, s, ev0, ev1);
+    return launch_multi_frag_p<DT, 2>(ma, total_blocks, k, frags, m, yt, nwaves, rtiles, s, ev0, ev1);
 }
 
 template <int DT>
@@ -656,11 +735,12 @@ hipError_t launch_multi_x(int xt, const MultiArgs &ma, int total_blocks, int64_t
 // aligned); otherwise `x` is the fragment buffer prepared for this format (m <= TURQ_GEMV_MAX_M; x_dtype and ldx unused).
 hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w, const int64_t *n, int64_t k, const void *x,
                                   int x_dtype, int64_t ldx, int64_t m, bool fused, void *const *y, int y_dtype, const int64_t *ldy,
-                                  const float *const *bias, int nwaves, hipStream_t stream, hipEvent_t ev_start,
+                                  const float *const *bias, int nwaves, int row_tiles, hipStream_t stream, hipEvent_t ev_start,
                                   hipEvent_t ev_stop) {
     if (count < 1 || count > kMaxMulti || m < 1 || m > (fused ? TURQ_GEMV_FUSED_MAX_M : TURQ_GEMV_MAX_M) || nwaves < 1 || nwaves > 16)
         return hipErrorInvalidValue;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (row_tiles != 1 && !(row_tiles == 2 && !fused && nwaves <= 4)) return hipErrorInvalidValue;
     MultiArgs ma{};
     int64_t blocks = 0;
     for (int i = 0; i < count; i++) {
@@ -670,17 +750,17 @@ hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w, co
         ma.n[i] = n[i];
         ma.ldy[i] = ldy[i];
         ma.first[i] = (int)blocks;
-        blocks += turq_tile_rows(n[i]);
+        blocks += (turq_tile_rows(n[i]) + row_tiles - 1) / row_tiles;
     }
     ma.count = count;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
     if (!fused) {
         switch (dtype) {
-        case TURQ_Q4_K: return launch_multi_frag<TURQ_Q4_K>(ma, (int)blocks, k, x, m, y_dtype, nwaves, stream, ev_start, ev_stop);
-        case TURQ_Q5_K: return launch_multi_frag<TURQ_Q5_K>(ma, (int)blocks, k, x, m, y_dtype, nwaves, stream, ev_start, ev_stop);
-        case TURQ_Q6_K: return launch_multi_frag<TURQ_Q6_K>(ma, (int)blocks, k, x, m, y_dtype, nwaves, stream, ev_start, ev_stop);
-        case TURQ_Q8_0: return launch_multi_frag<TURQ_Q8_0>(ma, (int)blocks, k, x, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+        case TURQ_Q4_K: return launch_multi_frag<TURQ_Q4_K>(ma, (int)blocks, k, x, m, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
+        case TURQ_Q5_K: return launch_multi_frag<TURQ_Q5_K>(ma, (int)blocks, k, x, m, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
+        case TURQ_Q6_K: return launch_multi_frag<TURQ_Q6_K>(ma, (int)blocks, k, x, m, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
+        case TURQ_Q8_0: return launch_multi_frag<TURQ_Q8_0>(ma, (int)blocks, k, x, m, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
         default: return hipErrorInvalidValue;
         }
     }

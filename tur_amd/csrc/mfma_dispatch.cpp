@@ -47,31 +47,32 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
         const uint8_t *xc = (const uint8_t *)x + (size_t)m0 * (size_t)ldx * xb;
         uint8_t *yc = (uint8_t *)y + (size_t)m0 * (size_t)ldy * yb;
         static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
-        hipEvent_t ev0 = nullptr, ev1 = nullptr;
-        TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
         // raw activation rows must be 16-byte (f32) / 8-byte (16-bit) aligned for the fused loads
         const bool aligned = ((uintptr_t)xc % 16 == 0) && ((size_t)ldx * xb) % 16 == 0;
         if (mc <= TURQ_GEMV_FUSED_MAX_M && aligned && !no_fuse) {
+            hipEvent_t ev0 = nullptr, ev1 = nullptr;
+            TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
             TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, xc, xt, ldx, mc, true, yc, yt, ldy, bias,
                                                 nwaves, ctx->stream, ev0, ev1));
             continue;
         }
-        int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep_bytes(w->dtype, mc, w->k));
+        // prepared fragments: the same path as a group of one weight
+        void *yv = yc;
+        const int rc = turq_qmatmul_multi_mfma(ctx, 1, &w, xc, xt, mc, ldx, &yv, yt, &ldy, bias ? &bias : nullptr);
         if (rc != TURQ_OK) return rc;
-        TURQ_HIP(ctx, turq_launch_act_prep(w->dtype, xc, xt, mc, w->k, ldx, ctx->act_prep, ctx->stream));
-        TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, TURQ_ACT_F16, 0, mc, false, yc, yt,
-                                            ldy, bias, nwaves, ctx->stream, ev0, ev1));
     }
     return TURQ_OK;
 }
 
 // Runs of neighbouring weights with the same format go out as one launch of the skinny kernel; the caller has
-// checked that all weights are tiled, share k and the device, that m <= TURQ_GEMV_MAX_M and, for
-// m <= TURQ_GEMV_FUSED_MAX_M, that the activation rows are 16-byte aligned.  Above that row count the activation
-// fragments are prepared once per fragment order (K-quants / Q8_0) and shared by all the weights.
+// checked that all weights are tiled, share k and the device and that m <= TURQ_GEMV_MAX_M.  Up to
+// TURQ_GEMV_FUSED_MAX_M rows with 16-byte aligned activation rows the kernel converts the activations itself; otherwise
+// the activation fragments are prepared once per fragment order (K-quants / Q8_0) and shared by all the weights.
 int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m,
                             int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias) {
-    const bool fused = m <= TURQ_GEMV_FUSED_MAX_M;
+    static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
+    const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
+    const bool fused = m <= TURQ_GEMV_FUSED_MAX_M && aligned && !no_fuse;
     int prepared = 0;  // fragment order currently in ctx->act_prep: 0 none, 1 K-quants, 2 Q8_0
     int i = 0;
     while (i < count) {
@@ -94,11 +95,18 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
             nn[t - i] = w[t]->n;
             rows += w[t]->n;
         }
-        const int nwaves = pick_waves(ctx, rows, w[i]->k);
+        // prepared fragments are the larger stream (9 - 18 KiB per column tile against 2 - 4 KiB per weight tile): with enough
+        // row tiles to keep every CU busy a workgroup takes two of them per set of fragments
+        static const int forced_r = [] { const char *e = getenv("TURQ_GEMV_ROWTILES"); return e ? atoi(e) : 0; }();
+        const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+        int rtiles = (!fused && turq_tile_rows(rows) >= 4 * cus) ? 2 : 1;
+        if (!fused && (forced_r == 1 || forced_r == 2)) rtiles = forced_r;
+        int nwaves = pick_waves(ctx, rows / rtiles, w[i]->k);
+        if (rtiles == 2) nwaves = std::min(nwaves, 4);
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
         TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
         TURQ_HIP(ctx, turq_launch_gemv_multi(w[i]->dtype, j - i, wp, nn, w[i]->k, fused ? x : ctx->act_prep, xt, ldx, m, fused, y + i, yt,
-                                             ldy + i, bias ? bias + i : nullptr, nwaves, ctx->stream, ev0, ev1));
+                                             ldy + i, bias ? bias + i : nullptr, nwaves, rtiles, ctx->stream, ev0, ev1));
         i = j;
     }
     return TURQ_OK;
