@@ -20,6 +20,16 @@ int pick_waves(const turq_ctx *ctx, int64_t n, int64_t k) {
     return (int)w;
 }
 
+// The skinny kernel can convert up to TURQ_GEMV_FUSED_MAX_M activation rows itself (no preparation launch), but every wave
+// then converts its own column tiles again for every row tile; measured, that pays for one row, and for two rows unless
+// the matrix is large enough for the two-row-tile form of the prepared path (LM head).
+// A matrix of a few MB is bound by the launch itself: there the extra preparation launch costs more than it saves.
+bool use_fused(const turq_ctx *ctx, int64_t m, int64_t row_tiles, size_t weight_bytes) {
+    const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+    if (m > TURQ_GEMV_FUSED_MAX_M) return false;
+    return m == 1 || weight_bytes < (8u << 20) || (m == 2 && row_tiles < 4 * cus);
+}
+
 }  // namespace
 
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
@@ -49,7 +59,7 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
         static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
         // raw activation rows must be 16-byte (f32) / 8-byte (16-bit) aligned for the fused loads
         const bool aligned = ((uintptr_t)xc % 16 == 0) && ((size_t)ldx * xb) % 16 == 0;
-        if (mc <= TURQ_GEMV_FUSED_MAX_M && aligned && !no_fuse) {
+        if (use_fused(ctx, mc, turq_tile_rows(w->n), w->dev_bytes) && aligned && !no_fuse) {
             hipEvent_t ev0 = nullptr, ev1 = nullptr;
             TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
             TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, xc, xt, ldx, mc, true, yc, yt, ldy, bias,
@@ -72,7 +82,13 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
                             int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias) {
     static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
     const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
-    const bool fused = m <= TURQ_GEMV_FUSED_MAX_M && aligned && !no_fuse;
+    int64_t all_tiles = 0;
+    size_t all_bytes = 0;
+    for (int t = 0; t < count; t++) {
+        all_tiles += turq_tile_rows(w[t]->n);
+        all_bytes += w[t]->dev_bytes;
+    }
+    const bool fused = use_fused(ctx, m, all_tiles, all_bytes) && aligned && !no_fuse;
     int prepared = 0;  // fragment order currently in ctx->act_prep: 0 none, 1 K-quants, 2 Q8_0
     int i = 0;
     while (i < count) {
