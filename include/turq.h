@@ -152,8 +152,8 @@ int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype
 
 /* The same product for `count` weights that take the same activations: ys[i][m, n_i] = x[m, k] * W_i^T (+ biases[i]).
  * All weights must share k.  With device pointers, tiled weights and m <= 32, neighbouring weights of one format
- * go out as ONE kernel launch (for 5 <= m <= 32, or activation rows that are not 16-byte aligned, after one
- * preparation of the activations for all the weights); every other case is exactly the turq_qmatmul calls one
+ * go out as ONE kernel launch (for more than one row on all but small matrices, or activation rows that are not
+ * 16-byte aligned, after one preparation of the activations for all the weights); every other case is exactly the turq_qmatmul calls one
  * after the other (including their errors).  `biases` may be NULL, and so may its entries.
  * Replaces: the back-to-back `forward` calls on one input in the reference's decoder layer - q_proj / k_proj /
  * v_proj (src/models/qwen3.rs:272-274) and gate_proj / up_proj (src/models/qwen3.rs:161-167). */

@@ -140,7 +140,8 @@ hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t 
 
 // largest m the skinny MFMA kernel takes; above it the LDS-tiled GEMM runs
 #define TURQ_GEMV_MAX_M 32
-// up to this many rows the skinny kernel prepares the activations itself (no separate launch)
+// largest m for which the skinny kernel can prepare the activations itself (no separate launch);
+// whether it does is decided per call in mfma_dispatch.cpp
 #define TURQ_GEMV_FUSED_MAX_M 4
 // MFMA paths on the tiled layout (activation preparation + kernel launch), see mfma_dispatch.cpp
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,

@@ -565,7 +565,7 @@ __device__ __forceinline__ void gemv_frag_body(const uint8_t *__restrict__ w, in
     }
 }
 
-// the same for 5 <= m <= 32: activation fragments prepared once by act_prep_kernel and shared by all the weights
+// the same with activation fragments prepared once by act_prep_kernel and shared by all the weights
 template <int DT, int MT, int P, int MAXT, int R>
 __global__ void __launch_bounds__(MAXT) gemv_multi_frag_kernel(MultiArgs a, int64_t k, const void *__restrict__ frags, int64_t m,
                                                                 int mpad, int yt) {

@@ -124,7 +124,7 @@ public:
                                        TURQ_MEM_DEVICE, TURQ_ALGO_AUTO));
     }
     // Several projections of one device tensor (q / k / v, gate / up: src/models/qwen3.rs:161-167, 272-274), ys[i] is
-    // [m, n_i] with row stride n_i: one kernel launch per run of equal formats for m <= 4, the single calls otherwise.
+    // [m, n_i] with row stride n_i: one kernel launch per run of equal formats for m <= 32, the single calls otherwise.
     static void forward_multi(const std::vector<const QMatMul *> &layers, const void *x_dev, int x_dtype, int64_t m, int64_t ldx,
                               const std::vector<void *> &ys_dev, int y_dtype) {
         if (layers.empty()) return;
