@@ -30,6 +30,22 @@ bool use_fused(const turq_ctx *ctx, int64_t m, int64_t row_tiles, size_t weight_
     return m == 1 || weight_bytes < (8u << 20) || (m == 2 && row_tiles < 4 * cus);
 }
 
+// one activation row, formats the sub-block-row kernel covers (TURQ_GEMV_NO_ROW1 keeps the general kernel, for comparison)
+bool use_row1(int dtype) {
+    static const bool off = getenv("TURQ_GEMV_NO_ROW1") != nullptr;
+    return !off && turq_gemv_row1_supports(dtype);
+}
+
+// Waves per workgroup of the one-row kernel: it is light on registers and on vector work, so what it wants is many waves
+// with few column tiles each (two by default), up to the largest workgroup.
+int pick_waves_row1(int64_t k) {
+    static const int forced = [] { const char *e = getenv("TURQ_GEMV_WAVES"); return e ? atoi(e) : 0; }();
+    static const int tpw = [] { const char *e = getenv("TURQ_ROW1_TPW"); return e && atoi(e) > 0 ? atoi(e) : 2; }();
+    const int64_t col_tiles = turq_tile_cols(k);
+    if (forced >= 1 && forced <= 16) return (int)std::min<int64_t>(forced, col_tiles);
+    return (int)std::max<int64_t>(1, std::min<int64_t>((col_tiles + tpw - 1) / tpw, 16));
+}
+
 }  // namespace
 
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
@@ -62,6 +78,13 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
         if (use_fused(ctx, mc, turq_tile_rows(w->n), w->dev_bytes) && aligned && !no_fuse) {
             hipEvent_t ev0 = nullptr, ev1 = nullptr;
             TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+            if (mc == 1 && use_row1(w->dtype)) {
+                const void *wp = w->dev;
+                void *yv = yc;
+                TURQ_HIP(ctx, turq_launch_gemv_row1(w->dtype, 1, &wp, &w->n, w->k, xc, xt, &yv, yt, bias ? &bias : nullptr,
+                                                    pick_waves_row1(w->k), ctx->stream, ev0, ev1));
+                continue;
+            }
             TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, xc, xt, ldx, mc, true, yc, yt, ldy, bias,
                                                 nwaves, ctx->stream, ev0, ev1));
             continue;
@@ -121,6 +144,12 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
         if (rtiles == 2) nwaves = std::min(nwaves, 4);
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
         TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+        if (fused && m == 1 && use_row1(w[i]->dtype)) {
+            TURQ_HIP(ctx, turq_launch_gemv_row1(w[i]->dtype, j - i, wp, nn, w[i]->k, x, xt, y + i, yt, bias ? bias + i : nullptr,
+                                                pick_waves_row1(w[i]->k), ctx->stream, ev0, ev1));
+            i = j;
+            continue;
+        }
         TURQ_HIP(ctx, turq_launch_gemv_multi(w[i]->dtype, j - i, wp, nn, w[i]->k, fused ? x : ctx->act_prep, xt, ldx, m, fused, y + i, yt,
                                              ldy + i, bias ? bias + i : nullptr, nwaves, rtiles, ctx->stream, ev0, ev1));
         i = j;
