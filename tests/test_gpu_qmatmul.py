@@ -246,6 +246,52 @@ def test_prefill_gemm_large_scales_fall_back(gpu, dt):
 
 
 # ---------------------------------------------------------------------------------------------
+# one activation row (decode): the kernel that applies the sub-block scales on the MFMA result
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ALL)
+@pytest.mark.parametrize("n,k", [(1, 256), (17, 256), (200, 2048), (100, 12288), (48, 4096 + 256)])
+def test_one_row(gpu, dt, n, k):
+    if dt == Q8_0:
+        k += 96                      # Q8_0 rows end inside a column tile
+    raw = synth.random_weight(dt, n, k, seed=dt + n + k)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    rng = np.random.default_rng(n * 7 + k)
+    base = synth.random_activation(1, k, seed=k + n)
+    sparse = base * (rng.random((1, k)) < 0.05)
+    cases = {
+        "normal": (base, 2e-5),
+        # no cancellation in sum(base * x): the accumulator starts 1024 * 32 * |x| away from the result
+        "one-sided": (np.abs(base) + 3.0, 1e-4),
+        "large": (base * 2000.0, 2e-5),
+        "tiny": (base * 1e-3, 2e-5),
+        "sparse": (sparse.astype(np.float32), 2e-5),
+    }
+    for name, (x, bar) in cases.items():
+        want = orc.matmul_dequant(dt, f16_round(x), raw, n, k)
+        y = gpu.qmatmul(w, x, n, k)
+        assert rel_l2(y, want) <= bar, (name, rel_l2(y, want))
+    # 16-bit activations and outputs, bias (errors measured against the product itself: a bias may cancel it)
+    x = synth.random_activation(1, k, seed=3, bf16=True)
+    bias = rng.standard_normal(n).astype(np.float32)
+    prod = orc.matmul_dequant(dt, x, raw, n, k)
+
+    def err(y, want):
+        return float(np.linalg.norm(y - want) / np.linalg.norm(prod))
+
+    assert err(gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, bias=bias), prod + bias) <= 2e-5
+    assert err(gpu.qmatmul(w, f16_round(x), n, k, x_dtype=capi.ACT_F16, bias=bias),
+               orc.matmul_dequant(dt, f16_round(x), raw, n, k) + bias) <= 2e-5
+    yb = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16, bias=bias)
+    assert rel_l2(yb, synth.from_bf16_bits(synth.to_bf16_bits(prod + bias)).reshape(1, n)) <= 2e-3
+    assert rel_l2(gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_F16, bias=bias), prod + bias) <= 5e-4
+    # the candle CPU path on the same input (its own activation quantisation is the difference: about 7e-3 once
+    # there are enough blocks to average over, more on a single super-block)
+    if k >= 2048:
+        assert rel_l2(gpu.qmatmul(w, base, n, k), orc.qmatmul(dt, base, raw, n, k)) <= 1e-2
+    gpu.release(w)
+
+
+# ---------------------------------------------------------------------------------------------
 # several weights against the same activations (q/k/v, gate/up): one launch per run of equal formats
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dts", [(Q4_K, Q4_K), (Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0), (Q4_K, Q4_K, Q6_K), (Q5_K, Q4_K, Q4_K, Q4_K, Q4_K, Q4_K)])

@@ -1,24 +1,27 @@
-// One activation row (decode) against Q4_K / Q5_K weights on the tiled layout.
+// One activation row (decode) against quantized weights on the tiled layout.
 //
 // With a single row fifteen of the sixteen A rows of v_mfma_f32_16x16x32_f16 are idle.  This kernel puts them to
-// work as SUB-BLOCK selectors: A row R of MFMA step i holds the activations of the step's 32 columns where they belong
-// to sub-block R's slot and zeros elsewhere, so after the eight steps of a 256-column tile the 16 x 16 result holds,
-// per weight row n, the eight per-sub-block dot products apart instead of their sum.  That moves the 6-bit sub-block
-// scales from the B operand (one v_pk_fma_f16 per two weights in the general kernel) to the result (one multiply-add per
-// sub-block and weight row): the B operand is the raw "magic number" f16 (base + nibble), one v_and_or_b32 per two weights
-// and nothing else.  The base is taken out through the accumulator: it starts at -sum(base * x) of the sub-block, which
-// depends on the activations only.  The result rows that no step writes carry the plain sub-block sums of x for the
-// "- dmin * m" term, so a lane finds all four factors of its four 6-bit header fields in its four result registers:
-//   result row 4g     = sum over sub-block 2g   of q * x        (field sc[2g])
-//   result row 4g + 1 = sum over sub-block 2g   of x            (field m[2g])
-//   result row 4g + 2 = sum over sub-block 2g+1 of q * x        (field sc[2g+1])
-//   result row 4g + 3 = sum over sub-block 2g+1 of x            (field m[2g+1])
-// which is the order of the 24-bit group g of the tile header.  Lane (n, g) adds d * (sc*r0 + sc'*r2) - dmin * (m*r1 + m'*r3)
-// to its partial y[n]; the four lane groups and the waves of the workgroup are summed through LDS at the end.
+// work as SUB-BLOCK selectors: A row R of an MFMA step holds the activations of the step's 32 columns where they belong
+// to the sub-block that result row R stands for and zeros elsewhere, so after the eight steps of a 256-column tile the
+// 16 x 16 result holds, per weight row n, the per-sub-block dot products apart instead of their sum.  That moves the
+// sub-block scales from the B operand (one v_pk_fma_f16 per two weights in the general kernel) to the result (one
+// multiply-add per sub-block and weight row): the B operand is the raw "magic number" f16 (base + quant), one or two
+// v_and_or_b32 per two weights and nothing else.  The base (and the format's zero point) is taken out through the
+// accumulator: it starts at -sum(base * x) over the sub-block, which depends on the activations only.
 //
-// Numerics: products are exact (integers below 2048 times f16), sums in f32.  The base term makes the partial sums about
-// 1024 * |x| large where the result is about 30 * |x|, which costs 5 bits of the f32 accumulator: measured rel-L2 against
-// the f32 matmul on dequantized weights stays below 3e-5 for bf16 activations.
+//   Q4_K / Q5_K  8 sub-blocks of 32.  Result rows 4g, 4g + 2 collect sub-blocks 2g, 2g + 1; rows 4g + 1, 4g + 3 are
+//                written by no step and carry the plain sums of x over those sub-blocks for the "- dmin * m" term.  A
+//                lane's four result registers thus meet the four 6-bit fields (sc, m, sc', m') of header group g:
+//                lane (n, g) adds d * (sc * r0 + sc' * r2) - dmin * (m * r1 + m' * r3) to its partial y[n].
+//   Q6_K         16 sub-blocks of 16, result row = sub-block: lane (n, g) holds sub-blocks 4g .. 4g + 3, whose int8
+//                scales are the dword it loads from the tile's scale plane.  Zero point 32: base 256 + 32.
+//   Q8_0         8 blocks of 32, result row = block (rows 8 .. 15 stay zero), f16 scale per block.  The tile stores
+//                the bytes offset by 128: base 1024 + 128.
+// The four lane groups and the waves of the workgroup are summed through LDS at the end.
+//
+// Numerics: products are exact (integers below 2048 times f16), sums in f32.  The base term makes the partial sums
+// up to 1024 * |x| large where the result is about 30 * |x|; measured rel-L2 against the f32 matmul on dequantized
+// weights with the same f16-rounded activations stays below 2e-5.
 //
 // Per workgroup: one 16-row tile, the waves split the column tiles; every wave converts its own slice of x (256 columns
 // per tile) to f16 through its own LDS region and computes the sub-block sums on the way.
@@ -32,41 +35,41 @@
 namespace {
 
 constexpr uint32_t kMagic1024 = 0x64006400u;  // 1024.0 in both halves: field at mantissa bit 0
+constexpr uint32_t kMagic256 = 0x5C005C00u;   // 256.0: field at mantissa bit 2
 constexpr uint32_t kMagic64 = 0x54005400u;    // 64.0: field at mantissa bit 4
 constexpr uint32_t kMagicHdr = 0x64005400u;   // header fields: low half at bit 4 of 64.0, high half at bit 0 of 1024.0
 
-// LDS region of one (wave, tile in flight): 256 f16 of x, 8 x (-base sum, plain sum), 64 bytes of zeros
+// LDS region of one (wave, tile in flight): 256 f16 of x, 16 floats the accumulator starts from, 64 bytes of zeros
 constexpr int kX = 0, kInit = 512, kZero = 576, kRegion = 640;
 
-template <int DT> struct W1Regs { uint4v qa, qb; uint2v hh; uint32_t hd, grp; };
-
-template <int DT>
-__device__ inline W1Regs<DT> load_tile1(const uint8_t *__restrict__ tile, int lane, int grp_off) {
-    using F = TiledFmt<DT>;
-    W1Regs<DT> w;
-    w.qa = *(const uint4v *)(tile + F::kQA + 16 * lane);
-    w.qb = *(const uint4v *)(tile + F::kQB + 16 * lane);
-    if constexpr (DT == TURQ_Q5_K) w.hh = *(const uint2v *)(tile + F::kQH + 8 * lane);
-    else w.hh = uint2v{0u, 0u};
-    const uint8_t *h = tile + F::kHDR + 16 * (lane & 15);
-    w.hd = *(const uint32_t *)h;                  // f16 d, f16 dmin
-    __builtin_memcpy(&w.grp, h + grp_off, 4);     // the (unaligned) dword that holds this lane's 24-bit group
-    return w;
+// v + (the same value from the lane `CTRL` points at), inside a row of 16 lanes
+template <int CTRL> __device__ inline float dpp_add(float v) {
+    const int o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false);
+    return v + __int_as_float(o);
 }
+__device__ inline float sum4(float v) {
+    v = dpp_add<0xB1>(v);  // quad_perm [1, 0, 3, 2]
+    return dpp_add<0x4E>(v);  // quad_perm [2, 3, 0, 1]
+}
+__device__ inline float sum8(float v) { return dpp_add<0x141>(sum4(v)); }  // row_half_mirror: lane i <- lane 7 - i of its half row
 
-// raw activations of one tile: 4 consecutive columns per lane, as two packed f16 registers
+__device__ inline float dot2(half2v a, _Float16 b0, float c) { return __builtin_amdgcn_fdot2(a, splat2(b0), c, false); }
+
+// raw activations of one tile: 4 consecutive columns per lane
 template <int XT> struct X1Regs { uint32_t r[XT == TURQ_ACT_F32 ? 4 : 2]; };
 
 template <int XT>
-__device__ inline X1Regs<XT> load_x1(const void *__restrict__ x, int64_t b, int lane) {
+__device__ inline X1Regs<XT> load_x1(const void *__restrict__ x, int64_t k, int64_t b, int lane) {
     X1Regs<XT> v;
-    const int64_t col = b * 256 + 4 * lane;
+    int64_t col = b * 256 + 4 * lane;
+    const bool ok = col < k;  // k is a multiple of 32 (Q8_0) or 256: four columns are in or out together
+    col = ok ? col : 0;
     if constexpr (XT == TURQ_ACT_F32) {
         const uint4v t = *(const uint4v *)((const float *)x + col);
-        v.r[0] = t.x; v.r[1] = t.y; v.r[2] = t.z; v.r[3] = t.w;
+        v.r[0] = ok ? t.x : 0u; v.r[1] = ok ? t.y : 0u; v.r[2] = ok ? t.z : 0u; v.r[3] = ok ? t.w : 0u;
     } else {
         const uint2v t = *(const uint2v *)((const uint16_t *)x + col);
-        v.r[0] = t.x; v.r[1] = t.y;
+        v.r[0] = ok ? t.x : 0u; v.r[1] = ok ? t.y : 0u;
     }
     return v;
 }
@@ -85,48 +88,183 @@ __device__ inline void to_half4(const X1Regs<XT> &v, half2v &h01, half2v &h23) {
     }
 }
 
-// v + (the same value from the lane `ctrl` points at), inside a row of 16 lanes
-template <int CTRL> __device__ inline float dpp_add(float v) {
-    const int o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false);
-    return v + __int_as_float(o);
-}
-// sum over the 8 lanes that share a 32-column sub-block
-__device__ inline float sum8(float v) {
-    v = dpp_add<0xB1>(v);   // quad_perm [1, 0, 3, 2]
-    v = dpp_add<0x4E>(v);   // quad_perm [2, 3, 0, 1]
-    v = dpp_add<0x141>(v);  // row_half_mirror: lane i <- lane 7 - i of its half row
-    return v;
-}
+// ---- per-format pieces ----
+//   Lane:   per-lane constants (LDS offsets of the A operand, header addressing)
+//   W:      what a lane loads from HBM for one tile
+//   sums(): what the accumulator starts from, from a lane's four staged columns (h01, h23), written to region + kInit
+//   tile(): the eight MFMA steps and the scales; returns the lane's contribution to its partial y
+template <int DT> struct Row1Fmt;
 
-// Stage one tile's activations: f16 values, and per sub-block (-sum(base * x), sum(x)).
-// The slots of an MFMA step alternate in pairs between fields at mantissa bit 0 (base 1024) and bit 4 (base 64):
-// of a lane's four columns the first two are of the first kind.
-template <int XT>
+template <int DT> struct Row1K45 {
+    static constexpr bool HIGH = DT == TURQ_Q5_K;
+    using F = TiledFmt<DT>;
+    struct Lane {
+        int offA, offB;   // steps 0..3 feed result row 4g (sub-block 2g), steps 4..7 row 4g + 2; other rows read zeros
+        int grp_off;      // header group g: bit 24 g of the 12 bytes after (d, dmin) = byte 3 g; group 3 is read one byte
+        uint32_t rot_s, rot_m;  // early so that the load ends with the header.  Rotations that put (sc, sc') / (m, m')
+    };                          // on bits 4..9 and 16..21.
+    struct W { uint4v qa, qb; uint2v hh; uint32_t hd, grp; };
+    __device__ static Lane lane_init(int r, int g) {
+        Lane l;
+        l.offA = r == 4 * g ? kX + 128 * g : kZero;
+        l.offB = r == 4 * g + 2 ? kX + 128 * g + 64 : kZero;
+        l.grp_off = 4 + 3 * g - (g == 3);
+        l.rot_s = g == 3 ? 4u : 28u;
+        l.rot_m = g == 3 ? 10u : 2u;
+        return l;
+    }
+    __device__ static W load(const uint8_t *__restrict__ tile, int lane, const Lane &l) {
+        W w;
+        w.qa = *(const uint4v *)(tile + F::kQA + 16 * lane);
+        w.qb = *(const uint4v *)(tile + F::kQB + 16 * lane);
+        if constexpr (HIGH) w.hh = *(const uint2v *)(tile + F::kQH + 8 * lane);
+        else w.hh = uint2v{0u, 0u};
+        const uint8_t *h = tile + F::kHDR + 16 * (lane & 15);
+        w.hd = *(const uint32_t *)h;               // f16 d, f16 dmin
+        __builtin_memcpy(&w.grp, h + l.grp_off, 4);  // the (unaligned) dword that holds this lane's 24-bit group
+        return w;
+    }
+    // The slots of a step alternate in pairs between fields at mantissa bit 0 (base 1024) and bit 4 (base 64): of a lane's
+    // four columns the first two are of the first kind.  Per sub-block (8 lanes): (-sum(base * x), sum(x)).
+    __device__ static void sums(half2v h01, half2v h23, uint8_t *region, int lane) {
+        const float s = sum8(dot2(h23, (_Float16)1.0f, dot2(h01, (_Float16)1.0f, 0.0f)));
+        const float nb = sum8(dot2(h23, (_Float16)-64.0f, dot2(h01, (_Float16)-1024.0f, 0.0f)));
+        if ((lane & 7) == 0) *(float2 *)(region + kInit + lane) = float2{nb, s};
+    }
+    __device__ static half8v operand(uint32_t w, uint32_t h0, uint32_t h1, int u0) {
+        const uint32_t w8 = w >> 8;
+        uint32_t t0 = and_or_u32(w, 0x000F000Fu, kMagic1024);
+        uint32_t t1 = and_or_u32(w, 0x00F000F0u, kMagic64);
+        uint32_t t2 = and_or_u32(w8, 0x000F000Fu, kMagic1024);
+        uint32_t t3 = and_or_u32(w8, 0x00F000F0u, kMagic64);
+        if (HIGH) {  // fifth bit: + 16, i.e. mantissa bit 4 next to base 1024 and bit 8 next to base 64
+            t0 = and_or_u32(rotr32(h0, (uint32_t)u0), 0x00100010u, t0);
+            t1 = and_or_u32(rotr32(h1, (uint32_t)u0), 0x01000100u, t1);
+            t2 = and_or_u32(rotr32(h0, (uint32_t)(u0 + 1)), 0x00100010u, t2);
+            t3 = and_or_u32(rotr32(h1, (uint32_t)(u0 + 1)), 0x01000100u, t3);
+        }
+        return make_half8(as_half2(t0), as_half2(t1), as_half2(t2), as_half2(t3));
+    }
+    __device__ static float tile(const W &w, const uint8_t *reg, const Lane &l, int g) {
+        float4v c = *(const float4v *)(reg + kInit + 16 * g);
+        const uint32_t wq[8] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w, w.qb.x, w.qb.y, w.qb.z, w.qb.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const half8v av = *(const half8v *)(reg + (i < 4 ? l.offA : l.offB) + 16 * (i & 3));
+            c = mfma16x16x32(av, operand(wq[i], w.hh.x, w.hh.y, 2 * i), c);
+        }
+        const half2v kb = {(_Float16)-64.0f, (_Float16)-1024.0f};
+        const half2v sc = and_or_h2(rotr32(w.grp, l.rot_s), 0x003F03F0u, kMagicHdr) + kb;
+        const half2v mn = and_or_h2(rotr32(w.grp, l.rot_m), 0x003F03F0u, kMagicHdr) + kb;
+        const half2v dd = as_half2(w.hd);
+        const float u = (float)sc.x * c[0] + (float)sc.y * c[2];
+        const float v = (float)mn.x * c[1] + (float)mn.y * c[3];
+        return (float)dd.x * u - (float)dd.y * v;
+    }
+};
+template <> struct Row1Fmt<TURQ_Q4_K> : Row1K45<TURQ_Q4_K> {};
+template <> struct Row1Fmt<TURQ_Q5_K> : Row1K45<TURQ_Q5_K> {};
+
+template <> struct Row1Fmt<TURQ_Q6_K> {
+    using F = TiledFmt<TURQ_Q6_K>;
+    struct Lane { int off[4]; };  // steps 2s, 2s + 1 feed result row 4g + s (sub-block 4g + s)
+    struct W { uint4v qla, qlb, qh; uint32_t scw, d16; };
+    __device__ static Lane lane_init(int r, int g) {
+        Lane l;
+#pragma unroll
+        for (int s = 0; s < 4; s++) l.off[s] = r == 4 * g + s ? kX + 128 * g + 32 * s : kZero;
+        return l;
+    }
+    __device__ static W load(const uint8_t *__restrict__ tile, int lane, const Lane &) {
+        W w;
+        w.qla = *(const uint4v *)(tile + F::kQLA + 16 * lane);
+        w.qlb = *(const uint4v *)(tile + F::kQLB + 16 * lane);
+        w.qh = *(const uint4v *)(tile + F::kQH + 16 * lane);
+        w.scw = *(const uint32_t *)(tile + F::kSC + 4 * lane);
+        w.d16 = *(const uint16_t *)(tile + F::kD + 2 * (lane & 15));
+        return w;
+    }
+    // every value is built in the mantissa of 256.0 and stands for q - 32: per sub-block (4 lanes) -288 * sum(x)
+    __device__ static void sums(half2v h01, half2v h23, uint8_t *region, int lane) {
+        const float nb = sum4(dot2(h23, (_Float16)-288.0f, dot2(h01, (_Float16)-288.0f, 0.0f)));
+        if ((lane & 3) == 0) *(float *)(region + kInit + lane) = nb;
+    }
+    __device__ static float tile(const W &w, const uint8_t *reg, const Lane &l, int g) {
+        float4v c = *(const float4v *)(reg + kInit + 16 * g);
+        const uint32_t wl[8] = {w.qla.x, w.qla.y, w.qla.z, w.qla.w, w.qlb.x, w.qlb.y, w.qlb.z, w.qlb.w};
+        const uint32_t wh[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            // pair t of the step: the nibbles sit 4 t bits above mantissa bits 2..5, the two high bits 2 t + 8 (i % 2)
+            // bits above mantissa bits 6..7; together the 6-bit quant in the mantissa of 256.0 (ulp 1/4)
+            uint32_t v[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const uint32_t lo = t ? rotr32(wl[i], 4u * t) : wl[i];
+                const uint32_t rh = 2u * t + 8u * (i & 1);
+                const uint32_t hi = rh ? rotr32(wh[i >> 1], rh) : wh[i >> 1];
+                v[t] = and_or_u32(hi, 0x00C000C0u, and_or_u32(lo, 0x003C003Cu, kMagic256));
+            }
+            const half8v av = *(const half8v *)(reg + l.off[i >> 1] + 16 * (i & 1));
+            c = mfma16x16x32(av, make_half8(as_half2(v[0]), as_half2(v[1]), as_half2(v[2]), as_half2(v[3])), c);
+        }
+        float u = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) u += (float)(int)(int8_t)(w.scw >> (8 * i)) * c[i];
+        _Float16 d;
+        const uint16_t db = (uint16_t)w.d16;
+        __builtin_memcpy(&d, &db, 2);
+        return (float)d * u;
+    }
+};
+
+template <> struct Row1Fmt<TURQ_Q8_0> {
+    using F = TiledFmt<TURQ_Q8_0>;
+    struct Lane { int off[8]; int d_off; };  // step q feeds result row q (block q); rows 8..15 stay zero
+    struct W { uint4v p[4]; uint2v dd; };
+    __device__ static Lane lane_init(int r, int g) {
+        Lane l;
+#pragma unroll
+        for (int q = 0; q < 8; q++) l.off[q] = r == q ? kX + 64 * q + 16 * g : kZero;
+        l.d_off = F::kD + 16 * r + 8 * (g & 1);  // the four block scales that belong to result rows 4 (g % 2) ..
+        return l;
+    }
+    __device__ static W load(const uint8_t *__restrict__ tile, int lane, const Lane &l) {
+        W w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w.p[i] = *(const uint4v *)(tile + 1024 * i + 16 * lane);
+        w.dd = *(const uint2v *)(tile + l.d_off);
+        return w;
+    }
+    // bytes are stored as q + 128 and unpacked into the mantissa of 1024.0: per block (8 lanes) -1152 * sum(x).
+    // Lane groups 2 and 3 read the second half of the init area, which stays zero.
+    __device__ static void sums(half2v h01, half2v h23, uint8_t *region, int lane) {
+        const float nb = sum8(dot2(h23, (_Float16)-1152.0f, dot2(h01, (_Float16)-1152.0f, 0.0f)));
+        if ((lane & 7) == 0) *(float *)(region + kInit + (lane >> 1)) = nb;
+    }
+    __device__ static float tile(const W &w, const uint8_t *reg, const Lane &l, int g) {
+        float4v c = *(const float4v *)(reg + kInit + 16 * g);
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const uint32_t w0 = (q & 1) ? w.p[q >> 1].z : w.p[q >> 1].x;
+            const uint32_t w1 = (q & 1) ? w.p[q >> 1].w : w.p[q >> 1].y;
+            const half8v bop = make_half8(and_or_h2(w0, 0x00FF00FFu, kMagic1024), and_or_h2(w0 >> 8, 0x00FF00FFu, kMagic1024),
+                                          and_or_h2(w1, 0x00FF00FFu, kMagic1024), and_or_h2(w1 >> 8, 0x00FF00FFu, kMagic1024));
+            const half8v av = *(const half8v *)(reg + l.off[q]);
+            c = mfma16x16x32(av, bop, c);
+        }
+        const half2v d01 = as_half2(w.dd.x), d23 = as_half2(w.dd.y);
+        return ((float)d01.x * c[0] + (float)d01.y * c[1]) + ((float)d23.x * c[2] + (float)d23.y * c[3]);
+    }
+};
+
+// Stage one tile's activations: f16 values at kX, the accumulator start values at kInit.
+template <int DT, int XT>
 __device__ inline void stage_x1(const X1Regs<XT> &v, uint8_t *region, int lane) {
     half2v h01, h23;
     to_half4<XT>(v, h01, h23);
     *(uint2v *)(region + kX + 8 * lane) = uint2v{as_u32(h01), as_u32(h23)};
-    const half2v one = splat2((_Float16)1.0f), b0 = splat2((_Float16)-1024.0f), b1 = splat2((_Float16)-64.0f);
-    const float s = sum8(__builtin_amdgcn_fdot2(h23, one, __builtin_amdgcn_fdot2(h01, one, 0.0f, false), false));
-    const float nbsum = sum8(__builtin_amdgcn_fdot2(h23, b1, __builtin_amdgcn_fdot2(h01, b0, 0.0f, false), false));
-    if ((lane & 7) == 0) *(float2 *)(region + kInit + lane) = float2{nbsum, s};  // sub-block lane / 8 at 8 bytes each
-}
-
-// eight raw f16 B values (base + nibble [+ 16 * high bit]) of one step dword
-template <bool HIGH>
-__device__ inline half8v raw_operand(uint32_t w, uint32_t h0, uint32_t h1, int u0) {
-    const uint32_t w8 = w >> 8;
-    uint32_t t0 = and_or_u32(w, 0x000F000Fu, kMagic1024);
-    uint32_t t1 = and_or_u32(w, 0x00F000F0u, kMagic64);
-    uint32_t t2 = and_or_u32(w8, 0x000F000Fu, kMagic1024);
-    uint32_t t3 = and_or_u32(w8, 0x00F000F0u, kMagic64);
-    if (HIGH) {  // fifth bit: + 16, i.e. mantissa bit 4 next to base 1024 and bit 8 next to base 64
-        t0 = and_or_u32(rotr32(h0, (uint32_t)u0), 0x00100010u, t0);
-        t1 = and_or_u32(rotr32(h1, (uint32_t)u0), 0x01000100u, t1);
-        t2 = and_or_u32(rotr32(h0, (uint32_t)(u0 + 1)), 0x00100010u, t2);
-        t3 = and_or_u32(rotr32(h1, (uint32_t)(u0 + 1)), 0x01000100u, t3);
-    }
-    return make_half8(as_half2(t0), as_half2(t1), as_half2(t2), as_half2(t3));
+    Row1Fmt<DT>::sums(h01, h23, region, lane);
 }
 
 constexpr int kMaxRow1 = 4;
@@ -143,7 +281,7 @@ struct Row1Args {
 template <int DT, int XT, int P, int MAXT>
 __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int yt) {
     extern __shared__ uint8_t smem[];
-    constexpr bool HIGH = DT == TURQ_Q5_K;
+    using Fmt = Row1Fmt<DT>;
     constexpr int TB = TiledFmt<DT>::kTileBytes;
     const int blk = (int)blockIdx.x;
     const uint8_t *w = a.w[0];
@@ -159,41 +297,34 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nwaves = blockDim.x >> 6;
-    const int r = lane & 15, g = lane >> 4;
-    const int64_t ntc = k / 256;
+    const int g = lane >> 4;
+    const int64_t ntc = turq_tile_cols(k);
     uint8_t *region = smem + (size_t)wave * (P * kRegion);
     float *red = (float *)(smem + (size_t)nwaves * (P * kRegion));
 
-    // the zeros that the idle A rows read
-    if (lane < 16)
+    // the zeros that the idle A rows read, and start values that no format overwrites
+    if (lane < 32)
 #pragma unroll
-        for (int p = 0; p < P; p++) *(uint32_t *)(region + p * kRegion + kZero + 4 * lane) = 0u;
-    // A operand: steps 0..3 carry the columns of sub-block 2g into result row 4g, steps 4..7 those of sub-block 2g+1 into
-    // row 4g + 2; every other row reads zeros.  Byte offsets inside a region; step i adds 16 * (i % 4).
-    const int offA = r == 4 * g ? kX + 128 * g : kZero;
-    const int offB = r == 4 * g + 2 ? kX + 128 * g + 64 : kZero;
-    // header group g sits at bit 24 g of the 12 bytes after (d, dmin): byte 3 g, except that group 3 is read one byte early
-    // so that the load ends with the header.  Rotations that put (sc, sc') / (m, m') on bits 4..9 and 16..21.
-    const int grp_off = 4 + 3 * g - (g == 3);
-    const uint32_t rot_s = g == 3 ? 4u : 28u, rot_m = g == 3 ? 10u : 2u;
+        for (int p = 0; p < P; p++) *(uint32_t *)(region + p * kRegion + kInit + 4 * lane) = 0u;
+    const typename Fmt::Lane lc = Fmt::lane_init(lane & 15, g);
 
     float acc = 0.0f;
     const uint8_t *wrow = w + rt * ntc * TB;
     for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
         X1Regs<XT> xr[P];
-        W1Regs<DT> wr[P];
+        typename Fmt::W wr[P];
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
-            xr[p] = load_x1<XT>(x, b < ntc ? b : b0, lane);
+            xr[p] = load_x1<XT>(x, k, b < ntc ? b : b0, lane);
         }
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
-            wr[p] = load_tile1<DT>(wrow + (b < ntc ? b : b0) * TB, lane, grp_off);
+            wr[p] = Fmt::load(wrow + (b < ntc ? b : b0) * TB, lane, lc);
         }
 #pragma unroll
-        for (int p = 0; p < P; p++) stage_x1<XT>(xr[p], region + p * kRegion, lane);
+        for (int p = 0; p < P; p++) stage_x1<DT, XT>(xr[p], region + p * kRegion, lane);
         // same-wave LDS traffic is processed in order; the fences keep the compiler from reordering
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -202,21 +333,7 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
             if (b >= ntc) continue;  // uniform per wave
-            const uint8_t *reg = region + p * kRegion;
-            float4v c = *(const float4v *)(reg + kInit + 16 * g);
-            const uint32_t wq[8] = {wr[p].qa.x, wr[p].qa.y, wr[p].qa.z, wr[p].qa.w, wr[p].qb.x, wr[p].qb.y, wr[p].qb.z, wr[p].qb.w};
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const half8v av = *(const half8v *)(reg + (i < 4 ? offA : offB) + 16 * (i & 3));
-                c = mfma16x16x32(av, raw_operand<HIGH>(wq[i], wr[p].hh.x, wr[p].hh.y, 2 * i), c);
-            }
-            const half2v kb = {(_Float16)-64.0f, (_Float16)-1024.0f};
-            const half2v sc = and_or_h2(rotr32(wr[p].grp, rot_s), 0x003F03F0u, kMagicHdr) + kb;
-            const half2v mn = and_or_h2(rotr32(wr[p].grp, rot_m), 0x003F03F0u, kMagicHdr) + kb;
-            const half2v dd = as_half2(wr[p].hd);
-            const float u = (float)sc.x * c[0] + (float)sc.y * c[2];
-            const float v = (float)mn.x * c[1] + (float)mn.y * c[3];
-            acc += (float)dd.x * u - (float)dd.y * v;
+            acc += Fmt::tile(wr[p], region + p * kRegion, lc, g);
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -229,8 +346,7 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
     const int n4 = lane >> 2, q = lane & 3;
     float s = 0.0f;
     for (int wv = 0; wv < nwaves; wv++) s += red[wv * 64 + n4 + 16 * q];
-    s = dpp_add<0xB1>(s);
-    s = dpp_add<0x4E>(s);
+    s = sum4(s);
     const int64_t col = rt * 16 + n4;
     if (q == 0 && col < n) {
         const float out = s + (bias ? bias[col] : 0.0f);
@@ -257,7 +373,7 @@ template <int DT, int XT>
 hipError_t launch_p(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
                     hipEvent_t ev1) {
     static const int forced = [] { const char *e = getenv("TURQ_ROW1_P"); return e ? atoi(e) : 0; }();
-    const int64_t per_wave = (k / 256 + nwaves - 1) / nwaves;
+    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
     int p = (int)(per_wave < 4 ? per_wave : 4);
     if (forced >= 1 && forced <= 4) p = forced;
     if (p == 1) return launch_final<DT, XT, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
@@ -279,13 +395,15 @@ hipError_t launch_x(int xt, const Row1Args &a, int blocks, int64_t k, const void
 
 }  // namespace
 
-bool turq_gemv_row1_supports(int dtype) { return dtype == TURQ_Q4_K || dtype == TURQ_Q5_K; }
+bool turq_gemv_row1_supports(int dtype) {
+    return dtype == TURQ_Q4_K || dtype == TURQ_Q5_K || dtype == TURQ_Q6_K || dtype == TURQ_Q8_0;
+}
 
-// count (1..4) weights of one format (Q4_K or Q5_K) and one k against ONE activation row x (16-byte aligned).
+// count (1..4) weights of one format and one k against ONE activation row x (16-byte aligned).
 hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, const int64_t *n, int64_t k, const void *x, int x_dtype,
                                  void *const *y, int y_dtype, const float *const *bias, int nwaves, hipStream_t stream,
                                  hipEvent_t ev_start, hipEvent_t ev_stop) {
-    if (count < 1 || count > kMaxRow1 || nwaves < 1 || nwaves > 16 || k % 256 != 0) return hipErrorInvalidValue;
+    if (count < 1 || count > kMaxRow1 || nwaves < 1 || nwaves > 16 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
     Row1Args a{};
     int64_t blocks = 0;
@@ -298,11 +416,13 @@ hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, con
         blocks += turq_tile_rows(n[i]);
     }
     a.count = count;
-    if (blocks == 0 || k == 0) return blocks == 0 ? hipSuccess : hipErrorInvalidValue;
-    if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    if (blocks == 0) return hipSuccess;
+    if (k == 0 || blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
     switch (dtype) {
     case TURQ_Q4_K: return launch_x<TURQ_Q4_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
     case TURQ_Q5_K: return launch_x<TURQ_Q5_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q6_K: return launch_x<TURQ_Q6_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q8_0: return launch_x<TURQ_Q8_0>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
     default: return hipErrorInvalidValue;
     }
 }
