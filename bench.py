@@ -41,7 +41,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # dense f16 / bf16 MFMA, vendor figure
 # WRITE_SIZE, scaled by the same counters on a copy kernel of known size (summaries under profiles/); keyed by
 # (workload, m, activations, one call per matrix?)
 TRAFFIC = {
-    ("q4k_mlp_8b", 1, "f32", False): 42_894_850,    # gate + up in one launch 56 986 200, down 28 803 500
+    ("q4k_mlp_8b", 1, "f32", False): 42_855_250,    # gate + up in one launch 56 915 500, down 28 795 000
     ("q4k_mlp_8b", 1, "f32", True): 28_680_000,
     ("q4k_prefill_up_8b", 512, "bf16", False): 76_827_600,   # every XCD's L2 fetches the activation fragments once
     ("q4k_prefill_up_8b", 512, "bf16", True): 76_827_600,
@@ -232,7 +232,7 @@ class Bench:
             roofline = {
                 "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls))),
-                "kernel": "gemv_mfma_kernel" if a.single_calls or self.m > 4 else "gemv_multi_kernel / gemv_mfma_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
+                "kernel": "gemv_row1_kernel" if self.m == 1 else "gemv_multi_frag_kernel / gemv_multi_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "algorithmic_bytes_per_launch": int(bytes_per_launch),
             }
             metric, value, unit = "quantized GEMV HBM GB/s (Q4_K/Q6_K, Qwen3-8B shapes)", gbps, "GB/s"
