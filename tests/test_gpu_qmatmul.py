@@ -337,3 +337,21 @@ def test_multi_weight_falls_back_to_single_calls(gpu):
     for w in ws:
         gpu.release(w)
 
+
+
+# ---------------------------------------------------------------------------------------------
+# every instantiation of the one-row kernel: the launch shape is normally derived from the matrix, so the
+# environment overrides (read once per process) are applied to a child process running the tests above
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("row_tiles,in_flight", [(1, 1), (1, 2), (1, 3), (2, 1), (2, 2)])
+def test_one_row_launch_shapes(row_tiles, in_flight):
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, TURQ_ROW1_R=str(row_tiles), TURQ_ROW1_P=str(in_flight))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "-k", "test_one_row and not launch_shapes",
+                          "-p", "no:cacheprovider", os.path.join(root, "tests", "test_gpu_qmatmul.py")],
+                         cwd=root, env=env, capture_output=True, text=True, timeout=170)
+    assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-1000:]

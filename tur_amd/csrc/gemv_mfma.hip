@@ -156,7 +156,8 @@ __device__ inline half8v k45_operand(uint32_t w, half2v s, half2v s16, half2v c1
 // the register allocator reuses them for VALU temporaries a few cycles after the MFMA issues, and
 // on MI355X the Q8_0 kernel then returned garbage (a write-after-write on the MFMA destination:
 // the MFMA's late result write clobbers the temporary).  Consuming all four rows keeps the
-// destination registers live until the MFMA has retired.
+// destination registers live until the MFMA has retired; mfma_done() (mfma_common.h) closes every chain
+// for the sister case, a C operand in other registers than the result.
 template <int DT, int MT, int NV> struct TileOp;
 
 template <int DT, int MT, int NV> struct TileOpK45 {
@@ -179,7 +180,9 @@ template <int DT, int MT, int NV> struct TileOpK45 {
         }
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
-            const float4v tmin = mfma16x16x32(f.a[mt][8], c.bmin, float4v{0.f, 0.f, 0.f, 0.f});
+            float4v tmin = mfma16x16x32(f.a[mt][8], c.bmin, float4v{0.f, 0.f, 0.f, 0.f});
+            mfma_done(tmp[mt]);
+            mfma_done(tmin);
 #pragma unroll
             for (int i = 0; i < NV; i++) acc[mt][i] += c.d * tmp[mt][i] - c.dmin * tmin[i];
         }
@@ -231,9 +234,11 @@ template <int MT, int NV> struct TileOp<TURQ_Q6_K, MT, NV> {
             }
         }
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++)
+        for (int mt = 0; mt < MT; mt++) {
+            mfma_done(tmp[mt]);
 #pragma unroll
             for (int i = 0; i < NV; i++) acc[mt][i] += d * tmp[mt][i];
+        }
     }
 };
 
@@ -253,7 +258,8 @@ template <int MT, int NV> struct TileOp<TURQ_Q8_0, MT, NV> {
             const float d = h2f_bits((q & 1) ? (dw[q >> 1] >> 16) : (dw[q >> 1] & 0xFFFFu));
 #pragma unroll
             for (int mt = 0; mt < MT; mt++) {
-                const float4v t = mfma16x16x32(f.a[mt][q], bop, float4v{0.f, 0.f, 0.f, 0.f});
+                float4v t = mfma16x16x32(f.a[mt][q], bop, float4v{0.f, 0.f, 0.f, 0.f});
+                mfma_done(t);
 #pragma unroll
                 for (int i = 0; i < NV; i++) acc[mt][i] += d * t[i];
             }

@@ -92,7 +92,8 @@ __device__ inline void to_half4(const X1Regs<XT> &v, half2v &h01, half2v &h23) {
 //   Lane:   per-lane constants (LDS offsets of the A operand, header addressing)
 //   W:      what a lane loads from HBM for one tile
 //   sums(): what the accumulator starts from, from a lane's four staged columns (h01, h23), written to region + kInit
-//   tile(): the eight MFMA steps and the scales; returns the lane's contribution to its partial y
+//   chain(): the eight MFMA steps of a tile;  scales(): the tile's scale factors;
+//   finish(): the scales on the result of the chain = the lane's contribution to its partial y
 template <int DT> struct Row1Fmt;
 
 template <int DT> struct Row1K45 {
@@ -145,7 +146,7 @@ template <int DT> struct Row1K45 {
         }
         return make_half8(as_half2(t0), as_half2(t1), as_half2(t2), as_half2(t3));
     }
-    __device__ static float tile(const W &w, const uint8_t *reg, const Lane &l, int g) {
+    __device__ static float4v chain(const W &w, const uint8_t *reg, const Lane &l, int g) {
         float4v c = *(const float4v *)(reg + kInit + 16 * g);
         const uint32_t wq[8] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w, w.qb.x, w.qb.y, w.qb.z, w.qb.w};
 #pragma unroll
@@ -153,13 +154,21 @@ template <int DT> struct Row1K45 {
             const half8v av = *(const half8v *)(reg + (i < 4 ? l.offA : l.offB) + 16 * (i & 3));
             c = mfma16x16x32(av, operand(wq[i], w.hh.x, w.hh.y, 2 * i), c);
         }
+        return c;
+    }
+    struct Sc { half2v sc, mn, dd; };  // (sc, sc'), (m, m'), (d, dmin)
+    __device__ static Sc scales(const W &w, const Lane &l) {
         const half2v kb = {(_Float16)-64.0f, (_Float16)-1024.0f};
-        const half2v sc = and_or_h2(rotr32(w.grp, l.rot_s), 0x003F03F0u, kMagicHdr) + kb;
-        const half2v mn = and_or_h2(rotr32(w.grp, l.rot_m), 0x003F03F0u, kMagicHdr) + kb;
-        const half2v dd = as_half2(w.hd);
-        const float u = (float)sc.x * c[0] + (float)sc.y * c[2];
-        const float v = (float)mn.x * c[1] + (float)mn.y * c[3];
-        return (float)dd.x * u - (float)dd.y * v;
+        Sc s;
+        s.sc = and_or_h2(rotr32(w.grp, l.rot_s), 0x003F03F0u, kMagicHdr) + kb;
+        s.mn = and_or_h2(rotr32(w.grp, l.rot_m), 0x003F03F0u, kMagicHdr) + kb;
+        s.dd = as_half2(w.hd);
+        return s;
+    }
+    __device__ static float finish(const Sc &s, const float4v &c) {
+        const float u = (float)s.sc.x * c[0] + (float)s.sc.y * c[2];
+        const float v = (float)s.mn.x * c[1] + (float)s.mn.y * c[3];
+        return (float)s.dd.x * u - (float)s.dd.y * v;
     }
 };
 template <> struct Row1Fmt<TURQ_Q4_K> : Row1K45<TURQ_Q4_K> {};
@@ -189,7 +198,7 @@ template <> struct Row1Fmt<TURQ_Q6_K> {
         const float nb = sum4(dot2(h23, (_Float16)-288.0f, dot2(h01, (_Float16)-288.0f, 0.0f)));
         if ((lane & 3) == 0) *(float *)(region + kInit + lane) = nb;
     }
-    __device__ static float tile(const W &w, const uint8_t *reg, const Lane &l, int g) {
+    __device__ static float4v chain(const W &w, const uint8_t *reg, const Lane &l, int g) {
         float4v c = *(const float4v *)(reg + kInit + 16 * g);
         const uint32_t wl[8] = {w.qla.x, w.qla.y, w.qla.z, w.qla.w, w.qlb.x, w.qlb.y, w.qlb.z, w.qlb.w};
         const uint32_t wh[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
@@ -208,13 +217,21 @@ template <> struct Row1Fmt<TURQ_Q6_K> {
             const half8v av = *(const half8v *)(reg + l.off[i >> 1] + 16 * (i & 1));
             c = mfma16x16x32(av, make_half8(as_half2(v[0]), as_half2(v[1]), as_half2(v[2]), as_half2(v[3])), c);
         }
-        float u = 0.0f;
+        return c;
+    }
+    struct Sc { float s[4]; float d; };
+    __device__ static Sc scales(const W &w, const Lane &) {
+        Sc s;
 #pragma unroll
-        for (int i = 0; i < 4; i++) u += (float)(int)(int8_t)(w.scw >> (8 * i)) * c[i];
+        for (int i = 0; i < 4; i++) s.s[i] = (float)(int)(int8_t)(w.scw >> (8 * i));
         _Float16 d;
         const uint16_t db = (uint16_t)w.d16;
         __builtin_memcpy(&d, &db, 2);
-        return (float)d * u;
+        s.d = (float)d;
+        return s;
+    }
+    __device__ static float finish(const Sc &s, const float4v &c) {
+        return s.d * ((s.s[0] * c[0] + s.s[1] * c[1]) + (s.s[2] * c[2] + s.s[3] * c[3]));
     }
 };
 
@@ -242,7 +259,7 @@ template <> struct Row1Fmt<TURQ_Q8_0> {
         const float nb = sum8(dot2(h23, (_Float16)-1152.0f, dot2(h01, (_Float16)-1152.0f, 0.0f)));
         if ((lane & 7) == 0) *(float *)(region + kInit + (lane >> 1)) = nb;
     }
-    __device__ static float tile(const W &w, const uint8_t *reg, const Lane &l, int g) {
+    __device__ static float4v chain(const W &w, const uint8_t *reg, const Lane &l, int g) {
         float4v c = *(const float4v *)(reg + kInit + 16 * g);
 #pragma unroll
         for (int q = 0; q < 8; q++) {
@@ -253,8 +270,12 @@ template <> struct Row1Fmt<TURQ_Q8_0> {
             const half8v av = *(const half8v *)(reg + l.off[q]);
             c = mfma16x16x32(av, bop, c);
         }
-        const half2v d01 = as_half2(w.dd.x), d23 = as_half2(w.dd.y);
-        return ((float)d01.x * c[0] + (float)d01.y * c[1]) + ((float)d23.x * c[2] + (float)d23.y * c[3]);
+        return c;
+    }
+    struct Sc { half2v d01, d23; };
+    __device__ static Sc scales(const W &w, const Lane &) { return Sc{as_half2(w.dd.x), as_half2(w.dd.y)}; }
+    __device__ static float finish(const Sc &s, const float4v &c) {
+        return ((float)s.d01.x * c[0] + (float)s.d01.y * c[1]) + ((float)s.d23.x * c[2] + (float)s.d23.y * c[3]);
     }
 };
 
@@ -277,8 +298,9 @@ struct Row1Args {
     int count;
 };
 
-// P = tiles a wave keeps in flight; MAXT = largest workgroup of the instantiation
-template <int DT, int XT, int P, int MAXT>
+// P = column tiles a wave keeps in flight; R = row tiles per workgroup (a wave stages the activations of a column tile once and
+// uses them for R weight tiles); MAXT = largest workgroup of the instantiation
+template <int DT, int XT, int P, int R, int MAXT>
 __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int yt) {
     extern __shared__ uint8_t smem[];
     using Fmt = Row1Fmt<DT>;
@@ -292,7 +314,7 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
 #pragma unroll
     for (int i = 1; i < kMaxRow1; i++)
         if (i < a.count && blk >= a.first[i]) { w = a.w[i], y = a.y[i], bias = a.bias[i], n = a.n[i], first = a.first[i]; }
-    const int64_t rt = blk - first;
+    const int64_t rt0 = (int64_t)(blk - first) * R, nrt = turq_tile_rows(n);
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -308,11 +330,16 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
         for (int p = 0; p < P; p++) *(uint32_t *)(region + p * kRegion + kInit + 4 * lane) = 0u;
     const typename Fmt::Lane lc = Fmt::lane_init(lane & 15, g);
 
-    float acc = 0.0f;
-    const uint8_t *wrow = w + rt * ntc * TB;
+    float acc[R];
+    const uint8_t *wrow[R];  // row tiles past the weight's last one re-read it; their results are not stored
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        acc[r] = 0.0f;
+        wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+    }
     for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
         X1Regs<XT> xr[P];
-        typename Fmt::W wr[P];
+        typename Fmt::W wr[P][R];
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
@@ -321,7 +348,8 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
-            wr[p] = Fmt::load(wrow + (b < ntc ? b : b0) * TB, lane, lc);
+#pragma unroll
+            for (int r = 0; r < R; r++) wr[p][r] = Fmt::load(wrow[r] + (b < ntc ? b : b0) * TB, lane, lc);
         }
 #pragma unroll
         for (int p = 0; p < P; p++) stage_x1<DT, XT>(xr[p], region + p * kRegion, lane);
@@ -329,66 +357,79 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // one tile after the other: chain, fence, scales (mfma_common.h: the chains of two tiles must not be interleaved, and
+        // nothing may overwrite registers of a chain while it is in flight)
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
             if (b >= ntc) continue;  // uniform per wave
-            acc += Fmt::tile(wr[p], region + p * kRegion, lc, g);
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                float4v c = Fmt::chain(wr[p][r], region + p * kRegion, lc, g);
+                mfma_done(c);
+                acc[r] += Fmt::finish(Fmt::scales(wr[p][r], lc), c);
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     }
 
-    // y[16 rt + n] = sum over lane groups and waves
-    red[wave * 64 + lane] = acc;
+    // y[16 rt + n] = sum over lane groups and waves; wave r adds up row tile r
+#pragma unroll
+    for (int r = 0; r < R; r++) red[(r * nwaves + wave) * 64 + lane] = acc[r];
     __syncthreads();
-    if (wave != 0) return;
     const int n4 = lane >> 2, q = lane & 3;
-    float s = 0.0f;
-    for (int wv = 0; wv < nwaves; wv++) s += red[wv * 64 + n4 + 16 * q];
-    s = sum4(s);
-    const int64_t col = rt * 16 + n4;
-    if (q == 0 && col < n) {
-        const float out = s + (bias ? bias[col] : 0.0f);
-        if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, col, out);
-        else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, col, out);
-        else turq_store_out<TURQ_ACT_F16>(y, col, out);
+    for (int r = wave; r < R; r += nwaves) {
+        float s = 0.0f;
+        for (int wv = 0; wv < nwaves; wv++) s += red[(r * nwaves + wv) * 64 + n4 + 16 * q];
+        s = sum4(s);
+        const int64_t col = (rt0 + r) * 16 + n4;
+        if (q == 0 && rt0 + r < nrt && col < n) {
+            const float out = s + (bias ? bias[col] : 0.0f);
+            if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, col, out);
+            else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, col, out);
+            else turq_store_out<TURQ_ACT_F16>(y, col, out);
+        }
     }
 }
 
-template <int DT, int XT, int P, int MAXT>
+template <int DT, int XT, int P, int R, int MAXT>
 hipError_t launch_final(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
                         hipEvent_t ev1) {
-    const size_t lds = (size_t)nwaves * P * kRegion + (size_t)nwaves * 64 * sizeof(float);
+    const size_t lds = (size_t)nwaves * P * kRegion + (size_t)nwaves * R * 64 * sizeof(float);
     if (ev0) {
-        hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, MAXT>), dim3((unsigned)blocks), dim3((unsigned)(64 * nwaves)), (unsigned)lds, s,
-                              ev0, ev1, 0, a, k, x, yt);
+        hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, R, MAXT>), dim3((unsigned)blocks), dim3((unsigned)(64 * nwaves)), (unsigned)lds,
+                              s, ev0, ev1, 0, a, k, x, yt);
         return hipGetLastError();
     }
-    gemv_row1_kernel<DT, XT, P, MAXT><<<(unsigned)blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(a, k, x, yt);
+    gemv_row1_kernel<DT, XT, P, R, MAXT><<<(unsigned)blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(a, k, x, yt);
     return hipGetLastError();
 }
 
 template <int DT, int XT>
-hipError_t launch_p(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
-                    hipEvent_t ev1) {
+hipError_t launch_p(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, int rtiles, hipStream_t s,
+                    hipEvent_t ev0, hipEvent_t ev1) {
     static const int forced = [] { const char *e = getenv("TURQ_ROW1_P"); return e ? atoi(e) : 0; }();
     const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
-    int p = (int)(per_wave < 4 ? per_wave : 4);
+    int p = (int)(per_wave < 3 ? per_wave : 3);  // four tiles in flight do not fit the registers of every format
     if (forced >= 1 && forced <= 4) p = forced;
-    if (p == 1) return launch_final<DT, XT, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    if (p == 2) return launch_final<DT, XT, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    if (p == 3) return launch_final<DT, XT, 3, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    return launch_final<DT, XT, 4, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    if (rtiles == 2) {
+        if (p == 1) return launch_final<DT, XT, 1, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+        return launch_final<DT, XT, 2, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    }
+    if (p == 1) return launch_final<DT, XT, 1, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    if (p == 2) return launch_final<DT, XT, 2, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    if (p == 3) return launch_final<DT, XT, 3, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    return launch_final<DT, XT, 4, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
 }
 
 template <int DT>
-hipError_t launch_x(int xt, const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
-                    hipEvent_t ev1) {
+hipError_t launch_x(int xt, const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, int rtiles, hipStream_t s,
+                    hipEvent_t ev0, hipEvent_t ev1) {
     switch (xt) {
-    case TURQ_ACT_F32: return launch_p<DT, TURQ_ACT_F32>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    case TURQ_ACT_BF16: return launch_p<DT, TURQ_ACT_BF16>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    case TURQ_ACT_F16: return launch_p<DT, TURQ_ACT_F16>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    case TURQ_ACT_F32: return launch_p<DT, TURQ_ACT_F32>(a, blocks, k, x, yt, nwaves, rtiles, s, ev0, ev1);
+    case TURQ_ACT_BF16: return launch_p<DT, TURQ_ACT_BF16>(a, blocks, k, x, yt, nwaves, rtiles, s, ev0, ev1);
+    case TURQ_ACT_F16: return launch_p<DT, TURQ_ACT_F16>(a, blocks, k, x, yt, nwaves, rtiles, s, ev0, ev1);
     default: return hipErrorInvalidValue;
     }
 }
@@ -399,11 +440,12 @@ bool turq_gemv_row1_supports(int dtype) {
     return dtype == TURQ_Q4_K || dtype == TURQ_Q5_K || dtype == TURQ_Q6_K || dtype == TURQ_Q8_0;
 }
 
-// count (1..4) weights of one format and one k against ONE activation row x (16-byte aligned).
+// count (1..4) weights of one format and one k against ONE activation row x (16-byte aligned); row_tiles (1 or 2) per workgroup.
 hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, const int64_t *n, int64_t k, const void *x, int x_dtype,
-                                 void *const *y, int y_dtype, const float *const *bias, int nwaves, hipStream_t stream,
+                                 void *const *y, int y_dtype, const float *const *bias, int nwaves, int row_tiles, hipStream_t stream,
                                  hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (count < 1 || count > kMaxRow1 || nwaves < 1 || nwaves > 16 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
+    if (row_tiles != 1 && row_tiles != 2) return hipErrorInvalidValue;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
     Row1Args a{};
     int64_t blocks = 0;
@@ -413,16 +455,16 @@ hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, con
         a.bias[i] = bias ? bias[i] : nullptr;
         a.n[i] = n[i];
         a.first[i] = (int)blocks;
-        blocks += turq_tile_rows(n[i]);
+        blocks += (turq_tile_rows(n[i]) + row_tiles - 1) / row_tiles;
     }
     a.count = count;
     if (blocks == 0) return hipSuccess;
     if (k == 0 || blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
     switch (dtype) {
-    case TURQ_Q4_K: return launch_x<TURQ_Q4_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
-    case TURQ_Q5_K: return launch_x<TURQ_Q5_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
-    case TURQ_Q6_K: return launch_x<TURQ_Q6_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
-    case TURQ_Q8_0: return launch_x<TURQ_Q8_0>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q4_K: return launch_x<TURQ_Q4_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
+    case TURQ_Q5_K: return launch_x<TURQ_Q5_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
+    case TURQ_Q6_K: return launch_x<TURQ_Q6_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
+    case TURQ_Q8_0: return launch_x<TURQ_Q8_0>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
     default: return hipErrorInvalidValue;
     }
 }

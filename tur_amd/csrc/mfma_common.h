@@ -74,6 +74,19 @@ __device__ inline float4v mfma16x16x32(half8v a, half8v b, float4v c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
+// Ends a chain of MFMAs: the result is consumed here, and no vector or matrix instruction is scheduled across this point
+// (memory instructions and scalar ones may be: their results arrive long after any MFMA has retired).  Without it the
+// compiler is free to place vector instructions that overwrite registers of the chain (a C operand that went to other
+// registers than the result, result registers that are dead) at its minimum distance behind an MFMA; on MI355X that
+// distance has produced wrong sums with v_mfma_f32_16x16x32_f16 (a second row tile per workgroup in the one-row kernel:
+// the scale fields of one tile landed in the registers of the other tile's previous MFMA), so every chain here ends with it.
+__device__ inline void mfma_consume(float4v &c) { asm volatile("; MFMA chain result" : "+v"(c)); }
+__device__ inline void mfma_fence() { __builtin_amdgcn_sched_barrier(0x10 | 0x80 | 0x4); }
+__device__ inline void mfma_done(float4v &c) {  // several chains may share one fence: consume each, then fence once
+    mfma_consume(c);
+    mfma_fence();
+}
+
 __device__ inline uint32_t rotr32(uint32_t v, uint32_t s) { return __builtin_amdgcn_alignbit(v, v, s); }
 
 __device__ inline uint16_t turq_f2bf(float f) {  // round to nearest even, NaN kept quiet
@@ -114,7 +127,7 @@ hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w_til
 bool turq_gemv_row1_supports(int dtype);
 hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w_tiled, const int64_t *n, int64_t k, const void *x,
                                  int x_dtype, void *const *y, int y_dtype, const float *const *bias, int waves_per_group,
-                                 hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
+                                 int row_tiles_per_group, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
 hipError_t turq_launch_gemm_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
                                  int y_dtype, int64_t ldy, const float *bias, hipStream_t stream, hipEvent_t ev_start,
                                  hipEvent_t ev_stop);

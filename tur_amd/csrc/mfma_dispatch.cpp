@@ -46,6 +46,15 @@ int pick_waves_row1(int64_t k) {
     return (int)std::max<int64_t>(1, std::min<int64_t>((col_tiles + tpw - 1) / tpw, 16));
 }
 
+// Row tiles per workgroup of the one-row kernel (TURQ_ROW1_R forces it).
+int pick_rows_row1(const turq_ctx *ctx, int64_t row_tiles) {
+    static const int forced = [] { const char *e = getenv("TURQ_ROW1_R"); return e ? atoi(e) : 0; }();
+    if (forced == 1 || forced == 2) return forced;
+    // two row tiles share the staged activations where there are row tiles to spare (the LM head: + 10 %)
+    const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+    return row_tiles >= 16 * cus ? 2 : 1;
+}
+
 }  // namespace
 
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
@@ -82,7 +91,8 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
                 const void *wp = w->dev;
                 void *yv = yc;
                 TURQ_HIP(ctx, turq_launch_gemv_row1(w->dtype, 1, &wp, &w->n, w->k, xc, xt, &yv, yt, bias ? &bias : nullptr,
-                                                    pick_waves_row1(w->k), ctx->stream, ev0, ev1));
+                                                    pick_waves_row1(w->k), pick_rows_row1(ctx, turq_tile_rows(w->n)), ctx->stream,
+                                                    ev0, ev1));
                 continue;
             }
             TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, xc, xt, ldx, mc, true, yc, yt, ldy, bias,
@@ -146,7 +156,8 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
         TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
         if (fused && m == 1 && use_row1(w[i]->dtype)) {
             TURQ_HIP(ctx, turq_launch_gemv_row1(w[i]->dtype, j - i, wp, nn, w[i]->k, x, xt, y + i, yt, bias ? bias + i : nullptr,
-                                                pick_waves_row1(w[i]->k), ctx->stream, ev0, ev1));
+                                                pick_waves_row1(w[i]->k), pick_rows_row1(ctx, turq_tile_rows(rows)), ctx->stream,
+                                                ev0, ev1));
             i = j;
             continue;
         }
