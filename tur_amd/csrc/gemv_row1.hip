@@ -413,10 +413,7 @@ hipError_t launch_p(const Row1Args &a, int blocks, int64_t k, const void *x, int
     const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
     int p = (int)(per_wave < 3 ? per_wave : 3);  // four tiles in flight do not fit the registers of every format
     if (forced >= 1 && forced <= 4) p = forced;
-    if (rtiles == 2) {
-        if (p == 1) return launch_final<DT, XT, 1, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-        return launch_final<DT, XT, 2, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    }
+    if (rtiles == 2) return launch_final<DT, XT, 2, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
     if (p == 1) return launch_final<DT, XT, 1, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
     if (p == 2) return launch_final<DT, XT, 2, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
     if (p == 3) return launch_final<DT, XT, 3, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
@@ -446,6 +443,9 @@ hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, con
                                  hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (count < 1 || count > kMaxRow1 || nwaves < 1 || nwaves > 16 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
     if (row_tiles != 1 && row_tiles != 2) return hipErrorInvalidValue;
+    // two row tiles per workgroup exist with two column tiles in flight only (the shape the tall matrices it is meant for get;
+    // the variant with one column tile in flight returned wrong sums in some builds and is not instantiated)
+    if (row_tiles == 2 && (turq_tile_cols(k) + nwaves - 1) / nwaves < 2) row_tiles = 1;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
     Row1Args a{};
     int64_t blocks = 0;
