@@ -343,7 +343,7 @@ def test_multi_weight_falls_back_to_single_calls(gpu):
 # every instantiation of the one-row kernel: the launch shape is normally derived from the matrix, so the
 # environment overrides (read once per process) are applied to a child process running the tests above
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("row_tiles,in_flight", [(1, 1), (1, 2), (1, 3), (2, 2)])
+@pytest.mark.parametrize("row_tiles,in_flight", [(1, 1), (1, 2), (1, 3), (2, 1), (2, 2)])
 def test_one_row_launch_shapes(row_tiles, in_flight):
     import os
     import subprocess

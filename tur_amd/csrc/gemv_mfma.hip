@@ -151,13 +151,10 @@ __device__ inline half8v k45_operand(uint32_t w, half2v s, half2v s16, half2v c1
 }
 
 // ---- per-format tile arithmetic: acc[mt] += (this tile's contribution) ----
-// NV = how many of a lane's four result rows get the f32 scale applied.  Always instantiated with 4:
-// with NV < 4 (skipping rows that are never stored) the unused MFMA result registers become free,
-// the register allocator reuses them for VALU temporaries a few cycles after the MFMA issues, and
-// on MI355X the Q8_0 kernel then returned garbage (a write-after-write on the MFMA destination:
-// the MFMA's late result write clobbers the temporary).  Consuming all four rows keeps the
-// destination registers live until the MFMA has retired; mfma_done() (mfma_common.h) closes every chain
-// for the sister case, a C operand in other registers than the result.
+// NV = how many of a lane's four result rows get the f32 scale applied.  Always instantiated with 4.  (NV < 4 once
+// returned garbage for Q8_0; that was at a time when the unpack's v_and_or_b32 was written as inline asm, which hides
+// from the compiler the wait states between such an instruction and an MFMA whose registers it reuses, see
+// mfma_common.h.  It has not been tried again since.)
 template <int DT, int MT, int NV> struct TileOp;
 
 template <int DT, int MT, int NV> struct TileOpK45 {
@@ -181,8 +178,6 @@ template <int DT, int MT, int NV> struct TileOpK45 {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
             float4v tmin = mfma16x16x32(f.a[mt][8], c.bmin, float4v{0.f, 0.f, 0.f, 0.f});
-            mfma_done(tmp[mt]);
-            mfma_done(tmin);
 #pragma unroll
             for (int i = 0; i < NV; i++) acc[mt][i] += c.d * tmp[mt][i] - c.dmin * tmin[i];
         }
@@ -235,7 +230,6 @@ template <int MT, int NV> struct TileOp<TURQ_Q6_K, MT, NV> {
         }
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
-            mfma_done(tmp[mt]);
 #pragma unroll
             for (int i = 0; i < NV; i++) acc[mt][i] += d * tmp[mt][i];
         }
@@ -259,7 +253,6 @@ template <int MT, int NV> struct TileOp<TURQ_Q8_0, MT, NV> {
 #pragma unroll
             for (int mt = 0; mt < MT; mt++) {
                 float4v t = mfma16x16x32(f.a[mt][q], bop, float4v{0.f, 0.f, 0.f, 0.f});
-                mfma_done(t);
 #pragma unroll
                 for (int i = 0; i < NV; i++) acc[mt][i] += d * t[i];
             }

@@ -265,8 +265,8 @@ template <> struct Row1Fmt<TURQ_Q8_0> {
         for (int q = 0; q < 8; q++) {
             const uint32_t w0 = (q & 1) ? w.p[q >> 1].z : w.p[q >> 1].x;
             const uint32_t w1 = (q & 1) ? w.p[q >> 1].w : w.p[q >> 1].y;
-            const half8v bop = make_half8(and_or_h2(w0, 0x00FF00FFu, kMagic1024), and_or_h2(w0 >> 8, 0x00FF00FFu, kMagic1024),
-                                          and_or_h2(w1, 0x00FF00FFu, kMagic1024), and_or_h2(w1 >> 8, 0x00FF00FFu, kMagic1024));
+            const half8v bop = make_half8(as_half2(and_or_u32(w0, 0x00FF00FFu, kMagic1024)), as_half2(and_or_u32(w0 >> 8, 0x00FF00FFu, kMagic1024)),
+                                          as_half2(and_or_u32(w1, 0x00FF00FFu, kMagic1024)), as_half2(and_or_u32(w1 >> 8, 0x00FF00FFu, kMagic1024)));
             const half8v av = *(const half8v *)(reg + l.off[q]);
             c = mfma16x16x32(av, bop, c);
         }
@@ -327,7 +327,7 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
     // the zeros that the idle A rows read, and start values that no format overwrites
     if (lane < 32)
 #pragma unroll
-        for (int p = 0; p < P; p++) *(uint32_t *)(region + p * kRegion + kInit + 4 * lane) = 0u;
+        for (int p = 0; p < P; p++) *(float *)(region + p * kRegion + kInit + 4 * lane) = 0.0f;  // float like the later writes
     const typename Fmt::Lane lc = Fmt::lane_init(lane & 15, g);
 
     float acc[R];
@@ -357,16 +357,13 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        // one tile after the other: chain, fence, scales (mfma_common.h: the chains of two tiles must not be interleaved, and
-        // nothing may overwrite registers of a chain while it is in flight)
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
             if (b >= ntc) continue;  // uniform per wave
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                float4v c = Fmt::chain(wr[p][r], region + p * kRegion, lc, g);
-                mfma_done(c);
+                const float4v c = Fmt::chain(wr[p][r], region + p * kRegion, lc, g);
                 acc[r] += Fmt::finish(Fmt::scales(wr[p][r], lc), c);
             }
         }
@@ -413,7 +410,10 @@ hipError_t launch_p(const Row1Args &a, int blocks, int64_t k, const void *x, int
     const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
     int p = (int)(per_wave < 3 ? per_wave : 3);  // four tiles in flight do not fit the registers of every format
     if (forced >= 1 && forced <= 4) p = forced;
-    if (rtiles == 2) return launch_final<DT, XT, 2, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    if (rtiles == 2) {  // two row tiles double the weights a wave holds: at most two column tiles in flight
+        if (p == 1) return launch_final<DT, XT, 1, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+        return launch_final<DT, XT, 2, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    }
     if (p == 1) return launch_final<DT, XT, 1, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
     if (p == 2) return launch_final<DT, XT, 2, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
     if (p == 3) return launch_final<DT, XT, 3, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
@@ -443,9 +443,6 @@ hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, con
                                  hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (count < 1 || count > kMaxRow1 || nwaves < 1 || nwaves > 16 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
     if (row_tiles != 1 && row_tiles != 2) return hipErrorInvalidValue;
-    // two row tiles per workgroup exist with two column tiles in flight only (the shape the tall matrices it is meant for get;
-    // the variant with one column tile in flight returned wrong sums in some builds and is not instantiated)
-    if (row_tiles == 2 && (turq_tile_cols(k) + nwaves - 1) / nwaves < 2) row_tiles = 1;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
     Row1Args a{};
     int64_t blocks = 0;

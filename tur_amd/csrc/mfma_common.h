@@ -50,12 +50,31 @@ __host__ __device__ inline size_t turq_act_prep_bytes(int dt, int64_t m, int64_t
 __device__ inline half2v as_half2(uint32_t u) { return __builtin_bit_cast(half2v, u); }
 __device__ inline uint32_t as_u32(half2v h) { return __builtin_bit_cast(uint32_t, h); }
 
-// (w & mask) | magic in ONE instruction.  v_and_or_b32 is a VOP3 encoding, which on this ISA takes no
-// literal operands; left to itself the compiler prefers v_and_b32 + v_or_b32 with literals.  Here the
-// (wave-uniform) mask is forced into a scalar register and the magic into a vector register.
+// (w & mask) | magic in ONE instruction, v_and_or_b32.  It is a VOP3 encoding, which on this ISA takes no literal
+// operands; given literal constants the compiler prefers v_and_b32 + v_or_b32.  So constant masks and magics are first
+// passed through an empty asm statement that pins them to a register (the wave-uniform mask to a scalar one) and that
+// the optimizer cannot fold but can still hoist and share; the and/or itself stays ordinary code, for which the compiler
+// then selects v_and_or_b32.  The result passes through an empty asm too, so that two of them in a row are not
+// re-associated into v_and + v_and + v_or3.
+//
+// The instruction itself must NOT be written as inline asm.  The compiler does not know what an asm statement executes
+// and keeps none of the wait states the hardware asks for around it: two between a vector instruction's write and an
+// MFMA that reads the register, more between an MFMA and a vector write to its registers.  With the v_and_or_b32 in an
+// asm statement, an MFMA one issue slot behind it has read the register's PREVIOUS contents (wrong sums that came and
+// went with the schedule).  No asm statement in these kernels emits a vector instruction.
+__device__ inline uint32_t reg_const_s(uint32_t c) {
+    asm("" : "+s"(c));
+    return c;
+}
+__device__ inline uint32_t reg_const_v(uint32_t c) {
+    asm("" : "+v"(c));
+    return c;
+}
 __device__ inline uint32_t and_or_u32(uint32_t w, uint32_t mask, uint32_t magic) {
-    uint32_t r;
-    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "s"(mask), "v"(magic));
+    const uint32_t m = __builtin_constant_p(mask) ? reg_const_s(mask) : mask;
+    const uint32_t g = __builtin_constant_p(magic) ? reg_const_v(magic) : magic;
+    uint32_t r = (w & m) | g;
+    asm("" : "+v"(r));
     return r;
 }
 __device__ inline half2v and_or_h2(uint32_t w, uint32_t mask, uint32_t magic) { return as_half2(and_or_u32(w, mask, magic)); }
@@ -72,19 +91,6 @@ __device__ inline half8v make_half8(half2v a, half2v b, half2v c, half2v d) {
 
 __device__ inline float4v mfma16x16x32(half8v a, half8v b, float4v c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
-}
-
-// Ends a chain of MFMAs: the result is consumed here, and no vector or matrix instruction is scheduled across this point
-// (memory instructions and scalar ones may be: their results arrive long after any MFMA has retired).  Without it the
-// compiler is free to place vector instructions that overwrite registers of the chain (a C operand that went to other
-// registers than the result, result registers that are dead) at its minimum distance behind an MFMA; on MI355X that
-// distance has produced wrong sums with v_mfma_f32_16x16x32_f16 (a second row tile per workgroup in the one-row kernel:
-// the scale fields of one tile landed in the registers of the other tile's previous MFMA), so every chain here ends with it.
-__device__ inline void mfma_consume(float4v &c) { asm volatile("; MFMA chain result" : "+v"(c)); }
-__device__ inline void mfma_fence() { __builtin_amdgcn_sched_barrier(0x10 | 0x80 | 0x4); }
-__device__ inline void mfma_done(float4v &c) {  // several chains may share one fence: consume each, then fence once
-    mfma_consume(c);
-    mfma_fence();
 }
 
 __device__ inline uint32_t rotr32(uint32_t v, uint32_t s) { return __builtin_amdgcn_alignbit(v, v, s); }
