@@ -233,9 +233,9 @@ template <> struct GFmt<TURQ_Q4_K> {
     __device__ static half8v bmin(const Consts &c) { return c.bmin; }
     template <int KS, int ST> __device__ static half8v operand(const Stage &st, const Consts &c) {
         const uint32_t w = word_of<ST>(st.q), w8 = w >> 8;
-        return make_half8(pk_fma(and_or_h2(w, 0x000F000Fu, kMagic1024), c.s[KS], c.c1[KS]), pk_fma(and_or_h2(w, 0x00F000F0u, kMagic64), c.s[KS], c.c2[KS]),
-                          pk_fma(and_or_h2(w8, 0x000F000Fu, kMagic1024), c.s[KS], c.c1[KS]),
-                          pk_fma(and_or_h2(w8, 0x00F000F0u, kMagic64), c.s[KS], c.c2[KS]));
+        return make_half8(pk_fma(and_or_asm_h2(w, 0x000F000Fu, kMagic1024), c.s[KS], c.c1[KS]), pk_fma(and_or_asm_h2(w, 0x00F000F0u, kMagic64), c.s[KS], c.c2[KS]),
+                          pk_fma(and_or_asm_h2(w8, 0x000F000Fu, kMagic1024), c.s[KS], c.c1[KS]),
+                          pk_fma(and_or_asm_h2(w8, 0x00F000F0u, kMagic64), c.s[KS], c.c2[KS]));
     }
 };
 
@@ -266,14 +266,14 @@ template <> struct GFmt<TURQ_Q5_K> {
         // (+16 on a nibble at bits 0..3) or bit 8 / 24 (+16 on a nibble at bits 4..7 read with 16 units per step)
         constexpr uint32_t u0 = 2 * (4 * (KS & 1) + ST);
         const uint32_t w = word_of<ST>(st.q), w8 = w >> 8;
-        uint32_t t0 = and_or_u32(w, 0x000F000Fu, kMagic1024);
-        uint32_t t1 = and_or_u32(w, 0x00F000F0u, kMagic1024);
-        uint32_t t2 = and_or_u32(w8, 0x000F000Fu, kMagic1024);
-        uint32_t t3 = and_or_u32(w8, 0x00F000F0u, kMagic1024);
-        t0 = and_or_u32(rotr32(st.hh.x, u0), 0x00100010u, t0);
-        t1 = and_or_u32(rotr32(st.hh.y, u0), 0x01000100u, t1);
-        t2 = and_or_u32(rotr32(st.hh.x, u0 + 1), 0x00100010u, t2);
-        t3 = and_or_u32(rotr32(st.hh.y, u0 + 1), 0x01000100u, t3);
+        uint32_t t0 = and_or_asm(w, 0x000F000Fu, kMagic1024);
+        uint32_t t1 = and_or_asm(w, 0x00F000F0u, kMagic1024);
+        uint32_t t2 = and_or_asm(w8, 0x000F000Fu, kMagic1024);
+        uint32_t t3 = and_or_asm(w8, 0x00F000F0u, kMagic1024);
+        t0 = and_or_asm(rotr32(st.hh.x, u0), 0x00100010u, t0);
+        t1 = and_or_asm(rotr32(st.hh.y, u0), 0x01000100u, t1);
+        t2 = and_or_asm(rotr32(st.hh.x, u0 + 1), 0x00100010u, t2);
+        t3 = and_or_asm(rotr32(st.hh.y, u0 + 1), 0x01000100u, t3);
         return make_half8(pk_fma(as_half2(t0), c.s[KS], c.c1[KS]), pk_fma(as_half2(t1), c.s16[KS], c.c2[KS]),
                           pk_fma(as_half2(t2), c.s[KS], c.c1[KS]), pk_fma(as_half2(t3), c.s16[KS], c.c2[KS]));
     }
@@ -325,11 +325,11 @@ template <> struct GFmt<TURQ_Q6_K> {
         half2v r[4];
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            const uint32_t lo = and_or_u32(t == 0 ? wl : rotr32(wl, 4 * t), 0x003C003Cu, kMagic256);
+            const uint32_t lo = and_or_asm(t == 0 ? wl : rotr32(wl, 4 * t), 0x003C003Cu, kMagic256);
             const uint32_t hi_src = (8 * (i & 1) + 2 * t) == 0 ? wh : rotr32(wh, (uint32_t)(8 * (i & 1) + 2 * t));
             // (256 + q) - 288 = q - 32 exactly, then one rounding in the product; a fused form would need the constant
             // -288 * d * sc, which f16 cannot hold exactly (288 is not a power of two)
-            r[t] = (as_half2(and_or_u32(hi_src, 0x00C000C0u, lo)) - splat2((_Float16)288.0f)) * c.s[grp];
+            r[t] = (as_half2(and_or_asm(hi_src, 0x00C000C0u, lo)) - splat2((_Float16)288.0f)) * c.s[grp];
         }
         return make_half8(r[0], r[1], r[2], r[3]);
     }

@@ -363,7 +363,13 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
             if (b >= ntc) continue;  // uniform per wave
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const float4v c = Fmt::chain(wr[p][r], region + p * kRegion, lc, g);
+                float4v c = Fmt::chain(wr[p][r], region + p * kRegion, lc, g);
+                // One tile after the other.  Left free, the scheduler interleaves the tiles' chains and scale arithmetic, the
+                // unpacked operands of several tiles are live at once and the 128 registers a wave of a 16-wave workgroup may
+                // use overflow (spills in the instantiations with four tiles per pass; the 510 MB LM head lost 20 %).  The
+                // empty asm consumes the chain's result; vector and matrix instructions may not cross the barrier.
+                asm volatile("" : "+v"(c));
+                __builtin_amdgcn_sched_barrier(0x10 | 0x80 | 0x4);
                 acc[r] += Fmt::finish(Fmt::scales(wr[p][r], lc), c);
             }
         }
