@@ -80,8 +80,8 @@ __device__ inline uint32_t and_or_u32(uint32_t w, uint32_t mask, uint32_t magic)
 __device__ inline half2v and_or_h2(uint32_t w, uint32_t mask, uint32_t magic) { return as_half2(and_or_u32(w, mask, magic)); }
 // The instruction as inline asm, ONLY for values that feed ordinary vector arithmetic (v_pk_fma_f16, ...), never an MFMA, in a
 // kernel whose MFMA results stay in their registers for the kernel's life (the prefill GEMM: its hand-placed LDS waits are
-// tuned around this form, the compiler-visible one above costs it 3 %).  Neither an MFMA operand nor an MFMA result is ever
-// the destination or the source of this instruction there, so none of the hidden wait states applies.
+// tuned around this form, the compiler-visible one above costs it 3 %).  No MFMA reads its result and no
+// register of an MFMA result is ever free for it there, so neither of the hidden wait states applies.
 __device__ inline uint32_t and_or_asm(uint32_t w, uint32_t mask, uint32_t magic) {
     uint32_t r;
     asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(w), "s"(mask), "v"(magic));
