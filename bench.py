@@ -227,7 +227,8 @@ class Bench:
                 "kernel": "gemm_kq_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "flops_per_launch": int(flops_per_launch),
             }
-            metric, value, unit = "quantized prefill GEMM TFLOP/s (Q4_K, Qwen3-8B up_proj)", self.step_flops / (dt_s / a.steps) / 1e12, "TFLOP/s"
+            what = "Q4_K, Qwen3-8B up_proj" if a.workload == "q4k_prefill_up_8b" else a.workload
+            metric, value, unit = f"quantized prefill GEMM TFLOP/s ({what})", self.step_flops / (dt_s / a.steps) / 1e12, "TFLOP/s"
         else:
             roofline = {
                 "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",

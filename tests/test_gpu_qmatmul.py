@@ -196,10 +196,10 @@ def test_error_paths(gpu):
 
 
 # ---------------------------------------------------------------------------------------------
-# prefill GEMM (m > 32, K-quants): weights carry the f16 product d * sc inside the kernel, so the
+# prefill GEMM (m > 32): weights carry the f16 product d * sc (Q8_0: q * d) inside the kernel, so the
 # sharp bar is looser than the GEMV's; the 1e-3 bar against the f32 matmul on dequantized weights holds
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("dt", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("dt", [Q4_K, Q5_K, Q6_K, Q8_0])
 @pytest.mark.parametrize("n,k,m", [(96, 256, 33), (200, 1024, 300), (512, 2048, 512), (100, 512, 700), (16, 768, 129)])
 def test_prefill_gemm(gpu, dt, n, k, m):
     raw = synth.random_weight(dt, n, k, seed=n + m)
@@ -228,14 +228,15 @@ def test_prefill_gemm(gpu, dt, n, k, m):
     gpu.release(w)
 
 
-@pytest.mark.parametrize("dt", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("dt", [Q4_K, Q5_K, Q6_K, Q8_0])
 def test_prefill_gemm_large_scales_fall_back(gpu, dt):
     # (base + q) * d * sc would overflow f16 inside the GEMM: the dispatcher must take the exact skinny kernel instead
     n, k, m = 64, 512, 80
-    bs = {Q4_K: 144, Q5_K: 176, Q6_K: 210}[dt]
+    bs = {Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_0: 34}[dt]
     raw = synth.random_weight(dt, n, k, seed=3).reshape(-1, bs)
     d_at = 208 if dt == Q6_K else 0
-    raw[:, d_at:d_at + 2] = np.array([3.0], np.float16).view(np.uint8)     # d = 3 -> 1024 * 63 * d, 256 * 128 * d > 65504
+    big = 600.0 if dt == Q8_0 else 3.0     # d = 3 -> 1024 * 63 * d, 256 * 128 * d > 65504; Q8_0: 127 * 600 > 65504
+    raw[:, d_at:d_at + 2] = np.array([big], np.float16).view(np.uint8)
     raw = raw.reshape(-1)
     x = synth.random_activation(m, k, seed=4, bf16=True)
     w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
@@ -243,6 +244,17 @@ def test_prefill_gemm_large_scales_fall_back(gpu, dt):
     gpu.release(w)
     assert np.all(np.isfinite(y))
     assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, k)) <= 2e-5
+
+
+def test_prefill_q8_0_ragged_k_takes_the_skinny_kernel(gpu):
+    # Q8_0 rows may end inside a 256-column tile; the GEMM wants whole tiles, so these shapes walk m in chunks
+    n, k, m = 80, 256 + 96, 70
+    raw = synth.random_weight(Q8_0, n, k, seed=11)
+    x = synth.random_activation(m, k, seed=12, bf16=True)
+    w = gpu.upload(Q8_0, n, k, raw, capi.LAYOUT_TILED)
+    y = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    gpu.release(w)
+    assert rel_l2(y, orc.matmul_dequant(Q8_0, x, raw, n, k)) <= 2e-5
 
 
 # ---------------------------------------------------------------------------------------------

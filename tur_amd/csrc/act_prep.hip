@@ -104,10 +104,12 @@ hipError_t launch(int dtype, const void *x, int64_t m, int64_t k, int64_t ldx, v
 // (r, g32) = r + 32 * g32 of step q holds x[32 mt + r][256 b + 128 g32 + 8 q + j], j = 0..7; step 16
 // holds for the four 32-column sub-blocks of the lane's 128 columns the sums of the f16-rounded
 // activations as (hi, lo) f16 pairs.  chunk index = ((mt * ntc + b) * 17 + q) * 64 + lane.
+// Q8_0 order (Q8 = true): step q holds x[32 mt + r][256 b + 32 (q / 2) + 16 g32 + 8 (q % 2) + j] — the lane takes lane
+// slots 2 g32 and 2 g32 + 1 (8 elements each) of every 32-element block, block by block; step 16 is not used.
 // One workgroup per (m-tile, column tile): 32 rows x 256 columns come in along the rows (a thread reads 8
 // neighbouring columns, 32 threads one row), are rounded to f16 and transposed through the LDS into fragment
 // order, and leave as one contiguous 17 KiB piece.
-template <int XT>
+template <int XT, bool Q8>
 __global__ void __launch_bounds__(256) act_prep32_kernel(const void *__restrict__ x, int64_t m, int64_t k, int64_t ldx,
                                                          int64_t ntc, half8v *__restrict__ frags) {
     __shared__ half8v out[17 * 64];
@@ -152,7 +154,7 @@ __global__ void __launch_bounds__(256) act_prep32_kernel(const void *__restrict_
             h[j] = (_Float16)v[j];
             sum += (float)h[j];
         }
-        const int g32 = cc >> 4, q = cc & 15;
+        const int g32 = Q8 ? (cc >> 1) & 1 : cc >> 4, q = Q8 ? 2 * (cc >> 2) + (cc & 1) : cc & 15;
         out[q * 64 + r + 32 * g32] = h;
         part[r][cc] = sum;
     }
@@ -185,15 +187,22 @@ hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m
     }
 }
 
-hipError_t turq_launch_act_prep32(const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags, hipStream_t stream) {
+hipError_t turq_launch_act_prep32(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
+                                  hipStream_t stream) {
     if (m == 0 || k == 0) return hipSuccess;
     const int64_t ntc = (k + 255) / 256;
     const unsigned grid = (unsigned)(((m + 31) / 32) * ntc);
+    const bool q8 = dtype == TURQ_Q8_0;
+#define TURQ_PREP32(XT)                                                                                       \
+    if (q8) act_prep32_kernel<XT, true><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, (half8v *)frags);        \
+    else act_prep32_kernel<XT, false><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, (half8v *)frags);          \
+    break
     switch (x_dtype) {
-    case TURQ_ACT_F32: act_prep32_kernel<TURQ_ACT_F32><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, (half8v *)frags); break;
-    case TURQ_ACT_BF16: act_prep32_kernel<TURQ_ACT_BF16><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, (half8v *)frags); break;
-    case TURQ_ACT_F16: act_prep32_kernel<TURQ_ACT_F16><<<grid, 256, 0, stream>>>(x, m, k, ldx, ntc, (half8v *)frags); break;
+    case TURQ_ACT_F32: TURQ_PREP32(TURQ_ACT_F32);
+    case TURQ_ACT_BF16: TURQ_PREP32(TURQ_ACT_BF16);
+    case TURQ_ACT_F16: TURQ_PREP32(TURQ_ACT_F16);
     default: return hipErrorInvalidValue;
     }
+#undef TURQ_PREP32
     return hipGetLastError();
 }

@@ -217,17 +217,18 @@ int turq_weight_upload(turq_ctx *ctx, int dt, int64_t n, int64_t k, const void *
     w->k = k;
     w->native_bytes = nbytes;
     const uint8_t *src = (const uint8_t *)host_bytes;
-    if (dt == TURQ_Q4_K || dt == TURQ_Q5_K || dt == TURQ_Q6_K) {
-        // bound on |d * sc| (6-bit scales <= 63, Q6_K int8 scales <= 128 in magnitude), see turq_weight::max_scale
+    if (turq_dt_is_quant(dt)) {
+        // bound on the scale a weight is multiplied by: |d * sc| for the K-quants (6-bit scales <= 63, Q6_K int8 scales <= 128
+        // in magnitude), |d| for Q8_0; see turq_weight::max_scale
         const int bs = turq_block_bytes(dt), d_at = dt == TURQ_Q6_K ? 208 : 0;
         float mx = 0.0f;
-        const int64_t nblk = n * (k / 256);
+        const int64_t nblk = n * (k / turq_dt_block_elems(dt));
         for (int64_t i = 0; i < nblk; i++) {
             const uint8_t *b = src + i * bs + d_at;
             const float d = std::fabs(half_bits_to_float((uint16_t)(b[0] | (b[1] << 8))));
             if (d > mx || d != d) mx = d;
         }
-        w->max_scale = mx * (dt == TURQ_Q6_K ? 128.0f : 63.0f);
+        w->max_scale = mx * (dt == TURQ_Q8_0 ? 1.0f : dt == TURQ_Q6_K ? 128.0f : 63.0f);
     }
     std::vector<uint8_t> tiled;
     if (layout == TURQ_LAYOUT_TILED) {

@@ -46,7 +46,7 @@
 // high-bit plane with one rotate and one v_and_or_b32 per packed register; Q6_K builds the whole 6-bit value in
 // the mantissa of 256.0 (low nibble at bits 2..5, high field rotated onto bits 6..7) and needs no sums term.  Their
 // tiles are larger (2816 / 3360 bytes), so their workgroup is 128 x 128 (wave tile 2 x 2) to keep three
-// super-blocks of weights in the LDS.  Q8_0 has no GEMM yet.
+// super-blocks of weights in the LDS.  Q8_0 (4352-byte tiles, f16 block scales, no sums term): 128 x 64, wave tile 2 x 1.
 //
 // Results leave through the LDS (free after the main loop): each wave transposes its 64 x 96 tile so
 // that a lane stores 16 contiguous bytes and a row segment is 192 (bf16, f16) or 384 (f32) bytes.
@@ -332,6 +332,49 @@ template <> struct GFmt<TURQ_Q6_K> {
             r[t] = (as_half2(and_or_asm(hi_src, 0x00C000C0u, lo)) - splat2((_Float16)288.0f)) * c.s[grp];
         }
         return make_half8(r[0], r[1], r[2], r[3]);
+    }
+};
+
+// Q8_0: the tile holds 8 blocks of 32 columns in four planes (plane i = blocks 2 i, 2 i + 1); stage ks is plane ks.  The lane
+// reads its two lane slots (2 g32, 2 g32 + 1: 8 bytes per block each) and takes, per block, first the 8 columns of the one,
+// then of the other: operand step st of the stage is block 2 ks + st / 2, slot st % 2 (the Q8_0 order of act_prep32_kernel).
+// Bytes are q + 128 (tiled layout), read as 1024 + 128 + q in the mantissa of 1024.0; (t - 1152) is q exactly and q * d is
+// rounded once.  The tiles are 4352 bytes: wave tile 2 x 1 (workgroup 128 x 64) keeps three super-blocks in the LDS.
+template <> struct GFmt<TURQ_Q8_0> {
+    using F = TiledFmt<TURQ_Q8_0>;
+    static constexpr int WN = 1, NSTG = 2, NHDR = 1;
+    static constexpr bool SUMS = false;
+    struct Stage { uint4v a, b; };     // lane slots 2 g32 and 2 g32 + 1 of the plane: (block 2 ks: lo, hi), (block 2 ks + 1: lo, hi)
+    struct Hdr { uint4v dd; };         // the row's 8 f16 block scales
+    struct Consts { half2v s[8]; };
+    struct Addr { uint32_t q, h; };
+    __device__ static Addr addr(uint32_t tile, int r16, int g32) {
+        return Addr{tile + 16u * (uint32_t)(r16 + 32 * g32), tile + (uint32_t)F::kD + 16u * (uint32_t)r16};
+    }
+    template <int KS, int OFF> __device__ static void read_stage(Stage &st, const Addr &a, uint32_t ring) {
+        lds_read128<OFF + KS * 1024>(st.a, a.q + ring);
+        lds_read128<OFF + KS * 1024 + 256>(st.b, a.q + ring);
+    }
+    template <int OFF> __device__ static void read_hdr(Hdr &h, const Addr &a, uint32_t ring) { lds_read128<OFF>(h.dd, a.h + ring); }
+    __device__ static void pin_stage(Stage &st) { pin(st.a); pin(st.b); }
+    __device__ static void pin_hdr(Hdr &h) { pin(h.dd); }
+    __device__ static Consts consts(const Hdr &h, int) {
+        const uint32_t dw[4] = {h.dd.x, h.dd.y, h.dd.z, h.dd.w};
+        Consts c;
+#pragma unroll
+        for (int i = 0; i < 8; i++) c.s[i] = splat2(h_from_bits((i & 1) ? dw[i >> 1] >> 16 : dw[i >> 1] & 0xFFFFu));
+        return c;
+    }
+    __device__ static half8v bmin(const Consts &) { return half8v{}; }
+    template <int KS, int ST> __device__ static half8v operand(const Stage &st, const Consts &c) {
+        constexpr int blk = 2 * KS + (ST >> 1);
+        const uint4v src = (ST & 1) ? st.b : st.a;
+        const uint32_t w0 = (ST >> 1) ? src.z : src.x, w1 = (ST >> 1) ? src.w : src.y;
+        const half2v k1152 = splat2((_Float16)1152.0f);
+        return make_half8((and_or_asm_h2(w0, 0x00FF00FFu, kMagic1024) - k1152) * c.s[blk],
+                          (and_or_asm_h2(w0 >> 8, 0x00FF00FFu, kMagic1024) - k1152) * c.s[blk],
+                          (and_or_asm_h2(w1, 0x00FF00FFu, kMagic1024) - k1152) * c.s[blk],
+                          (and_or_asm_h2(w1 >> 8, 0x00FF00FFu, kMagic1024) - k1152) * c.s[blk]);
     }
 };
 
@@ -653,7 +696,7 @@ hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, i
 
 }  // namespace
 
-// frags: activations prepared by turq_launch_act_prep32 for all m rows
+// frags: activations prepared by turq_launch_act_prep32 (in the order of the same dtype) for all m rows
 hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
                                  int y_dtype, int64_t ldy, const float *bias, hipStream_t stream, hipEvent_t ev_start,
                                  hipEvent_t ev_stop) {
@@ -663,6 +706,7 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
     case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
     case TURQ_Q5_K: return launch_gemm<TURQ_Q5_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
     case TURQ_Q6_K: return launch_gemm<TURQ_Q6_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
+    case TURQ_Q8_0: return launch_gemm<TURQ_Q8_0>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
     default: return hipErrorInvalidValue;
     }
 }

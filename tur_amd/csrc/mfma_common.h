@@ -129,7 +129,8 @@ __host__ __device__ inline size_t turq_act_prep32_bytes(int64_t m, int64_t k) {
 }
 
 // launchers (act_prep.hip, gemv_mfma.hip)
-hipError_t turq_launch_act_prep32(const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags, hipStream_t stream);
+hipError_t turq_launch_act_prep32(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
+                                  hipStream_t stream);
 hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
                                 hipStream_t stream);
 hipError_t turq_launch_gemv_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *xin, int x_dtype,
