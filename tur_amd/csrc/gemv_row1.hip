@@ -51,24 +51,43 @@ __device__ inline float sum4(float v) {
     v = dpp_add<0xB1>(v);  // quad_perm [1, 0, 3, 2]
     return dpp_add<0x4E>(v);  // quad_perm [2, 3, 0, 1]
 }
-__device__ inline float sum8(float v) { return dpp_add<0x141>(sum4(v)); }  // row_half_mirror: lane i <- lane 7 - i of its half row
+// row_half_mirror: lane i <- lane 7 - i of its half row.  The result is pinned here: the callers store it from one lane in eight,
+// and an add that the compiler sinks into that branch no longer merges with its DPP move.
+__device__ inline float sum8(float v) {
+    float r = dpp_add<0x141>(sum4(v));
+    asm volatile("" : "+v"(r));
+    return r;
+}
 
 __device__ inline float dot2(half2v a, _Float16 b0, float c) { return __builtin_amdgcn_fdot2(a, splat2(b0), c, false); }
 
 // raw activations of one tile: 4 consecutive columns per lane
 template <int XT> struct X1Regs { uint32_t r[XT == TURQ_ACT_F32 ? 4 : 2]; };
 
-template <int XT>
-__device__ inline X1Regs<XT> load_x1(const void *__restrict__ x, int64_t k, int64_t b, int lane) {
+// 32-bit per-lane byte offsets of the global loads.  An offset computed (and widened to 64 bits) outside the loop reaches
+// the loads as a register pair and costs a 64-bit vector add per load; one that is widened next to the load folds into the
+// load's own addressing (scalar base + 32-bit lane offset).  touch() at the top of every pass makes the offsets new values
+// for the compiler there, at no instruction.
+struct GOff {
+    uint32_t o16, o8, o4, hdr, aux;  // 16, 8, 4 bytes per lane; the lane's header row; a format's second header offset
+    __device__ void touch() { asm volatile("" : "+v"(o16), "+v"(o8), "+v"(o4), "+v"(hdr), "+v"(aux)); }
+};
+
+// RAGGED: k may end inside the tile (Q8_0: a multiple of 32, four columns are in or out together); the K-quants' k is a
+// multiple of 256 and needs no test
+template <int XT, bool RAGGED>
+__device__ inline X1Regs<XT> load_x1(const void *__restrict__ x, int64_t k, int64_t b, int lane, const GOff &o) {
     X1Regs<XT> v;
-    int64_t col = b * 256 + 4 * lane;
-    const bool ok = col < k;  // k is a multiple of 32 (Q8_0) or 256: four columns are in or out together
-    col = ok ? col : 0;
+    constexpr int ES = XT == TURQ_ACT_F32 ? 4 : 2;
+    const bool ok = !RAGGED || b * 256 + 4 * lane < k;
+    const uint32_t off = XT == TURQ_ACT_F32 ? o.o16 : o.o8;
+    const uint8_t *src = (const uint8_t *)x + b * (256 * ES) + (ok ? off : 0u);
+    if (RAGGED && !ok) src = (const uint8_t *)x;
     if constexpr (XT == TURQ_ACT_F32) {
-        const uint4v t = *(const uint4v *)((const float *)x + col);
+        const uint4v t = *(const uint4v *)src;
         v.r[0] = ok ? t.x : 0u; v.r[1] = ok ? t.y : 0u; v.r[2] = ok ? t.z : 0u; v.r[3] = ok ? t.w : 0u;
     } else {
-        const uint2v t = *(const uint2v *)((const uint16_t *)x + col);
+        const uint2v t = *(const uint2v *)src;
         v.r[0] = ok ? t.x : 0u; v.r[1] = ok ? t.y : 0u;
     }
     return v;
@@ -77,8 +96,8 @@ __device__ inline X1Regs<XT> load_x1(const void *__restrict__ x, int64_t k, int6
 template <int XT>
 __device__ inline void to_half4(const X1Regs<XT> &v, half2v &h01, half2v &h23) {
     if constexpr (XT == TURQ_ACT_F32) {
-        h01 = half2v{(_Float16)__uint_as_float(v.r[0]), (_Float16)__uint_as_float(v.r[1])};
-        h23 = half2v{(_Float16)__uint_as_float(v.r[2]), (_Float16)__uint_as_float(v.r[3])};
+        h01 = __builtin_convertvector(float2v{__uint_as_float(v.r[0]), __uint_as_float(v.r[1])}, half2v);
+        h23 = __builtin_convertvector(float2v{__uint_as_float(v.r[2]), __uint_as_float(v.r[3])}, half2v);
     } else if constexpr (XT == TURQ_ACT_BF16) {
         h01 = half2v{(_Float16)__uint_as_float(v.r[0] << 16), (_Float16)__uint_as_float(v.r[0] & 0xFFFF0000u)};
         h23 = half2v{(_Float16)__uint_as_float(v.r[1] << 16), (_Float16)__uint_as_float(v.r[1] & 0xFFFF0000u)};
@@ -101,28 +120,28 @@ template <int DT> struct Row1K45 {
     using F = TiledFmt<DT>;
     struct Lane {
         int offA, offB;   // steps 0..3 feed result row 4g (sub-block 2g), steps 4..7 row 4g + 2; other rows read zeros
-        int grp_off;      // header group g: bit 24 g of the 12 bytes after (d, dmin) = byte 3 g; group 3 is read one byte
-        uint32_t rot_s, rot_m;  // early so that the load ends with the header.  Rotations that put (sc, sc') / (m, m')
-    };                          // on bits 4..9 and 16..21.
+        uint32_t rot_s, rot_m;  // rotations that put (sc, sc') / (m, m') of the lane's header group on bits 4..9 and 16..21
+    };
     struct W { uint4v qa, qb; uint2v hh; uint32_t hd, grp; };
     __device__ static Lane lane_init(int r, int g) {
         Lane l;
         l.offA = r == 4 * g ? kX + 128 * g : kZero;
         l.offB = r == 4 * g + 2 ? kX + 128 * g + 64 : kZero;
-        l.grp_off = 4 + 3 * g - (g == 3);
         l.rot_s = g == 3 ? 4u : 28u;
         l.rot_m = g == 3 ? 10u : 2u;
         return l;
     }
-    __device__ static W load(const uint8_t *__restrict__ tile, int lane, const Lane &l) {
+    // header group g sits at bit 24 g of the 12 bytes after (d, dmin) = byte 3 g; group 3 is read one byte early so that the
+    // load ends with the header
+    __device__ static uint32_t aux_off(int r, int g) { return 16u * (uint32_t)r + 4u + 3u * (uint32_t)g - (g == 3 ? 1u : 0u); }
+    __device__ static W load(const uint8_t *__restrict__ tile, const GOff &o) {
         W w;
-        w.qa = *(const uint4v *)(tile + F::kQA + 16 * lane);
-        w.qb = *(const uint4v *)(tile + F::kQB + 16 * lane);
-        if constexpr (HIGH) w.hh = *(const uint2v *)(tile + F::kQH + 8 * lane);
+        w.qa = *(const uint4v *)(tile + F::kQA + o.o16);
+        w.qb = *(const uint4v *)(tile + F::kQB + o.o16);
+        if constexpr (HIGH) w.hh = *(const uint2v *)(tile + F::kQH + o.o8);
         else w.hh = uint2v{0u, 0u};
-        const uint8_t *h = tile + F::kHDR + 16 * (lane & 15);
-        w.hd = *(const uint32_t *)h;               // f16 d, f16 dmin
-        __builtin_memcpy(&w.grp, h + l.grp_off, 4);  // the (unaligned) dword that holds this lane's 24-bit group
+        w.hd = *(const uint32_t *)(tile + F::kHDR + o.hdr);  // f16 d, f16 dmin
+        __builtin_memcpy(&w.grp, tile + F::kHDR + o.aux, 4);  // the (unaligned) dword that holds this lane's 24-bit group
         return w;
     }
     // The slots of a step alternate in pairs between fields at mantissa bit 0 (base 1024) and bit 4 (base 64): of a lane's
@@ -184,13 +203,14 @@ template <> struct Row1Fmt<TURQ_Q6_K> {
         for (int s = 0; s < 4; s++) l.off[s] = r == 4 * g + s ? kX + 128 * g + 32 * s : kZero;
         return l;
     }
-    __device__ static W load(const uint8_t *__restrict__ tile, int lane, const Lane &) {
+    __device__ static uint32_t aux_off(int r, int) { return 2u * (uint32_t)r; }  // the row's d
+    __device__ static W load(const uint8_t *__restrict__ tile, const GOff &o) {
         W w;
-        w.qla = *(const uint4v *)(tile + F::kQLA + 16 * lane);
-        w.qlb = *(const uint4v *)(tile + F::kQLB + 16 * lane);
-        w.qh = *(const uint4v *)(tile + F::kQH + 16 * lane);
-        w.scw = *(const uint32_t *)(tile + F::kSC + 4 * lane);
-        w.d16 = *(const uint16_t *)(tile + F::kD + 2 * (lane & 15));
+        w.qla = *(const uint4v *)(tile + F::kQLA + o.o16);
+        w.qlb = *(const uint4v *)(tile + F::kQLB + o.o16);
+        w.qh = *(const uint4v *)(tile + F::kQH + o.o16);
+        w.scw = *(const uint32_t *)(tile + F::kSC + o.o4);
+        w.d16 = *(const uint16_t *)(tile + F::kD + o.aux);
         return w;
     }
     // every value is built in the mantissa of 256.0 and stands for q - 32: per sub-block (4 lanes) -288 * sum(x)
@@ -237,20 +257,21 @@ template <> struct Row1Fmt<TURQ_Q6_K> {
 
 template <> struct Row1Fmt<TURQ_Q8_0> {
     using F = TiledFmt<TURQ_Q8_0>;
-    struct Lane { int off[8]; int d_off; };  // step q feeds result row q (block q); rows 8..15 stay zero
+    struct Lane { int off[8]; };  // step q feeds result row q (block q); rows 8..15 stay zero
     struct W { uint4v p[4]; uint2v dd; };
     __device__ static Lane lane_init(int r, int g) {
         Lane l;
 #pragma unroll
         for (int q = 0; q < 8; q++) l.off[q] = r == q ? kX + 64 * q + 16 * g : kZero;
-        l.d_off = F::kD + 16 * r + 8 * (g & 1);  // the four block scales that belong to result rows 4 (g % 2) ..
         return l;
     }
-    __device__ static W load(const uint8_t *__restrict__ tile, int lane, const Lane &l) {
+    // the four block scales that belong to result rows 4 (g % 2) .. 4 (g % 2) + 3
+    __device__ static uint32_t aux_off(int r, int g) { return (uint32_t)F::kD + 16u * (uint32_t)r + 8u * (uint32_t)(g & 1); }
+    __device__ static W load(const uint8_t *__restrict__ tile, const GOff &o) {
         W w;
 #pragma unroll
-        for (int i = 0; i < 4; i++) w.p[i] = *(const uint4v *)(tile + 1024 * i + 16 * lane);
-        w.dd = *(const uint2v *)(tile + l.d_off);
+        for (int i = 0; i < 4; i++) w.p[i] = *(const uint4v *)(tile + 1024 * i + o.o16);
+        w.dd = *(const uint2v *)(tile + o.aux);
         return w;
     }
     // bytes are stored as q + 128 and unpacked into the mantissa of 1024.0: per block (8 lanes) -1152 * sum(x).
@@ -329,6 +350,7 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
 #pragma unroll
         for (int p = 0; p < P; p++) *(float *)(region + p * kRegion + kInit + 4 * lane) = 0.0f;  // float like the later writes
     const typename Fmt::Lane lc = Fmt::lane_init(lane & 15, g);
+    GOff go{16u * (uint32_t)lane, 8u * (uint32_t)lane, 4u * (uint32_t)lane, 16u * (uint32_t)(lane & 15), Fmt::aux_off(lane & 15, g)};
 
     float acc[R];
     const uint8_t *wrow[R];  // row tiles past the weight's last one re-read it; their results are not stored
@@ -340,16 +362,17 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
     for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
         X1Regs<XT> xr[P];
         typename Fmt::W wr[P][R];
+        go.touch();
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
-            xr[p] = load_x1<XT>(x, k, b < ntc ? b : b0, lane);
+            xr[p] = load_x1<XT, DT == TURQ_Q8_0>(x, k, b < ntc ? b : b0, lane, go);
         }
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
 #pragma unroll
-            for (int r = 0; r < R; r++) wr[p][r] = Fmt::load(wrow[r] + (b < ntc ? b : b0) * TB, lane, lc);
+            for (int r = 0; r < R; r++) wr[p][r] = Fmt::load(wrow[r] + (b < ntc ? b : b0) * TB, go);
         }
 #pragma unroll
         for (int p = 0; p < P; p++) stage_x1<DT, XT>(xr[p], region + p * kRegion, lane);
