@@ -42,41 +42,46 @@ template <> struct WRegs<TURQ_Q5_K> { uint4v qa, qb, hd; uint2v hh; };
 template <> struct WRegs<TURQ_Q6_K> { uint4v qla, qlb, qh; uint32_t scw; uint32_t d16; };
 template <> struct WRegs<TURQ_Q8_0> { uint4v p[4]; uint4v dd; };
 
-template <int DT> __device__ inline WRegs<DT> load_tile(const uint8_t *__restrict__ tile, int lane);
-template <> __device__ inline WRegs<TURQ_Q4_K> load_tile<TURQ_Q4_K>(const uint8_t *__restrict__ tile, int lane) {
+// o: the lane's byte offsets (aux = 2 bytes per weight row); `tile` is wave-uniform
+template <int DT> __device__ inline WRegs<DT> load_tile(const uint8_t *__restrict__ tile, const GOff &o);
+template <> __device__ inline WRegs<TURQ_Q4_K> load_tile<TURQ_Q4_K>(const uint8_t *__restrict__ tile, const GOff &o) {
     using F = TiledFmt<TURQ_Q4_K>;
     WRegs<TURQ_Q4_K> w;
-    w.qa = *(const uint4v *)(tile + F::kQA + 16 * lane);
-    w.qb = *(const uint4v *)(tile + F::kQB + 16 * lane);
-    w.hd = *(const uint4v *)(tile + F::kHDR + 16 * (lane & 15));
+    w.qa = *(const uint4v *)(tile + F::kQA + o.o16);
+    w.qb = *(const uint4v *)(tile + F::kQB + o.o16);
+    w.hd = *(const uint4v *)(tile + F::kHDR + o.hdr);
     return w;
 }
-template <> __device__ inline WRegs<TURQ_Q5_K> load_tile<TURQ_Q5_K>(const uint8_t *__restrict__ tile, int lane) {
+template <> __device__ inline WRegs<TURQ_Q5_K> load_tile<TURQ_Q5_K>(const uint8_t *__restrict__ tile, const GOff &o) {
     using F = TiledFmt<TURQ_Q5_K>;
     WRegs<TURQ_Q5_K> w;
-    w.qa = *(const uint4v *)(tile + F::kQA + 16 * lane);
-    w.qb = *(const uint4v *)(tile + F::kQB + 16 * lane);
-    w.hh = *(const uint2v *)(tile + F::kQH + 8 * lane);
-    w.hd = *(const uint4v *)(tile + F::kHDR + 16 * (lane & 15));
+    w.qa = *(const uint4v *)(tile + F::kQA + o.o16);
+    w.qb = *(const uint4v *)(tile + F::kQB + o.o16);
+    w.hh = *(const uint2v *)(tile + F::kQH + o.o8);
+    w.hd = *(const uint4v *)(tile + F::kHDR + o.hdr);
     return w;
 }
-template <> __device__ inline WRegs<TURQ_Q6_K> load_tile<TURQ_Q6_K>(const uint8_t *__restrict__ tile, int lane) {
+template <> __device__ inline WRegs<TURQ_Q6_K> load_tile<TURQ_Q6_K>(const uint8_t *__restrict__ tile, const GOff &o) {
     using F = TiledFmt<TURQ_Q6_K>;
     WRegs<TURQ_Q6_K> w;
-    w.qla = *(const uint4v *)(tile + F::kQLA + 16 * lane);
-    w.qlb = *(const uint4v *)(tile + F::kQLB + 16 * lane);
-    w.qh = *(const uint4v *)(tile + F::kQH + 16 * lane);
-    w.scw = *(const uint32_t *)(tile + F::kSC + 4 * lane);
-    w.d16 = *(const uint16_t *)(tile + F::kD + 2 * (lane & 15));
+    w.qla = *(const uint4v *)(tile + F::kQLA + o.o16);
+    w.qlb = *(const uint4v *)(tile + F::kQLB + o.o16);
+    w.qh = *(const uint4v *)(tile + F::kQH + o.o16);
+    w.scw = *(const uint32_t *)(tile + F::kSC + o.o4);
+    w.d16 = *(const uint16_t *)(tile + F::kD + o.aux);
     return w;
 }
-template <> __device__ inline WRegs<TURQ_Q8_0> load_tile<TURQ_Q8_0>(const uint8_t *__restrict__ tile, int lane) {
+template <> __device__ inline WRegs<TURQ_Q8_0> load_tile<TURQ_Q8_0>(const uint8_t *__restrict__ tile, const GOff &o) {
     using F = TiledFmt<TURQ_Q8_0>;
     WRegs<TURQ_Q8_0> w;
 #pragma unroll
-    for (int i = 0; i < 4; i++) w.p[i] = *(const uint4v *)(tile + 1024 * i + 16 * lane);
-    w.dd = *(const uint4v *)(tile + F::kD + 16 * (lane & 15));
+    for (int i = 0; i < 4; i++) w.p[i] = *(const uint4v *)(tile + 1024 * i + o.o16);
+    w.dd = *(const uint4v *)(tile + F::kD + o.hdr);
     return w;
+}
+__device__ inline GOff lane_offsets(int lane, int mpad) {
+    const uint32_t l = (uint32_t)lane, r = l & 15u;
+    return GOff{16u * l, 8u * l, 4u * l, 16u * r, 2u * r, 16u * ((l >> 4) * (uint32_t)mpad + (r & (uint32_t)(mpad - 1)))};
 }
 
 // ---- activation fragments of one tile: NQ steps for each of MT m-tiles ----
@@ -87,15 +92,18 @@ template <int DT, int MT> struct AFrags {
     half8v a[MT][NQ];
 };
 
+// tile_frags (wave-uniform): the fragments of column tile b of m-tile 0; step q of m-tile mt starts mt * mt_stride + 4 q mpad
+// chunks of 16 bytes further on, and lane (r, g) takes chunk g * mpad + r % mpad of it (o.frag)
 template <int DT, int MT>
 __device__ inline AFrags<DT, MT> load_frags_global(const half8v *__restrict__ tile_frags, int64_t mt_stride, int mpad,
-                                                   int lane) {
+                                                   const GOff &o) {
     AFrags<DT, MT> f;
-    const int g = lane >> 4, r = (lane & 15) & (mpad - 1);
+    const uint8_t *base = (const uint8_t *)tile_frags;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-        for (int q = 0; q < AFrags<DT, MT>::NQ; q++) f.a[mt][q] = tile_frags[mt * mt_stride + (q * 4 + g) * mpad + r];
+        for (int q = 0; q < AFrags<DT, MT>::NQ; q++)
+            f.a[mt][q] = *(const half8v *)(base + 16 * (mt * mt_stride + (int64_t)(q * 4) * mpad) + o.frag);
     return f;
 }
 
@@ -352,14 +360,16 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ w, int64_t
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) acc[mt] = float4v{0.f, 0.f, 0.f, 0.f};
     const uint8_t *wrow = w + rt * ntc * TB;
+    GOff go = lane_offsets(lane, mpad);
     for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
         WRegs<DT> wr[P];
         XRegs<XT, MP> xr[P];
+        go.touch();
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
             const int64_t bc = b < ntc ? b : b0;  // keep the address in bounds; the result is not used
-            wr[p] = load_tile<DT>(wrow + bc * TB, lane);
+            wr[p] = load_tile<DT>(wrow + bc * TB, go);
             if constexpr (FUSED) xr[p] = load_x<XT, MP>(xin, ldx, m, k, bc, lane);
         }
 #pragma unroll
@@ -371,7 +381,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ w, int64_t
                     TileOp<DT, 1, 4>::run(wr[p], f, lane, acc);
                 } else {
                     const AFrags<DT, MT> f =
-                        load_frags_global<DT, MT>((const half8v *)xin + b * tile_chunks, mt_stride, mpad, lane);
+                        load_frags_global<DT, MT>((const half8v *)xin + b * tile_chunks, mt_stride, mpad, go);
                     TileOp<DT, MT, 4>::run(wr[p], f, lane, acc);
                 }
             }
@@ -515,20 +525,22 @@ __device__ __forceinline__ void gemv_frag_body(const uint8_t *__restrict__ w, in
     const uint8_t *wrow[R];  // row tiles past the end re-read the last one; their results are not stored
 #pragma unroll
     for (int r = 0; r < R; r++) wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+    GOff go = lane_offsets(lane, mpad);
     for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
         WRegs<DT> wr[P][R];
+        go.touch();
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
             const int64_t bc = b < ntc ? b : b0;
 #pragma unroll
-            for (int r = 0; r < R; r++) wr[p][r] = load_tile<DT>(wrow[r] + bc * TB, lane);
+            for (int r = 0; r < R; r++) wr[p][r] = load_tile<DT>(wrow[r] + bc * TB, go);
         }
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
             if (b < ntc) {  // uniform per wave
-                const AFrags<DT, MT> f = load_frags_global<DT, MT>((const half8v *)frags + b * tile_chunks, mt_stride, mpad, lane);
+                const AFrags<DT, MT> f = load_frags_global<DT, MT>((const half8v *)frags + b * tile_chunks, mt_stride, mpad, go);
 #pragma unroll
                 for (int r = 0; r < R; r++) TileOp<DT, MT, 4>::run(wr[p][r], f, lane, acc[r]);
             }

@@ -64,15 +64,6 @@ __device__ inline float dot2(half2v a, _Float16 b0, float c) { return __builtin_
 // raw activations of one tile: 4 consecutive columns per lane
 template <int XT> struct X1Regs { uint32_t r[XT == TURQ_ACT_F32 ? 4 : 2]; };
 
-// 32-bit per-lane byte offsets of the global loads.  An offset computed (and widened to 64 bits) outside the loop reaches
-// the loads as a register pair and costs a 64-bit vector add per load; one that is widened next to the load folds into the
-// load's own addressing (scalar base + 32-bit lane offset).  touch() at the top of every pass makes the offsets new values
-// for the compiler there, at no instruction.
-struct GOff {
-    uint32_t o16, o8, o4, hdr, aux;  // 16, 8, 4 bytes per lane; the lane's header row; a format's second header offset
-    __device__ void touch() { asm volatile("" : "+v"(o16), "+v"(o8), "+v"(o4), "+v"(hdr), "+v"(aux)); }
-};
-
 // RAGGED: k may end inside the tile (Q8_0: a multiple of 32, four columns are in or out together); the K-quants' k is a
 // multiple of 256 and needs no test
 template <int XT, bool RAGGED>
@@ -350,7 +341,7 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
 #pragma unroll
         for (int p = 0; p < P; p++) *(float *)(region + p * kRegion + kInit + 4 * lane) = 0.0f;  // float like the later writes
     const typename Fmt::Lane lc = Fmt::lane_init(lane & 15, g);
-    GOff go{16u * (uint32_t)lane, 8u * (uint32_t)lane, 4u * (uint32_t)lane, 16u * (uint32_t)(lane & 15), Fmt::aux_off(lane & 15, g)};
+    GOff go{16u * (uint32_t)lane, 8u * (uint32_t)lane, 4u * (uint32_t)lane, 16u * (uint32_t)(lane & 15), Fmt::aux_off(lane & 15, g), 0u};
 
     float acc[R];
     const uint8_t *wrow[R];  // row tiles past the weight's last one re-read it; their results are not stored

@@ -104,6 +104,18 @@ __device__ inline float4v mfma16x16x32(half8v a, half8v b, float4v c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
 }
 
+// 32-bit per-lane byte offsets of the global loads.  An offset computed (and widened to 64 bits) outside the loop reaches
+// the loads as a register pair and costs a 64-bit vector add per load; one that is widened next to the load folds into the
+// load's own addressing (scalar base + 32-bit lane offset).  touch() at the top of every pass makes the offsets new values
+// for the compiler there, at no instruction.
+struct GOff {
+    uint32_t o16, o8, o4;  // 16, 8, 4 bytes per lane
+    uint32_t hdr;          // 16 bytes per weight row of the tile (lane % 16)
+    uint32_t aux;          // a second header offset, by format
+    uint32_t frag;         // the lane's chunk inside one step of prepared activation fragments
+    __device__ void touch() { asm volatile("" : "+v"(o16), "+v"(o8), "+v"(o4), "+v"(hdr), "+v"(aux), "+v"(frag)); }
+};
+
 __device__ inline uint32_t rotr32(uint32_t v, uint32_t s) { return __builtin_amdgcn_alignbit(v, v, s); }
 
 __device__ inline uint16_t turq_f2bf(float f) {  // round to nearest even, NaN kept quiet
