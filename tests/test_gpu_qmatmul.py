@@ -246,6 +246,28 @@ def test_prefill_gemm_large_scales_fall_back(gpu, dt):
     assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, k)) <= 2e-5
 
 
+@pytest.mark.parametrize("dt", [Q4_K, Q5_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("shrink", [1 / 300, 1 / 3000])
+def test_prefill_gemm_small_scales(gpu, dt, shrink):
+    # real checkpoints carry super-block scales around 1e-5 .. 1e-4, where d * sc (and d * sc / 16 of Q5_K) would sit in
+    # the f16 subnormals: the GEMM multiplies the scales of a tensor by a power of two first and divides the result
+    n, k, m = 256, 2048, 64
+    bs = {Q4_K: 144, Q5_K: 176, Q6_K: 210, Q8_0: 34}[dt]
+    x = synth.random_activation(m, k, seed=m, bf16=True)
+    # Q4_K / Q5_K a second time with dmin left as it is: the power of two must leave room for dmin * m as well
+    for fields in ([[208]] if dt == Q6_K else [[0]] if dt == Q8_0 else [[0, 2], [0]]):
+        raw = synth.random_weight(dt, n, k, seed=5).reshape(-1, bs).copy()
+        for at in fields:
+            d = raw[:, at:at + 2].copy().view(np.float16).astype(np.float32) * np.float32(shrink)
+            raw[:, at:at + 2] = d.astype(np.float16).view(np.uint8)
+        raw = raw.reshape(-1)
+        w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+        y = gpu.qmatmul(w, x, n, k, algo=capi.ALGO_GEMM, x_dtype=capi.ACT_BF16)
+        gpu.release(w)
+        assert np.all(np.isfinite(y))
+        assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, k)) <= 4e-4, fields
+
+
 def test_prefill_q8_0_ragged_k_takes_the_skinny_kernel(gpu):
     # Q8_0 rows may end inside a 256-column tile; the GEMM wants whole tiles, so these shapes walk m in chunks
     n, k, m = 80, 256 + 96, 70

@@ -219,14 +219,20 @@ int turq_weight_upload(turq_ctx *ctx, int dt, int64_t n, int64_t k, const void *
     const uint8_t *src = (const uint8_t *)host_bytes;
     if (turq_dt_is_quant(dt)) {
         // bound on the scale a weight is multiplied by: |d * sc| for the K-quants (6-bit scales <= 63, Q6_K int8 scales <= 128
-        // in magnitude), |d| for Q8_0; see turq_weight::max_scale
+        // in magnitude), |d| for Q8_0; see turq_weight::max_scale.  Q4_K / Q5_K: dmin counts with 1 / 1024 of its size, which
+        // is what its packed-f16 constant (dmin * m, no base of 1024 on it) needs next to those of d.
         const int bs = turq_block_bytes(dt), d_at = dt == TURQ_Q6_K ? 208 : 0;
+        const bool has_min = dt == TURQ_Q4_K || dt == TURQ_Q5_K;
         float mx = 0.0f;
         const int64_t nblk = n * (k / turq_dt_block_elems(dt));
         for (int64_t i = 0; i < nblk; i++) {
             const uint8_t *b = src + i * bs + d_at;
             const float d = std::fabs(half_bits_to_float((uint16_t)(b[0] | (b[1] << 8))));
             if (d > mx || d != d) mx = d;
+            if (has_min) {
+                const float dm = std::fabs(half_bits_to_float((uint16_t)(b[2] | (b[3] << 8)))) * (1.0f / 1024.0f);
+                if (dm > mx || dm != dm) mx = dm;
+            }
         }
         w->max_scale = mx * (dt == TURQ_Q8_0 ? 1.0f : dt == TURQ_Q6_K ? 128.0f : 63.0f);
     }

@@ -179,7 +179,7 @@ struct K4Consts {
 };
 
 // constants of the lane's four sub-blocks u (sub-block 4 * g32 + u of the super-block) from a Q4_K / Q5_K header row
-__device__ inline K4Consts k4_consts(uint4v hd, int g32) {
+__device__ inline K4Consts k4_consts(uint4v hd, int g32, _Float16 ws) {
     // 24-bit groups of lane slots 2*g32 and 2*g32+1 inside the 96-bit field hd.y, hd.z, hd.w
     // (both candidates are computed and selected: a divergent branch would cost more than the two shifts)
     const uint32_t g0a = hd.y, g0b = __builtin_amdgcn_alignbit(hd.w, hd.z, 16);
@@ -188,8 +188,8 @@ __device__ inline K4Consts k4_consts(uint4v hd, int g32) {
     const uint32_t G0 = (g0a & ~msk) | (g0b & msk);
     const uint32_t G1 = (g1a & ~msk) | (g1b & msk);
     const half2v k1024 = splat2((_Float16)1024.0f);
-    const half2v dd = splat2(h_from_bits(hd.x & 0xFFFFu));
-    const half2v dm = splat2((_Float16)(-(float)h_from_bits(hd.x >> 16)));
+    const half2v dd = splat2(h_from_bits(hd.x & 0xFFFFu) * ws);  // ws is a power of two: exact
+    const half2v dm = splat2(-h_from_bits(hd.x >> 16) * ws);
     K4Consts c;
     half2v mn[2];
 #pragma unroll
@@ -229,7 +229,7 @@ template <> struct GFmt<TURQ_Q4_K> {
     template <int OFF> __device__ static void read_hdr(Hdr &h, const Addr &a, uint32_t ring) { lds_read128<OFF>(h.hd, a.h + ring); }
     __device__ static void pin_stage(Stage &st) { pin(st.q); }
     __device__ static void pin_hdr(Hdr &h) { pin(h.hd); }
-    __device__ static Consts consts(const Hdr &h, int g32) { return k4_consts(h.hd, g32); }
+    __device__ static Consts consts(const Hdr &h, int g32, _Float16 ws) { return k4_consts(h.hd, g32, ws); }
     __device__ static half8v bmin(const Consts &c) { return c.bmin; }
     template <int KS, int ST> __device__ static half8v operand(const Stage &st, const Consts &c) {
         const uint32_t w = word_of<ST>(st.q), w8 = w >> 8;
@@ -258,7 +258,7 @@ template <> struct GFmt<TURQ_Q5_K> {
     template <int OFF> __device__ static void read_hdr(Hdr &h, const Addr &a, uint32_t ring) { lds_read128<OFF>(h.hd, a.h + ring); }
     __device__ static void pin_stage(Stage &st) { pin(st.q); pin(st.hh); }
     __device__ static void pin_hdr(Hdr &h) { pin(h.hd); }
-    __device__ static Consts consts(const Hdr &h, int g32) { return k4_consts(h.hd, g32); }
+    __device__ static Consts consts(const Hdr &h, int g32, _Float16 ws) { return k4_consts(h.hd, g32, ws); }
     __device__ static half8v bmin(const Consts &c) { return c.bmin; }
     template <int KS, int ST> __device__ static half8v operand(const Stage &st, const Consts &c) {
         // step i of the slot; with v = 4 i + t the packed register t, u = v >> 1: its two high bits sit in H0 (even t) at
@@ -303,8 +303,8 @@ template <> struct GFmt<TURQ_Q6_K> {
     }
     __device__ static void pin_stage(Stage &st) { pin(st.ql); pin(st.qh); }
     __device__ static void pin_hdr(Hdr &h) { pin(h.sc0); pin(h.sc1); pin(h.d16); }
-    __device__ static Consts consts(const Hdr &h, int) {
-        const float d = (float)h_from_bits(h.d16);
+    __device__ static Consts consts(const Hdr &h, int, _Float16 ws) {
+        const float d = (float)h_from_bits(h.d16) * (float)ws;
         Consts c;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -358,11 +358,11 @@ template <> struct GFmt<TURQ_Q8_0> {
     template <int OFF> __device__ static void read_hdr(Hdr &h, const Addr &a, uint32_t ring) { lds_read128<OFF>(h.dd, a.h + ring); }
     __device__ static void pin_stage(Stage &st) { pin(st.a); pin(st.b); }
     __device__ static void pin_hdr(Hdr &h) { pin(h.dd); }
-    __device__ static Consts consts(const Hdr &h, int) {
+    __device__ static Consts consts(const Hdr &h, int, _Float16 ws) {
         const uint32_t dw[4] = {h.dd.x, h.dd.y, h.dd.z, h.dd.w};
         Consts c;
 #pragma unroll
-        for (int i = 0; i < 8; i++) c.s[i] = splat2(h_from_bits((i & 1) ? dw[i >> 1] >> 16 : dw[i >> 1] & 0xFFFFu));
+        for (int i = 0; i < 8; i++) c.s[i] = splat2(h_from_bits((i & 1) ? dw[i >> 1] >> 16 : dw[i >> 1] & 0xFFFFu) * ws);
         return c;
     }
     __device__ static half8v bmin(const Consts &) { return half8v{}; }
@@ -384,11 +384,15 @@ template <int DT>
 __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
                                                       const uint8_t *__restrict__ frags, int64_t m, void *__restrict__ y,
                                                       int yt, int64_t ldy, const float *__restrict__ bias, int nblocks_n,
-                                                      int nblocks_m, int vec_out) {
+                                                      int nblocks_m, int vec_out, float wscale, float inv_ws) {
     using Fm = GFmt<DT>;
     using G = Geo<DT, Fm::WN>;
     constexpr int WN = Fm::WN, TB = G::TB;
     constexpr bool SUMS = Fm::SUMS;
+    // every block scale is multiplied by wscale (a power of two chosen per tensor so that the largest packed-f16 weight
+    // lands near 2^15) and the results by its inverse: small scales keep their precision instead of dropping into the
+    // f16 subnormals (d * sc / 16 of Q5_K does so from d around 1e-4)
+    const _Float16 ws = (_Float16)wscale;  // inv_ws = 1 / wscale comes from the host
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -501,7 +505,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
 #pragma unroll
     for (int j = 0; j < WN; j++) {
         Fm::pin_hdr(hd[j]);
-        cs[j] = Fm::consts(hd[j], g32);
+        cs[j] = Fm::consts(hd[j], g32, ws);
     }
 
     for (int b = 0; b < ntc; b++) {
@@ -528,7 +532,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
 #pragma unroll
                             for (int j = 0; j < WN; j++) {
                                 Fm::pin_hdr(hd[j]);
-                                cs_next[j] = Fm::consts(hd[j], g32);
+                                cs_next[j] = Fm::consts(hd[j], g32, ws);
                             }
                         }
                     }
@@ -616,7 +620,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
             for (int i = 0; i < WM; i++)
 #pragma unroll
                 for (int e = 0; e < 16; e++)
-                    stage[(32 * i + 8 * (e >> 2) + 4 * g32 + (e & 3)) * OUT_PITCH + 32 * j + n32] = acc[i][j][e] + bv;
+                    stage[(32 * i + 8 * (e >> 2) + 4 * g32 + (e & 3)) * OUT_PITCH + 32 * j + n32] = acc[i][j][e] * inv_ws + bv;
         }
         // each wave reads back only what it wrote itself; LDS operations of one wave complete in order
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -659,7 +663,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                 for (int e = 0; e < 16; e++) {
                     const int64_t row = row0 + 32 * i + 8 * (e >> 2) + 4 * g32 + (e & 3);
                     if (row < m) {
-                        const float v = acc[i][j][e] + bv;
+                        const float v = acc[i][j][e] * inv_ws + bv;
                         if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, row * ldy + col, v);
                         else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, row * ldy + col, v);
                         else turq_store_out<TURQ_ACT_F16>(y, row * ldy + col, v);
@@ -671,7 +675,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
 
 template <int DT>
 hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y, int y_dtype, int64_t ldy,
-                       const float *bias, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+                       const float *bias, float wscale, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
     using G = Geo<DT, GFmt<DT>::WN>;
     constexpr int LDS_BYTES = G::S_OFF + (GFmt<DT>::SUMS ? NS * S_BYTES : 0);
     static_assert(LDS_BYTES <= 160 * 1024 && 4 * 64 * G::OUT_PITCH * 4 <= LDS_BYTES, "LDS of one workgroup; result staging fits");
@@ -686,10 +690,10 @@ hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, i
     const int vec_out = ((uintptr_t)y % 16 == 0 && ((uint64_t)ldy * es) % 16 == 0 && n % 8 == 0) ? 1 : 0;
     if (ev_start) {
         hipExtLaunchKernelGGL(gemm_kq_kernel<DT>, grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
-                              (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out);
+                              (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale);
     } else {
         gemm_kq_kernel<DT><<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype, ldy,
-                                                               bias, nbn, nbm, vec_out);
+                                                               bias, nbn, nbm, vec_out, wscale, 1.0f / wscale);
     }
     return hipGetLastError();
 }
@@ -697,16 +701,17 @@ hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, i
 }  // namespace
 
 // frags: activations prepared by turq_launch_act_prep32 (in the order of the same dtype) for all m rows
+// wscale: a power of two in [2^-14, 2^15] by which the kernel multiplies every block scale (see turq_gemm_weight_scale)
 hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
-                                 int y_dtype, int64_t ldy, const float *bias, hipStream_t stream, hipEvent_t ev_start,
-                                 hipEvent_t ev_stop) {
+                                 int y_dtype, int64_t ldy, const float *bias, float wscale, hipStream_t stream,
+                                 hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (n == 0 || m == 0) return hipSuccess;
-    if (k <= 0 || k % 256 != 0) return hipErrorInvalidValue;
+    if (k <= 0 || k % 256 != 0 || !(wscale >= 6.103515625e-5f && wscale <= 32768.0f)) return hipErrorInvalidValue;
     switch (dtype) {
-    case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
-    case TURQ_Q5_K: return launch_gemm<TURQ_Q5_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
-    case TURQ_Q6_K: return launch_gemm<TURQ_Q6_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
-    case TURQ_Q8_0: return launch_gemm<TURQ_Q8_0>(w, n, k, frags, m, y, y_dtype, ldy, bias, stream, ev_start, ev_stop);
+    case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+    case TURQ_Q5_K: return launch_gemm<TURQ_Q5_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+    case TURQ_Q6_K: return launch_gemm<TURQ_Q6_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+    case TURQ_Q8_0: return launch_gemm<TURQ_Q8_0>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
     default: return hipErrorInvalidValue;
     }
 }

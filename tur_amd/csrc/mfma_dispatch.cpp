@@ -60,10 +60,15 @@ int pick_rows_row1(const turq_ctx *ctx, int64_t row_tiles) {
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
                       int yt, int64_t ldy, const float *bias, int algo) {
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
-    // prefill chunks: LDS-tiled MFMA GEMM.  The largest packed-f16 value of the unpack must stay inside f16:
-    // (base + q) * d * sc with base 1024 for the nibbles of Q4_K / Q5_K and 256 for the 6-bit values of Q6_K; q * d for Q8_0
+    // prefill chunks: LDS-tiled MFMA GEMM.  Its weights are packed f16 values (base + q) * d * sc (base 1024 for the nibbles of
+    // Q4_K / Q5_K, 256 for the 6-bit values of Q6_K; q * d for Q8_0), the scales multiplied by a power of two that puts the
+    // largest of them near 2^15 (small scales would otherwise lose bits in the f16 subnormals); a tensor whose largest value
+    // does not fit f16 even unscaled goes through the exact skinny kernel instead
     const float top = w->dtype == TURQ_Q4_K ? 1039.0f : w->dtype == TURQ_Q5_K ? 1055.0f : w->dtype == TURQ_Q6_K ? 319.0f : 128.0f;
     const bool gemm_ok = turq_dt_is_quant(w->dtype) && w->k % 256 == 0 && w->max_scale * top < 60000.0f;
+    float wscale = 1.0f;
+    if (gemm_ok && w->max_scale > 0.0f)
+        while (wscale < 32768.0f && w->max_scale * top * wscale * 2.0f < 40000.0f) wscale *= 2.0f;
     if (algo == TURQ_ALGO_GEMM && !gemm_ok && m > TURQ_GEMV_MAX_M)
         algo = TURQ_ALGO_GEMV;  // scales too large for f16 operands, ragged Q8_0 columns: walk m in chunks through the skinny kernel
     if (m > TURQ_GEMV_MAX_M && algo == TURQ_ALGO_GEMM) {
@@ -72,7 +77,7 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
         TURQ_HIP(ctx, turq_launch_act_prep32(w->dtype, x, xt, m, w->k, ldx, ctx->act_prep, ctx->stream));
         TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
-        TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, ctx->stream, ev0, ev1));
+        TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, wscale, ctx->stream, ev0, ev1));
         return TURQ_OK;
     }
     const int nwaves = pick_waves(ctx, w->n, w->k);
