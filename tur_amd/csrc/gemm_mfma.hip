@@ -601,6 +601,15 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
         wr2 = t;
     }
     wait_lds<0>();
+    // The last stage boundary has issued the first LDS reads of a stage that does not exist.  Nothing uses them, but they
+    // are asm statements: the compiler takes their destination registers for written when the statement executes and, the
+    // values being dead, hands the registers out again at once, while the data arrives whenever the LDS delivers it.  (A
+    // division placed here by the compiler lost its temporaries that way, in whole wave tiles of some launches.)  Naming
+    // the registers after the wait keeps them reserved until the reads have landed.
+    pin(af[0][0]);
+    pin(af[0][1]);
+#pragma unroll
+    for (int j = 0; j < WN; j++) Fm::pin_stage(wq[0][j]);
     wait_vmcnt<0>();  // the trailing copies must neither outlive the workgroup's LDS nor land in the staged results
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
