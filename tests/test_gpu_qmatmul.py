@@ -348,6 +348,27 @@ def test_multi_weight_launch(gpu, dts, m):
         gpu.release(w)
 
 
+@pytest.mark.parametrize("dts", [(Q4_K, Q6_K), (Q4_K, Q4_K, Q4_K, Q6_K), (Q4_K, Q6_K, Q6_K), (Q6_K, Q4_K), (Q4_K,) * 4 + (Q6_K,)])
+@pytest.mark.parametrize("k", [256, 4096, 12288])
+def test_two_formats_in_one_row_launch(gpu, dts, k):
+    # one activation row against Q4_K weights followed by Q6_K ones (q, k, v of a Q4_K_M file): one launch when they are at
+    # most four; other orders and longer lists go out run by run.  Either way every result equals the single call.
+    ns = [80, 16, 33, 272, 48][: len(dts)]
+    raws = [synth.random_weight(dt, n, k, seed=7 * i + n + k) for i, (dt, n) in enumerate(zip(dts, ns))]
+    ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
+    x = synth.random_activation(1, k, seed=k, bf16=True)
+    biases = [None if i == 0 else np.random.default_rng(i).standard_normal(n).astype(np.float32) for i, n in enumerate(ns)]
+    for x_dtype in (capi.ACT_F32, capi.ACT_BF16):
+        ys = gpu.qmatmul_multi(ws, x, ns, k, x_dtype=x_dtype, biases=biases)
+        for dt, n, raw, w, y, b in zip(dts, ns, raws, ws, ys, biases):
+            want = orc.matmul_dequant(dt, x, raw, n, k) + (0 if b is None else b)
+            assert rel_l2(y, want) <= 2e-5, (dt, n)
+            single = gpu.qmatmul(w, x, n, k, x_dtype=x_dtype, bias=b)
+            assert np.array_equal(y, single), (dt, n)      # same kernel body, same split over waves
+    for w in ws:
+        gpu.release(w)
+
+
 def test_multi_weight_falls_back_to_single_calls(gpu):
     # more than 32 rows, or host pointers: the same as the calls one after the other
     k, ns, dts = 512, [48, 80], (Q4_K, Q4_K)

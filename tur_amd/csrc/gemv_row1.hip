@@ -308,25 +308,19 @@ struct Row1Args {
     int64_t n[kMaxRow1];
     int first[kMaxRow1];
     int count;
+    int second;  // two-format launches: weights [0, second) are of the first format, [second, count) of the second
 };
 
+// the work of one workgroup: row tiles rtb * R .. rtb * R + R - 1 of one weight.
 // P = column tiles a wave keeps in flight; R = row tiles per workgroup (a wave stages the activations of a column tile once and
-// uses them for R weight tiles); MAXT = largest workgroup of the instantiation
-template <int DT, int XT, int P, int R, int MAXT>
-__global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int yt) {
+// uses them for R weight tiles)
+template <int DT, int XT, int P, int R>
+__device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *__restrict__ y, const float *__restrict__ bias,
+                                          int64_t n, int64_t rtb, int64_t k, const void *__restrict__ x, int yt) {
     extern __shared__ uint8_t smem[];
     using Fmt = Row1Fmt<DT>;
     constexpr int TB = TiledFmt<DT>::kTileBytes;
-    const int blk = (int)blockIdx.x;
-    const uint8_t *w = a.w[0];
-    void *y = a.y[0];
-    const float *bias = a.bias[0];
-    int64_t n = a.n[0];
-    int first = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxRow1; i++)
-        if (i < a.count && blk >= a.first[i]) { w = a.w[i], y = a.y[i], bias = a.bias[i], n = a.n[i], first = a.first[i]; }
-    const int64_t rt0 = (int64_t)(blk - first) * R, nrt = turq_tile_rows(n);
+    const int64_t rt0 = rtb * R, nrt = turq_tile_rows(n);
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -410,6 +404,33 @@ __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, 
     }
 }
 
+// which weight of the launch this workgroup works on
+struct Row1Pick { const uint8_t *w; void *y; const float *bias; int64_t n; int first; int index; };
+__device__ inline Row1Pick row1_pick(const Row1Args &a, int blk) {
+    Row1Pick p{a.w[0], a.y[0], a.bias[0], a.n[0], 0, 0};
+#pragma unroll
+    for (int i = 1; i < kMaxRow1; i++)
+        if (i < a.count && blk >= a.first[i]) p = Row1Pick{a.w[i], a.y[i], a.bias[i], a.n[i], a.first[i], i};
+    return p;
+}
+
+// MAXT = largest workgroup of the instantiation
+template <int DT, int XT, int P, int R, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int yt) {
+    const Row1Pick p = row1_pick(a, (int)blockIdx.x);
+    row1_body<DT, XT, P, R>(p.w, p.y, p.bias, p.n, (int64_t)((int)blockIdx.x - p.first), k, x, yt);
+}
+
+// weights of two formats that share an input (q, k Q4_K and v Q6_K of a Q4_K_M file) in one launch: the workgroup's weight
+// decides which body runs
+template <int DTA, int DTB, int XT, int P, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_row1_mixed_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int yt) {
+    const Row1Pick p = row1_pick(a, (int)blockIdx.x);
+    const int64_t rtb = (int64_t)((int)blockIdx.x - p.first);
+    if (p.index < a.second) row1_body<DTA, XT, P, 1>(p.w, p.y, p.bias, p.n, rtb, k, x, yt);
+    else row1_body<DTB, XT, P, 1>(p.w, p.y, p.bias, p.n, rtb, k, x, yt);
+}
+
 template <int DT, int XT, int P, int R, int MAXT>
 hipError_t launch_final(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
                         hipEvent_t ev1) {
@@ -451,6 +472,28 @@ hipError_t launch_x(int xt, const Row1Args &a, int blocks, int64_t k, const void
     }
 }
 
+template <int DTA, int DTB, int XT, int P>
+hipError_t launch_mixed_final(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
+                              hipEvent_t ev1) {
+    const size_t lds = (size_t)nwaves * P * kRegion + (size_t)nwaves * 64 * sizeof(float);
+    if (ev0) {
+        hipExtLaunchKernelGGL((gemv_row1_mixed_kernel<DTA, DTB, XT, P, 1024>), dim3((unsigned)blocks), dim3((unsigned)(64 * nwaves)),
+                              (unsigned)lds, s, ev0, ev1, 0, a, k, x, yt);
+        return hipGetLastError();
+    }
+    gemv_row1_mixed_kernel<DTA, DTB, XT, P, 1024><<<(unsigned)blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(a, k, x, yt);
+    return hipGetLastError();
+}
+
+template <int DTA, int DTB, int XT>
+hipError_t launch_mixed_p(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
+                          hipEvent_t ev1) {
+    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
+    if (per_wave <= 1) return launch_mixed_final<DTA, DTB, XT, 1>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    if (per_wave == 2) return launch_mixed_final<DTA, DTB, XT, 2>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    return launch_mixed_final<DTA, DTB, XT, 3>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+}
+
 }  // namespace
 
 bool turq_gemv_row1_supports(int dtype) {
@@ -482,6 +525,39 @@ hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, con
     case TURQ_Q5_K: return launch_x<TURQ_Q5_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
     case TURQ_Q6_K: return launch_x<TURQ_Q6_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
     case TURQ_Q8_0: return launch_x<TURQ_Q8_0>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+bool turq_gemv_row1_mixed_supports(int dtype_a, int dtype_b) { return dtype_a == TURQ_Q4_K && dtype_b == TURQ_Q6_K; }
+
+// count (2..4) weights of one k against ONE activation row: the first `second` of format dtype_a, the others of dtype_b
+// (a pair turq_gemv_row1_mixed_supports accepts); one row tile per workgroup.
+hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w, const int64_t *n,
+                                       int64_t k, const void *x, int x_dtype, void *const *y, int y_dtype, const float *const *bias,
+                                       int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+    if (!turq_gemv_row1_mixed_supports(dtype_a, dtype_b) || count < 2 || count > kMaxRow1 || second < 1 || second >= count ||
+        nwaves < 1 || nwaves > 16 || k % 256 != 0)
+        return hipErrorInvalidValue;
+    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    Row1Args a{};
+    int64_t blocks = 0;
+    for (int i = 0; i < count; i++) {
+        a.w[i] = (const uint8_t *)w[i];
+        a.y[i] = y[i];
+        a.bias[i] = bias ? bias[i] : nullptr;
+        a.n[i] = n[i];
+        a.first[i] = (int)blocks;
+        blocks += turq_tile_rows(n[i]);
+    }
+    a.count = count;
+    a.second = second;
+    if (blocks == 0) return hipSuccess;
+    if (k == 0 || blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    switch (x_dtype) {
+    case TURQ_ACT_F32: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_F32>(a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_ACT_BF16: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_BF16>(a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_ACT_F16: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_F16>(a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
     default: return hipErrorInvalidValue;
     }
 }

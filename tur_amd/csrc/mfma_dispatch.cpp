@@ -131,6 +131,27 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
     while (i < count) {
         int j = i + 1;
         while (j < count && j - i < 4 && w[j]->dtype == w[i]->dtype) j++;
+        // one activation row: a run of a second format joins the launch where the kernel has that pair (q, k Q4_K + v Q6_K)
+        static const bool no_mixed = getenv("TURQ_GEMV_NO_MIXED") != nullptr;
+        if (fused && m == 1 && !no_mixed && j < count && use_row1(w[i]->dtype) && use_row1(w[j]->dtype) &&
+            turq_gemv_row1_mixed_supports(w[i]->dtype, w[j]->dtype)) {
+            int j2 = j + 1;
+            while (j2 < count && w[j2]->dtype == w[j]->dtype) j2++;
+            if (j2 - i <= 4) {
+                const void *wp[4];
+                int64_t nn[4];
+                for (int t = i; t < j2; t++) {
+                    wp[t - i] = w[t]->dev;
+                    nn[t - i] = w[t]->n;
+                }
+                hipEvent_t ev0 = nullptr, ev1 = nullptr;
+                TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+                TURQ_HIP(ctx, turq_launch_gemv_row1_mixed(w[i]->dtype, w[j]->dtype, j2 - i, j - i, wp, nn, w[i]->k, x, xt, y + i, yt,
+                                                          bias ? bias + i : nullptr, pick_waves_row1(w[i]->k), ctx->stream, ev0, ev1));
+                i = j2;
+                continue;
+            }
+        }
         if (!fused) {
             const int order = w[i]->dtype == TURQ_Q8_0 ? 2 : 1;
             if (prepared != order) {
