@@ -480,6 +480,7 @@ struct MultiArgs {
     int64_t n[kMaxMulti], ldy[kMaxMulti];
     int first[kMaxMulti];
     int count;
+    int second;  // two-format launches: weights [0, second) are of the first format, [second, count) of the second
 };
 
 template <int DT, int XT, int MP, int P, int MAXT>
@@ -593,6 +594,26 @@ __global__ void __launch_bounds__(MAXT) gemv_multi_frag_kernel(MultiArgs a, int6
         }
     if constexpr (R == 1) gemv_body<DT, MT, TURQ_ACT_F16, false, 1, P>(w, n, k, frags, 0, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
     else gemv_frag_body<DT, MT, P, R>(w, n, k, frags, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
+}
+
+// prepared fragments, weights of two formats with the same fragment order (Q4_K weights followed by Q6_K ones: q, k and v of a
+// Q4_K_M file): the workgroup's weight decides which body runs.  One row tile per workgroup.
+template <int DTA, int DTB, int MT, int P, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_multi_frag_mixed_kernel(MultiArgs a, int64_t k, const void *__restrict__ frags, int64_t m,
+                                                                      int mpad, int yt) {
+    const int blk = (int)blockIdx.x;
+    const uint8_t *w = a.w[0];
+    void *y = a.y[0];
+    const float *bias = a.bias[0];
+    int64_t n = a.n[0], ldy = a.ldy[0];
+    int first = 0, index = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxMulti; i++)
+        if (i < a.count && blk >= a.first[i]) {
+            w = a.w[i], y = a.y[i], bias = a.bias[i], n = a.n[i], ldy = a.ldy[i], first = a.first[i], index = i;
+        }
+    if (index < a.second) gemv_body<DTA, MT, TURQ_ACT_F16, false, 1, P>(w, n, k, frags, 0, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
+    else gemv_body<DTB, MT, TURQ_ACT_F16, false, 1, P>(w, n, k, frags, 0, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
 }
 
 struct GemvArgs {
@@ -740,6 +761,35 @@ hipError_t launch_multi_x(int xt, const MultiArgs &ma, int total_blocks, int64_t
     }
 }
 
+template <int DTA, int DTB, int MT, int P, int MAXT>
+hipError_t launch_multi_frag_mixed_final(const MultiArgs &ma, int total_blocks, int64_t k, const void *frags, int64_t m, int yt,
+                                         int nwaves, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    const int mpad = MT > 1 ? 16 : turq_mpad(m);
+    const size_t lds = nwaves > 1 ? (size_t)nwaves * MT * 64 * sizeof(float4v) : 0;
+    if (ev0) {
+        hipExtLaunchKernelGGL((gemv_multi_frag_mixed_kernel<DTA, DTB, MT, P, MAXT>), dim3((unsigned)total_blocks),
+                              dim3((unsigned)(64 * nwaves)), (unsigned)lds, s, ev0, ev1, 0, ma, k, frags, m, mpad, yt);
+        return hipGetLastError();
+    }
+    gemv_multi_frag_mixed_kernel<DTA, DTB, MT, P, MAXT><<<(unsigned)total_blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(ma, k, frags, m,
+                                                                                                                        mpad, yt);
+    return hipGetLastError();
+}
+
+// the launch shapes of launch_multi_frag_p with one row tile per workgroup
+template <int DTA, int DTB, int MT>
+hipError_t launch_multi_frag_mixed_p(const MultiArgs &ma, int total_blocks, int64_t k, const void *frags, int64_t m, int yt, int nwaves,
+                                     hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
+    if (nwaves <= 4) {
+        if (per_wave <= 1) return launch_multi_frag_mixed_final<DTA, DTB, MT, 1, 256>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+        if (per_wave <= 2) return launch_multi_frag_mixed_final<DTA, DTB, MT, 2, 256>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+        return launch_multi_frag_mixed_final<DTA, DTB, MT, 4, 256>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+    }
+    if (per_wave <= 1 || MT > 1) return launch_multi_frag_mixed_final<DTA, DTB, MT, 1, 1024>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+    return launch_multi_frag_mixed_final<DTA, DTB, MT, 2, 1024>(ma, total_blocks, k, frags, m, yt, nwaves, s, ev0, ev1);
+}
+
 }  // namespace
 
 // count (2..4) weights of one format and one k.  fused: `x` are the raw activations (m <= TURQ_GEMV_FUSED_MAX_M, rows 16-byte
@@ -782,6 +832,38 @@ hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w, co
     case TURQ_Q8_0: return launch_multi_x<TURQ_Q8_0>(x_dtype, ma, (int)blocks, k, x, ldx, m, y_dtype, nwaves, stream, ev_start, ev_stop);
     default: return hipErrorInvalidValue;
     }
+}
+
+bool turq_gemv_multi_mixed_supports(int dtype_a, int dtype_b) { return dtype_a == TURQ_Q4_K && dtype_b == TURQ_Q6_K; }
+
+// count (2..4) weights of one k against prepared fragments (K-quant order) of m <= TURQ_GEMV_MAX_M rows: the first `second` of
+// format dtype_a, the others of dtype_b (a pair turq_gemv_multi_mixed_supports accepts); one row tile per workgroup.
+hipError_t turq_launch_gemv_multi_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w, const int64_t *n,
+                                        int64_t k, const void *frags, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
+                                        const float *const *bias, int nwaves, hipStream_t stream, hipEvent_t ev_start,
+                                        hipEvent_t ev_stop) {
+    if (!turq_gemv_multi_mixed_supports(dtype_a, dtype_b) || count < 2 || count > kMaxMulti || second < 1 || second >= count || m < 1 ||
+        m > TURQ_GEMV_MAX_M || nwaves < 1 || nwaves > 16)
+        return hipErrorInvalidValue;
+    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    MultiArgs ma{};
+    int64_t blocks = 0;
+    for (int i = 0; i < count; i++) {
+        ma.w[i] = (const uint8_t *)w[i];
+        ma.y[i] = y[i];
+        ma.bias[i] = bias ? bias[i] : nullptr;
+        ma.n[i] = n[i];
+        ma.ldy[i] = ldy[i];
+        ma.first[i] = (int)blocks;
+        blocks += turq_tile_rows(n[i]);
+    }
+    ma.count = count;
+    ma.second = second;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    if (m <= 16)
+        return launch_multi_frag_mixed_p<TURQ_Q4_K, TURQ_Q6_K, 1>(ma, (int)blocks, k, frags, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+    return launch_multi_frag_mixed_p<TURQ_Q4_K, TURQ_Q6_K, 2>(ma, (int)blocks, k, frags, m, y_dtype, nwaves, stream, ev_start, ev_stop);
 }
 
 // `xin` is the prepared fragment buffer (fused == false; ldx and x_dtype unused) or the raw

@@ -158,6 +158,11 @@ bool turq_gemv_row1_supports(int dtype);
 hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w_tiled, const int64_t *n, int64_t k, const void *x,
                                  int x_dtype, void *const *y, int y_dtype, const float *const *bias, int waves_per_group,
                                  int row_tiles_per_group, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
+bool turq_gemv_multi_mixed_supports(int dtype_a, int dtype_b);
+hipError_t turq_launch_gemv_multi_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w_tiled, const int64_t *n,
+                                        int64_t k, const void *frags, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
+                                        const float *const *bias, int waves_per_group, hipStream_t stream, hipEvent_t ev_start,
+                                        hipEvent_t ev_stop);
 bool turq_gemv_row1_mixed_supports(int dtype_a, int dtype_b);
 hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w_tiled, const int64_t *n,
                                        int64_t k, const void *x, int x_dtype, void *const *y, int y_dtype, const float *const *bias,

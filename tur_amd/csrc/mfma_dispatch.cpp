@@ -161,6 +161,30 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
                 prepared = order;
             }
         }
+        // prepared fragments: the same for a second format of the same fragment order, while one row tile per workgroup is the
+        // launch shape anyway
+        if (!fused && !no_mixed && j < count && turq_gemv_multi_mixed_supports(w[i]->dtype, w[j]->dtype)) {
+            int j2 = j + 1;
+            while (j2 < count && w[j2]->dtype == w[j]->dtype) j2++;
+            int64_t rows2 = 0;
+            for (int t = i; t < j2; t++) rows2 += w[t]->n;
+            const int64_t cus2 = ctx->compute_units > 0 ? ctx->compute_units : 256;
+            if (j2 - i <= 4 && turq_tile_rows(rows2) < 4 * cus2) {
+                const void *wp2[4];
+                int64_t nn2[4];
+                for (int t = i; t < j2; t++) {
+                    wp2[t - i] = w[t]->dev;
+                    nn2[t - i] = w[t]->n;
+                }
+                hipEvent_t e0 = nullptr, e1 = nullptr;
+                TURQ_HIP(ctx, turq_prof_next(ctx, &e0, &e1));
+                TURQ_HIP(ctx, turq_launch_gemv_multi_mixed(w[i]->dtype, w[j]->dtype, j2 - i, j - i, wp2, nn2, w[i]->k, ctx->act_prep, m,
+                                                           y + i, yt, ldy + i, bias ? bias + i : nullptr,
+                                                           pick_waves(ctx, rows2, w[i]->k), ctx->stream, e0, e1));
+                i = j2;
+                continue;
+            }
+        }
         const void *wp[4];
         int64_t nn[4];
         int64_t rows = 0;
