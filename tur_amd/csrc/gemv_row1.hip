@@ -374,7 +374,8 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
                 float4v c = Fmt::chain(wr[p][r], region + p * kRegion, lc, g);
                 // One tile after the other.  Left free, the scheduler interleaves the tiles' chains and scale arithmetic, the
                 // unpacked operands of several tiles are live at once and the 128 registers a wave of a 16-wave workgroup may
-                // use overflow (spills in the instantiations with four tiles per pass; the 510 MB LM head lost 20 %).  The
+                // use overflow (spills in the instantiations with four tiles per workgroup pass; the 510 MB LM head lost
+                // 20 %).  The
                 // empty asm consumes the chain's result; vector and matrix instructions may not cross the barrier.
                 asm volatile("" : "+v"(c));
                 __builtin_amdgcn_sched_barrier(0x10 | 0x80 | 0x4);
@@ -450,15 +451,14 @@ hipError_t launch_p(const Row1Args &a, int blocks, int64_t k, const void *x, int
     static const int forced = [] { const char *e = getenv("TURQ_ROW1_P"); return e ? atoi(e) : 0; }();
     const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
     int p = (int)(per_wave < 3 ? per_wave : 3);  // four tiles in flight do not fit the registers of every format
-    if (forced >= 1 && forced <= 4) p = forced;
+    if (forced >= 1 && forced <= 3) p = forced;
     if (rtiles == 2) {  // two row tiles double the weights a wave holds: at most two column tiles in flight
         if (p == 1) return launch_final<DT, XT, 1, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
         return launch_final<DT, XT, 2, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
     }
     if (p == 1) return launch_final<DT, XT, 1, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
     if (p == 2) return launch_final<DT, XT, 2, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    if (p == 3) return launch_final<DT, XT, 3, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    return launch_final<DT, XT, 4, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    return launch_final<DT, XT, 3, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
 }
 
 template <int DT>
