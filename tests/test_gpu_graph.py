@@ -1,0 +1,132 @@
+"""A decode / prefill step captured into a HIP graph and replayed: every replay must give what the same calls give eagerly.
+
+The step mixes the launch kinds a model step has: a q / k / v group of two formats (one launch at m = 1 and with prepared
+fragments), a single call of a third format, and (m > 32) the prefill GEMM with its preparation kernel.  Between the replays
+the program does its own eager work and synchronises, and the activations change in place, as they do between decode steps.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import capi as orc
+from tests.helpers import Gpu, rel_l2
+from tur_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+Q8_0, Q4_K, Q6_K = capi.Q8_0, capi.Q4_K, capi.Q6_K
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    g = Gpu()
+    yield g
+    g.close()
+
+
+class Step:
+    """q / k / v (Q4_K, Q4_K, Q6_K) through turq_qmatmul_multi plus one Q8_0 matrix, everything in device memory."""
+
+    def __init__(self, gpu, m, k=1024):
+        self.gpu, self.m, self.k = gpu, m, k
+        L, ctx = gpu.L, gpu.ctx
+        self.dts = (Q4_K, Q4_K, Q6_K, Q8_0)
+        self.ns = (80, 48, 33, 64)
+        self.raws = [synth.random_weight(dt, n, k, seed=3 * i + n) for i, (dt, n) in enumerate(zip(self.dts, self.ns))]
+        self.ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(self.dts, self.ns, self.raws)]
+        self.bufs = []
+        self.x = self._dev(m * k * 4)
+        self.ys = [self._dev(m * n * 4) for n in self.ns]
+        self.warr = (ctypes.c_void_p * 3)(*[w.value for w in self.ws[:3]])
+        self.yarr = (ctypes.c_void_p * 3)(*[y.value for y in self.ys[:3]])
+        self.ldys = (ctypes.c_int64 * 3)(*self.ns[:3])
+
+    def _dev(self, nbytes):
+        p = ctypes.c_void_p()
+        capi.check(self.gpu.L.turq_dev_alloc(self.gpu.ctx, nbytes, ctypes.byref(p)), self.gpu.ctx)
+        self.bufs.append(p)
+        return p
+
+    def close(self):
+        for b in self.bufs:
+            capi.check(self.gpu.L.turq_dev_free(self.gpu.ctx, b), self.gpu.ctx)
+        for w in self.ws:
+            self.gpu.release(w)
+
+    def set_x(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        capi.check(self.gpu.L.turq_memcpy_h2d(self.gpu.ctx, self.x, capi.ptr(x), x.nbytes), self.gpu.ctx)
+
+    def clear_outputs(self):
+        for y, n in zip(self.ys, self.ns):
+            z = np.full(self.m * n, np.nan, np.float32)
+            capi.check(self.gpu.L.turq_memcpy_h2d(self.gpu.ctx, y, capi.ptr(z), z.nbytes), self.gpu.ctx)
+
+    def outputs(self):
+        capi.check(self.gpu.L.turq_sync(self.gpu.ctx), self.gpu.ctx)
+        outs = []
+        for y, n in zip(self.ys, self.ns):
+            o = np.empty((self.m, n), np.float32)
+            capi.check(self.gpu.L.turq_memcpy_d2h(self.gpu.ctx, capi.ptr(o), y, o.nbytes), self.gpu.ctx)
+            outs.append(o)
+        return outs
+
+    def calls(self):
+        L, ctx, m, k = self.gpu.L, self.gpu.ctx, self.m, self.k
+        capi.check(L.turq_qmatmul_multi(ctx, 3, self.warr, self.x, capi.ACT_F32, m, k, self.yarr, capi.ACT_F32, self.ldys, None,
+                                        capi.MEM_DEVICE, capi.ALGO_AUTO), ctx)
+        capi.check(L.turq_qmatmul(ctx, self.ws[3], self.x, capi.ACT_F32, m, k, self.ys[3], capi.ACT_F32, self.ns[3], None,
+                                  capi.MEM_DEVICE, capi.ALGO_AUTO), ctx)
+
+
+@pytest.mark.parametrize("m", [1, 8, 64])
+def test_graph_replays_equal_the_eager_calls(gpu, m):
+    L, ctx = gpu.L, gpu.ctx
+    st = Step(gpu, m)
+    other = Step(gpu, 3, k=512)          # the program's own eager work between replays
+    other.set_x(synth.random_activation(3, 512, seed=99))
+    try:
+        st.set_x(synth.random_activation(m, st.k, seed=1))
+        st.calls()                        # scratch buffers reach their final size outside the capture
+        capi.check(L.turq_sync(ctx), ctx)
+        capi.check(L.turq_graph_begin(ctx), ctx)
+        st.calls()
+        g = ctypes.c_void_p()
+        capi.check(L.turq_graph_end(ctx, ctypes.byref(g)), ctx)
+        assert g.value
+        for rep in range(4):
+            x = synth.random_activation(m, st.k, seed=10 + rep)
+            st.set_x(x)
+            st.clear_outputs()
+            st.calls()
+            want = st.outputs()
+            for dt, n, raw, y in zip(st.dts, st.ns, st.raws, want):
+                assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, st.k)) <= 1e-3, (rep, dt)
+            other.calls()                 # eager work of another shape: the shared scratch buffers are rewritten
+            other.outputs()
+            st.clear_outputs()
+            capi.check(L.turq_graph_launch(ctx, g), ctx)
+            got = st.outputs()
+            for dt, y, w in zip(st.dts, got, want):
+                assert np.array_equal(y, w), (rep, dt)
+        L.turq_graph_destroy(g)
+    finally:
+        st.close()
+        other.close()
+
+
+def test_graph_misuse_is_an_error_not_a_crash(gpu):
+    L, ctx = gpu.L, gpu.ctx
+    g = ctypes.c_void_p()
+    assert L.turq_graph_end(ctx, ctypes.byref(g)) == capi.ERR_INVALID          # no capture running
+    assert L.turq_graph_launch(ctx, None) == capi.ERR_INVALID
+    capi.check(L.turq_graph_begin(ctx), ctx)
+    assert L.turq_graph_begin(ctx) == capi.ERR_INVALID                         # already capturing
+    capi.check(L.turq_graph_end(ctx, ctypes.byref(g)), ctx)                    # an empty graph is still a graph
+    capi.check(L.turq_graph_launch(ctx, g), ctx)
+    capi.check(L.turq_sync(ctx), ctx)
+    L.turq_graph_destroy(g)
+    L.turq_graph_destroy(None)
