@@ -7,9 +7,11 @@
 // hidden under the MFMAs (about 2 cycles per VALU instruction on top of the 32 of an MFMA, also with
 // two waves per SIMD), so the loop is written to spend as few other instructions as it can.
 //
-// Tiling.  Workgroup tile 128 (m) x 192 (n), 4 waves as 2 x 2, wave tile 64 x 96 = 2 x 3 MFMA tiles
-// (96 accumulator registers).  The activations are the expensive operand here (2 bytes per element
-// against 0.56 for the weights), hence the wide n.
+// Tiling.  A workgroup is 4 waves and takes 128 rows of m.  Q4_K: tile 128 (m) x 192 (n), waves as 2 x 2, wave tile
+// 64 x 96 = 2 x 3 MFMA tiles (96 accumulator registers).  The activations are the expensive operand here (2 bytes per
+// element against 0.56 for the weights), hence the wide n.  Q5_K / Q6_K, whose unpack is two to three times as long: tile
+// 128 x 128 with the waves as 1 x 4, wave tile 128 x 32 = 4 x 1 MFMA tiles, so that every weight is unpacked by one wave
+// instead of two (the 2 x 2 grid is 18 % slower for Q6_K, 7 % for Q5_K).
 //
 // Everything reaches the LDS by global_load_lds_dwordx4 (no registers, no ds_write):
 //   * activations, prepared in 32-row A-fragment order (act_prep32_kernel), 64 columns (4 operand
@@ -42,16 +44,16 @@
 // weights this costs about 3e-4 relative L2 (bar: 1e-3).  The dispatcher only uses this kernel while
 // 1024 * d * sc stays inside f16.
 //
-// Formats.  Q4_K as above (wave tile 2 x 3, workgroup 128 x 192).  Q5_K adds the fifth bit from the tile's
+// Formats.  Q4_K as above.  Q5_K adds the fifth bit from the tile's
 // high-bit plane with one rotate and one v_and_or_b32 per packed register; Q6_K builds the whole 6-bit value in
 // the mantissa of 256.0 (low nibble at bits 2..5, high field rotated onto bits 6..7) and needs no sums term.  Their
-// tiles are larger (2816 / 3360 bytes), so their workgroup is 128 x 128 (wave tile 2 x 2) to keep three
-// super-blocks of weights in the LDS.  Q8_0 (4352-byte tiles, f16 block scales, no sums term): 128 x 64, wave tile 2 x 1.
+// tiles are larger (2816 / 3360 bytes), so their workgroup is 128 x 128 to keep three super-blocks of weights in the LDS.  Q8_0 (4352-byte tiles, f16 block scales, no sums term): 128 x 64, wave tile 2 x 1.
 //
 // Results leave through the LDS (free after the main loop): each wave transposes its 64 x 96 tile so
 // that a lane stores 16 contiguous bytes and a row segment is 192 (bf16, f16) or 384 (f32) bytes.
 #include <hip/hip_ext.h>
 
+#include <cstdlib>
 #include <type_traits>
 #include <utility>
 
@@ -67,20 +69,31 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 constexpr uint32_t kMagic1024 = 0x64006400u;  // 1024.0: a nibble in mantissa bits 0..3 reads as 1024 + n
 constexpr uint32_t kMagic64 = 0x54005400u;    // 64.0:   a nibble in mantissa bits 4..7 reads as 64 + n
 constexpr uint32_t kMagic256 = 0x5C005C00u;   // 256.0:  a 6-bit value in mantissa bits 2..7 reads as 256 + q
-constexpr int WGM = 2, WGN = 2;               // waves of a workgroup along m and n
-constexpr int WM = 2;                         // 32x32 MFMA tiles per wave along m
-constexpr int BM = WGM * WM * 32;             // 128
+// A workgroup is 4 waves and covers 128 rows of m (4 m-tiles of 32): as 2 x 2 waves with 2 m-tiles each (WGM = 2), or as
+// 1 x 4 waves that all take the 4 m-tiles (WGM = 1: every weight is unpacked by ONE wave instead of two, at twice the
+// activation reads per wave; for the formats whose unpack is long)
+constexpr int BM = 128;
 constexpr int MT = BM / 32;                   // m-tiles per workgroup; wave w copies m-tile w
 constexpr int A_STAGE = MT * 4 * 1024;        // [m-tile][step] blocks of 1 KiB
 constexpr int NA = 4;                         // stage ring; 4 stages per super-block, so stage ks lives in buffer ks
 constexpr int NW = 3;                         // weight ring (super-blocks)
 constexpr int S_BYTES = MT * 1024;
 constexpr int NS = 2;
-static_assert(MT == 4 && WGM * WGN == 4 && WM == 2, "the copy and read schedules below are written for this shape");
+static_assert(MT == 4, "the copy and read schedules below are written for this shape");
 
-// geometry that depends on the format: WN = 32x32 tiles per wave along n
-template <int DT, int WN_> struct Geo {
-    static constexpr int WN = WN_;
+// 32x32 tiles per wave along n in the 2 x 2 wave grid, by format (the per-format pieces are further down)
+template <int DT> struct GFmtWN;
+template <> struct GFmtWN<TURQ_Q4_K> { static constexpr int value = 3; };
+template <> struct GFmtWN<TURQ_Q5_K> { static constexpr int value = 2; };
+template <> struct GFmtWN<TURQ_Q6_K> { static constexpr int value = 2; };
+template <> struct GFmtWN<TURQ_Q8_0> { static constexpr int value = 1; };
+
+// geometry that depends on the format and the wave grid: WGM x WGN waves, WM x WN 32x32 tiles per wave
+template <int DT, int WGM_> struct Geo {
+    static_assert(WGM_ == 1 || (WGM_ == 2), "wave grid 2 x 2 or 1 x 4");
+    static_assert(WGM_ == 2 || GFmtWN<DT>::value % 2 == 0, "the 1 x 4 grid halves the format's tiles per wave along n");
+    static constexpr int WGM = WGM_, WGN = 4 / WGM_, WM = MT / WGM_;
+    static constexpr int WN = WGM_ == 2 ? GFmtWN<DT>::value : GFmtWN<DT>::value / 2;
     static constexpr int BN = WGN * WN * 32;
     static constexpr int NT16 = BN / 16;                           // 16-row weight tiles per workgroup
     static constexpr int TB = TiledFmt<DT>::kTileBytes;
@@ -213,7 +226,7 @@ __device__ inline K4Consts k4_consts(uint4v hd, int g32, _Float16 ws) {
 
 template <> struct GFmt<TURQ_Q4_K> {
     using F = TiledFmt<TURQ_Q4_K>;
-    static constexpr int WN = 3, NSTG = 1, NHDR = 1;
+    static constexpr int NSTG = 1;
     static constexpr bool SUMS = true;
     struct Stage { uint4v q; };
     struct Hdr { uint4v hd; };
@@ -241,7 +254,7 @@ template <> struct GFmt<TURQ_Q4_K> {
 
 template <> struct GFmt<TURQ_Q5_K> {
     using F = TiledFmt<TURQ_Q5_K>;
-    static constexpr int WN = 2, NSTG = 2, NHDR = 1;
+    static constexpr int NSTG = 2;
     static constexpr bool SUMS = true;
     struct Stage { uint4v q; uint2v hh; };
     struct Hdr { uint4v hd; };
@@ -281,7 +294,7 @@ template <> struct GFmt<TURQ_Q5_K> {
 
 template <> struct GFmt<TURQ_Q6_K> {
     using F = TiledFmt<TURQ_Q6_K>;
-    static constexpr int WN = 2, NSTG = 2, NHDR = 3;
+    static constexpr int NSTG = 2;
     static constexpr bool SUMS = false;
     struct Stage { uint4v ql, qh; };
     struct Hdr { uint32_t sc0, sc1, d16; };  // the four int8 scales of lane slots 2 g32 and 2 g32 + 1; the row's d
@@ -342,7 +355,7 @@ template <> struct GFmt<TURQ_Q6_K> {
 // rounded once.  The tiles are 4352 bytes: wave tile 2 x 1 (workgroup 128 x 64) keeps three super-blocks in the LDS.
 template <> struct GFmt<TURQ_Q8_0> {
     using F = TiledFmt<TURQ_Q8_0>;
-    static constexpr int WN = 1, NSTG = 2, NHDR = 1;
+    static constexpr int NSTG = 2;
     static constexpr bool SUMS = false;
     struct Stage { uint4v a, b; };     // lane slots 2 g32 and 2 g32 + 1 of the plane: (block 2 ks: lo, hi), (block 2 ks + 1: lo, hi)
     struct Hdr { uint4v dd; };         // the row's 8 f16 block scales
@@ -380,14 +393,14 @@ template <> struct GFmt<TURQ_Q8_0> {
 
 // frags: 32-row fragments, 1 KiB block index (mt * ntc + b) * 17 + q
 // vec_out: rows of y can be written as aligned 16-byte pieces
-template <int DT>
+template <int DT, int WGM_>
 __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
                                                       const uint8_t *__restrict__ frags, int64_t m, void *__restrict__ y,
                                                       int yt, int64_t ldy, const float *__restrict__ bias, int nblocks_n,
                                                       int nblocks_m, int vec_out, float wscale, float inv_ws) {
     using Fm = GFmt<DT>;
-    using G = Geo<DT, Fm::WN>;
-    constexpr int WN = Fm::WN, TB = G::TB;
+    using G = Geo<DT, WGM_>;
+    constexpr int WGN = G::WGN, WM = G::WM, WN = G::WN, TB = G::TB;
     constexpr bool SUMS = Fm::SUMS;
     // every block scale is multiplied by wscale (a power of two chosen per tensor so that the largest packed-f16 weight
     // lands near 2^15) and the results by its inverse: small scales keep their precision instead of dropping into the
@@ -397,7 +410,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WGN, wn = wave % WGN;
     const int n32 = lane & 31, g32 = lane >> 5;
     const int r16 = n32 & 15, tsel = n32 >> 4;
     // Workgroups of one XCD (blockIdx % 8) get consecutive logical ids and the m-blocks of one n-block are
@@ -499,8 +512,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
         Fm::template read_hdr<j * 2 * TB>(hd[j], w_rd, wr0);
         Fm::template read_stage<0, j * 2 * TB>(wq[0][j], w_rd, wr0);
     });
-    lds_read128<0>(af[0][0], a_rd);
-    lds_read128<4096>(af[0][1], a_rd);
+    static_for<WM>([&](auto I) { lds_read128<decltype(I)::value * 4096>(af[0][decltype(I)::value], a_rd); });
     wait_lds<0>();
 #pragma unroll
     for (int j = 0; j < WN; j++) {
@@ -520,11 +532,13 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                 constexpr int pa = st & 1;
                 if constexpr (st < 3) {
                     // next step's activation fragments come in while this step computes
-                    lds_read128<ks * A_STAGE + (st + 1) * 1024>(af[pa ^ 1][0], a_rd);
-                    lds_read128<ks * A_STAGE + 4096 + (st + 1) * 1024>(af[pa ^ 1][1], a_rd);
-                    wait_lds<2>();  // everything but the two reads just issued
-                    pin(af[pa][0]);
-                    pin(af[pa][1]);
+                    static_for<WM>([&](auto I) {
+                        constexpr int i = decltype(I)::value;
+                        lds_read128<ks * A_STAGE + i * 4096 + (st + 1) * 1024>(af[pa ^ 1][i], a_rd);
+                    });
+                    wait_lds<WM>();  // everything but the reads just issued
+#pragma unroll
+                    for (int i = 0; i < WM; i++) pin(af[pa][i]);
                     if constexpr (st == 0) {
 #pragma unroll
                         for (int j = 0; j < WN; j++) Fm::pin_stage(wq[cur][j]);
@@ -539,8 +553,8 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                 } else {
                     // ---- stage boundary, before the last step: the next stage becomes readable ----
                     wait_lds<0>();  // step 3's fragments are in registers: this wave is done with the stage's LDS
-                    pin(af[1][0]);
-                    pin(af[1][1]);
+#pragma unroll
+                    for (int i = 0; i < WM; i++) pin(af[1][i]);
                     // The next stage's copies were issued three boundaries ago; younger than them are that
                     // boundary's weight (and sums) copies and everything of the two boundaries since.
                     if constexpr (ks == 0 || !SUMS) wait_vmcnt<14>(); else wait_vmcnt<15>();
@@ -552,8 +566,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                     if constexpr (ks == 0) issue_s(b1);
                     // first reads of the next stage, hidden under step 3's MFMAs
                     if constexpr (ks == 3 && SUMS) {
-                        lds_read128<0>(sf[0], s_cur);
-                        lds_read128<1024>(sf[1], s_cur);
+                        static_for<WM>([&](auto I) { lds_read128<decltype(I)::value * 1024>(sf[decltype(I)::value], s_cur); });
                     }
                     constexpr int nks = (ks + 1) & 3;
                     const uint32_t ring_from = ks == 3 ? wr1 : wr0;
@@ -567,8 +580,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                             Fm::template read_hdr<j * 2 * TB>(hd[j], w_rd, wr1);
                         });
                     }
-                    lds_read128<nks * A_STAGE>(af[0][0], a_rd);
-                    lds_read128<nks * A_STAGE + 4096>(af[0][1], a_rd);
+                    static_for<WM>([&](auto I) { lds_read128<nks * A_STAGE + decltype(I)::value * 4096>(af[0][decltype(I)::value], a_rd); });
                 }
                 // operand step 4 ks + st of the lane's 128 columns
                 half8v bop[WN];
@@ -582,9 +594,9 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
             if constexpr (ks == 3) {
                 if constexpr (SUMS) {
                     // "- dmin * m" term against the sub-block sums
-                    wait_lds<WN * Fm::NSTG + 2>();  // all but the weight and fragment reads of the next stage
-                    pin(sf[0]);
-                    pin(sf[1]);
+                    wait_lds<WN * Fm::NSTG + WM>();  // all but the weight and fragment reads of the next stage
+#pragma unroll
+                    for (int i = 0; i < WM; i++) pin(sf[i]);
 #pragma unroll
                     for (int i = 0; i < WM; i++)
 #pragma unroll
@@ -606,8 +618,8 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     // values being dead, hands the registers out again at once, while the data arrives whenever the LDS delivers it.  (A
     // division placed here by the compiler lost its temporaries that way, in whole wave tiles of some launches.)  Naming
     // the registers after the wait keeps them reserved until the reads have landed.
-    pin(af[0][0]);
-    pin(af[0][1]);
+#pragma unroll
+    for (int i = 0; i < WM; i++) pin(af[0][i]);
 #pragma unroll
     for (int j = 0; j < WN; j++) Fm::pin_stage(wq[0][j]);
     wait_vmcnt<0>();  // the trailing copies must neither outlive the workgroup's LDS nor land in the staged results
@@ -620,7 +632,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     const int64_t row0 = (int64_t)mb * BM + wm * (WM * 32);
     const int64_t col0 = (int64_t)nb * G::BN + wn * (WN * 32);
     if (vec_out) {
-        float *stage = (float *)lds + (size_t)wave * (64 * OUT_PITCH);
+        float *stage = (float *)lds + (size_t)wave * (WM * 32 * OUT_PITCH);
 #pragma unroll
         for (int j = 0; j < WN; j++) {
             const int64_t col = col0 + 32 * j + n32;
@@ -638,7 +650,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
         if (yt == TURQ_ACT_F32) {
             constexpr int CPR = WN * 32 / 4;  // 16-byte pieces per row
 #pragma unroll 4
-            for (int it = 0; it < CPR; it++) {
+            for (int it = 0; it < WM * 32 * CPR / 64; it++) {
                 const int c = it * 64 + lane;
                 const int r = c / CPR, cc = c - r * CPR;
                 const float4v v = *(const float4v *)(stage + r * OUT_PITCH + 4 * cc);
@@ -647,7 +659,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
         } else {
             constexpr int CPR = WN * 32 / 8;
 #pragma unroll 4
-            for (int it = 0; it < CPR; it++) {
+            for (int it = 0; it < WM * 32 * CPR / 64; it++) {
                 const int c = it * 64 + lane;
                 const int r = c / CPR, cc = c - r * CPR;
                 const float4v v0 = *(const float4v *)(stage + r * OUT_PITCH + 8 * cc);
@@ -682,27 +694,27 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     }
 }
 
-template <int DT>
+template <int DT, int WGM_>
 hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y, int y_dtype, int64_t ldy,
                        const float *bias, float wscale, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
-    using G = Geo<DT, GFmt<DT>::WN>;
+    using G = Geo<DT, WGM_>;
     constexpr int LDS_BYTES = G::S_OFF + (GFmt<DT>::SUMS ? NS * S_BYTES : 0);
-    static_assert(LDS_BYTES <= 160 * 1024 && 4 * 64 * G::OUT_PITCH * 4 <= LDS_BYTES, "LDS of one workgroup; result staging fits");
+    static_assert(LDS_BYTES <= 160 * 1024 && 4 * G::WM * 32 * G::OUT_PITCH * 4 <= LDS_BYTES, "LDS of one workgroup; result staging fits");
     // per-lane weight offsets are 32-bit
     if ((uint64_t)G::NT16 * (uint64_t)(k / 256) * G::TB >= (1ull << 32)) return hipErrorInvalidValue;
     static const hipError_t attr =
-        hipFuncSetAttribute((const void *)gemm_kq_kernel<DT>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        hipFuncSetAttribute((const void *)gemm_kq_kernel<DT, WGM_>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (attr != hipSuccess) return attr;
     const int nbn = (int)((n + G::BN - 1) / G::BN), nbm = (int)((m + BM - 1) / BM);
     const dim3 grid((unsigned)(nbn * nbm)), block(256);
     const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
     const int vec_out = ((uintptr_t)y % 16 == 0 && ((uint64_t)ldy * es) % 16 == 0 && n % 8 == 0) ? 1 : 0;
     if (ev_start) {
-        hipExtLaunchKernelGGL(gemm_kq_kernel<DT>, grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
+        hipExtLaunchKernelGGL((gemm_kq_kernel<DT, WGM_>), grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
                               (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale);
     } else {
-        gemm_kq_kernel<DT><<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype, ldy,
-                                                               bias, nbn, nbm, vec_out, wscale, 1.0f / wscale);
+        gemm_kq_kernel<DT, WGM_><<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype,
+                                                                      ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale);
     }
     return hipGetLastError();
 }
@@ -716,11 +728,16 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
                                  hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (n == 0 || m == 0) return hipSuccess;
     if (k <= 0 || k % 256 != 0 || !(wscale >= 6.103515625e-5f && wscale <= 32768.0f)) return hipErrorInvalidValue;
+    static const bool tall = getenv("TURQ_GEMM_GRID_2X2") == nullptr;  // Q5_K / Q6_K: 1 x 4 waves unless told otherwise
     switch (dtype) {
-    case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-    case TURQ_Q5_K: return launch_gemm<TURQ_Q5_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-    case TURQ_Q6_K: return launch_gemm<TURQ_Q6_K>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-    case TURQ_Q8_0: return launch_gemm<TURQ_Q8_0>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+    case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+    case TURQ_Q5_K:
+        if (tall) return launch_gemm<TURQ_Q5_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+        return launch_gemm<TURQ_Q5_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+    case TURQ_Q6_K:
+        if (tall) return launch_gemm<TURQ_Q6_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+        return launch_gemm<TURQ_Q6_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+    case TURQ_Q8_0: return launch_gemm<TURQ_Q8_0, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
     default: return hipErrorInvalidValue;
     }
 }
