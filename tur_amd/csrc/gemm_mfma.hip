@@ -90,10 +90,9 @@ template <> struct GFmtWN<TURQ_Q8_0> { static constexpr int value = 1; };
 
 // geometry that depends on the format and the wave grid: WGM x WGN waves, WM x WN 32x32 tiles per wave
 template <int DT, int WGM_> struct Geo {
-    static_assert(WGM_ == 1 || (WGM_ == 2), "wave grid 2 x 2 or 1 x 4");
-    static_assert(WGM_ == 2 || GFmtWN<DT>::value % 2 == 0, "the 1 x 4 grid halves the format's tiles per wave along n");
+    static_assert(WGM_ == 1 || WGM_ == 2, "wave grid 2 x 2 or 1 x 4");
     static constexpr int WGM = WGM_, WGN = 4 / WGM_, WM = MT / WGM_;
-    static constexpr int WN = WGM_ == 2 ? GFmtWN<DT>::value : GFmtWN<DT>::value / 2;
+    static constexpr int WN = WGM_ == 2 ? GFmtWN<DT>::value : 1;  // 1 x 4 waves: 128 rows of n, whatever the format
     static constexpr int BN = WGN * WN * 32;
     static constexpr int NT16 = BN / 16;                           // 16-row weight tiles per workgroup
     static constexpr int TB = TiledFmt<DT>::kTileBytes;
@@ -722,15 +721,21 @@ hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, i
 }  // namespace
 
 // frags: activations prepared by turq_launch_act_prep32 (in the order of the same dtype) for all m rows
-// wscale: a power of two in [2^-14, 2^15] by which the kernel multiplies every block scale (see turq_gemm_weight_scale)
+// wscale: a power of two in [2^-14, 2^15] by which the kernel multiplies every block scale; compute_units: CUs of the device
+// (0: unknown), for the choice of the tile shape
 hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
-                                 int y_dtype, int64_t ldy, const float *bias, float wscale, hipStream_t stream,
+                                 int y_dtype, int64_t ldy, const float *bias, float wscale, int compute_units, hipStream_t stream,
                                  hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (n == 0 || m == 0) return hipSuccess;
     if (k <= 0 || k % 256 != 0 || !(wscale >= 6.103515625e-5f && wscale <= 32768.0f)) return hipErrorInvalidValue;
     static const bool tall = getenv("TURQ_GEMM_GRID_2X2") == nullptr;  // Q5_K / Q6_K: 1 x 4 waves unless told otherwise
     switch (dtype) {
-    case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+    case TURQ_Q4_K:
+        // 128 x 192 tiles of 2 x 2 waves, unless the 128 x 128 tiles of the 1 x 4 grid still fit the machine in one round:
+        // then there are half as many again to spread (m = 128: 96 workgroups instead of 64, 34 us instead of 45)
+        if (compute_units > 0 && ((n + 127) / 128) * ((m + BM - 1) / BM) <= compute_units)
+            return launch_gemm<TURQ_Q4_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+        return launch_gemm<TURQ_Q4_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
     case TURQ_Q5_K:
         if (tall) return launch_gemm<TURQ_Q5_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
         return launch_gemm<TURQ_Q5_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);

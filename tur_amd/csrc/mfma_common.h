@@ -168,5 +168,5 @@ hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int 
                                        int64_t k, const void *x, int x_dtype, void *const *y, int y_dtype, const float *const *bias,
                                        int waves_per_group, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
 hipError_t turq_launch_gemm_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
-                                 int y_dtype, int64_t ldy, const float *bias, float wscale, hipStream_t stream,
+                                 int y_dtype, int64_t ldy, const float *bias, float wscale, int compute_units, hipStream_t stream,
                                  hipEvent_t ev_start, hipEvent_t ev_stop);

@@ -77,7 +77,7 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
         TURQ_HIP(ctx, turq_launch_act_prep32(w->dtype, x, xt, m, w->k, ldx, ctx->act_prep, ctx->stream));
         TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
-        TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, wscale, ctx->stream, ev0, ev1));
+        TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, wscale, ctx->compute_units, ctx->stream, ev0, ev1));
         return TURQ_OK;
     }
     const int nwaves = pick_waves(ctx, w->n, w->k);
