@@ -369,6 +369,43 @@ def test_two_formats_in_one_row_launch(gpu, dts, k):
         gpu.release(w)
 
 
+@pytest.mark.parametrize("dt", ALL)
+def test_two_rows_on_a_large_weight(gpu, dt):
+    # two activation rows on a weight of more than 8 MiB go through the one-row kernel's two-row form (no preparation launch);
+    # smaller weights and more rows take the general kernel
+    n, k = 4096, 4096 + (96 if dt == Q8_0 else 0)
+    raw = synth.random_weight(dt, n, k, seed=dt)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    x = synth.random_activation(2, k, seed=5)
+    bias = np.random.default_rng(2).standard_normal(n).astype(np.float32)
+    y = gpu.qmatmul(w, x, n, k, bias=bias, ldx=k + 4, ldy=n + 5)
+    want = orc.matmul_dequant(dt, f16_round(x), raw, n, k) + bias
+    assert rel_l2(y, want) <= 2e-5
+    for m in (1, 3):       # the rows are independent of each other: row i of any batch equals the one-row result
+        ym = gpu.qmatmul(w, np.concatenate([x, x])[:m], n, k, bias=bias)
+        assert rel_l2(ym, want[:1] if m == 1 else np.concatenate([want, want])[:m]) <= 2e-5
+    xb = synth.random_activation(2, k, seed=6, bf16=True)
+    yb = gpu.qmatmul(w, xb, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16)
+    assert rel_l2(yb, orc.matmul_dequant(dt, xb, raw, n, k)) <= 4e-3      # bf16 store
+    gpu.release(w)
+
+
+def test_two_rows_two_formats(gpu):
+    # q, k (Q4_K) and v (Q6_K) against two activation rows: one launch of the two-format kernel
+    k, ns, dts = 4096, [4096, 1024, 1000], (Q4_K, Q4_K, Q6_K)
+    raws = [synth.random_weight(dt, n, k, seed=n + i) for i, (dt, n) in enumerate(zip(dts, ns))]
+    ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
+    x = synth.random_activation(2, k, seed=8, bf16=True)
+    for x_dtype in (capi.ACT_F32, capi.ACT_BF16):
+        ys = gpu.qmatmul_multi(ws, x, ns, k, x_dtype=x_dtype)
+        for dt, n, raw, w, y in zip(dts, ns, raws, ws, ys):
+            assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, k)) <= 2e-5, (dt, n)
+            # (the single call of a small weight takes another kernel: equal up to the order of the sums)
+            assert rel_l2(y, gpu.qmatmul(w, x, n, k, x_dtype=x_dtype)) <= 1e-5, (dt, n)
+    for w in ws:
+        gpu.release(w)
+
+
 def test_multi_weight_falls_back_to_single_calls(gpu):
     # more than 32 rows, or host pointers: the same as the calls one after the other
     k, ns, dts = 512, [48, 80], (Q4_K, Q4_K)

@@ -68,6 +68,7 @@ template <int XT> struct X1Regs { uint32_t r[XT == TURQ_ACT_F32 ? 4 : 2]; };
 // multiple of 256 and needs no test
 template <int XT, bool RAGGED>
 __device__ inline X1Regs<XT> load_x1(const void *__restrict__ x, int64_t k, int64_t b, int lane, const GOff &o) {
+    // x: the activation row (wave-uniform pointer)
     X1Regs<XT> v;
     constexpr int ES = XT == TURQ_ACT_F32 ? 4 : 2;
     const bool ok = !RAGGED || b * 256 + 4 * lane < k;
@@ -156,15 +157,20 @@ template <int DT> struct Row1K45 {
         }
         return make_half8(as_half2(t0), as_half2(t1), as_half2(t2), as_half2(t3));
     }
-    __device__ static float4v chain(const W &w, const uint8_t *reg, const Lane &l, int g) {
-        float4v c = *(const float4v *)(reg + kInit + 16 * g);
+    // M activation rows: their regions follow each other; every operand is unpacked once and used for all of them
+    template <int M> __device__ static void chain(const W &w, const uint8_t *reg, const Lane &l, int g, float4v *c) {
+#pragma unroll
+        for (int mm = 0; mm < M; mm++) c[mm] = *(const float4v *)(reg + mm * kRegion + kInit + 16 * g);
         const uint32_t wq[8] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w, w.qb.x, w.qb.y, w.qb.z, w.qb.w};
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const half8v av = *(const half8v *)(reg + (i < 4 ? l.offA : l.offB) + 16 * (i & 3));
-            c = mfma16x16x32(av, operand(wq[i], w.hh.x, w.hh.y, 2 * i), c);
+            const half8v bop = operand(wq[i], w.hh.x, w.hh.y, 2 * i);
+#pragma unroll
+            for (int mm = 0; mm < M; mm++) {
+                const half8v av = *(const half8v *)(reg + mm * kRegion + (i < 4 ? l.offA : l.offB) + 16 * (i & 3));
+                c[mm] = mfma16x16x32(av, bop, c[mm]);
+            }
         }
-        return c;
     }
     struct Sc { half2v sc, mn, dd; };  // (sc, sc'), (m, m'), (d, dmin)
     __device__ static Sc scales(const W &w, const Lane &l) {
@@ -209,8 +215,9 @@ template <> struct Row1Fmt<TURQ_Q6_K> {
         const float nb = sum4(dot2(h23, (_Float16)-288.0f, dot2(h01, (_Float16)-288.0f, 0.0f)));
         if ((lane & 3) == 0) *(float *)(region + kInit + lane) = nb;
     }
-    __device__ static float4v chain(const W &w, const uint8_t *reg, const Lane &l, int g) {
-        float4v c = *(const float4v *)(reg + kInit + 16 * g);
+    template <int M> __device__ static void chain(const W &w, const uint8_t *reg, const Lane &l, int g, float4v *c) {
+#pragma unroll
+        for (int mm = 0; mm < M; mm++) c[mm] = *(const float4v *)(reg + mm * kRegion + kInit + 16 * g);
         const uint32_t wl[8] = {w.qla.x, w.qla.y, w.qla.z, w.qla.w, w.qlb.x, w.qlb.y, w.qlb.z, w.qlb.w};
         const uint32_t wh[4] = {w.qh.x, w.qh.y, w.qh.z, w.qh.w};
 #pragma unroll
@@ -225,10 +232,13 @@ template <> struct Row1Fmt<TURQ_Q6_K> {
                 const uint32_t hi = rh ? rotr32(wh[i >> 1], rh) : wh[i >> 1];
                 v[t] = and_or_u32(hi, 0x00C000C0u, and_or_u32(lo, 0x003C003Cu, kMagic256));
             }
-            const half8v av = *(const half8v *)(reg + l.off[i >> 1] + 16 * (i & 1));
-            c = mfma16x16x32(av, make_half8(as_half2(v[0]), as_half2(v[1]), as_half2(v[2]), as_half2(v[3])), c);
+            const half8v bop = make_half8(as_half2(v[0]), as_half2(v[1]), as_half2(v[2]), as_half2(v[3]));
+#pragma unroll
+            for (int mm = 0; mm < M; mm++) {
+                const half8v av = *(const half8v *)(reg + mm * kRegion + l.off[i >> 1] + 16 * (i & 1));
+                c[mm] = mfma16x16x32(av, bop, c[mm]);
+            }
         }
-        return c;
     }
     struct Sc { float s[4]; float d; };
     __device__ static Sc scales(const W &w, const Lane &) {
@@ -271,18 +281,21 @@ template <> struct Row1Fmt<TURQ_Q8_0> {
         const float nb = sum8(dot2(h23, (_Float16)-1152.0f, dot2(h01, (_Float16)-1152.0f, 0.0f)));
         if ((lane & 7) == 0) *(float *)(region + kInit + (lane >> 1)) = nb;
     }
-    __device__ static float4v chain(const W &w, const uint8_t *reg, const Lane &l, int g) {
-        float4v c = *(const float4v *)(reg + kInit + 16 * g);
+    template <int M> __device__ static void chain(const W &w, const uint8_t *reg, const Lane &l, int g, float4v *c) {
+#pragma unroll
+        for (int mm = 0; mm < M; mm++) c[mm] = *(const float4v *)(reg + mm * kRegion + kInit + 16 * g);
 #pragma unroll
         for (int q = 0; q < 8; q++) {
             const uint32_t w0 = (q & 1) ? w.p[q >> 1].z : w.p[q >> 1].x;
             const uint32_t w1 = (q & 1) ? w.p[q >> 1].w : w.p[q >> 1].y;
             const half8v bop = make_half8(as_half2(and_or_u32(w0, 0x00FF00FFu, kMagic1024)), as_half2(and_or_u32(w0 >> 8, 0x00FF00FFu, kMagic1024)),
                                           as_half2(and_or_u32(w1, 0x00FF00FFu, kMagic1024)), as_half2(and_or_u32(w1 >> 8, 0x00FF00FFu, kMagic1024)));
-            const half8v av = *(const half8v *)(reg + l.off[q]);
-            c = mfma16x16x32(av, bop, c);
+#pragma unroll
+            for (int mm = 0; mm < M; mm++) {
+                const half8v av = *(const half8v *)(reg + mm * kRegion + l.off[q]);
+                c[mm] = mfma16x16x32(av, bop, c[mm]);
+            }
         }
-        return c;
     }
     struct Sc { half2v d01, d23; };
     __device__ static Sc scales(const W &w, const Lane &) { return Sc{as_half2(w.dd.x), as_half2(w.dd.y)}; }
@@ -305,21 +318,22 @@ struct Row1Args {
     const uint8_t *w[kMaxRow1];
     void *y[kMaxRow1];
     const float *bias[kMaxRow1];
-    int64_t n[kMaxRow1];
+    int64_t n[kMaxRow1], ldy[kMaxRow1];
     int first[kMaxRow1];
     int count;
     int second;  // two-format launches: weights [0, second) are of the first format, [second, count) of the second
 };
 
-// the work of one workgroup: row tiles rtb * R .. rtb * R + R - 1 of one weight.
+// the work of one workgroup: row tiles rtb * R .. rtb * R + R - 1 of one weight, against m <= M activation rows.
 // P = column tiles a wave keeps in flight; R = row tiles per workgroup (a wave stages the activations of a column tile once and
-// uses them for R weight tiles)
-template <int DT, int XT, int P, int R>
-__device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *__restrict__ y, const float *__restrict__ bias,
-                                          int64_t n, int64_t rtb, int64_t k, const void *__restrict__ x, int yt) {
+// uses them for R weight tiles); M = activation rows the instantiation holds (rows past m repeat row 0 and are not stored)
+template <int DT, int XT, int P, int R, int M>
+__device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *__restrict__ y, int64_t ldy, const float *__restrict__ bias,
+                                          int64_t n, int64_t rtb, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt) {
     extern __shared__ uint8_t smem[];
     using Fmt = Row1Fmt<DT>;
     constexpr int TB = TiledFmt<DT>::kTileBytes;
+    constexpr int ES = XT == TURQ_ACT_F32 ? 4 : 2;
     const int64_t rt0 = rtb * R, nrt = turq_tile_rows(n);
 
     const int lane = threadIdx.x & 63;
@@ -327,31 +341,36 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
     const int nwaves = blockDim.x >> 6;
     const int g = lane >> 4;
     const int64_t ntc = turq_tile_cols(k);
-    uint8_t *region = smem + (size_t)wave * (P * kRegion);
-    float *red = (float *)(smem + (size_t)nwaves * (P * kRegion));
+    uint8_t *region = smem + (size_t)wave * (P * M * kRegion);  // [p][activation row]
+    float *red = (float *)(smem + (size_t)nwaves * (P * M * kRegion));
 
     // the zeros that the idle A rows read, and start values that no format overwrites
     if (lane < 32)
 #pragma unroll
-        for (int p = 0; p < P; p++) *(float *)(region + p * kRegion + kInit + 4 * lane) = 0.0f;  // float like the later writes
+        for (int p = 0; p < P * M; p++) *(float *)(region + p * kRegion + kInit + 4 * lane) = 0.0f;  // float like the later writes
     const typename Fmt::Lane lc = Fmt::lane_init(lane & 15, g);
     GOff go{16u * (uint32_t)lane, 8u * (uint32_t)lane, 4u * (uint32_t)lane, 16u * (uint32_t)(lane & 15), Fmt::aux_off(lane & 15, g), 0u};
 
-    float acc[R];
+    float acc[R][M];
     const uint8_t *wrow[R];  // row tiles past the weight's last one re-read it; their results are not stored
+    const uint8_t *xrow[M];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        acc[r] = 0.0f;
+#pragma unroll
+        for (int mm = 0; mm < M; mm++) acc[r][mm] = 0.0f;
         wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
     }
+#pragma unroll
+    for (int mm = 0; mm < M; mm++) xrow[mm] = (const uint8_t *)x + (mm < m ? mm : 0) * ldx * ES;
     for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
-        X1Regs<XT> xr[P];
+        X1Regs<XT> xr[P][M];
         typename Fmt::W wr[P][R];
         go.touch();
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int64_t b = b0 + (int64_t)p * nwaves;
-            xr[p] = load_x1<XT, DT == TURQ_Q8_0>(x, k, b < ntc ? b : b0, lane, go);
+#pragma unroll
+            for (int mm = 0; mm < M; mm++) xr[p][mm] = load_x1<XT, DT == TURQ_Q8_0>(xrow[mm], k, b < ntc ? b : b0, lane, go);
         }
 #pragma unroll
         for (int p = 0; p < P; p++) {
@@ -360,7 +379,9 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
             for (int r = 0; r < R; r++) wr[p][r] = Fmt::load(wrow[r] + (b < ntc ? b : b0) * TB, go);
         }
 #pragma unroll
-        for (int p = 0; p < P; p++) stage_x1<DT, XT>(xr[p], region + p * kRegion, lane);
+        for (int p = 0; p < P; p++)
+#pragma unroll
+            for (int mm = 0; mm < M; mm++) stage_x1<DT, XT>(xr[p][mm], region + (p * M + mm) * kRegion, lane);
         // same-wave LDS traffic is processed in order; the fences keep the compiler from reordering
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -371,127 +392,175 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
             if (b >= ntc) continue;  // uniform per wave
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                float4v c = Fmt::chain(wr[p][r], region + p * kRegion, lc, g);
+                float4v c[M];
+                Fmt::template chain<M>(wr[p][r], region + p * M * kRegion, lc, g, c);
                 // One tile after the other.  Left free, the scheduler interleaves the tiles' chains and scale arithmetic, the
                 // unpacked operands of several tiles are live at once and the 128 registers a wave of a 16-wave workgroup may
                 // use overflow (spills in the instantiations with four tiles per workgroup pass; the 510 MB LM head lost
-                // 20 %).  The
-                // empty asm consumes the chain's result; vector and matrix instructions may not cross the barrier.
-                asm volatile("" : "+v"(c));
+                // 20 %).  The empty asm consumes the chains' results; vector and matrix instructions may not cross the barrier.
+#pragma unroll
+                for (int mm = 0; mm < M; mm++) asm volatile("" : "+v"(c[mm]));
                 __builtin_amdgcn_sched_barrier(0x10 | 0x80 | 0x4);
-                acc[r] += Fmt::finish(Fmt::scales(wr[p][r], lc), c);
+                const typename Fmt::Sc sc = Fmt::scales(wr[p][r], lc);
+#pragma unroll
+                for (int mm = 0; mm < M; mm++) acc[r][mm] += Fmt::finish(sc, c[mm]);
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     }
 
-    // y[16 rt + n] = sum over lane groups and waves; wave r adds up row tile r
+    // y[mm][16 rt + n] = sum over lane groups and waves; wave i adds up the i-th (row tile, activation row) pair
 #pragma unroll
-    for (int r = 0; r < R; r++) red[(r * nwaves + wave) * 64 + lane] = acc[r];
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int mm = 0; mm < M; mm++) red[((r * M + mm) * nwaves + wave) * 64 + lane] = acc[r][mm];
     __syncthreads();
     const int n4 = lane >> 2, q = lane & 3;
-    for (int r = wave; r < R; r += nwaves) {
+    for (int i = wave; i < R * M; i += nwaves) {
+        const int r = i / M, mm = i - r * M;
         float s = 0.0f;
-        for (int wv = 0; wv < nwaves; wv++) s += red[(r * nwaves + wv) * 64 + n4 + 16 * q];
+        for (int wv = 0; wv < nwaves; wv++) s += red[(i * nwaves + wv) * 64 + n4 + 16 * q];
         s = sum4(s);
         const int64_t col = (rt0 + r) * 16 + n4;
-        if (q == 0 && rt0 + r < nrt && col < n) {
+        if (q == 0 && rt0 + r < nrt && col < n && mm < m) {
             const float out = s + (bias ? bias[col] : 0.0f);
-            if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, col, out);
-            else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, col, out);
-            else turq_store_out<TURQ_ACT_F16>(y, col, out);
+            const int64_t at = (int64_t)mm * ldy + col;
+            if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, at, out);
+            else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, at, out);
+            else turq_store_out<TURQ_ACT_F16>(y, at, out);
         }
     }
 }
 
 // which weight of the launch this workgroup works on
-struct Row1Pick { const uint8_t *w; void *y; const float *bias; int64_t n; int first; int index; };
+struct Row1Pick { const uint8_t *w; void *y; const float *bias; int64_t n, ldy; int first; int index; };
 __device__ inline Row1Pick row1_pick(const Row1Args &a, int blk) {
-    Row1Pick p{a.w[0], a.y[0], a.bias[0], a.n[0], 0, 0};
+    Row1Pick p{a.w[0], a.y[0], a.bias[0], a.n[0], a.ldy[0], 0, 0};
 #pragma unroll
     for (int i = 1; i < kMaxRow1; i++)
-        if (i < a.count && blk >= a.first[i]) p = Row1Pick{a.w[i], a.y[i], a.bias[i], a.n[i], a.first[i], i};
+        if (i < a.count && blk >= a.first[i]) p = Row1Pick{a.w[i], a.y[i], a.bias[i], a.n[i], a.ldy[i], a.first[i], i};
     return p;
 }
 
-// MAXT = largest workgroup of the instantiation
-template <int DT, int XT, int P, int R, int MAXT>
-__global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int yt) {
+// m <= M activation rows of stride ldx; MAXT = largest workgroup of the instantiation
+template <int DT, int XT, int P, int R, int M, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt) {
     const Row1Pick p = row1_pick(a, (int)blockIdx.x);
-    row1_body<DT, XT, P, R>(p.w, p.y, p.bias, p.n, (int64_t)((int)blockIdx.x - p.first), k, x, yt);
+    row1_body<DT, XT, P, R, M>(p.w, p.y, p.ldy, p.bias, p.n, (int64_t)((int)blockIdx.x - p.first), k, x, ldx, m, yt);
 }
 
 // weights of two formats that share an input (q, k Q4_K and v Q6_K of a Q4_K_M file) in one launch: the workgroup's weight
 // decides which body runs
-template <int DTA, int DTB, int XT, int P, int MAXT>
-__global__ void __launch_bounds__(MAXT) gemv_row1_mixed_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int yt) {
+template <int DTA, int DTB, int XT, int P, int M, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_row1_mixed_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int64_t ldx, int m,
+                                                                int yt) {
     const Row1Pick p = row1_pick(a, (int)blockIdx.x);
     const int64_t rtb = (int64_t)((int)blockIdx.x - p.first);
-    if (p.index < a.second) row1_body<DTA, XT, P, 1>(p.w, p.y, p.bias, p.n, rtb, k, x, yt);
-    else row1_body<DTB, XT, P, 1>(p.w, p.y, p.bias, p.n, rtb, k, x, yt);
+    if (p.index < a.second) row1_body<DTA, XT, P, 1, M>(p.w, p.y, p.ldy, p.bias, p.n, rtb, k, x, ldx, m, yt);
+    else row1_body<DTB, XT, P, 1, M>(p.w, p.y, p.ldy, p.bias, p.n, rtb, k, x, ldx, m, yt);
 }
 
-template <int DT, int XT, int P, int R, int MAXT>
-hipError_t launch_final(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
-                        hipEvent_t ev1) {
-    const size_t lds = (size_t)nwaves * P * kRegion + (size_t)nwaves * R * 64 * sizeof(float);
-    if (ev0) {
-        hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, R, MAXT>), dim3((unsigned)blocks), dim3((unsigned)(64 * nwaves)), (unsigned)lds,
-                              s, ev0, ev1, 0, a, k, x, yt);
+struct Row1Launch {
+    Row1Args a;
+    int blocks;
+    int64_t k;
+    const void *x;
+    int64_t ldx;
+    int m, yt, nwaves, rtiles;
+    hipStream_t s;
+    hipEvent_t ev0, ev1;
+};
+
+template <int P, int R, int M> size_t row1_lds(int nwaves) {
+    return (size_t)nwaves * P * M * kRegion + (size_t)nwaves * R * M * 64 * sizeof(float);
+}
+
+template <int DT, int XT, int P, int R, int M>
+hipError_t launch_final(const Row1Launch &l) {
+    const size_t lds = row1_lds<P, R, M>(l.nwaves);
+    const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
+    if (l.ev0) {
+        hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, R, M, 1024>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k, l.x,
+                              l.ldx, l.m, l.yt);
         return hipGetLastError();
     }
-    gemv_row1_kernel<DT, XT, P, R, MAXT><<<(unsigned)blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(a, k, x, yt);
+    gemv_row1_kernel<DT, XT, P, R, M, 1024><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
     return hipGetLastError();
 }
 
-template <int DT, int XT>
-hipError_t launch_p(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, int rtiles, hipStream_t s,
-                    hipEvent_t ev0, hipEvent_t ev1) {
+// column tiles in flight per wave: up to three for one activation row (four do not fit the registers of every format), up to
+// two for several rows, whose raw activations are held next to the weights until they are staged
+inline int row1_in_flight(int64_t k, int nwaves, int m) {
     static const int forced = [] { const char *e = getenv("TURQ_ROW1_P"); return e ? atoi(e) : 0; }();
     const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
-    int p = (int)(per_wave < 3 ? per_wave : 3);  // four tiles in flight do not fit the registers of every format
-    if (forced >= 1 && forced <= 3) p = forced;
-    if (rtiles == 2) {  // two row tiles double the weights a wave holds: at most two column tiles in flight
-        if (p == 1) return launch_final<DT, XT, 1, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-        return launch_final<DT, XT, 2, 2, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    }
-    if (p == 1) return launch_final<DT, XT, 1, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    if (p == 2) return launch_final<DT, XT, 2, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    return launch_final<DT, XT, 3, 1, 1024>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+    const int most = m > 1 ? 2 : 3;
+    int p = (int)(per_wave < most ? per_wave : most);
+    if (forced >= 1 && forced <= most) p = forced;
+    return p;
+}
+
+template <int DT, int XT>
+hipError_t launch_p(const Row1Launch &l) {
+    const int p = row1_in_flight(l.k, l.nwaves, l.m);
+    static_assert(TURQ_ROW1_MAX_M == 2, "instantiations for one and two activation rows");
+    if (l.m == 2) return p == 1 ? launch_final<DT, XT, 1, 1, 2>(l) : launch_final<DT, XT, 2, 1, 2>(l);
+    if (l.rtiles == 2)  // two row tiles double the weights a wave holds: at most two column tiles in flight
+        return p == 1 ? launch_final<DT, XT, 1, 2, 1>(l) : launch_final<DT, XT, 2, 2, 1>(l);
+    if (p == 1) return launch_final<DT, XT, 1, 1, 1>(l);
+    if (p == 2) return launch_final<DT, XT, 2, 1, 1>(l);
+    return launch_final<DT, XT, 3, 1, 1>(l);
 }
 
 template <int DT>
-hipError_t launch_x(int xt, const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, int rtiles, hipStream_t s,
-                    hipEvent_t ev0, hipEvent_t ev1) {
+hipError_t launch_x(int xt, const Row1Launch &l) {
     switch (xt) {
-    case TURQ_ACT_F32: return launch_p<DT, TURQ_ACT_F32>(a, blocks, k, x, yt, nwaves, rtiles, s, ev0, ev1);
-    case TURQ_ACT_BF16: return launch_p<DT, TURQ_ACT_BF16>(a, blocks, k, x, yt, nwaves, rtiles, s, ev0, ev1);
-    case TURQ_ACT_F16: return launch_p<DT, TURQ_ACT_F16>(a, blocks, k, x, yt, nwaves, rtiles, s, ev0, ev1);
+    case TURQ_ACT_F32: return launch_p<DT, TURQ_ACT_F32>(l);
+    case TURQ_ACT_BF16: return launch_p<DT, TURQ_ACT_BF16>(l);
+    case TURQ_ACT_F16: return launch_p<DT, TURQ_ACT_F16>(l);
     default: return hipErrorInvalidValue;
     }
 }
 
-template <int DTA, int DTB, int XT, int P>
-hipError_t launch_mixed_final(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
-                              hipEvent_t ev1) {
-    const size_t lds = (size_t)nwaves * P * kRegion + (size_t)nwaves * 64 * sizeof(float);
-    if (ev0) {
-        hipExtLaunchKernelGGL((gemv_row1_mixed_kernel<DTA, DTB, XT, P, 1024>), dim3((unsigned)blocks), dim3((unsigned)(64 * nwaves)),
-                              (unsigned)lds, s, ev0, ev1, 0, a, k, x, yt);
+template <int DTA, int DTB, int XT, int P, int M>
+hipError_t launch_mixed_final(const Row1Launch &l) {
+    const size_t lds = row1_lds<P, 1, M>(l.nwaves);
+    const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
+    if (l.ev0) {
+        hipExtLaunchKernelGGL((gemv_row1_mixed_kernel<DTA, DTB, XT, P, M, 1024>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a,
+                              l.k, l.x, l.ldx, l.m, l.yt);
         return hipGetLastError();
     }
-    gemv_row1_mixed_kernel<DTA, DTB, XT, P, 1024><<<(unsigned)blocks, dim3((unsigned)(64 * nwaves)), lds, s>>>(a, k, x, yt);
+    gemv_row1_mixed_kernel<DTA, DTB, XT, P, M, 1024><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
     return hipGetLastError();
 }
 
 template <int DTA, int DTB, int XT>
-hipError_t launch_mixed_p(const Row1Args &a, int blocks, int64_t k, const void *x, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
-                          hipEvent_t ev1) {
-    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
-    if (per_wave <= 1) return launch_mixed_final<DTA, DTB, XT, 1>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    if (per_wave == 2) return launch_mixed_final<DTA, DTB, XT, 2>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
-    return launch_mixed_final<DTA, DTB, XT, 3>(a, blocks, k, x, yt, nwaves, s, ev0, ev1);
+hipError_t launch_mixed_p(const Row1Launch &l) {
+    const int p = row1_in_flight(l.k, l.nwaves, l.m);
+    if (l.m == 2) return p == 1 ? launch_mixed_final<DTA, DTB, XT, 1, 2>(l) : launch_mixed_final<DTA, DTB, XT, 2, 2>(l);
+    if (p == 1) return launch_mixed_final<DTA, DTB, XT, 1, 1>(l);
+    if (p == 2) return launch_mixed_final<DTA, DTB, XT, 2, 1>(l);
+    return launch_mixed_final<DTA, DTB, XT, 3, 1>(l);
+}
+
+// fills the argument block; returns false for arguments no launch accepts
+bool row1_args(Row1Launch &l, int count, const void *const *w, const int64_t *n, void *const *y, const int64_t *ldy,
+               const float *const *bias, int row_tiles) {
+    int64_t blocks = 0;
+    for (int i = 0; i < count; i++) {
+        l.a.w[i] = (const uint8_t *)w[i];
+        l.a.y[i] = y[i];
+        l.a.bias[i] = bias ? bias[i] : nullptr;
+        l.a.n[i] = n[i];
+        l.a.ldy[i] = ldy ? ldy[i] : n[i];
+        l.a.first[i] = (int)blocks;
+        blocks += (turq_tile_rows(n[i]) + row_tiles - 1) / row_tiles;
+    }
+    l.a.count = count;
+    if (blocks > 0x7FFFFFFF) return false;
+    l.blocks = (int)blocks;
+    return true;
 }
 
 }  // namespace
@@ -500,64 +569,52 @@ bool turq_gemv_row1_supports(int dtype) {
     return dtype == TURQ_Q4_K || dtype == TURQ_Q5_K || dtype == TURQ_Q6_K || dtype == TURQ_Q8_0;
 }
 
-// count (1..4) weights of one format and one k against ONE activation row x (16-byte aligned); row_tiles (1 or 2) per workgroup.
+// count (1..4) weights of one format and one k against m (1..TURQ_ROW1_MAX_M) activation rows of stride ldx (rows 16-byte
+// aligned); results to y[i] with row stride ldy[i] (null: n[i]); row_tiles (1 or 2; 2 with one activation row only) per workgroup.
 hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, const int64_t *n, int64_t k, const void *x, int x_dtype,
-                                 void *const *y, int y_dtype, const float *const *bias, int nwaves, int row_tiles, hipStream_t stream,
-                                 hipEvent_t ev_start, hipEvent_t ev_stop) {
+                                 int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy, const float *const *bias,
+                                 int nwaves, int row_tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (count < 1 || count > kMaxRow1 || nwaves < 1 || nwaves > 16 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
-    if (row_tiles != 1 && row_tiles != 2) return hipErrorInvalidValue;
+    if (m < 1 || m > TURQ_ROW1_MAX_M || (row_tiles != 1 && !(row_tiles == 2 && m == 1))) return hipErrorInvalidValue;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
-    Row1Args a{};
-    int64_t blocks = 0;
-    for (int i = 0; i < count; i++) {
-        a.w[i] = (const uint8_t *)w[i];
-        a.y[i] = y[i];
-        a.bias[i] = bias ? bias[i] : nullptr;
-        a.n[i] = n[i];
-        a.first[i] = (int)blocks;
-        blocks += (turq_tile_rows(n[i]) + row_tiles - 1) / row_tiles;
-    }
-    a.count = count;
-    if (blocks == 0) return hipSuccess;
-    if (k == 0 || blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    Row1Launch l{};
+    if (!row1_args(l, count, w, n, y, ldy, bias, row_tiles)) return hipErrorInvalidValue;
+    if (l.blocks == 0) return hipSuccess;
+    if (k == 0) return hipErrorInvalidValue;
+    l.k = k, l.x = x, l.ldx = ldx, l.m = (int)m, l.yt = y_dtype, l.nwaves = nwaves, l.rtiles = row_tiles;
+    l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop;
     switch (dtype) {
-    case TURQ_Q4_K: return launch_x<TURQ_Q4_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
-    case TURQ_Q5_K: return launch_x<TURQ_Q5_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
-    case TURQ_Q6_K: return launch_x<TURQ_Q6_K>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
-    case TURQ_Q8_0: return launch_x<TURQ_Q8_0>(x_dtype, a, (int)blocks, k, x, y_dtype, nwaves, row_tiles, stream, ev_start, ev_stop);
+    case TURQ_Q4_K: return launch_x<TURQ_Q4_K>(x_dtype, l);
+    case TURQ_Q5_K: return launch_x<TURQ_Q5_K>(x_dtype, l);
+    case TURQ_Q6_K: return launch_x<TURQ_Q6_K>(x_dtype, l);
+    case TURQ_Q8_0: return launch_x<TURQ_Q8_0>(x_dtype, l);
     default: return hipErrorInvalidValue;
     }
 }
 
 bool turq_gemv_row1_mixed_supports(int dtype_a, int dtype_b) { return dtype_a == TURQ_Q4_K && dtype_b == TURQ_Q6_K; }
 
-// count (2..4) weights of one k against ONE activation row: the first `second` of format dtype_a, the others of dtype_b
+// count (2..4) weights of one k against m activation rows: the first `second` of format dtype_a, the others of dtype_b
 // (a pair turq_gemv_row1_mixed_supports accepts); one row tile per workgroup.
 hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w, const int64_t *n,
-                                       int64_t k, const void *x, int x_dtype, void *const *y, int y_dtype, const float *const *bias,
-                                       int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+                                       int64_t k, const void *x, int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype,
+                                       const int64_t *ldy, const float *const *bias, int nwaves, hipStream_t stream,
+                                       hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (!turq_gemv_row1_mixed_supports(dtype_a, dtype_b) || count < 2 || count > kMaxRow1 || second < 1 || second >= count ||
-        nwaves < 1 || nwaves > 16 || k % 256 != 0)
+        nwaves < 1 || nwaves > 16 || k % 256 != 0 || m < 1 || m > TURQ_ROW1_MAX_M)
         return hipErrorInvalidValue;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
-    Row1Args a{};
-    int64_t blocks = 0;
-    for (int i = 0; i < count; i++) {
-        a.w[i] = (const uint8_t *)w[i];
-        a.y[i] = y[i];
-        a.bias[i] = bias ? bias[i] : nullptr;
-        a.n[i] = n[i];
-        a.first[i] = (int)blocks;
-        blocks += turq_tile_rows(n[i]);
-    }
-    a.count = count;
-    a.second = second;
-    if (blocks == 0) return hipSuccess;
-    if (k == 0 || blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    Row1Launch l{};
+    if (!row1_args(l, count, w, n, y, ldy, bias, 1)) return hipErrorInvalidValue;
+    l.a.second = second;
+    if (l.blocks == 0) return hipSuccess;
+    if (k == 0) return hipErrorInvalidValue;
+    l.k = k, l.x = x, l.ldx = ldx, l.m = (int)m, l.yt = y_dtype, l.nwaves = nwaves, l.rtiles = 1;
+    l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop;
     switch (x_dtype) {
-    case TURQ_ACT_F32: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_F32>(a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
-    case TURQ_ACT_BF16: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_BF16>(a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
-    case TURQ_ACT_F16: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_F16>(a, (int)blocks, k, x, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_ACT_F32: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_F32>(l);
+    case TURQ_ACT_BF16: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_BF16>(l);
+    case TURQ_ACT_F16: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_F16>(l);
     default: return hipErrorInvalidValue;
     }
 }

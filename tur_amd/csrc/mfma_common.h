@@ -154,10 +154,15 @@ hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w_til
                                   int x_dtype, int64_t ldx, int64_t m, bool fused, void *const *y, int y_dtype, const int64_t *ldy,
                                   const float *const *bias, int waves_per_group, int row_tiles_per_group, hipStream_t stream,
                                   hipEvent_t ev_start, hipEvent_t ev_stop);
+// Activation rows the one-row kernel takes in one launch.  The body is written for any number M (every unpacked operand feeds
+// M MFMAs); with four rows it is bound by its vector instructions (staging and scales per row) and loses 6 - 13 % to the
+// preparation launch + general kernel, with two it wins 5 - 12 % on matrices of tens of MB.
+#define TURQ_ROW1_MAX_M 2
 bool turq_gemv_row1_supports(int dtype);
 hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w_tiled, const int64_t *n, int64_t k, const void *x,
-                                 int x_dtype, void *const *y, int y_dtype, const float *const *bias, int waves_per_group,
-                                 int row_tiles_per_group, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
+                                 int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
+                                 const float *const *bias, int waves_per_group, int row_tiles_per_group, hipStream_t stream,
+                                 hipEvent_t ev_start, hipEvent_t ev_stop);
 bool turq_gemv_multi_mixed_supports(int dtype_a, int dtype_b);
 hipError_t turq_launch_gemv_multi_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w_tiled, const int64_t *n,
                                         int64_t k, const void *frags, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
@@ -165,8 +170,9 @@ hipError_t turq_launch_gemv_multi_mixed(int dtype_a, int dtype_b, int count, int
                                         hipEvent_t ev_stop);
 bool turq_gemv_row1_mixed_supports(int dtype_a, int dtype_b);
 hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w_tiled, const int64_t *n,
-                                       int64_t k, const void *x, int x_dtype, void *const *y, int y_dtype, const float *const *bias,
-                                       int waves_per_group, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
+                                       int64_t k, const void *x, int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype,
+                                       const int64_t *ldy, const float *const *bias, int waves_per_group, hipStream_t stream,
+                                       hipEvent_t ev_start, hipEvent_t ev_stop);
 hipError_t turq_launch_gemm_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
                                  int y_dtype, int64_t ldy, const float *bias, float wscale, int compute_units, hipStream_t stream,
                                  hipEvent_t ev_start, hipEvent_t ev_stop);

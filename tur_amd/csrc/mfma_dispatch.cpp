@@ -36,6 +36,14 @@ bool use_row1(int dtype) {
     return !off && turq_gemv_row1_supports(dtype);
 }
 
+// The one-row kernel stages the raw activations itself, once per wave and column tile, and needs no preparation launch.
+// One activation row: always.  Two: where the weights of the call are large enough for its launch to beat the fused general
+// kernel (measured: + 5 .. 12 % at 28 MB and more, - 10 % at 3 MB).  TURQ_ROW1_M = 1 keeps it to one row, for comparison.
+bool row1_takes(int64_t m, size_t weight_bytes) {
+    static const int most = [] { const char *e = getenv("TURQ_ROW1_M"); const int x = e ? atoi(e) : TURQ_ROW1_MAX_M; return x < 1 ? 1 : x > TURQ_ROW1_MAX_M ? TURQ_ROW1_MAX_M : x; }();
+    return m == 1 || (m <= most && weight_bytes >= (8u << 20));
+}
+
 // Waves per workgroup of the one-row kernel: it is light on registers and on vector work, so what it wants is many waves
 // with few column tiles each (two by default), up to the largest workgroup.
 int pick_waves_row1(int64_t k) {
@@ -88,17 +96,19 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
         static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
         // raw activation rows must be 16-byte (f32) / 8-byte (16-bit) aligned for the fused loads
         const bool aligned = ((uintptr_t)xc % 16 == 0) && ((size_t)ldx * xb) % 16 == 0;
+        if (aligned && !no_fuse && row1_takes(mc, w->dev_bytes) && use_row1(w->dtype)) {
+            hipEvent_t ev0 = nullptr, ev1 = nullptr;
+            TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+            const void *wp = w->dev;
+            void *yv = yc;
+            TURQ_HIP(ctx, turq_launch_gemv_row1(w->dtype, 1, &wp, &w->n, w->k, xc, xt, ldx, mc, &yv, yt, &ldy, bias ? &bias : nullptr,
+                                                pick_waves_row1(w->k), mc == 1 ? pick_rows_row1(ctx, turq_tile_rows(w->n)) : 1,
+                                                ctx->stream, ev0, ev1));
+            continue;
+        }
         if (use_fused(ctx, mc, turq_tile_rows(w->n), w->dev_bytes) && aligned && !no_fuse) {
             hipEvent_t ev0 = nullptr, ev1 = nullptr;
             TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
-            if (mc == 1 && use_row1(w->dtype)) {
-                const void *wp = w->dev;
-                void *yv = yc;
-                TURQ_HIP(ctx, turq_launch_gemv_row1(w->dtype, 1, &wp, &w->n, w->k, xc, xt, &yv, yt, bias ? &bias : nullptr,
-                                                    pick_waves_row1(w->k), pick_rows_row1(ctx, turq_tile_rows(w->n)), ctx->stream,
-                                                    ev0, ev1));
-                continue;
-            }
             TURQ_HIP(ctx, turq_launch_gemv_mfma(w->dtype, w->dev, w->n, w->k, xc, xt, ldx, mc, true, yc, yt, ldy, bias,
                                                 nwaves, ctx->stream, ev0, ev1));
             continue;
@@ -133,7 +143,8 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
         while (j < count && j - i < 4 && w[j]->dtype == w[i]->dtype) j++;
         // one activation row: a run of a second format joins the launch where the kernel has that pair (q, k Q4_K + v Q6_K)
         static const bool no_mixed = getenv("TURQ_GEMV_NO_MIXED") != nullptr;
-        if (fused && m == 1 && !no_mixed && j < count && use_row1(w[i]->dtype) && use_row1(w[j]->dtype) &&
+        const bool row1_ok = aligned && !no_fuse && row1_takes(m, all_bytes);
+        if (row1_ok && !no_mixed && j < count && use_row1(w[i]->dtype) && use_row1(w[j]->dtype) &&
             turq_gemv_row1_mixed_supports(w[i]->dtype, w[j]->dtype)) {
             int j2 = j + 1;
             while (j2 < count && w[j2]->dtype == w[j]->dtype) j2++;
@@ -146,11 +157,29 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
                 }
                 hipEvent_t ev0 = nullptr, ev1 = nullptr;
                 TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
-                TURQ_HIP(ctx, turq_launch_gemv_row1_mixed(w[i]->dtype, w[j]->dtype, j2 - i, j - i, wp, nn, w[i]->k, x, xt, y + i, yt,
-                                                          bias ? bias + i : nullptr, pick_waves_row1(w[i]->k), ctx->stream, ev0, ev1));
+                TURQ_HIP(ctx, turq_launch_gemv_row1_mixed(w[i]->dtype, w[j]->dtype, j2 - i, j - i, wp, nn, w[i]->k, x, xt, ldx, m, y + i,
+                                                          yt, ldy + i, bias ? bias + i : nullptr, pick_waves_row1(w[i]->k), ctx->stream,
+                                                          ev0, ev1));
                 i = j2;
                 continue;
             }
+        }
+        if (row1_ok && use_row1(w[i]->dtype)) {
+            const void *wp[4];
+            int64_t nn[4];
+            int64_t rows = 0;
+            for (int t = i; t < j; t++) {
+                wp[t - i] = w[t]->dev;
+                nn[t - i] = w[t]->n;
+                rows += w[t]->n;
+            }
+            hipEvent_t ev0 = nullptr, ev1 = nullptr;
+            TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+            TURQ_HIP(ctx, turq_launch_gemv_row1(w[i]->dtype, j - i, wp, nn, w[i]->k, x, xt, ldx, m, y + i, yt, ldy + i,
+                                                bias ? bias + i : nullptr, pick_waves_row1(w[i]->k),
+                                                m == 1 ? pick_rows_row1(ctx, turq_tile_rows(rows)) : 1, ctx->stream, ev0, ev1));
+            i = j;
+            continue;
         }
         if (!fused) {
             const int order = w[i]->dtype == TURQ_Q8_0 ? 2 : 1;
@@ -203,13 +232,6 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
         if (rtiles == 2) nwaves = std::min(nwaves, 4);
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
         TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
-        if (fused && m == 1 && use_row1(w[i]->dtype)) {
-            TURQ_HIP(ctx, turq_launch_gemv_row1(w[i]->dtype, j - i, wp, nn, w[i]->k, x, xt, y + i, yt, bias ? bias + i : nullptr,
-                                                pick_waves_row1(w[i]->k), pick_rows_row1(ctx, turq_tile_rows(rows)), ctx->stream,
-                                                ev0, ev1));
-            i = j;
-            continue;
-        }
         TURQ_HIP(ctx, turq_launch_gemv_multi(w[i]->dtype, j - i, wp, nn, w[i]->k, fused ? x : ctx->act_prep, xt, ldx, m, fused, y + i, yt,
                                              ldy + i, bias ? bias + i : nullptr, nwaves, rtiles, ctx->stream, ev0, ev1));
         i = j;
