@@ -390,6 +390,46 @@ def test_two_rows_on_a_large_weight(gpu, dt):
     gpu.release(w)
 
 
+@pytest.mark.parametrize("dt", ALL)
+@pytest.mark.parametrize("m", [3, 4])
+def test_up_to_four_rows_on_a_large_weight(gpu, dt, m):
+    # Q4_K / Q5_K: pairs of activation rows share an MFMA chain in the one-row kernel (three rows: the fourth repeats the
+    # first and is not stored); the other formats take the general kernel.  Distinct rows, strides, bias, every activation type.
+    n, k = 4100, 4096 + (96 if dt == Q8_0 else 0)
+    raw = synth.random_weight(dt, n, k, seed=dt + m)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    x = synth.random_activation(m, k, seed=11 + m)
+    bias = np.random.default_rng(3).standard_normal(n).astype(np.float32)
+    y = gpu.qmatmul(w, x, n, k, bias=bias, ldx=k + 8, ldy=n + 3)
+    want = orc.matmul_dequant(dt, f16_round(x), raw, n, k) + bias
+    assert y.shape == (m, n) and rel_l2(y, want) <= 2e-5
+    for i in range(m):      # row i alone gives the same numbers up to the order of the sums
+        assert rel_l2(gpu.qmatmul(w, x[i:i + 1], n, k, bias=bias), y[i:i + 1]) <= 1e-5, i
+    xb = synth.random_activation(m, k, seed=21, bf16=True)
+    yb = gpu.qmatmul(w, xb, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_F32)
+    assert rel_l2(yb, orc.matmul_dequant(dt, xb, raw, n, k)) <= 2e-5
+    xh = f16_round(x)
+    yh = gpu.qmatmul(w, xh, n, k, x_dtype=capi.ACT_F16, y_dtype=capi.ACT_F32)
+    assert rel_l2(yh, want - bias) <= 2e-5
+    gpu.release(w)
+
+
+@pytest.mark.parametrize("dt", [Q4_K, Q5_K])
+def test_four_rows_several_weights_one_launch(gpu, dt):
+    # gate + up against four rows: one launch of the packed form; every output equals the single call's bit for bit
+    k, ns = 4096, [6144, 6100]
+    raws = [synth.random_weight(dt, n, k, seed=n) for n in ns]
+    ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for n, raw in zip(ns, raws)]
+    for m in (3, 4):
+        x = synth.random_activation(m, k, seed=30 + m)
+        ys = gpu.qmatmul_multi(ws, x, ns, k)
+        for n, raw, w, y in zip(ns, raws, ws, ys):
+            assert rel_l2(y, orc.matmul_dequant(dt, f16_round(x), raw, n, k)) <= 2e-5, (m, n)
+            assert rel_l2(y, gpu.qmatmul(w, x, n, k)) <= 1e-5, (m, n)
+    for w in ws:
+        gpu.release(w)
+
+
 def test_two_rows_two_formats(gpu):
     # q, k (Q4_K) and v (Q6_K) against two activation rows: one launch of the two-format kernel
     k, ns, dts = 4096, [4096, 1024, 1000], (Q4_K, Q4_K, Q6_K)

@@ -29,6 +29,8 @@
 
 #include <cstdlib>
 
+#include <algorithm>
+
 #include "layout.h"
 #include "mfma_common.h"
 
@@ -41,6 +43,9 @@ constexpr uint32_t kMagicHdr = 0x64005400u;   // header fields: low half at bit 
 
 // LDS region of one (wave, tile in flight): 256 f16 of x, 16 floats the accumulator starts from, 64 bytes of zeros
 constexpr int kX = 0, kInit = 512, kZero = 576, kRegion = 640;
+// LDS region of one (wave, tile in flight, PAIR of activation rows) in the packed form, where the sixteen A rows of an MFMA are
+// eight sub-blocks x two activation rows: 2 x 256 f16 of x, 16 start values, 16 sums of x (for the mins), 64 bytes of zeros
+constexpr int kPX = 0, kPInit = 1024, kPSum = 1088, kPZero = 1152, kPairRegion = 1216;
 
 // v + (the same value from the lane `CTRL` points at), inside a row of 16 lanes
 template <int CTRL> __device__ inline float dpp_add(float v) {
@@ -172,6 +177,41 @@ template <int DT> struct Row1K45 {
             }
         }
     }
+    // ---- packed form: two activation rows per chain.  A row R = 4 g' + 2 s + a carries sub-block 2 g' + s of activation row
+    // a of the pair, so lane (n, g) of the result finds (sub-block 2g, row 0), (2g, row 1), (2g + 1, row 0), (2g + 1, row 1) in
+    // its four registers; no row is left for sum(x), which the staging keeps in the LDS instead (kPSum, same index).
+    static constexpr bool kPacked = true;
+    struct LanePK { int offA, offB; };
+    __device__ static LanePK lane_init_pk(int r, int g) {
+        const int gq = r >> 2, s = (r >> 1) & 1, a = r & 1;
+        LanePK l;
+        l.offA = (g == gq && s == 0) ? kPX + 512 * a + 128 * g : kPZero;
+        l.offB = (g == gq && s == 1) ? kPX + 512 * a + 128 * g + 64 : kPZero;
+        return l;
+    }
+    __device__ static void sums_pk(half2v h01, half2v h23, uint8_t *pr, int lane, int a) {
+        const float s = sum8(dot2(h23, (_Float16)1.0f, dot2(h01, (_Float16)1.0f, 0.0f)));
+        const float nb = sum8(dot2(h23, (_Float16)-64.0f, dot2(h01, (_Float16)-1024.0f, 0.0f)));
+        if ((lane & 7) == 0) {
+            const int at = 4 * (2 * (lane >> 3) + a);  // sub-block lane / 8
+            *(float *)(pr + kPInit + at) = nb;
+            *(float *)(pr + kPSum + at) = s;
+        }
+    }
+    template <int NP> __device__ static void chain_pk(const W &w, const uint8_t *pr, const LanePK &l, int g, float4v *c) {
+#pragma unroll
+        for (int np = 0; np < NP; np++) c[np] = *(const float4v *)(pr + np * kPairRegion + kPInit + 16 * g);
+        const uint32_t wq[8] = {w.qa.x, w.qa.y, w.qa.z, w.qa.w, w.qb.x, w.qb.y, w.qb.z, w.qb.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const half8v bop = operand(wq[i], w.hh.x, w.hh.y, 2 * i);
+#pragma unroll
+            for (int np = 0; np < NP; np++) {
+                const half8v av = *(const half8v *)(pr + np * kPairRegion + (i < 4 ? l.offA : l.offB) + 16 * (i & 3));
+                c[np] = mfma16x16x32(av, bop, c[np]);
+            }
+        }
+    }
     struct Sc { half2v sc, mn, dd; };  // (sc, sc'), (m, m'), (d, dmin)
     __device__ static Sc scales(const W &w, const Lane &l) {
         const half2v kb = {(_Float16)-64.0f, (_Float16)-1024.0f};
@@ -186,6 +226,13 @@ template <int DT> struct Row1K45 {
         const float v = (float)s.mn.x * c[1] + (float)s.mn.y * c[3];
         return (float)s.dd.x * u - (float)s.dd.y * v;
     }
+    // sx: the sums of x in the order of c
+    __device__ static void finish_pk(const Sc &s, const float4v &c, const float4v &sx, float &y0, float &y1) {
+        const float sc0 = (float)s.sc.x, sc1 = (float)s.sc.y, m0 = (float)s.mn.x, m1 = (float)s.mn.y;
+        const float d = (float)s.dd.x, dmin = (float)s.dd.y;
+        y0 += d * (sc0 * c[0] + sc1 * c[2]) - dmin * (m0 * sx[0] + m1 * sx[2]);
+        y1 += d * (sc0 * c[1] + sc1 * c[3]) - dmin * (m0 * sx[1] + m1 * sx[3]);
+    }
 };
 template <> struct Row1Fmt<TURQ_Q4_K> : Row1K45<TURQ_Q4_K> {};
 template <> struct Row1Fmt<TURQ_Q5_K> : Row1K45<TURQ_Q5_K> {};
@@ -193,6 +240,7 @@ template <> struct Row1Fmt<TURQ_Q5_K> : Row1K45<TURQ_Q5_K> {};
 template <> struct Row1Fmt<TURQ_Q6_K> {
     using F = TiledFmt<TURQ_Q6_K>;
     struct Lane { int off[4]; };  // steps 2s, 2s + 1 feed result row 4g + s (sub-block 4g + s)
+    static constexpr bool kPacked = false;  // no packed form: rows are handled one MFMA chain each
     struct W { uint4v qla, qlb, qh; uint32_t scw, d16; };
     __device__ static Lane lane_init(int r, int g) {
         Lane l;
@@ -259,6 +307,7 @@ template <> struct Row1Fmt<TURQ_Q6_K> {
 template <> struct Row1Fmt<TURQ_Q8_0> {
     using F = TiledFmt<TURQ_Q8_0>;
     struct Lane { int off[8]; };  // step q feeds result row q (block q); rows 8..15 stay zero
+    static constexpr bool kPacked = false;  // no packed form: rows are handled one MFMA chain each
     struct W { uint4v p[4]; uint2v dd; };
     __device__ static Lane lane_init(int r, int g) {
         Lane l;
@@ -341,13 +390,24 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
     const int nwaves = blockDim.x >> 6;
     const int g = lane >> 4;
     const int64_t ntc = turq_tile_cols(k);
-    uint8_t *region = smem + (size_t)wave * (P * M * kRegion);  // [p][activation row]
-    float *red = (float *)(smem + (size_t)nwaves * (P * M * kRegion));
+    // several rows of a format that has the packed form: two rows per MFMA chain, regions per pair of rows
+    constexpr bool PK = Fmt::kPacked && M > 1;
+    constexpr int NP = M / 2;
+    constexpr int PSTRIDE = PK ? NP * kPairRegion : M * kRegion;  // LDS of one tile in flight
+    static_assert(!PK || M % 2 == 0, "packed pairs");
+    uint8_t *region = smem + (size_t)wave * (P * PSTRIDE);  // [p][activation row] or [p][pair]
+    float *red = (float *)(smem + (size_t)nwaves * (P * PSTRIDE));
 
     // the zeros that the idle A rows read, and start values that no format overwrites
-    if (lane < 32)
+    if constexpr (PK) {
+        if (lane < 48)
 #pragma unroll
-        for (int p = 0; p < P * M; p++) *(float *)(region + p * kRegion + kInit + 4 * lane) = 0.0f;  // float like the later writes
+            for (int p = 0; p < P * NP; p++) *(float *)(region + p * kPairRegion + kPInit + 4 * lane) = 0.0f;
+    } else {
+        if (lane < 32)
+#pragma unroll
+            for (int p = 0; p < P * M; p++) *(float *)(region + p * kRegion + kInit + 4 * lane) = 0.0f;  // float like the later writes
+    }
     const typename Fmt::Lane lc = Fmt::lane_init(lane & 15, g);
     GOff go{16u * (uint32_t)lane, 8u * (uint32_t)lane, 4u * (uint32_t)lane, 16u * (uint32_t)(lane & 15), Fmt::aux_off(lane & 15, g), 0u};
 
@@ -381,7 +441,17 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
 #pragma unroll
         for (int p = 0; p < P; p++)
 #pragma unroll
-            for (int mm = 0; mm < M; mm++) stage_x1<DT, XT>(xr[p][mm], region + (p * M + mm) * kRegion, lane);
+            for (int mm = 0; mm < M; mm++) {
+                if constexpr (PK) {
+                    uint8_t *pr = region + p * PSTRIDE + (mm >> 1) * kPairRegion;
+                    half2v h01, h23;
+                    to_half4<XT>(xr[p][mm], h01, h23);
+                    *(uint2v *)(pr + kPX + 512 * (mm & 1) + 8 * lane) = uint2v{as_u32(h01), as_u32(h23)};
+                    Fmt::sums_pk(h01, h23, pr, lane, mm & 1);
+                } else {
+                    stage_x1<DT, XT>(xr[p][mm], region + p * PSTRIDE + mm * kRegion, lane);
+                }
+            }
         // same-wave LDS traffic is processed in order; the fences keep the compiler from reordering
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -392,8 +462,23 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
             if (b >= ntc) continue;  // uniform per wave
 #pragma unroll
             for (int r = 0; r < R; r++) {
+                if constexpr (PK) {
+                    const typename Fmt::LanePK lpk = Fmt::lane_init_pk(lane & 15, g);
+                    float4v c[NP];
+                    Fmt::template chain_pk<NP>(wr[p][r], region + p * PSTRIDE, lpk, g, c);
+#pragma unroll
+                    for (int np = 0; np < NP; np++) asm volatile("" : "+v"(c[np]));
+                    __builtin_amdgcn_sched_barrier(0x10 | 0x80 | 0x4);
+                    const typename Fmt::Sc sc = Fmt::scales(wr[p][r], lc);
+#pragma unroll
+                    for (int np = 0; np < NP; np++) {
+                        const float4v sx = *(const float4v *)(region + p * PSTRIDE + np * kPairRegion + kPSum + 16 * g);
+                        Fmt::finish_pk(sc, c[np], sx, acc[r][2 * np], acc[r][2 * np + 1]);
+                    }
+                    continue;
+                }
                 float4v c[M];
-                Fmt::template chain<M>(wr[p][r], region + p * M * kRegion, lc, g, c);
+                Fmt::template chain<M>(wr[p][r], region + p * PSTRIDE, lc, g, c);
                 // One tile after the other.  Left free, the scheduler interleaves the tiles' chains and scale arithmetic, the
                 // unpacked operands of several tiles are live at once and the 128 registers a wave of a 16-wave workgroup may
                 // use overflow (spills in the instantiations with four tiles per workgroup pass; the 510 MB LM head lost
@@ -472,13 +557,14 @@ struct Row1Launch {
     hipEvent_t ev0, ev1;
 };
 
-template <int P, int R, int M> size_t row1_lds(int nwaves) {
-    return (size_t)nwaves * P * M * kRegion + (size_t)nwaves * R * M * 64 * sizeof(float);
+template <int DT, int P, int R, int M> size_t row1_lds(int nwaves) {
+    const size_t tile = (Row1Fmt<DT>::kPacked && M > 1) ? (size_t)(M / 2) * kPairRegion : (size_t)M * kRegion;
+    return (size_t)nwaves * P * tile + (size_t)nwaves * R * M * 64 * sizeof(float);
 }
 
 template <int DT, int XT, int P, int R, int M>
 hipError_t launch_final(const Row1Launch &l) {
-    const size_t lds = row1_lds<P, R, M>(l.nwaves);
+    const size_t lds = row1_lds<DT, P, R, M>(l.nwaves);
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
     if (l.ev0) {
         hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, R, M, 1024>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k, l.x,
@@ -503,7 +589,11 @@ inline int row1_in_flight(int64_t k, int nwaves, int m) {
 template <int DT, int XT>
 hipError_t launch_p(const Row1Launch &l) {
     const int p = row1_in_flight(l.k, l.nwaves, l.m);
-    static_assert(TURQ_ROW1_MAX_M == 2, "instantiations for one and two activation rows");
+    static_assert(TURQ_ROW1_MAX_M == 4, "instantiations for one, two and (packed formats) four activation rows");
+    if (l.m > 2) {
+        if constexpr (Row1Fmt<DT>::kPacked) return p == 1 ? launch_final<DT, XT, 1, 1, 4>(l) : launch_final<DT, XT, 2, 1, 4>(l);
+        else return hipErrorInvalidValue;  // turq_gemv_row1_rows() says so
+    }
     if (l.m == 2) return p == 1 ? launch_final<DT, XT, 1, 1, 2>(l) : launch_final<DT, XT, 2, 1, 2>(l);
     if (l.rtiles == 2)  // two row tiles double the weights a wave holds: at most two column tiles in flight
         return p == 1 ? launch_final<DT, XT, 1, 2, 1>(l) : launch_final<DT, XT, 2, 2, 1>(l);
@@ -524,7 +614,7 @@ hipError_t launch_x(int xt, const Row1Launch &l) {
 
 template <int DTA, int DTB, int XT, int P, int M>
 hipError_t launch_mixed_final(const Row1Launch &l) {
-    const size_t lds = row1_lds<P, 1, M>(l.nwaves);
+    const size_t lds = std::max(row1_lds<DTA, P, 1, M>(l.nwaves), row1_lds<DTB, P, 1, M>(l.nwaves));
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
     if (l.ev0) {
         hipExtLaunchKernelGGL((gemv_row1_mixed_kernel<DTA, DTB, XT, P, M, 1024>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a,
@@ -538,6 +628,7 @@ hipError_t launch_mixed_final(const Row1Launch &l) {
 template <int DTA, int DTB, int XT>
 hipError_t launch_mixed_p(const Row1Launch &l) {
     const int p = row1_in_flight(l.k, l.nwaves, l.m);
+    if (l.m > 2) return hipErrorInvalidValue;
     if (l.m == 2) return p == 1 ? launch_mixed_final<DTA, DTB, XT, 1, 2>(l) : launch_mixed_final<DTA, DTB, XT, 2, 2>(l);
     if (p == 1) return launch_mixed_final<DTA, DTB, XT, 1, 1>(l);
     if (p == 2) return launch_mixed_final<DTA, DTB, XT, 2, 1>(l);
@@ -567,6 +658,16 @@ bool row1_args(Row1Launch &l, int count, const void *const *w, const int64_t *n,
 
 bool turq_gemv_row1_supports(int dtype) {
     return dtype == TURQ_Q4_K || dtype == TURQ_Q5_K || dtype == TURQ_Q6_K || dtype == TURQ_Q8_0;
+}
+// activation rows one launch takes for this format: four where two rows share an MFMA chain, else two
+int turq_gemv_row1_rows(int dtype) {
+    switch (dtype) {
+    case TURQ_Q4_K: return Row1Fmt<TURQ_Q4_K>::kPacked ? 4 : 2;
+    case TURQ_Q5_K: return Row1Fmt<TURQ_Q5_K>::kPacked ? 4 : 2;
+    case TURQ_Q6_K: return Row1Fmt<TURQ_Q6_K>::kPacked ? 4 : 2;
+    case TURQ_Q8_0: return Row1Fmt<TURQ_Q8_0>::kPacked ? 4 : 2;
+    default: return 0;
+    }
 }
 
 // count (1..4) weights of one format and one k against m (1..TURQ_ROW1_MAX_M) activation rows of stride ldx (rows 16-byte

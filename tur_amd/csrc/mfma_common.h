@@ -155,9 +155,10 @@ hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w_til
                                   const float *const *bias, int waves_per_group, int row_tiles_per_group, hipStream_t stream,
                                   hipEvent_t ev_start, hipEvent_t ev_stop);
 // Activation rows the one-row kernel takes in one launch.  The body is written for any number M (every unpacked operand feeds
-// M MFMAs); with four rows it is bound by its vector instructions (staging and scales per row) and loses 6 - 13 % to the
-// preparation launch + general kernel, with two it wins 5 - 12 % on matrices of tens of MB.
-#define TURQ_ROW1_MAX_M 2
+// the MFMAs of all rows).  Formats with 8 sub-blocks per tile pack two activation rows into the 16 A rows of one MFMA chain
+// (turq_gemv_row1_rows() = 4); Q6_K, whose 16 sub-blocks fill the A rows, and Q8_0 take a chain per row and stop at two.
+#define TURQ_ROW1_MAX_M 4
+int turq_gemv_row1_rows(int dtype);
 bool turq_gemv_row1_supports(int dtype);
 hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w_tiled, const int64_t *n, int64_t k, const void *x,
                                  int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,

@@ -37,11 +37,18 @@ bool use_row1(int dtype) {
 }
 
 // The one-row kernel stages the raw activations itself, once per wave and column tile, and needs no preparation launch.
-// One activation row: always.  Two: where the weights of the call are large enough for its launch to beat the fused general
-// kernel (measured: + 5 .. 12 % at 28 MB and more, - 10 % at 3 MB).  TURQ_ROW1_M = 1 keeps it to one row, for comparison.
-bool row1_takes(int64_t m, size_t weight_bytes) {
+// One activation row: always.  Two rows: where the weights of the call are large enough for its launch to beat the fused
+// general kernel (+ 5 .. 12 % at 28 MB and more, - 10 % at 3 MB).  Three and four rows (formats whose kernel packs pairs of
+// rows): the 16 MFMAs and LDS operand reads per tile then cost as much as the tile's bytes, so only up to a size where the
+// general kernel's preparation launch and its tail still weigh more (Q4_K: + 6 .. 40 % up to 57 MB, - 4 % at 75 MB,
+// - 19 % at 350 MB; Q5_K: + 7 % at 92 MB, - 12 % at 430 MB).  TURQ_ROW1_M lowers the row limit, for comparison.
+bool row1_takes(int64_t m, size_t weight_bytes, int dtype) {
     static const int most = [] { const char *e = getenv("TURQ_ROW1_M"); const int x = e ? atoi(e) : TURQ_ROW1_MAX_M; return x < 1 ? 1 : x > TURQ_ROW1_MAX_M ? TURQ_ROW1_MAX_M : x; }();
-    return m == 1 || (m <= most && weight_bytes >= (8u << 20));
+    const size_t least = (size_t)8 << 20;  // below: the general kernel is level or up to 10 % ahead, for any number of rows
+    if (m == 1) return true;
+    if (m > most || m > turq_gemv_row1_rows(dtype) || weight_bytes < least) return false;
+    if (m <= 2) return true;
+    return weight_bytes <= ((size_t)(dtype == TURQ_Q4_K ? 64 : 128) << 20);
 }
 
 // Waves per workgroup of the one-row kernel: it is light on registers and on vector work, so what it wants is many waves
@@ -96,7 +103,7 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
         static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
         // raw activation rows must be 16-byte (f32) / 8-byte (16-bit) aligned for the fused loads
         const bool aligned = ((uintptr_t)xc % 16 == 0) && ((size_t)ldx * xb) % 16 == 0;
-        if (aligned && !no_fuse && row1_takes(mc, w->dev_bytes) && use_row1(w->dtype)) {
+        if (aligned && !no_fuse && use_row1(w->dtype) && row1_takes(mc, w->dev_bytes, w->dtype)) {
             hipEvent_t ev0 = nullptr, ev1 = nullptr;
             TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
             const void *wp = w->dev;
@@ -143,8 +150,10 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
         while (j < count && j - i < 4 && w[j]->dtype == w[i]->dtype) j++;
         // one activation row: a run of a second format joins the launch where the kernel has that pair (q, k Q4_K + v Q6_K)
         static const bool no_mixed = getenv("TURQ_GEMV_NO_MIXED") != nullptr;
-        const bool row1_ok = aligned && !no_fuse && row1_takes(m, all_bytes);
-        if (row1_ok && !no_mixed && j < count && use_row1(w[i]->dtype) && use_row1(w[j]->dtype) &&
+        // (more than two rows: only a call of one format, which would otherwise lose the launch it shares with a second one)
+        const bool row1_ok = aligned && !no_fuse && use_row1(w[i]->dtype) && row1_takes(m, all_bytes, w[i]->dtype) &&
+                             (m <= 2 || (i == 0 && j == count));
+        if (row1_ok && m <= 2 && !no_mixed && j < count && use_row1(w[j]->dtype) &&
             turq_gemv_row1_mixed_supports(w[i]->dtype, w[j]->dtype)) {
             int j2 = j + 1;
             while (j2 < count && w[j2]->dtype == w[j]->dtype) j2++;
@@ -164,7 +173,7 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
                 continue;
             }
         }
-        if (row1_ok && use_row1(w[i]->dtype)) {
+        if (row1_ok) {
             const void *wp[4];
             int64_t nn[4];
             int64_t rows = 0;
