@@ -41,10 +41,10 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # dense f16 / bf16 MFMA, vendor figure
 # WRITE_SIZE, scaled by the same counters on a copy kernel of known size (summaries under profiles/); keyed by
 # (workload, m, activations, one call per matrix?)
 TRAFFIC = {
-    ("q4k_mlp_8b", 1, "f32", False): 42_868_400,    # gate + up in one launch 56 925 200, down 28 811 600
+    ("q4k_mlp_8b", 1, "f32", False): 42_858_500,    # gate + up in one launch 56 920 900, down 28 796 200
     ("q4k_mlp_8b", 1, "f32", True): 28_680_000,
-    ("q4k_prefill_up_8b", 512, "bf16", False): 76_827_600,   # every XCD's L2 fetches the activation fragments once
-    ("q4k_prefill_up_8b", 512, "bf16", True): 76_827_600,
+    ("q4k_prefill_up_8b", 512, "bf16", False): 76_833_700,   # every XCD's L2 fetches the activation fragments once
+    ("q4k_prefill_up_8b", 512, "bf16", True): 76_833_700,
 }
 
 WORKLOADS = {
