@@ -415,6 +415,19 @@ def test_up_to_four_rows_on_a_large_weight(gpu, dt, m):
 
 
 @pytest.mark.parametrize("dt", [Q4_K, Q5_K])
+def test_four_rows_wide_weight(gpu, dt):
+    # 48 column tiles: sixteen waves per workgroup, two tiles in flight and two pairs of rows each (94 KiB of LDS)
+    n, k = 2048, 12288
+    raw = synth.random_weight(dt, n, k, seed=dt + 40)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    for m in (3, 4):
+        x = synth.random_activation(m, k, seed=50 + m)
+        y = gpu.qmatmul(w, x, n, k)
+        assert rel_l2(y, orc.matmul_dequant(dt, f16_round(x), raw, n, k)) <= 2e-5, m
+    gpu.release(w)
+
+
+@pytest.mark.parametrize("dt", [Q4_K, Q5_K])
 def test_four_rows_several_weights_one_launch(gpu, dt):
     # gate + up against four rows: one launch of the packed form; every output equals the single call's bit for bit
     k, ns = 4096, [6144, 6100]

@@ -566,6 +566,11 @@ template <int DT, int XT, int P, int R, int M>
 hipError_t launch_final(const Row1Launch &l) {
     const size_t lds = row1_lds<DT, P, R, M>(l.nwaves);
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
+    if (lds > (64u << 10)) {  // 16 waves x two tiles in flight x two pairs of rows: 94 KiB
+        static const hipError_t raised = hipFuncSetAttribute((const void *)gemv_row1_kernel<DT, XT, P, R, M, 1024>,
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10);
+        if (raised != hipSuccess) return raised;
+    }
     if (l.ev0) {
         hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, R, M, 1024>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k, l.x,
                               l.ldx, l.m, l.yt);
