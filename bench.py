@@ -61,6 +61,15 @@ OUT = {"f32": (capi.ACT_F32, 4), "bf16": (capi.ACT_BF16, 2)}
 ACT = {"f32": (capi.ACT_F32, 4, np.float32), "bf16": (capi.ACT_BF16, 2, np.uint16)}
 
 
+# projections that the reference applies to one and the same tensor (src/models/qwen3.rs:272-274 and :161-167); o_proj and
+# down_proj have inputs of their own
+SHARED_INPUT = ({"q", "k", "v"}, {"gate", "up"})
+
+
+def shares_input(a, b):
+    return any(a in g and b in g for g in SHARED_INPUT)
+
+
 def algorithmic_bytes(dt, n, k, m, xbytes, ybytes):
     return synth.weight_nbytes(dt, n, k) + m * k * xbytes + m * n * ybytes
 
@@ -131,7 +140,7 @@ class Bench:
             i = 0
             while i < len(self.mats):
                 j = i + 1
-                while j < len(self.mats) and self.mats[j][3] == self.mats[i][3]:
+                while j < len(self.mats) and self.mats[j][3] == self.mats[i][3] and shares_input(self.mats[i][0], self.mats[j][0]):
                     j += 1
                 cnt = j - i
                 warr = (ctypes.c_void_p * cnt)(*[w.value for w in layer[i:j]])
