@@ -161,6 +161,24 @@ int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weigh
                        int64_t ldx, void *const *ys, int y_dtype, const int64_t *ldys, const float *const *biases, int mem,
                        int algo);
 
+/* Activation functions of turq_qmatmul_gate_up (candle_nn::Activation; the reference reads it from the model's config,
+ * `act_fn: cfg.hidden_act`, src/models/qwen3.rs:156; Qwen3 and Granite use SiLU). */
+enum { TURQ_ACTFN_SILU = 0 };
+
+/* The first half of the reference's MLP in one call: y[m, n] = act(x * gate^T + bias_gate) * (x * up^T + bias_up), with
+ * act = SiLU, v / (1 + exp(-v)), computed in f32.  gate and up are two weights of one shape [n, k]; x, y, the strides, the
+ * biases (NULL: none) and `mem` as in turq_qmatmul.  With device pointers, tiled weights of one format and one activation
+ * row (two on 8 MiB of weights and more) the activation and the product are applied inside the matmul kernel, which then is
+ * the one launch of the call and writes one output instead of two; every other case computes the two products through
+ * turq_qmatmul_multi into scratch memory of the context (which grows on demand, never inside a graph capture) and combines
+ * them in one elementwise pass.  Errors as turq_qmatmul; gate and up of different shapes: TURQ_ERR_SHAPE; an activation other
+ * than TURQ_ACTFN_SILU: TURQ_ERR_INVALID.
+ * Replaces: `x.apply(&self.gate_proj)?.apply(&self.act_fn)?` times `x.apply(&self.up_proj)?` in `Qwen3MLP::forward`
+ * (src/models/qwen3.rs:161-167; the Granite MLP, src/models/granite_41.rs:151-155, has the same form). */
+int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int x_dtype, int64_t m,
+                         int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up, int act,
+                         int mem);
+
 /* ---- activation quantisation (candle's VecDotType::from_float, bit-exact) ---- */
 /* x f32 [m, k] (row stride k) -> Q8_0 blocks (34 B per 32) / Q8_K blocks (292 B per 256).
  * The GPU forward path does not use them (it keeps activations in f16); they are the device

@@ -220,3 +220,14 @@ def qmatmul(dtype: int, x: np.ndarray, raw, n: int, k: int) -> np.ndarray:
             s = s + sums[:, l]
         out[r] = sumf + s
     return out
+
+
+def silu_mul(gate: np.ndarray, up: np.ndarray) -> np.ndarray:
+    """``act(gate) * up`` of the reference's MLP, src/models/qwen3.rs:161-167 (``x.apply(&gate_proj)?.apply(&act_fn)? *
+    x.apply(&up_proj)?``) with ``act_fn`` = SiLU, candle's ``v / (1 + exp(-v))``; evaluated in f64 and rounded once to f32.
+    Pinned by closed forms (tests/test_oracle_kat.py): silu(0) = 0, silu(v) - silu(-v) = v, silu(v) -> v for large v,
+    the minimum -0.27846 at v = -1.27846; candle's own f32 evaluation order is not reproduced (tolerance test, not bit test)."""
+    g = np.asarray(gate, np.float64)
+    with np.errstate(over="ignore"):
+        act = g / (1.0 + np.exp(-g))
+    return (act * np.asarray(up, np.float64)).astype(_f32)

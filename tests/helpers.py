@@ -113,6 +113,46 @@ class Gpu:
             capi.check(L.turq_dev_free(ctx, p), ctx)
         return outs
 
+    def gate_up(self, wg, wu, x, n, k, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_F32, bias_gate=None, bias_up=None,
+                mem=capi.MEM_DEVICE, ldx=None, ldy=None):
+        """act(x gate^T) * (x up^T) through turq_qmatmul_gate_up; returns f32 [m, n]"""
+        L, ctx = self.L, self.ctx
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
+        m = x.shape[0]
+        ldx, ldy = ldx or k, ldy or n
+        xbuf = np.zeros((m, ldx), np.float32)
+        xbuf[:, :k] = x
+        xsend = (synth.to_bf16_bits(xbuf).reshape(m, ldx) if x_dtype == capi.ACT_BF16
+                 else xbuf.astype(np.float16) if x_dtype == capi.ACT_F16 else xbuf)
+        ydt = {capi.ACT_F32: np.float32, capi.ACT_BF16: np.uint16, capi.ACT_F16: np.float16}[y_dtype]
+        y = np.full((m, ldy), 0, ydt)
+        bg = None if bias_gate is None else np.ascontiguousarray(bias_gate, np.float32)
+        bu = None if bias_up is None else np.ascontiguousarray(bias_up, np.float32)
+        freed = []
+
+        def dev(arr):
+            p = ctypes.c_void_p()
+            capi.check(L.turq_dev_alloc(ctx, max(arr.nbytes, 16), ctypes.byref(p)), ctx)
+            freed.append(p)
+            capi.check(L.turq_memcpy_h2d(ctx, p, capi.ptr(arr), arr.nbytes), ctx)
+            return p
+
+        if mem == capi.MEM_DEVICE:
+            xp, yp = dev(xsend), dev(y)
+            bgp = None if bg is None else dev(bg)
+            bup = None if bu is None else dev(bu)
+        else:
+            xp, yp, bgp, bup = capi.ptr(xsend), capi.ptr(y), capi.ptr(bg), capi.ptr(bu)
+        rc = L.turq_qmatmul_gate_up(ctx, wg, wu, xp, x_dtype, m, ldx, yp, y_dtype, ldy, bgp, bup, 0, mem)
+        capi.check(rc, ctx)
+        if mem == capi.MEM_DEVICE:
+            capi.check(L.turq_memcpy_d2h(ctx, capi.ptr(y), yp, y.nbytes), ctx)
+        for p in freed:
+            capi.check(L.turq_dev_free(ctx, p), ctx)
+        if y_dtype == capi.ACT_BF16:
+            y = synth.from_bf16_bits(y).reshape(m, ldy)
+        return np.asarray(y, np.float32)[:, :n]
+
     def quantize(self, x, kind):
         x = np.ascontiguousarray(x, np.float32)
         m, k = x.shape

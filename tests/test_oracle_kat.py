@@ -326,3 +326,21 @@ def test_vec_dot_integer_part_is_exact():
     y = orc.qmatmul(Q4_K, x[None, :], blk, 1, k)[0, 0]
     w = orc.dequantize(Q4_K, blk)
     assert y == np.float32(np.dot(w.astype(np.float64), x.astype(np.float64)))
+
+
+def test_silu_mul_closed_forms():
+    # the activation of the reference's MLP (src/models/qwen3.rs:161-167): silu(v) = v * sigmoid(v)
+    from oracle import oracle_np as onp
+    one = np.ones(1, np.float32)
+    assert onp.silu_mul(np.zeros(1, np.float32), one)[0] == 0.0
+    v = np.linspace(-12, 12, 97).astype(np.float32)
+    ones = np.ones_like(v)
+    # silu(v) - silu(-v) = v (sigmoid(v) + sigmoid(-v) = 1)
+    assert np.allclose(onp.silu_mul(v, ones) - onp.silu_mul(-v, ones), v, rtol=0, atol=2e-6)
+    # large arguments: the identity and zero; no overflow of exp(-v) for very negative v
+    assert onp.silu_mul(np.float32([40.0]), one)[0] == np.float32(40.0)
+    assert abs(onp.silu_mul(np.float32([-200.0]), one)[0]) == 0.0
+    # the minimum of silu: -0.2784645 at v = -1.2784645
+    assert abs(onp.silu_mul(np.float32([-1.2784645]), one)[0] + 0.2784645) < 1e-6
+    # a known value and the product: silu(1) = 1 / (1 + e^-1) = 0.7310586
+    assert abs(onp.silu_mul(np.float32([1.0]), np.float32([3.0]))[0] - 3 * 0.7310586) < 1e-6

@@ -127,6 +127,7 @@ void turq_ctx_destroy(turq_ctx *ctx) {
     if (ctx->stage_x) (void)hipFree(ctx->stage_x);
     if (ctx->stage_y) (void)hipFree(ctx->stage_y);
     if (ctx->act_prep) (void)hipFree(ctx->act_prep);
+    if (ctx->gate_up) (void)hipFree(ctx->gate_up);
     if (ctx->stage_b) (void)hipFree(ctx->stage_b);
     for (auto &p : ctx->prof_events) { (void)hipEventDestroy(p.first); (void)hipEventDestroy(p.second); }
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -429,6 +430,76 @@ int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weigh
         return TURQ_OK;
     }
     return turq_qmatmul_multi_mfma(ctx, count, weights, x, xt, m, ldx, ys, yt, ldys, biases);
+}
+
+namespace {
+uint16_t host_bf16(float v) {  // round to nearest even, as the kernels store it
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40);
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+}  // namespace
+
+int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m, int64_t ldx,
+                         void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, int act, int mem) {
+    TURQ_ENTER(ctx);
+    if (!gate || !up) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_gate_up: null weight");
+    if (act != TURQ_ACTFN_SILU) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_gate_up: activation %d is not supported", act);
+    if (gate->n != up->n || gate->k != up->k)
+        return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul_gate_up: gate is [%lld, %lld], up is [%lld, %lld]", (long long)gate->n,
+                         (long long)gate->k, (long long)up->n, (long long)up->k);
+    if (mem != TURQ_MEM_DEVICE && mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_gate_up: bad mem %d", mem);
+    const int yb = turq_act_bytes(yt);
+    if (!yb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul_gate_up: output dtype %d", yt);
+    if (m < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul_gate_up: m=%lld is negative", (long long)m);
+    if (ldy < gate->n) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul_gate_up: ldy=%lld is smaller than n=%lld", (long long)ldy, (long long)gate->n);
+    const int64_t n = gate->n;
+    const turq_weight *ws[2] = {gate, up};
+    const float *biases[2] = {bias_gate, bias_up};
+    const int64_t ldys[2] = {n, n};
+    if (mem == TURQ_MEM_HOST) {
+        // the two products through the host path, the expression on the host (the remaining argument checks are turq_qmatmul's)
+        std::vector<float> prod;
+        try { prod.resize((size_t)(2 * m * n)); } catch (...) { return turq_fail(ctx, TURQ_ERR_OOM, "turq_qmatmul_gate_up: host scratch"); }
+        for (int i = 0; i < 2; i++) {
+            const int rc = turq_qmatmul(ctx, ws[i], x, xt, m, ldx, prod.data() + (size_t)i * m * n, TURQ_ACT_F32, n, biases[i], mem, TURQ_ALGO_AUTO);
+            if (rc != TURQ_OK) return rc;
+        }
+        if (m == 0 || n == 0) return TURQ_OK;
+        if (!y) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_gate_up: null output pointer");
+        for (int64_t r = 0; r < m; r++)
+            for (int64_t c = 0; c < n; c++) {
+                const float g = prod[(size_t)(r * n + c)], u = prod[(size_t)((m + r) * n + c)];
+                const float out = g / (1.0f + expf(-g)) * u;
+                const size_t at = (size_t)(r * ldy + c);
+                if (yt == TURQ_ACT_F32) ((float *)y)[at] = out;
+                else if (yt == TURQ_ACT_BF16) ((uint16_t *)y)[at] = host_bf16(out);
+                else {
+                    const _Float16 h = (_Float16)out;
+                    memcpy((uint16_t *)y + at, &h, 2);
+                }
+            }
+        return TURQ_OK;
+    }
+    if (m > 0 && n > 0 && x && y && gate->device == ctx->device && up->device == ctx->device && gate->k > 0 && ldx >= gate->k &&
+        turq_act_bytes(xt)) {
+        bool taken = false;
+        const int rc = turq_qmatmul_gate_up_mfma(ctx, gate, up, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, &taken);
+        if (rc != TURQ_OK || taken) return rc;
+    }
+    // general path: both products as f32 into scratch (one call, so they share a launch or an activation preparation where
+    // turq_qmatmul_multi does that), then one elementwise pass
+    const size_t half = (size_t)(m > 0 ? m : 0) * (size_t)n;
+    int rc = turq_ctx_reserve(ctx, &ctx->gate_up, &ctx->gate_up_cap, 2 * half * sizeof(float) + 16);
+    if (rc != TURQ_OK) return rc;
+    void *ys[2] = {ctx->gate_up, (float *)ctx->gate_up + half};
+    rc = turq_qmatmul_multi(ctx, 2, ws, x, xt, m, ldx, ys, TURQ_ACT_F32, ldys, biases, mem, TURQ_ALGO_AUTO);
+    if (rc != TURQ_OK) return rc;
+    if (m == 0 || n == 0) return TURQ_OK;
+    if (!y) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_gate_up: null output pointer");
+    TURQ_HIP(ctx, turq_launch_silu_mul((const float *)ys[0], (const float *)ys[1], m, n, y, yt, ldy, ctx->stream));
+    return TURQ_OK;
 }
 
 // ---- graphs and kernel timing ----

@@ -72,6 +72,7 @@ struct turq_ctx {
     void *stage_y = nullptr;  size_t stage_y_cap = 0;
     void *stage_b = nullptr;  size_t stage_b_cap = 0;
     void *act_prep = nullptr; size_t act_prep_cap = 0;
+    void *gate_up = nullptr;  size_t gate_up_cap = 0;  // the two f32 products of turq_qmatmul_gate_up's general path
     // kernel timing (turq_profile_*): event pairs recorded around matmul kernels
     bool profiling = false;
     bool capturing = false;
@@ -146,5 +147,11 @@ hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t 
 // MFMA paths on the tiled layout (activation preparation + kernel launch), see mfma_dispatch.cpp
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
                       int yt, int64_t ldy, const float *bias, int algo);
+// act(gate) * up on two f32 matrices [m, n] of row stride n (act_mul.hip)
+hipError_t turq_launch_silu_mul(const float *gate, const float *up, int64_t m, int64_t n, void *y, int y_dtype, int64_t ldy,
+                                hipStream_t stream);
+// act(gate) * up inside the one-row kernel; *taken = false (and nothing launched) where that kernel does not apply
+int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m,
+                              int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, bool *taken);
 int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m,
                             int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias);

@@ -376,14 +376,18 @@ struct Row1Args {
 // the work of one workgroup: row tiles rtb * R .. rtb * R + R - 1 of one weight, against m <= M activation rows.
 // P = column tiles a wave keeps in flight; R = row tiles per workgroup (a wave stages the activations of a column tile once and
 // uses them for R weight tiles); M = activation rows the instantiation holds (rows past m repeat row 0 and are not stored)
-template <int DT, int XT, int P, int R, int M>
+// GU (R = 2): the two "row tiles" are row tile rtb of a gate weight (w) and of an up weight (w2) of the same shape, and
+// what is stored is act(gate) * up (src/models/qwen3.rs:161-167 computes that product from the two projections' outputs)
+template <int DT, int XT, int P, int R, int M, bool GU = false>
 __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *__restrict__ y, int64_t ldy, const float *__restrict__ bias,
-                                          int64_t n, int64_t rtb, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt) {
+                                          int64_t n, int64_t rtb, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt,
+                                          const uint8_t *__restrict__ w2 = nullptr, const float *__restrict__ bias2 = nullptr) {
+    static_assert(!GU || R == 2, "gate and up take the places of two row tiles");
     extern __shared__ uint8_t smem[];
     using Fmt = Row1Fmt<DT>;
     constexpr int TB = TiledFmt<DT>::kTileBytes;
     constexpr int ES = XT == TURQ_ACT_F32 ? 4 : 2;
-    const int64_t rt0 = rtb * R, nrt = turq_tile_rows(n);
+    const int64_t rt0 = GU ? rtb : rtb * R, nrt = turq_tile_rows(n);
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -418,7 +422,8 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
     for (int r = 0; r < R; r++) {
 #pragma unroll
         for (int mm = 0; mm < M; mm++) acc[r][mm] = 0.0f;
-        wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+        if constexpr (GU) wrow[r] = (r == 0 ? w : w2) + rt0 * ntc * TB;
+        else wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
     }
 #pragma unroll
     for (int mm = 0; mm < M; mm++) xrow[mm] = (const uint8_t *)x + (mm < m ? mm : 0) * ldx * ES;
@@ -502,6 +507,27 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
         for (int mm = 0; mm < M; mm++) red[((r * M + mm) * nwaves + wave) * 64 + lane] = acc[r][mm];
     __syncthreads();
     const int n4 = lane >> 2, q = lane & 3;
+    if constexpr (GU) {
+        for (int mm = wave; mm < M; mm += nwaves) {
+            float sg = 0.0f, su = 0.0f;
+            for (int wv = 0; wv < nwaves; wv++) {
+                sg += red[(mm * nwaves + wv) * 64 + n4 + 16 * q];
+                su += red[((M + mm) * nwaves + wv) * 64 + n4 + 16 * q];
+            }
+            sg = sum4(sg);
+            su = sum4(su);
+            const int64_t col = rt0 * 16 + n4;
+            if (q == 0 && col < n && mm < m) {
+                const float gate = sg + (bias ? bias[col] : 0.0f), up = su + (bias2 ? bias2[col] : 0.0f);
+                const float out = gate / (1.0f + expf(-gate)) * up;  // SiLU
+                const int64_t at = (int64_t)mm * ldy + col;
+                if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, at, out);
+                else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, at, out);
+                else turq_store_out<TURQ_ACT_F16>(y, at, out);
+            }
+        }
+        return;
+    }
     for (int i = wave; i < R * M; i += nwaves) {
         const int r = i / M, mm = i - r * M;
         float s = 0.0f;
@@ -533,6 +559,16 @@ template <int DT, int XT, int P, int R, int M, int MAXT>
 __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt) {
     const Row1Pick p = row1_pick(a, (int)blockIdx.x);
     row1_body<DT, XT, P, R, M>(p.w, p.y, p.ldy, p.bias, p.n, (int64_t)((int)blockIdx.x - p.first), k, x, ldx, m, yt);
+}
+
+// gate_proj and up_proj of one MLP in one launch, the activation and the product applied before the store: workgroup b
+// takes row tile b of both weights
+template <int DT, int XT, int P, int M, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_row1_gateup_kernel(const uint8_t *__restrict__ wg, const uint8_t *__restrict__ wu,
+                                                                 const float *__restrict__ bg, const float *__restrict__ bu, int64_t n,
+                                                                 int64_t k, const void *__restrict__ x, int64_t ldx, int m,
+                                                                 void *__restrict__ y, int64_t ldy, int yt) {
+    row1_body<DT, XT, P, 2, M, true>(wg, y, ldy, bg, n, (int64_t)blockIdx.x, k, x, ldx, m, yt, wu, bu);
 }
 
 // weights of two formats that share an input (q, k Q4_K and v Q6_K of a Q4_K_M file) in one launch: the workgroup's weight
@@ -721,6 +757,66 @@ hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int 
     case TURQ_ACT_F32: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_F32>(l);
     case TURQ_ACT_BF16: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_BF16>(l);
     case TURQ_ACT_F16: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_F16>(l);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+namespace {
+template <int DT, int XT, int P, int M>
+hipError_t launch_gateup_final(const void *wg, const void *wu, const float *bg, const float *bu, int64_t n, int64_t k, const void *x,
+                               int64_t ldx, int m, void *y, int64_t ldy, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
+                               hipEvent_t ev1) {
+    const size_t lds = row1_lds<DT, P, 2, M>(nwaves);
+    const dim3 grid((unsigned)turq_tile_rows(n)), block((unsigned)(64 * nwaves));
+    if (ev0) {
+        hipExtLaunchKernelGGL((gemv_row1_gateup_kernel<DT, XT, P, M, 1024>), grid, block, (unsigned)lds, s, ev0, ev1, 0,
+                              (const uint8_t *)wg, (const uint8_t *)wu, bg, bu, n, k, x, ldx, m, y, ldy, yt);
+        return hipGetLastError();
+    }
+    gemv_row1_gateup_kernel<DT, XT, P, M, 1024><<<grid, block, lds, s>>>((const uint8_t *)wg, (const uint8_t *)wu, bg, bu, n, k, x, ldx,
+                                                                          m, y, ldy, yt);
+    return hipGetLastError();
+}
+
+template <int DT, int XT>
+hipError_t launch_gateup_p(const void *wg, const void *wu, const float *bg, const float *bu, int64_t n, int64_t k, const void *x,
+                           int64_t ldx, int m, void *y, int64_t ldy, int yt, int nwaves, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    // two weights double what a wave holds per column tile: at most two column tiles in flight
+    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
+    if (m == 2) {
+        if (per_wave <= 1) return launch_gateup_final<DT, XT, 1, 2>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+        return launch_gateup_final<DT, XT, 2, 2>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    }
+    if (per_wave <= 1) return launch_gateup_final<DT, XT, 1, 1>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    return launch_gateup_final<DT, XT, 2, 1>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+}
+
+template <int DT>
+hipError_t launch_gateup_x(int xt, const void *wg, const void *wu, const float *bg, const float *bu, int64_t n, int64_t k,
+                           const void *x, int64_t ldx, int m, void *y, int64_t ldy, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
+                           hipEvent_t ev1) {
+    switch (xt) {
+    case TURQ_ACT_F32: return launch_gateup_p<DT, TURQ_ACT_F32>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    case TURQ_ACT_BF16: return launch_gateup_p<DT, TURQ_ACT_BF16>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    case TURQ_ACT_F16: return launch_gateup_p<DT, TURQ_ACT_F16>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    default: return hipErrorInvalidValue;
+    }
+}
+}  // namespace
+
+// y[mm][c] = silu(x[mm] . gate[c] + bias_gate[c]) * (x[mm] . up[c] + bias_up[c]) for m = 1 or 2 activation rows: gate and up are
+// two tiled weights of one format and one shape [n, k]; rows of x 16-byte aligned
+hipError_t turq_launch_gemv_row1_gateup(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x,
+                                        int x_dtype, int64_t ldx, int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate,
+                                        const float *bias_up, int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+    if (nwaves < 1 || nwaves > 16 || m < 1 || m > 2 || k <= 0 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
+    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (n == 0) return hipSuccess;
+    switch (dtype) {
+    case TURQ_Q4_K: return launch_gateup_x<TURQ_Q4_K>(x_dtype, w_gate, w_up, bias_gate, bias_up, n, k, x, ldx, (int)m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q5_K: return launch_gateup_x<TURQ_Q5_K>(x_dtype, w_gate, w_up, bias_gate, bias_up, n, k, x, ldx, (int)m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q6_K: return launch_gateup_x<TURQ_Q6_K>(x_dtype, w_gate, w_up, bias_gate, bias_up, n, k, x, ldx, (int)m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q8_0: return launch_gateup_x<TURQ_Q8_0>(x_dtype, w_gate, w_up, bias_gate, bias_up, n, k, x, ldx, (int)m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
     default: return hipErrorInvalidValue;
     }
 }

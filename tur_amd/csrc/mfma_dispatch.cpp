@@ -128,6 +128,25 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
     return TURQ_OK;
 }
 
+// gate_proj and up_proj of an MLP with the activation and the product in the kernel: one or two activation rows (two: on
+// weights large enough for the one-row kernel, as in row1_takes), tiled weights of one format, 16-byte aligned rows
+int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m,
+                              int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, bool *taken) {
+    static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
+    *taken = false;
+    const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
+    if (no_fuse || !aligned || m < 1 || m > 2 || gate->dtype != up->dtype || !use_row1(gate->dtype) ||
+        gate->layout != TURQ_LAYOUT_TILED || up->layout != TURQ_LAYOUT_TILED)
+        return TURQ_OK;
+    if (!row1_takes(m, gate->dev_bytes + up->dev_bytes, gate->dtype)) return TURQ_OK;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+    TURQ_HIP(ctx, turq_launch_gemv_row1_gateup(gate->dtype, gate->dev, up->dev, gate->n, gate->k, x, xt, ldx, m, y, yt, ldy, bias_gate,
+                                               bias_up, pick_waves_row1(gate->k), ctx->stream, ev0, ev1));
+    *taken = true;
+    return TURQ_OK;
+}
+
 // Runs of neighbouring weights with the same format go out as one launch of the skinny kernel; the caller has
 // checked that all weights are tiled, share k and the device and that m <= TURQ_GEMV_MAX_M.  Up to
 // TURQ_GEMV_FUSED_MAX_M rows with 16-byte aligned activation rows the kernel converts the activations itself; otherwise
