@@ -80,6 +80,19 @@ int main(int argc, char **argv) {
                 if (std::fabs(y4[i] - y5[i]) > 1e-4f * (1.0f + std::fabs(y5[i]))) return fail("forward_multi differs from forward (second layer)");
         }
 
+        // silu(gate(x)) * up(x) in one call (same weight in both places): equal to the expression on the single call's result
+        {
+            turq::DeviceBuffer yg(dev, (size_t)m * n * 4);
+            turq::QMatMul::forward_gate_up(copy.qmatmul(), copy.qmatmul(), xd.ptr(), TURQ_ACT_F32, m, k, yg.ptr(), TURQ_ACT_F32, n);
+            dev.synchronize();
+            std::vector<float> y6((size_t)m * n);
+            yg.download(y6.data(), y6.size() * 4);
+            for (size_t i = 0; i < y.size(); i++) {
+                const double v = y[i], want = v / (1.0 + std::exp(-v)) * v;
+                if (std::fabs(y6[i] - want) > 1e-4 * (1.0 + std::fabs(want))) return fail("forward_gate_up differs from silu(forward) * forward");
+            }
+        }
+
         // dequantize of the norm weight (F32 tensor) is a copy
         std::vector<float> norm = b0.pp("attn_norm").get({k}, "weight").dequantize();
         std::printf("norm %zu %.9g %.9g\n", norm.size(), norm.front(), norm.back());

@@ -96,6 +96,23 @@ def test_qkv_projections_in_one_call(model):
         qlinear.QMatMul.forward_multi([l.qmatmul for l in layers], x[..., :-1].copy())
 
 
+def test_mlp_gate_up_in_one_call(model):
+    # Qwen3MLP::forward, first half (qwen3.rs:161-167): silu(gate_proj(x)) * up_proj(x)
+    dev, vb, tensors, _, _ = model
+    gate = qlinear.linear(HID, FFN, vb.pp("blk").pp(0).pp("ffn_gate"))
+    up = qlinear.linear(HID, FFN, vb.pp("blk").pp(0).pp("ffn_up"))
+    x = (np.random.default_rng(6).standard_normal((2, 3, HID)) / 64).astype(np.float32)
+    y = qlinear.QMatMul.forward_gate_up(gate.qmatmul, up.qmatmul, x)
+    assert y.shape == (2, 3, FFN)
+    g, u = gate.forward(x).astype(np.float64), up.forward(x).astype(np.float64)
+    assert rel_l2(y, (g / (1 + np.exp(-g)) * u).astype(np.float32)) <= 1e-6
+    with pytest.raises(capi.TurqError):
+        qlinear.QMatMul.forward_gate_up(gate.qmatmul, up.qmatmul, x[..., :-1].copy())
+    down = qlinear.linear(FFN, HID, vb.pp("blk").pp(0).pp("ffn_down"))
+    with pytest.raises(capi.TurqError):       # gate and up of different shapes
+        qlinear.QMatMul.forward_gate_up(gate.qmatmul, down.qmatmul, x)
+
+
 def test_bias_is_dequantized_at_load_and_added(model):
     dev, vb, tensors, bias, _ = model
     layer = qlinear.linear(HID, 96, vb.pp("blk").pp(0).pp("biased"))

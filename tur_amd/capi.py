@@ -16,6 +16,7 @@ ACT_F32, ACT_BF16, ACT_F16 = 0, 1, 2
 LAYOUT_NATIVE, LAYOUT_TILED = 0, 1
 MEM_HOST, MEM_DEVICE = 0, 1
 ALGO_AUTO, ALGO_SIMPLE, ALGO_GEMV, ALGO_GEMM = 0, 1, 2, 3
+ACTFN_SILU = 0
 
 # every symbol include/turq.h declares: (restype, argtypes)
 _SIGS = {

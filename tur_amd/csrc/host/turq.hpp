@@ -139,6 +139,14 @@ public:
         d.check(turq_qmatmul_multi(d.ctx(), (int)w.size(), w.data(), x_dev, x_dtype, m, ldx, ys_dev.data(), y_dtype, ldy.data(), nullptr,
                                    TURQ_MEM_DEVICE, TURQ_ALGO_AUTO));
     }
+    // silu(x gate^T) * (x up^T) of a device tensor, the first half of Qwen3MLP::forward (src/models/qwen3.rs:161-167): for one
+    // or two rows one kernel launch that writes the product, otherwise two products and an elementwise pass
+    static void forward_gate_up(const QMatMul &gate, const QMatMul &up, const void *x_dev, int x_dtype, int64_t m, int64_t ldx,
+                                void *y_dev, int y_dtype, int64_t ldy) {
+        const Device &d = gate.t_.device();
+        d.check(turq_qmatmul_gate_up(d.ctx(), gate.t_.handle(), up.t_.handle(), x_dev, x_dtype, m, ldx, y_dev, y_dtype, ldy, nullptr,
+                                     nullptr, TURQ_ACTFN_SILU, TURQ_MEM_DEVICE));
+    }
     const QTensor &qtensor() const { return t_; }
 
 private:

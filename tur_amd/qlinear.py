@@ -173,6 +173,30 @@ class QMatMul:
         return [y.reshape(lead + (y.shape[1],)) for y in ys]
 
 
+    @staticmethod
+    def forward_gate_up(gate: "QMatMul", up: "QMatMul", xs: np.ndarray, bias_gate: Optional[np.ndarray] = None,
+                        bias_up: Optional[np.ndarray] = None) -> np.ndarray:
+        """``silu(x @ gate.T) * (x @ up.T)``, the first half of ``Qwen3MLP::forward`` (src/models/qwen3.rs:161-167), through
+        ``turq_qmatmul_gate_up``.  With host arrays, as here, the two products go through the host path and are combined on the
+        host; with device-resident activations and one or two rows it is one kernel launch that writes the product."""
+        xs = np.asarray(xs)
+        n, k = gate.qtensor._n, gate.qtensor._k
+        if xs.ndim < 2 or xs.shape[-1] != k:
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch in matmul: input {xs.shape}, layers need last dim {k}")
+        if xs.dtype != np.float32 or not xs.flags["C_CONTIGUOUS"]:
+            raise TurqError(capi.ERR_INVALID, "forward_gate_up needs a contiguous f32 input")
+        lead = xs.shape[:-1]
+        m = int(np.prod(lead)) if lead else 1
+        y = np.empty((m, n), np.float32)
+        bg = None if bias_gate is None else np.ascontiguousarray(bias_gate, np.float32)
+        bu = None if bias_up is None else np.ascontiguousarray(bias_up, np.float32)
+        dev = gate.qtensor.device
+        capi.check(dev.L.turq_qmatmul_gate_up(dev.ctx, gate.qtensor.handle, up.qtensor.handle, capi.ptr(xs), capi.ACT_F32, m, k,
+                                              capi.ptr(y), capi.ACT_F32, n, capi.ptr(bg), capi.ptr(bu), capi.ACTFN_SILU,
+                                              capi.MEM_HOST), dev.ctx)
+        return y.reshape(lead + (n,))
+
+
 class LinearX:
     """``LinearX::Quantized { qmatmul, bias }`` (src/models/layers/linear.rs:8-31)."""
 
