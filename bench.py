@@ -146,15 +146,25 @@ class Bench:
                 warr = (ctypes.c_void_p * cnt)(*[w.value for w in layer[i:j]])
                 yarr = (ctypes.c_void_p * cnt)(*[y.value for y in self.y_dev[i:j]])
                 ldys = (ctypes.c_int64 * cnt)(*[mt[2] for mt in self.mats[i:j]])
-                self.groups.append((cnt, warr, self.x_dev[self.mats[i][3]], yarr, ldys, self.mats[i][3]))
+                fused = bool(getattr(self.args, "gate_up", False)) and [mt[0] for mt in self.mats[i:j]] == ["gate", "up"]
+                self.groups.append((cnt, warr, self.x_dev[self.mats[i][3]], yarr, ldys, self.mats[i][3], fused))
                 i = j
         self.step_bytes = layers * sum(algorithmic_bytes(dt, n, k, self.m, self.xbytes, self.ybytes) for _, dt, n, k in self.mats)
+        if getattr(self.args, "gate_up", False):
+            # turq_qmatmul_gate_up reads the shared activations once and writes one output for the pair
+            self.step_bytes -= layers * sum(self.m * (n * self.ybytes + k * self.xbytes) for lb, _, n, k in self.mats if lb == "up")
         self.step_flops = layers * sum(2 * self.m * n * k for _, _, n, k in self.mats)
 
     def step_eager(self):
         L, ctx, m, xt = self.L, self.ctx, self.m, self.xt
         if not self.args.single_calls:
-            for cnt, warr, x, yarr, ldys, k in self.groups:
+            for cnt, warr, x, yarr, ldys, k, fused in self.groups:
+                if fused:
+                    rc = L.turq_qmatmul_gate_up(ctx, warr[0], warr[1], x, xt, m, k, yarr[0], self.yt, ldys[0], None, None,
+                                                capi.ACTFN_SILU, capi.MEM_DEVICE)
+                    if rc:
+                        capi.check(rc, ctx)
+                    continue
                 rc = L.turq_qmatmul_multi(ctx, cnt, warr, x, xt, m, k, yarr, self.yt, ldys, None, capi.MEM_DEVICE, capi.ALGO_AUTO)
                 if rc:
                     capi.check(rc, ctx)
@@ -173,7 +183,10 @@ class Bench:
         self.step_eager()
         self.sync()
         worst = 0.0
+        fused = bool(getattr(self.args, "gate_up", False)) and not self.args.single_calls
         for (label, dt, n, k), y in zip(self.mats, self.y_dev):
+            if fused and label == "up":
+                continue      # its product went into the gate's output
             got = np.empty((self.m, n), np.float32 if self.yt == capi.ACT_F32 else np.uint16)
             capi.check(self.L.turq_memcpy_d2h(self.ctx, capi.ptr(got), y, got.nbytes), self.ctx)
             if self.yt != capi.ACT_F32:
@@ -182,6 +195,10 @@ class Bench:
             got = got[:, rows]
             sub = self.host_raw[label].reshape(n, -1)[rows].reshape(-1)
             want = orc.matmul_dequant(dt, self.x_host[k], sub, len(rows), k)
+            if fused and label == "gate":
+                from oracle import oracle_np as onp
+                sub_up = self.host_raw["up"].reshape(n, -1)[rows].reshape(-1)
+                want = onp.silu_mul(want, orc.matmul_dequant(dt, self.x_host[k], sub_up, len(rows), k))
             rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
             worst = max(worst, rel)
         bar = 1e-3 if self.yt == capi.ACT_F32 else 4e-3      # a bf16 store alone costs about 1.6e-3
@@ -232,7 +249,7 @@ class Bench:
             tfl = flops_per_launch / (avg_us * 1e-6) / 1e12
             roofline = {
                 "bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(tfl / MFMA_F16_PEAK_TFLOPS, 4), "traffic": TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls))),
+                "frac": round(tfl / MFMA_F16_PEAK_TFLOPS, 4), "traffic": (None if a.gate_up else TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls)))),
                 "kernel": "gemm_kq_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "flops_per_launch": int(flops_per_launch),
             }
@@ -241,7 +258,7 @@ class Bench:
         else:
             roofline = {
                 "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls))),
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": (None if a.gate_up else TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls)))),
                 "kernel": "gemv_row1_kernel" if self.m == 1 else "gemv_multi_frag_kernel / gemv_multi_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "algorithmic_bytes_per_launch": int(bytes_per_launch),
             }
@@ -253,7 +270,7 @@ class Bench:
             "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": f"{a.workload}: {self.desc}", "m": self.m, "layers": a.layers,
                        "activations": a.act, "outputs": a.out, "launch": "eager" if a.eager else "hip-graph",
-                       "calls": "turq_qmatmul" if a.single_calls else "turq_qmatmul_multi",
+                       "calls": "turq_qmatmul" if a.single_calls else ("turq_qmatmul_gate_up + turq_qmatmul_multi" if a.gate_up else "turq_qmatmul_multi"),
                        "step_bytes": int(self.step_bytes), "device": self.device, "compute_units": self.cus,
                        "max_rel_l2_vs_oracle": float(f"{rel:.3e}")},
             "whole_step_gbps": round(gbps, 1), "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
@@ -317,6 +334,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--single-calls", action="store_true",
                     help="one turq_qmatmul per matrix instead of turq_qmatmul_multi per group of matrices with a common input")
+    ap.add_argument("--gate-up", action="store_true",
+                    help="gate_proj / up_proj through turq_qmatmul_gate_up (SiLU and the product applied in the call, one output)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the workload, run a plain copy kernel of known size (dequantize of an F32 tensor: 256 MiB "
                          "read + 256 MiB written) three times, as the yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
