@@ -320,6 +320,56 @@ class Bench:
         self.L.turq_ctx_destroy(self.ctx)
 
 
+def run_embedding(args):
+    """Side measurement (not the headline): turq_embedding_lookup of --m token ids on a token_embd-sized table
+    [151936, 4096] Q6_K in the native layout, ids and output in HBM; a step is one call, replayed from a HIP graph."""
+    from oracle import capi as orc
+    L = capi.lib()
+    ctx = ctypes.c_void_p()
+    capi.check(L.turq_ctx_create(0, ctypes.byref(ctx)))
+    n, k, dt, count = 151936, 4096, synth.Q6_K, args.m
+    raw = synth.random_weight(dt, n, k, seed=77)
+    w = ctypes.c_void_p()
+    capi.check(L.turq_weight_upload(ctx, dt, n, k, capi.ptr(raw), raw.size, capi.LAYOUT_NATIVE, ctypes.byref(w)), ctx)
+    ids = np.random.default_rng(5).integers(0, n, count).astype(np.uint32)
+    idd, outd = ctypes.c_void_p(), ctypes.c_void_p()
+    capi.check(L.turq_dev_alloc(ctx, max(ids.nbytes, 16), ctypes.byref(idd)), ctx)
+    capi.check(L.turq_dev_alloc(ctx, count * k * 4, ctypes.byref(outd)), ctx)
+    capi.check(L.turq_memcpy_h2d(ctx, idd, capi.ptr(ids), ids.nbytes), ctx)
+    call = lambda: capi.check(L.turq_embedding_lookup(ctx, w, idd, count, outd, capi.ACT_F32, k, capi.MEM_DEVICE), ctx)
+    call()
+    got = np.empty((count, k), np.float32)
+    capi.check(L.turq_memcpy_d2h(ctx, capi.ptr(got), outd, got.nbytes), ctx)
+    rows = raw.reshape(n, -1)[ids[:64]].reshape(-1)
+    if not np.array_equal(got[:64].view(np.uint32), orc.dequantize(dt, rows).reshape(-1, k).view(np.uint32)):
+        raise SystemExit("bench: embedding rows differ from the oracle's dequantize")
+    reps = 64      # calls per graph: one graph launch costs the host about 20 us, more than a small lookup takes
+    capi.check(L.turq_graph_begin(ctx), ctx)
+    for _ in range(reps):
+        call()
+    g = ctypes.c_void_p()
+    capi.check(L.turq_graph_end(ctx, ctypes.byref(g)), ctx)
+    one = lambda: capi.check(L.turq_graph_launch(ctx, g), ctx)
+    for _ in range(args.warmup):
+        one()
+    capi.check(L.turq_sync(ctx), ctx)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one()
+    capi.check(L.turq_sync(ctx), ctx)
+    dt_s = (time.perf_counter() - t0) / (args.steps * reps)
+    nbytes = count * (k // 256 * 210 + 4 + 4 * k)      # blocks of the rows + the ids read, f32 rows written
+    print(json.dumps({"metric": "embedding lookup HBM GB/s (token_embd Q6_K 151936x4096, rows dequantized on gather)",
+                      "value": round(nbytes / dt_s / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                      "ms_per_step": round(dt_s * 1e3, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": "token_embd_q6k_8b", "ids": count, "layout": "native", "launch": "hip-graph of 64 calls", "step": "one call",
+                                 "bytes_per_step": nbytes, "checked": "first 64 rows bit-equal to the oracle"}}))
+    L.turq_graph_destroy(g)
+    capi.check(L.turq_weight_release(w))
+    L.turq_ctx_destroy(ctx)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -336,12 +386,16 @@ def main():
                     help="one turq_qmatmul per matrix instead of turq_qmatmul_multi per group of matrices with a common input")
     ap.add_argument("--gate-up", action="store_true",
                     help="gate_proj / up_proj through turq_qmatmul_gate_up (SiLU and the product applied in the call, one output)")
+    ap.add_argument("--embedding", action="store_true",
+                    help="side measurement: turq_embedding_lookup of --m ids on a [151936, 4096] Q6_K table instead of a matmul workload")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the workload, run a plain copy kernel of known size (dequantize of an F32 tensor: 256 MiB "
                          "read + 256 MiB written) three times, as the yardstick for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.embedding:
+        return run_embedding(args)
     if args.layers is None:
         # enough distinct weight copies that a step streams well over the 256 MB Infinity Cache
         per_layer = sum(synth.weight_nbytes(dt, n, k) for _, dt, n, k in WORKLOADS[args.workload][1])

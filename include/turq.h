@@ -134,6 +134,17 @@ int turq_untile_host(int ggml_dtype, int64_t n, int64_t k, const void *tiled, vo
  * src/models/layers/mod.rs:37; src/models/layers/norm.rs:84; src/models/layers/linear.rs:66). */
 int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem);
 
+/* Rows of the dequantized tensor picked by index: out[i, 0..k) = dequantize(w)[ids[i], :] for i < count, the same numbers
+ * as turq_dequantize bit for bit (then rounded once if out_dtype is bf16 or f16), without the f32 copy of the whole table
+ * (2.5 GB for the 151936 x 4096 token_embd of Qwen3-8B against 0.5 GB quantized).  Any ggml dtype turq_dequantize takes,
+ * either layout.  `out` has row stride ldo >= k elements; `mem` says where ids and out live.  An index >= n is
+ * TURQ_ERR_INVALID with host pointers; with device pointers, where the call cannot look at the indices, that row of `out`
+ * is filled with NaN.
+ * Replaces: candle's `Embedding::forward` (index_select) on the table that `layers::embedding` dequantizes whole at load
+ * (src/models/layers/mod.rs:30-37). */
+int turq_embedding_lookup(turq_ctx *ctx, const turq_weight *w, const uint32_t *ids, int64_t count, void *out, int out_dtype,
+                          int64_t ldo, int mem);
+
 /* ---- forward ---- */
 /* y[m, n] = x[m, k] * W^T  (+ bias[n] when bias != NULL).
  *   x: m rows of k elements of `x_dtype`, row stride ldx elements (ldx >= k);

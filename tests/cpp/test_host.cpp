@@ -93,6 +93,18 @@ int main(int argc, char **argv) {
             }
         }
 
+        // embedding rows of the quantized table = rows of its full dequantize
+        {
+            turq::QTensor table = b0.pp("ffn_gate").get({n, k}, "weight");
+            const std::vector<float> full = table.dequantize();
+            turq::Embedding emb(table, k);
+            const std::vector<uint32_t> ids = {0, (uint32_t)(n - 1), 5, 5};
+            const std::vector<float> rows = emb.forward(ids);
+            for (size_t i = 0; i < ids.size(); i++)
+                if (std::memcmp(rows.data() + i * k, full.data() + (size_t)ids[i] * k, (size_t)k * 4) != 0) return fail("embedding row differs from dequantize");
+            try { emb.forward({(uint32_t)n}); return fail("index outside the table accepted"); } catch (const turq::Error &) {}
+        }
+
         // dequantize of the norm weight (F32 tensor) is a copy
         std::vector<float> norm = b0.pp("attn_norm").get({k}, "weight").dequantize();
         std::printf("norm %zu %.9g %.9g\n", norm.size(), norm.front(), norm.back());

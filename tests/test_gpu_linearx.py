@@ -113,6 +113,26 @@ def test_mlp_gate_up_in_one_call(model):
         qlinear.QMatMul.forward_gate_up(gate.qmatmul, down.qmatmul, x)
 
 
+def test_embedding_over_the_quantized_table(model):
+    # layers::embedding (layers/mod.rs:11-50): table [vocab, hidden], forward(ids) -> ids.shape + [hidden]
+    dev, vb, tensors, _, _ = model
+    emb, vocab = qlinear.embedding(None, HID, vb.pp("output"))          # the 1000 x 512 Q8_0 tensor of the fixture
+    assert vocab == 1000
+    emb2, vocab2 = qlinear.embedding(1000, HID, vb.pp("output"))
+    assert vocab2 == 1000
+    with pytest.raises(capi.TurqError):
+        qlinear.embedding(999, HID, vb.pp("output"))                    # shape mismatch as in gguf_varbuilder.rs:62-66
+    ids = np.array([[0, 999, 7], [7, 7, 3]])
+    y = emb.forward(ids)
+    assert y.shape == (2, 3, HID)
+    raw = tensors["output.weight"][3]
+    table = orc.dequantize(Q8_0, raw).reshape(1000, HID)
+    assert np.array_equal(y, table[ids])
+    assert np.array_equal(emb2.forward(ids), y)
+    with pytest.raises(capi.TurqError):
+        emb.forward(np.array([1000]))
+
+
 def test_bias_is_dequantized_at_load_and_added(model):
     dev, vb, tensors, bias, _ = model
     layer = qlinear.linear(HID, 96, vb.pp("blk").pp(0).pp("biased"))

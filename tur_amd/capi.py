@@ -43,6 +43,7 @@ _SIGS = {
     "turq_tile_host": (c_int, [c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "turq_untile_host": (c_int, [c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "turq_dequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_int]),
+    "turq_embedding_lookup": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int]),
     "turq_qmatmul": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int, c_int]),
     "turq_qmatmul_multi": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p, c_void_p,
                                    c_int, c_int]),

@@ -342,6 +342,41 @@ int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem
     return TURQ_OK;
 }
 
+int turq_embedding_lookup(turq_ctx *ctx, const turq_weight *w, const uint32_t *ids, int64_t count, void *out, int out_dtype,
+                          int64_t ldo, int mem) {
+    TURQ_ENTER(ctx);
+    if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_embedding_lookup: null weight");
+    if (w->device != ctx->device) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_embedding_lookup: weight lives on device %d, context on %d", w->device, ctx->device);
+    if (!turq_dt_is_quant(w->dtype) && w->dtype != TURQ_F32 && w->dtype != TURQ_F16 && w->dtype != TURQ_BF16)
+        return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_embedding_lookup: unsupported dtype %d", w->dtype);
+    const int ob = turq_act_bytes(out_dtype);
+    if (!ob) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_embedding_lookup: output dtype %d", out_dtype);
+    if (count < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_embedding_lookup: count=%lld is negative", (long long)count);
+    if (ldo < w->k) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_embedding_lookup: ldo=%lld is smaller than the row length %lld", (long long)ldo, (long long)w->k);
+    if (count == 0 || w->k == 0) return TURQ_OK;
+    if (!ids || !out) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_embedding_lookup: null index or output pointer");
+    if (mem == TURQ_MEM_DEVICE) {
+        TURQ_HIP(ctx, turq_launch_gather_rows(w->dtype, w->layout, w->dev, w->n, w->k, ids, count, out, out_dtype, ldo, ctx->stream));
+        return TURQ_OK;
+    }
+    if (mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_embedding_lookup: bad mem %d", mem);
+    for (int64_t i = 0; i < count; i++)  // host indices can be checked before anything runs (candle's index_select refuses them too)
+        if ((int64_t)ids[i] >= w->n)
+            return turq_fail(ctx, TURQ_ERR_INVALID, "turq_embedding_lookup: index %u at position %lld is outside the table of %lld rows",
+                             ids[i], (long long)i, (long long)w->n);
+    const size_t row = (size_t)w->k * (size_t)ob;
+    int rc = turq_ctx_reserve(ctx, &ctx->stage_x, &ctx->stage_x_cap, (size_t)count * sizeof(uint32_t));
+    if (rc != TURQ_OK) return rc;
+    rc = turq_ctx_reserve(ctx, &ctx->stage_y, &ctx->stage_y_cap, row * (size_t)count);
+    if (rc != TURQ_OK) return rc;
+    TURQ_HIP(ctx, hipMemcpyAsync(ctx->stage_x, ids, (size_t)count * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
+    TURQ_HIP(ctx, turq_launch_gather_rows(w->dtype, w->layout, w->dev, w->n, w->k, (const uint32_t *)ctx->stage_x, count, ctx->stage_y,
+                                          out_dtype, w->k, ctx->stream));
+    TURQ_HIP(ctx, hipMemcpy2DAsync(out, (size_t)ldo * ob, ctx->stage_y, row, row, (size_t)count, hipMemcpyDeviceToHost, ctx->stream));
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return TURQ_OK;
+}
+
 // ---- forward ----
 
 static int qmatmul_device(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,

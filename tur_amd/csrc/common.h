@@ -131,6 +131,8 @@ int turq_ctx_reserve(turq_ctx *ctx, void **buf, size_t *cap, size_t need);
 
 // ---- kernel launchers implemented in the .hip translation units ----
 // All are asynchronous on `stream` and return hipGetLastError() of the launch.
+hipError_t turq_launch_gather_rows(int dtype, int layout, const void *w, int64_t n, int64_t k, const uint32_t *ids, int64_t count,
+                                   void *out, int out_dtype, int64_t ldo, hipStream_t stream);
 hipError_t turq_launch_dequant(int dtype, int layout, const void *w, int64_t n, int64_t k, float *out,
                                hipStream_t stream);
 hipError_t turq_launch_quantize_q8_0(const float *x, int64_t nblocks, void *out, hipStream_t stream);

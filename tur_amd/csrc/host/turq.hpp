@@ -170,6 +170,30 @@ private:
     std::optional<std::vector<float>> bias_;
 };
 
+// candle's Embedding over a table that stays quantized: forward gathers and dequantizes the rows of the given token ids where
+// the reference dequantizes the whole table at load (src/models/layers/mod.rs:30-37)
+class Embedding {
+public:
+    Embedding(QTensor table, int64_t hidden_size) : t_(std::move(table)) {
+        if (t_.cols() != hidden_size) throw Error(TURQ_ERR_SHAPE, "shape mismatch for weight: row length is not the hidden size");
+    }
+    // host ids -> host rows [ids.size(), hidden]
+    std::vector<float> forward(const std::vector<uint32_t> &ids) const {
+        std::vector<float> out(ids.size() * (size_t)t_.cols());
+        t_.device().check(turq_embedding_lookup(t_.device().ctx(), t_.handle(), ids.data(), (int64_t)ids.size(), out.data(), TURQ_ACT_F32,
+                                                t_.cols(), TURQ_MEM_HOST));
+        return out;
+    }
+    // device ids -> device rows, asynchronous on the device's stream
+    void forward(const uint32_t *ids_dev, int64_t count, void *out_dev, int out_dtype, int64_t ldo) const {
+        t_.device().check(turq_embedding_lookup(t_.device().ctx(), t_.handle(), ids_dev, count, out_dev, out_dtype, ldo, TURQ_MEM_DEVICE));
+    }
+    int64_t vocab_size() const { return t_.rows(); }
+
+private:
+    QTensor t_;
+};
+
 class QVarBuilder {
 public:
     static QVarBuilder from_gguf(const std::string &path, const Device &d, int layout = TURQ_LAYOUT_TILED) {

@@ -296,3 +296,34 @@ def linear(in_dim: int, out_dim: int, vb: QVarBuilder) -> LinearX:
         except TurqError:
             bias = None     # the reference looks the bias up with `.ok()`
     return LinearX(QMatMul.from_arc(qweight), bias)
+
+
+class Embedding:
+    """candle's ``Embedding`` over a table that stays quantized in HBM: ``forward(ids)`` gathers and dequantizes the rows
+    (``turq_embedding_lookup``) where the reference dequantizes the whole table at load (src/models/layers/mod.rs:30-37)."""
+
+    def __init__(self, table: QTensor, hidden_size: int):
+        if table._k != hidden_size:
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch for weight, got [{table._n}, {table._k}], expected [*, {hidden_size}]")
+        self.table = table
+        self.hidden_size = hidden_size
+
+    def forward(self, ids: np.ndarray) -> np.ndarray:
+        ids = np.asarray(ids)
+        if ids.dtype.kind not in "iu":
+            raise TurqError(capi.ERR_DTYPE, f"token ids must be integers, got {ids.dtype}")
+        if ids.size and (ids.min() < 0 or ids.max() >= self.table._n):
+            raise TurqError(capi.ERR_INVALID, f"index outside the table of {self.table._n} rows")
+        flat = np.ascontiguousarray(ids.reshape(-1), np.uint32)
+        out = np.empty((flat.size, self.hidden_size), np.float32)
+        dev = self.table.device
+        capi.check(dev.L.turq_embedding_lookup(dev.ctx, self.table.handle, capi.ptr(flat), flat.size, capi.ptr(out), capi.ACT_F32,
+                                               self.hidden_size, capi.MEM_HOST), dev.ctx)
+        return out.reshape(ids.shape + (self.hidden_size,))
+
+
+def embedding(vocab_size: Optional[int], hidden_size: int, vb: QVarBuilder) -> Tuple[Embedding, int]:
+    """GGUF arm of ``layers::embedding`` (src/models/layers/mod.rs:11-50): the shape check when the vocabulary size is given,
+    ``get_no_shape`` otherwise; returns the layer and the vocabulary size."""
+    t = vb.get((vocab_size, hidden_size), "weight") if vocab_size is not None else vb.get_no_shape("weight")
+    return Embedding(t, hidden_size), (vocab_size if vocab_size is not None else t._n)
