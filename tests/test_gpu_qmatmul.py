@@ -328,7 +328,8 @@ def test_one_row(gpu, dt, n, k):
 # ---------------------------------------------------------------------------------------------
 # several weights against the same activations (q/k/v, gate/up): one launch per run of equal formats
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("dts", [(Q4_K, Q4_K), (Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0), (Q4_K, Q4_K, Q6_K), (Q5_K, Q4_K, Q4_K, Q4_K, Q4_K, Q4_K)])
+@pytest.mark.parametrize("dts", [(Q4_K, Q4_K), (Q6_K, Q6_K, Q6_K), (Q8_0, Q8_0), (Q4_K, Q4_K, Q6_K), (Q5_K, Q5_K, Q6_K),
+                                 (Q5_K, Q4_K, Q4_K, Q4_K, Q4_K, Q4_K)])
 @pytest.mark.parametrize("m", [1, 3, 8, 20, 32])
 def test_multi_weight_launch(gpu, dts, m):
     k = 1024
@@ -348,11 +349,12 @@ def test_multi_weight_launch(gpu, dts, m):
         gpu.release(w)
 
 
-@pytest.mark.parametrize("dts", [(Q4_K, Q6_K), (Q4_K, Q4_K, Q4_K, Q6_K), (Q4_K, Q6_K, Q6_K), (Q6_K, Q4_K), (Q4_K,) * 4 + (Q6_K,)])
+@pytest.mark.parametrize("dts", [(Q4_K, Q6_K), (Q4_K, Q4_K, Q4_K, Q6_K), (Q4_K, Q6_K, Q6_K), (Q6_K, Q4_K), (Q4_K,) * 4 + (Q6_K,),
+                                 (Q5_K, Q5_K, Q6_K), (Q5_K, Q6_K, Q6_K), (Q4_K, Q5_K, Q6_K)])
 @pytest.mark.parametrize("k", [256, 4096, 12288])
 def test_two_formats_in_one_row_launch(gpu, dts, k):
-    # one activation row against Q4_K weights followed by Q6_K ones (q, k, v of a Q4_K_M file): one launch when they are at
-    # most four; other orders and longer lists go out run by run.  Either way every result equals the single call.
+    # one activation row against Q4_K (or Q5_K) weights followed by Q6_K ones (q, k, v of a Q4_K_M / Q5_K_M file): one launch
+    # when they are at most four; other orders and longer lists go out run by run.  Either way every result equals the single call.
     ns = [80, 16, 33, 272, 48][: len(dts)]
     raws = [synth.random_weight(dt, n, k, seed=7 * i + n + k) for i, (dt, n) in enumerate(zip(dts, ns))]
     ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
@@ -443,9 +445,10 @@ def test_four_rows_several_weights_one_launch(gpu, dt):
         gpu.release(w)
 
 
-def test_two_rows_two_formats(gpu):
-    # q, k (Q4_K) and v (Q6_K) against two activation rows: one launch of the two-format kernel
-    k, ns, dts = 4096, [4096, 1024, 1000], (Q4_K, Q4_K, Q6_K)
+@pytest.mark.parametrize("first", [Q4_K, Q5_K])
+def test_two_rows_two_formats(gpu, first):
+    # q, k (Q4_K or Q5_K) and v (Q6_K) against two activation rows: one launch of the two-format kernel
+    k, ns, dts = 4096, [4096, 1024, 1000], (first, first, Q6_K)
     raws = [synth.random_weight(dt, n, k, seed=n + i) for i, (dt, n) in enumerate(zip(dts, ns))]
     ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
     x = synth.random_activation(2, k, seed=8, bf16=True)

@@ -834,7 +834,10 @@ hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w, co
     }
 }
 
-bool turq_gemv_multi_mixed_supports(int dtype_a, int dtype_b) { return dtype_a == TURQ_Q4_K && dtype_b == TURQ_Q6_K; }
+// the pairs of a Q4_K_M and of a Q5_K_M file
+bool turq_gemv_multi_mixed_supports(int dtype_a, int dtype_b) {
+    return (dtype_a == TURQ_Q4_K || dtype_a == TURQ_Q5_K) && dtype_b == TURQ_Q6_K;
+}
 
 // count (2..4) weights of one k against prepared fragments (K-quant order) of m <= TURQ_GEMV_MAX_M rows: the first `second` of
 // format dtype_a, the others of dtype_b (a pair turq_gemv_multi_mixed_supports accepts); one row tile per workgroup.
@@ -861,6 +864,11 @@ hipError_t turq_launch_gemv_multi_mixed(int dtype_a, int dtype_b, int count, int
     ma.second = second;
     if (blocks == 0) return hipSuccess;
     if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    if (dtype_a == TURQ_Q5_K) {
+        if (m <= 16)
+            return launch_multi_frag_mixed_p<TURQ_Q5_K, TURQ_Q6_K, 1>(ma, (int)blocks, k, frags, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+        return launch_multi_frag_mixed_p<TURQ_Q5_K, TURQ_Q6_K, 2>(ma, (int)blocks, k, frags, m, y_dtype, nwaves, stream, ev_start, ev_stop);
+    }
     if (m <= 16)
         return launch_multi_frag_mixed_p<TURQ_Q4_K, TURQ_Q6_K, 1>(ma, (int)blocks, k, frags, m, y_dtype, nwaves, stream, ev_start, ev_stop);
     return launch_multi_frag_mixed_p<TURQ_Q4_K, TURQ_Q6_K, 2>(ma, (int)blocks, k, frags, m, y_dtype, nwaves, stream, ev_start, ev_stop);

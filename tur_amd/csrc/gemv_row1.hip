@@ -734,7 +734,10 @@ hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, con
     }
 }
 
-bool turq_gemv_row1_mixed_supports(int dtype_a, int dtype_b) { return dtype_a == TURQ_Q4_K && dtype_b == TURQ_Q6_K; }
+// the pairs of a Q4_K_M and of a Q5_K_M file
+bool turq_gemv_row1_mixed_supports(int dtype_a, int dtype_b) {
+    return (dtype_a == TURQ_Q4_K || dtype_a == TURQ_Q5_K) && dtype_b == TURQ_Q6_K;
+}
 
 // count (2..4) weights of one k against m activation rows: the first `second` of format dtype_a, the others of dtype_b
 // (a pair turq_gemv_row1_mixed_supports accepts); one row tile per workgroup.
@@ -753,6 +756,14 @@ hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int 
     if (k == 0) return hipErrorInvalidValue;
     l.k = k, l.x = x, l.ldx = ldx, l.m = (int)m, l.yt = y_dtype, l.nwaves = nwaves, l.rtiles = 1;
     l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop;
+    if (dtype_a == TURQ_Q5_K) {
+        switch (x_dtype) {
+        case TURQ_ACT_F32: return launch_mixed_p<TURQ_Q5_K, TURQ_Q6_K, TURQ_ACT_F32>(l);
+        case TURQ_ACT_BF16: return launch_mixed_p<TURQ_Q5_K, TURQ_Q6_K, TURQ_ACT_BF16>(l);
+        case TURQ_ACT_F16: return launch_mixed_p<TURQ_Q5_K, TURQ_Q6_K, TURQ_ACT_F16>(l);
+        default: return hipErrorInvalidValue;
+        }
+    }
     switch (x_dtype) {
     case TURQ_ACT_F32: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_F32>(l);
     case TURQ_ACT_BF16: return launch_mixed_p<TURQ_Q4_K, TURQ_Q6_K, TURQ_ACT_BF16>(l);
