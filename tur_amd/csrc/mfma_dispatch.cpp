@@ -141,8 +141,13 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
     if (!row1_takes(m, gate->dev_bytes + up->dev_bytes, gate->dtype)) return TURQ_OK;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+    // a wave holds a tile of each weight per column tile: half as many column tiles per wave as in the plain launch, i.e. twice
+    // the waves (K = 4096: 16 waves of one column tile; 8 waves of two cost the MLP step 2.7 %)
+    static const bool forced = getenv("TURQ_GEMV_WAVES") != nullptr;
+    int nwaves = pick_waves_row1(gate->k);
+    if (!forced) nwaves = (int)std::min<int64_t>({2 * (int64_t)nwaves, 16, turq_tile_cols(gate->k)});
     TURQ_HIP(ctx, turq_launch_gemv_row1_gateup(gate->dtype, gate->dev, up->dev, gate->n, gate->k, x, xt, ldx, m, y, yt, ldy, bias_gate,
-                                               bias_up, pick_waves_row1(gate->k), ctx->stream, ev0, ev1));
+                                               bias_up, nwaves, ctx->stream, ev0, ev1));
     *taken = true;
     return TURQ_OK;
 }
