@@ -85,3 +85,30 @@ def test_prefill_up_proj(gpu, m):
     want = orc.matmul_dequant(Q4_K, x, sub, len(rows), k)
     assert np.all(np.isfinite(y))
     assert rel_l2(y[:, rows], want) <= 1e-3
+
+
+def test_mlp_gate_up_and_token_embd(gpu):
+    # the two calls that widen the path, at Qwen3-8B sizes: gate / up with SiLU (12288 x 4096 Q4_K, one launch for one row, the two
+    # products plus an elementwise pass for sixteen) and token_embd rows (151936 x 4096 Q6_K) against the full dequantize
+    from oracle import oracle_np as onp
+    n, k = 12288, 4096
+    raw_g = synth.random_weight(Q4_K, n, k, seed=1)
+    raw_u = synth.random_weight(Q4_K, n, k, seed=2)
+    wg = gpu.upload(Q4_K, n, k, raw_g, capi.LAYOUT_TILED)
+    wu = gpu.upload(Q4_K, n, k, raw_u, capi.LAYOUT_TILED)
+    for m in (1, 2, 16):
+        x = synth.random_activation(m, k, seed=40 + m, bf16=True)
+        y = gpu.gate_up(wg, wu, x, n, k, x_dtype=capi.ACT_BF16)
+        want = onp.silu_mul(orc.matmul_dequant(Q4_K, x, raw_g, n, k), orc.matmul_dequant(Q4_K, x, raw_u, n, k))
+        assert rel_l2(y, want) <= 5e-5, m
+    gpu.release(wg)
+    gpu.release(wu)
+    n = 151936
+    raw = synth.random_weight(Q6_K, n, k, seed=3)
+    w = gpu.upload(Q6_K, n, k, raw, capi.LAYOUT_NATIVE)
+    ids = np.concatenate([[0, n - 1], np.random.default_rng(4).integers(0, n, 510)]).astype(np.uint32)
+    out = np.zeros((len(ids), k), np.float32)
+    capi.check(gpu.L.turq_embedding_lookup(gpu.ctx, w, capi.ptr(ids), len(ids), capi.ptr(out), capi.ACT_F32, k, capi.MEM_HOST), gpu.ctx)
+    rows = raw.reshape(n, -1)[ids].reshape(-1)
+    assert np.array_equal(out.view(np.uint32), orc.dequantize(Q6_K, rows).reshape(len(ids), k).view(np.uint32))
+    gpu.release(w)
