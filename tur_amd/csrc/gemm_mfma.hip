@@ -89,19 +89,27 @@ template <> struct GFmtWN<TURQ_Q6_K> { static constexpr int value = 2; };
 template <> struct GFmtWN<TURQ_Q8_0> { static constexpr int value = 1; };
 
 // geometry that depends on the format and the wave grid: WGM x WGN waves, WM x WN 32x32 tiles per wave
+// WGM_ = 3 is the WIDE form of the 1 x 4 grid: two 32x32 tiles per wave along n (workgroup tile 128 x 256), which halves the
+// activation bytes a launch pulls through the L2 per flop; to fit the LDS its rings are two deep (activation stages and
+// weight super-blocks alike) and the weights of a super-block are requested in two halves, at the last boundary of the
+// super-block before the previous one and at the first of the previous one.
 template <int DT, int WGM_> struct Geo {
-    static_assert(WGM_ == 1 || WGM_ == 2, "wave grid 2 x 2 or 1 x 4");
-    static constexpr int WGM = WGM_, WGN = 4 / WGM_, WM = MT / WGM_;
-    static constexpr int WN = WGM_ == 2 ? GFmtWN<DT>::value : 1;  // 1 x 4 waves: 128 rows of n, whatever the format
+    static_assert(WGM_ == 1 || WGM_ == 2 || WGM_ == 3, "wave grid 2 x 2, 1 x 4, or 1 x 4 with the wide tile");
+    static constexpr bool WIDE = WGM_ == 3;
+    static constexpr int WGM = WIDE ? 1 : WGM_, WGN = 4 / WGM, WM = MT / WGM;
+    static constexpr int WN = WGM_ == 2 ? GFmtWN<DT>::value : (WIDE ? 2 : 1);  // 1 x 4 waves: 128 (wide: 256) rows of n
+    static constexpr int RA = WIDE ? 2 : NA, RW = WIDE ? 2 : NW;               // ring depths
     static constexpr int BN = WGN * WN * 32;
     static constexpr int NT16 = BN / 16;                           // 16-row weight tiles per workgroup
     static constexpr int TB = TiledFmt<DT>::kTileBytes;
     static constexpr int W_BYTES = NT16 * TB;
     static constexpr int W_CHUNKS = (W_BYTES + 1023) / 1024;       // copies of 1 KiB; the last may be partial
     static constexpr int W_STRIDE = W_CHUNKS * 1024;               // ring stride: a partial last copy lands in padding
-    static constexpr int A_OFF = 0, W_OFF = NA * A_STAGE, S_OFF = W_OFF + NW * W_STRIDE;
+    static constexpr int CPW = 2 * ((W_CHUNKS + 7) / 8);           // wide form: weight copies per wave and super-block (even)
+    static constexpr int A_OFF = 0, W_OFF = RA * A_STAGE, S_OFF = W_OFF + RW * W_STRIDE;
     static constexpr int OUT_PITCH = WN * 32 + 8;                  // floats per staged result row: rows r and r + 4 land 32 banks apart
-    static_assert(W_CHUNKS <= 32, "weight copies: two per wave and group");
+    static_assert(WIDE || W_CHUNKS <= 32, "weight copies: two per wave and group");
+    static_assert(!WIDE || (CPW % 2 == 0 && CPW <= 24), "wide form: two halves of CPW / 2 copies per wave");
 };
 
 template <int... I, typename F> __device__ inline void static_for_impl(std::integer_sequence<int, I...>, F &&f) {
@@ -436,13 +444,15 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     // tiles re-read the last 16 bytes into the padding of the ring entry)
     const int tile0 = nb * G::NT16;
     const uint8_t *w_src = uniform_ptr(w + (size_t)tile0 * ntc * TB);  // + b * TB
-    uint32_t w_voff[4][2];
-    uint32_t w_dst[4][2];
+    // (wide form: copies wave, wave + 4, ... of the super-block, CPW per wave, in two halves)
+    constexpr int NG = G::WIDE ? G::CPW : 4, NI = G::WIDE ? 1 : 2;
+    uint32_t w_voff[NG][NI];
+    uint32_t w_dst[NG][NI];
 #pragma unroll
-    for (int g = 0; g < 4; g++)
+    for (int g = 0; g < NG; g++)
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            int c = i == 0 ? 4 * g + wave : 16 + 4 * g + wave;
+        for (int i = 0; i < NI; i++) {
+            int c = G::WIDE ? 4 * g + wave : (i == 0 ? 4 * g + wave : 16 + 4 * g + wave);
             c = c < G::W_CHUNKS ? c : G::W_CHUNKS - 1;
             uint32_t o = (uint32_t)c * 1024u + lane_off;
             o = o < (uint32_t)G::W_BYTES ? o : (uint32_t)G::W_BYTES - 16u;
@@ -456,17 +466,22 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     // ring offsets of the weight buffers of super-blocks b, b + 1, b + 2
     uint32_t wr0 = 0, wr1 = G::W_STRIDE, wr2 = 2 * G::W_STRIDE;
 
-    auto issue_a = [&](int bb, int ks) {  // stage (bb, ks) -> stage buffer ks
+    auto issue_a = [&](int bb, int ks) {  // stage (bb, ks) -> stage buffer ks (wide form: ks % 2)
         const uint8_t *src = a_src + ((size_t)(bb * 17 + 4 * ks) << 10);
-        dma_set<0>(lane_off, src, a_dst + (uint32_t)ks * A_STAGE);
+        dma_set<0>(lane_off, src, a_dst + (uint32_t)(ks % G::RA) * A_STAGE);
         dma_more<1024>(lane_off, src);
         dma_more<2048>(lane_off, src);
         dma_more<3072>(lane_off, src);
     };
     auto issue_w = [&](int bb, int g, uint32_t ring) {  // group g of super-block bb
         const uint8_t *src = w_src + (size_t)bb * TB;
-        dma_set<0>(w_voff[g][0], src, w_dst[g][0] + ring);
-        dma_set<0>(w_voff[g][1], src, w_dst[g][1] + ring);
+        if constexpr (G::WIDE) {  // half g of the wave's copies
+#pragma unroll
+            for (int i = 0; i < G::CPW / 2; i++) dma_set<0>(w_voff[g * (G::CPW / 2) + i][0], src, w_dst[g * (G::CPW / 2) + i][0] + ring);
+        } else {
+            dma_set<0>(w_voff[g][0], src, w_dst[g][0] + ring);
+            dma_set<0>(w_voff[g][1], src, w_dst[g][1] + ring);
+        }
     };
     auto issue_s = [&](int bb) {
         if constexpr (SUMS) dma_set<0>(lane_off, a_src + ((size_t)(bb * 17 + 16) << 10), s_dst + (uint32_t)(bb & 1) * S_BYTES);
@@ -489,14 +504,24 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
 
     // ---- prologue: super-block 0 complete, weights of 1 and the first group of 2 on their way ----
     const int last = ntc - 1;
+    if constexpr (G::WIDE) {
+        // stages 0 and 1 and the weights of super-block 0 complete, the first half of super-block 1 on its way
+        issue_a(0, 0);
+        issue_a(0, 1);
+        issue_w(0, 0, wr0);
+        issue_w(0, 1, wr0);
+        issue_w(1 < last ? 1 : last, 0, wr1);
+        issue_s(0);
+    } else {
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) issue_a(0, ks);
+        for (int ks = 0; ks < 4; ks++) issue_a(0, ks);
 #pragma unroll
-    for (int g = 0; g < 4; g++) issue_w(0, g, wr0);
+        for (int g = 0; g < 4; g++) issue_w(0, g, wr0);
 #pragma unroll
-    for (int g = 0; g < 4; g++) issue_w(1 < last ? 1 : last, g, wr1);
-    issue_w(2 < last ? 2 : last, 0, wr2);
-    issue_s(0);
+        for (int g = 0; g < 4; g++) issue_w(1 < last ? 1 : last, g, wr1);
+        issue_w(2 < last ? 2 : last, 0, wr2);
+        issue_s(0);
+    }
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -533,7 +558,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                     // next step's activation fragments come in while this step computes
                     static_for<WM>([&](auto I) {
                         constexpr int i = decltype(I)::value;
-                        lds_read128<ks * A_STAGE + i * 4096 + (st + 1) * 1024>(af[pa ^ 1][i], a_rd);
+                        lds_read128<(ks % G::RA) * A_STAGE + i * 4096 + (st + 1) * 1024>(af[pa ^ 1][i], a_rd);
                     });
                     wait_lds<WM>();  // everything but the reads just issued
 #pragma unroll
@@ -556,6 +581,20 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                     for (int i = 0; i < WM; i++) pin(af[1][i]);
                     // The next stage's copies were issued three boundaries ago; younger than them are that
                     // boundary's weight (and sums) copies and everything of the two boundaries since.
+                    if constexpr (G::WIDE) {
+                        // The next stage's copies were issued at the previous boundary, first of what was issued there; the
+                        // boundaries (b, 3) and (b, 0) add half a super-block of weights after them, (b, 1) the sums.  The
+                        // waits at (b, 2) and (b, 3) leave nothing in flight, which also completes super-block b + 1 before
+                        // its header is read.
+                        if constexpr (ks == 0 || ks == 1) wait_vmcnt<G::CPW / 2>(); else wait_vmcnt<0>();
+                        __builtin_amdgcn_s_barrier();
+                        asm volatile("" ::: "memory");
+                        // stage buffer ks % 2 is free: the stage after the next goes there
+                        if constexpr (ks < 2) issue_a(b, ks + 2); else issue_a(b1, ks - 2);
+                        if constexpr (ks == 0) issue_w(b1, 1, wr1);       // second half of super-block b + 1
+                        if constexpr (ks == 3) issue_w(b2, 0, wr0);       // first half of super-block b + 2: b's buffer is free
+                        if constexpr (ks == 1) issue_s(b1);
+                    } else {
                     if constexpr (ks == 0 || !SUMS) wait_vmcnt<14>(); else wait_vmcnt<15>();
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
@@ -563,6 +602,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                     issue_a(b1, ks);
                     if constexpr (ks == 3) issue_w(b3, 0, wr0); else issue_w(b2, ks + 1, wr2);
                     if constexpr (ks == 0) issue_s(b1);
+                    }
                     // first reads of the next stage, hidden under step 3's MFMAs
                     if constexpr (ks == 3 && SUMS) {
                         static_for<WM>([&](auto I) { lds_read128<decltype(I)::value * 1024>(sf[decltype(I)::value], s_cur); });
@@ -579,7 +619,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                             Fm::template read_hdr<j * 2 * TB>(hd[j], w_rd, wr1);
                         });
                     }
-                    static_for<WM>([&](auto I) { lds_read128<nks * A_STAGE + decltype(I)::value * 4096>(af[0][decltype(I)::value], a_rd); });
+                    static_for<WM>([&](auto I) { lds_read128<(nks % G::RA) * A_STAGE + decltype(I)::value * 4096>(af[0][decltype(I)::value], a_rd); });
                 }
                 // operand step 4 ks + st of the lane's 128 columns
                 half8v bop[WN];
@@ -608,8 +648,12 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
         });
         const uint32_t t = wr0;
         wr0 = wr1;
-        wr1 = wr2;
-        wr2 = t;
+        if constexpr (G::WIDE) {
+            wr1 = t;
+        } else {
+            wr1 = wr2;
+            wr2 = t;
+        }
     }
     wait_lds<0>();
     // The last stage boundary has issued the first LDS reads of a stage that does not exist.  Nothing uses them, but they
@@ -697,8 +741,9 @@ template <int DT, int WGM_>
 hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y, int y_dtype, int64_t ldy,
                        const float *bias, float wscale, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
     using G = Geo<DT, WGM_>;
-    constexpr int LDS_BYTES = G::S_OFF + (GFmt<DT>::SUMS ? NS * S_BYTES : 0);
-    static_assert(LDS_BYTES <= 160 * 1024 && 4 * G::WM * 32 * G::OUT_PITCH * 4 <= LDS_BYTES, "LDS of one workgroup; result staging fits");
+    constexpr int RING_BYTES = G::S_OFF + (GFmt<DT>::SUMS ? NS * S_BYTES : 0), STAGING_BYTES = 4 * G::WM * 32 * G::OUT_PITCH * 4;
+    constexpr int LDS_BYTES = RING_BYTES > STAGING_BYTES ? RING_BYTES : STAGING_BYTES;
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS of one workgroup: the rings, or the staged results after the main loop");
     // per-lane weight offsets are 32-bit
     if ((uint64_t)G::NT16 * (uint64_t)(k / 256) * G::TB >= (1ull << 32)) return hipErrorInvalidValue;
     static const hipError_t attr =
@@ -729,17 +774,38 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
     if (n == 0 || m == 0) return hipSuccess;
     if (k <= 0 || k % 256 != 0 || !(wscale >= 6.103515625e-5f && wscale <= 32768.0f)) return hipErrorInvalidValue;
     static const bool tall = getenv("TURQ_GEMM_GRID_2X2") == nullptr;  // Q5_K / Q6_K: 1 x 4 waves unless told otherwise
+    // The wide tile (128 x 256, Geo<.., 3>) pulls fewer activation bytes through the L2 per flop (Q4_K: + 12 % at m = 2048 and
+    // 4096; LM head Q5_K / Q6_K: + 4 .. 21 % from m = 64 to 512) but makes fewer, larger workgroups: it is taken where its
+    // gain outweighs what its workgroup count loses in the last round over the CUs, and only where there are workgroups
+    // enough to matter.  TURQ_GEMM_WIDE = 0 / 1 overrides the rule.
+    static const int wide_env = [] { const char *e = getenv("TURQ_GEMM_WIDE"); return e ? (atoi(e) != 0 ? 1 : 0) : -1; }();
+    const int64_t cus = compute_units > 0 ? compute_units : 256;
+    auto fill = [&](int64_t bn, int64_t *count) {  // share of the CU-rounds a launch with this tile width keeps busy
+        const int64_t wgs = ((n + bn - 1) / bn) * ((m + BM - 1) / BM), rounds = (wgs + cus - 1) / cus;
+        if (count) *count = wgs;
+        return (double)wgs / (double)(rounds * cus);
+    };
+    int64_t wide_wgs = 0;
+    const double fill_wide = fill(256, &wide_wgs);
+    auto pick_wide = [&](int64_t bn_other, double gain) {
+        if (wide_env >= 0) return wide_env == 1;
+        return 2 * wide_wgs >= cus && fill_wide * gain >= fill(bn_other, nullptr);
+    };
     switch (dtype) {
     case TURQ_Q4_K:
+        if (wide_env == 1) return launch_gemm<TURQ_Q4_K, 3>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
         // 128 x 192 tiles of 2 x 2 waves, unless the 128 x 128 tiles of the 1 x 4 grid still fit the machine in one round:
         // then there are half as many again to spread (m = 128: 96 workgroups instead of 64, 34 us instead of 45)
         if (compute_units > 0 && ((n + 127) / 128) * ((m + BM - 1) / BM) <= compute_units)
             return launch_gemm<TURQ_Q4_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+        if (pick_wide(192, 1.10)) return launch_gemm<TURQ_Q4_K, 3>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
         return launch_gemm<TURQ_Q4_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
     case TURQ_Q5_K:
+        if (pick_wide(128, 1.25)) return launch_gemm<TURQ_Q5_K, 3>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
         if (tall) return launch_gemm<TURQ_Q5_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
         return launch_gemm<TURQ_Q5_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
     case TURQ_Q6_K:
+        if (pick_wide(128, 1.25)) return launch_gemm<TURQ_Q6_K, 3>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
         if (tall) return launch_gemm<TURQ_Q6_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
         return launch_gemm<TURQ_Q6_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
     case TURQ_Q8_0: return launch_gemm<TURQ_Q8_0, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
