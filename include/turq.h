@@ -178,11 +178,12 @@ enum { TURQ_ACTFN_SILU = 0 };
 
 /* The first half of the reference's MLP in one call: y[m, n] = act(x * gate^T + bias_gate) * (x * up^T + bias_up), with
  * act = SiLU, v / (1 + exp(-v)), computed in f32.  gate and up are two weights of one shape [n, k]; x, y, the strides, the
- * biases (NULL: none) and `mem` as in turq_qmatmul.  With device pointers, tiled weights of one format and one activation
- * row (two on 8 MiB of weights and more) the activation and the product are applied inside the matmul kernel, which then is
- * the one launch of the call and writes one output instead of two; every other case computes the two products through
- * turq_qmatmul_multi into scratch memory of the context (which grows on demand, never inside a graph capture) and combines
- * them in one elementwise pass.  Errors as turq_qmatmul; gate and up of different shapes: TURQ_ERR_SHAPE; an activation other
+ * biases (NULL: none) and `mem` as in turq_qmatmul.  With device pointers, tiled weights of one format and up to 32
+ * activation rows the activation and the product are applied inside the matmul kernel, which writes one output instead of
+ * two: for one row (two on 8 MiB of weights and more) that kernel is the one launch of the call, for more rows it follows
+ * one preparation of the activations (scratch memory of the context, which grows on demand, never inside a graph
+ * capture).  Every other case computes the two products through turq_qmatmul_multi into scratch memory of the context and
+ * combines them in one elementwise pass.  Errors as turq_qmatmul; gate and up of different shapes: TURQ_ERR_SHAPE; an activation other
  * than TURQ_ACTFN_SILU: TURQ_ERR_INVALID.
  * Replaces: `x.apply(&self.gate_proj)?.apply(&self.act_fn)?` times `x.apply(&self.up_proj)?` in `Qwen3MLP::forward`
  * (src/models/qwen3.rs:161-167; the Granite MLP, src/models/granite_41.rs:151-155, has the same form). */

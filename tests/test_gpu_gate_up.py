@@ -44,7 +44,8 @@ def expected(dt, x, raw_g, raw_u, n, k, bg=None, bu=None):
 @pytest.mark.parametrize("dt", ALL)
 @pytest.mark.parametrize("m", [1, 2, 3, 8, 40])
 def test_gate_up_matches_the_two_calls(gpu, dt, m):
-    # one row: inside the one-row kernel; more rows on this small pair: two products + the elementwise pass (m = 40: the GEMM)
+    # one row: inside the one-row kernel; up to 32 rows: inside the prepared-fragment kernel; m = 40: the two GEMM products + the
+    # elementwise pass
     n, k = 200, 1024 + (64 if dt == Q8_0 else 0)
     raw_g = synth.random_weight(dt, n, k, seed=dt + 1)
     raw_u = synth.random_weight(dt, n, k, seed=dt + 2)

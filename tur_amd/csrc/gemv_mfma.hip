@@ -503,10 +503,14 @@ __global__ void __launch_bounds__(MAXT) gemv_multi_kernel(MultiArgs a, int64_t k
 
 // Prepared fragments, R row tiles per workgroup: a wave applies the fragments of a column tile, once fetched, to R weight
 // tiles, which divides the fragment traffic through L2 (9 - 18 KiB per column tile against 2 - 4 KiB per weight tile) by R.
-template <int DT, int MT, int P, int R>
+// GU (R = 2): the two row tiles are row tile rtg of a gate weight (w) and of an up weight (w2) of one shape, and what is stored
+// is silu(gate) * up (src/models/qwen3.rs:161-167).
+template <int DT, int MT, int P, int R, bool GU = false>
 __device__ __forceinline__ void gemv_frag_body(const uint8_t *__restrict__ w, int64_t n, int64_t k, const void *__restrict__ frags,
                                                int64_t m, int mpad, void *__restrict__ y, int yt, int64_t ldy,
-                                               const float *__restrict__ bias, int64_t rtg) {
+                                               const float *__restrict__ bias, int64_t rtg, const uint8_t *__restrict__ w2 = nullptr,
+                                               const float *__restrict__ bias2 = nullptr) {
+    static_assert(!GU || R == 2, "gate and up take the places of two row tiles");
     extern __shared__ uint8_t smem[];
     constexpr int NQ = DT == TURQ_Q8_0 ? TURQ_NQ_Q8_0 : TURQ_NQ_KQUANT;
     constexpr int TB = TiledFmt<DT>::kTileBytes;
@@ -514,7 +518,7 @@ __device__ __forceinline__ void gemv_frag_body(const uint8_t *__restrict__ w, in
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nwaves = blockDim.x >> 6;
     const int64_t ntc = turq_tile_cols(k), nrt = turq_tile_rows(n);
-    const int64_t rt0 = rtg * R;
+    const int64_t rt0 = GU ? rtg : rtg * R;
     const int64_t tile_chunks = (int64_t)NQ * 4 * mpad;
     const int64_t mt_stride = ntc * tile_chunks;
     float4v *red = (float4v *)smem;
@@ -525,7 +529,10 @@ __device__ __forceinline__ void gemv_frag_body(const uint8_t *__restrict__ w, in
         for (int mt = 0; mt < MT; mt++) acc[r][mt] = float4v{0.f, 0.f, 0.f, 0.f};
     const uint8_t *wrow[R];  // row tiles past the end re-read the last one; their results are not stored
 #pragma unroll
-    for (int r = 0; r < R; r++) wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+    for (int r = 0; r < R; r++) {
+        if constexpr (GU) wrow[r] = (r == 0 ? w : w2) + rt0 * ntc * TB;
+        else wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+    }
     GOff go = lane_offsets(lane, mpad);
     for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
         WRegs<DT> wr[P][R];
@@ -562,6 +569,20 @@ __device__ __forceinline__ void gemv_frag_body(const uint8_t *__restrict__ w, in
     }
     // lane (nn, g) holds y[16 mt + 4 g + i][16 (rt0 + r) + nn], i = 0..3
     const int nn = lane & 15, g = lane >> 4;
+    if constexpr (GU) {
+        const int64_t col = rt0 * 16 + nn;
+        if (col >= n) return;
+        const float bg = bias ? bias[col] : 0.0f, bu = bias2 ? bias2[col] : 0.0f;
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int64_t row = 16 * mt + 4 * g + i;
+                const float gate = acc[0][mt][i] + bg, up = acc[1][mt][i] + bu;
+                if (row < m) turq_store_any(y, yt, row * ldy + col, gate / (1.0f + expf(-gate)) * up);
+            }
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int64_t col = (rt0 + r) * 16 + nn;
@@ -594,6 +615,16 @@ __global__ void __launch_bounds__(MAXT) gemv_multi_frag_kernel(MultiArgs a, int6
         }
     if constexpr (R == 1) gemv_body<DT, MT, TURQ_ACT_F16, false, 1, P>(w, n, k, frags, 0, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
     else gemv_frag_body<DT, MT, P, R>(w, n, k, frags, m, mpad, y, yt, ldy, bias, (int64_t)(blk - first));
+}
+
+// gate_proj and up_proj of one MLP against prepared fragments, SiLU and the product applied before the store: workgroup b takes
+// row tile b of both weights
+template <int DT, int MT, int P, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_gateup_frag_kernel(const uint8_t *__restrict__ wg, const uint8_t *__restrict__ wu,
+                                                                 const float *__restrict__ bg, const float *__restrict__ bu, int64_t n,
+                                                                 int64_t k, const void *__restrict__ frags, int64_t m, int mpad,
+                                                                 void *__restrict__ y, int64_t ldy, int yt) {
+    gemv_frag_body<DT, MT, P, 2, true>(wg, n, k, frags, m, mpad, y, yt, ldy, bg, (int64_t)blockIdx.x, wu, bu);
 }
 
 // prepared fragments, weights of two formats with the same fragment order (Q4_K weights followed by Q6_K ones: q, k and v of a
@@ -890,6 +921,54 @@ hipError_t turq_launch_gemv_mfma(int dtype, const void *w, int64_t n, int64_t k,
     case TURQ_Q5_K: return launch_x<TURQ_Q5_K>(x_dtype, fused, a);
     case TURQ_Q6_K: return launch_x<TURQ_Q6_K>(x_dtype, fused, a);
     case TURQ_Q8_0: return launch_x<TURQ_Q8_0>(x_dtype, fused, a);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+namespace {
+template <int DT, int MT, int P>
+hipError_t launch_gateup_frag_final(const void *wg, const void *wu, const float *bg, const float *bu, int64_t n, int64_t k,
+                                    const void *frags, int64_t m, void *y, int64_t ldy, int yt, int nwaves, hipStream_t s,
+                                    hipEvent_t ev0, hipEvent_t ev1) {
+    const int mpad = MT > 1 ? 16 : turq_mpad(m);
+    const size_t lds = nwaves > 1 ? (size_t)nwaves * 2 * MT * 64 * sizeof(float4v) : 0;
+    const dim3 grid((unsigned)turq_tile_rows(n)), block((unsigned)(64 * nwaves));
+    if (ev0) {
+        hipExtLaunchKernelGGL((gemv_gateup_frag_kernel<DT, MT, P, 256>), grid, block, (unsigned)lds, s, ev0, ev1, 0, (const uint8_t *)wg,
+                              (const uint8_t *)wu, bg, bu, n, k, frags, m, mpad, y, ldy, yt);
+        return hipGetLastError();
+    }
+    gemv_gateup_frag_kernel<DT, MT, P, 256><<<grid, block, lds, s>>>((const uint8_t *)wg, (const uint8_t *)wu, bg, bu, n, k, frags, m, mpad,
+                                                                      y, ldy, yt);
+    return hipGetLastError();
+}
+
+template <int DT>
+hipError_t launch_gateup_frag(const void *wg, const void *wu, const float *bg, const float *bu, int64_t n, int64_t k, const void *frags,
+                              int64_t m, void *y, int64_t ldy, int yt, int nwaves, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
+    if (m <= 16) {
+        if (per_wave <= 1) return launch_gateup_frag_final<DT, 1, 1>(wg, wu, bg, bu, n, k, frags, m, y, ldy, yt, nwaves, s, ev0, ev1);
+        return launch_gateup_frag_final<DT, 1, 2>(wg, wu, bg, bu, n, k, frags, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    }
+    if (per_wave <= 1) return launch_gateup_frag_final<DT, 2, 1>(wg, wu, bg, bu, n, k, frags, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    return launch_gateup_frag_final<DT, 2, 2>(wg, wu, bg, bu, n, k, frags, m, y, ldy, yt, nwaves, s, ev0, ev1);
+}
+}  // namespace
+
+// y[r][c] = silu(x[r] . gate[c] + bias_gate[c]) * (x[r] . up[c] + bias_up[c]) for m <= TURQ_GEMV_MAX_M rows whose fragments
+// turq_launch_act_prep prepared for this format; gate and up: two tiled weights of one format and shape [n, k]; up to four waves
+hipError_t turq_launch_gemv_gateup_frag(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *frags,
+                                        int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up,
+                                        int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+    if (nwaves < 1 || nwaves > 4 || m < 1 || m > TURQ_GEMV_MAX_M || k <= 0 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
+    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (n == 0) return hipSuccess;
+    switch (dtype) {
+    case TURQ_Q4_K: return launch_gateup_frag<TURQ_Q4_K>(w_gate, w_up, bias_gate, bias_up, n, k, frags, m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q5_K: return launch_gateup_frag<TURQ_Q5_K>(w_gate, w_up, bias_gate, bias_up, n, k, frags, m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q6_K: return launch_gateup_frag<TURQ_Q6_K>(w_gate, w_up, bias_gate, bias_up, n, k, frags, m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q8_0: return launch_gateup_frag<TURQ_Q8_0>(w_gate, w_up, bias_gate, bias_up, n, k, frags, m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
     default: return hipErrorInvalidValue;
     }
 }

@@ -159,6 +159,9 @@ hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w_til
 // (turq_gemv_row1_rows() = 4); Q6_K, whose 16 sub-blocks fill the A rows, and Q8_0 take a chain per row and stop at two.
 #define TURQ_ROW1_MAX_M 4
 int turq_gemv_row1_rows(int dtype);
+hipError_t turq_launch_gemv_gateup_frag(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *frags,
+                                        int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up,
+                                        int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
 bool turq_gemv_row1_supports(int dtype);
 hipError_t turq_launch_gemv_row1_gateup(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x,
                                         int x_dtype, int64_t ldx, int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate,

@@ -137,11 +137,25 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
     static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
     *taken = false;
     const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
-    if (no_fuse || !aligned || m < 1 || m > 2 || gate->dtype != up->dtype || !use_row1(gate->dtype) ||
-        gate->layout != TURQ_LAYOUT_TILED || up->layout != TURQ_LAYOUT_TILED)
+    if (m < 1 || m > TURQ_GEMV_MAX_M || gate->dtype != up->dtype || !turq_dt_is_quant(gate->dtype) || gate->layout != TURQ_LAYOUT_TILED ||
+        up->layout != TURQ_LAYOUT_TILED)
         return TURQ_OK;
-    if (!row1_takes(m, gate->dev_bytes + up->dev_bytes, gate->dtype)) return TURQ_OK;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    if (no_fuse || !aligned || m > 2 || !use_row1(gate->dtype) || !row1_takes(m, gate->dev_bytes + up->dev_bytes, gate->dtype)) {
+        // up to 32 rows: fragments prepared once, then one launch whose workgroups take row tile b of both weights (the shape
+        // of the two-row-tile kernel: at most four waves) and store the product
+        static const bool no_frag = getenv("TURQ_GATEUP_NO_FRAG") != nullptr;
+        if (no_frag) return TURQ_OK;
+        int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep_bytes(gate->dtype, m, gate->k));
+        if (rc != TURQ_OK) return rc;
+        TURQ_HIP(ctx, turq_launch_act_prep(gate->dtype, x, xt, m, gate->k, ldx, ctx->act_prep, ctx->stream));
+        TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+        const int nw = std::min(pick_waves(ctx, gate->n, gate->k), 4);
+        TURQ_HIP(ctx, turq_launch_gemv_gateup_frag(gate->dtype, gate->dev, up->dev, gate->n, gate->k, ctx->act_prep, m, y, yt, ldy,
+                                                   bias_gate, bias_up, nw, ctx->stream, ev0, ev1));
+        *taken = true;
+        return TURQ_OK;
+    }
     TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
     // a wave holds a tile of each weight per column tile: half as many column tiles per wave as in the plain launch, i.e. twice
     // the waves (K = 4096: 16 waves of one column tile; 8 waves of two cost the MLP step 2.7 %)
