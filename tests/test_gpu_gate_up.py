@@ -42,7 +42,7 @@ def expected(dt, x, raw_g, raw_u, n, k, bg=None, bu=None):
 
 
 @pytest.mark.parametrize("dt", ALL)
-@pytest.mark.parametrize("m", [1, 2, 3, 8, 40])
+@pytest.mark.parametrize("m", [1, 2, 3, 8, 16, 20, 32, 40])
 def test_gate_up_matches_the_two_calls(gpu, dt, m):
     # one row: inside the one-row kernel; up to 32 rows: inside the prepared-fragment kernel; m = 40: the two GEMM products + the
     # elementwise pass
@@ -87,6 +87,27 @@ def test_gate_up_two_rows_on_large_weights(gpu, dt):
         # (f16 activations; an f16 OUTPUT could not hold these synthetic products, which pass 65504)
         yh = gpu.gate_up(wg, wu, f16_round(x), n, k, x_dtype=capi.ACT_F16)
         assert rel_l2(yh, expected(dt, f16_round(x), raw_g, raw_u, n, k)) <= 5e-5, m
+    gpu.release(wg)
+    gpu.release(wu)
+
+
+@pytest.mark.parametrize("dt", ALL)
+def test_gate_up_several_rows_bias_strides_and_stores(gpu, dt):
+    # the prepared-fragment form on a pair large enough for several waves per workgroup: biases, row strides, bf16 in and out
+    n, k = 1030, 4096 + (32 if dt == Q8_0 else 0)
+    raw_g = synth.random_weight(dt, n, k, seed=61)
+    raw_u = synth.random_weight(dt, n, k, seed=62)
+    wg = gpu.upload(dt, n, k, raw_g, capi.LAYOUT_TILED)
+    wu = gpu.upload(dt, n, k, raw_u, capi.LAYOUT_TILED)
+    bg = np.random.default_rng(3).standard_normal(n).astype(np.float32)
+    bu = np.random.default_rng(4).standard_normal(n).astype(np.float32)
+    for m in (5, 16, 29):
+        x = synth.random_activation(m, k, seed=70 + m, bf16=True)
+        want = expected(dt, x, raw_g, raw_u, n, k, bg, bu)
+        y = gpu.gate_up(wg, wu, x, n, k, bias_gate=bg, bias_up=bu, ldx=k + 8, ldy=n + 2)
+        assert rel_l2(y, want) <= 5e-5, m
+        yb = gpu.gate_up(wg, wu, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16, bias_gate=bg, bias_up=bu)
+        assert rel_l2(yb, want) <= 4e-3, m
     gpu.release(wg)
     gpu.release(wu)
 
