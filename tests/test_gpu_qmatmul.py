@@ -505,16 +505,17 @@ def test_one_row_launch_shapes(row_tiles, in_flight):
     assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-1000:]
 
 
-# The prefill GEMM picks its tile (128 x 128, 128 x 192 or the wide 128 x 256 with two-deep rings) from the problem size; the
-# small matrices of the tests above would never reach the wide one, so they run once more in a child process with it forced,
-# and once with it forbidden (the rule takes it for some of the full-size cases).
-@pytest.mark.parametrize("wide", ["1", "0"])
-def test_prefill_tile_shapes(wide):
+# The prefill GEMM picks its tile (128 x 128, 128 x 192, the wide 128 x 256 with two-deep rings, or the low 64 x 128 for launches
+# that would leave CUs idle) from the problem size; the small matrices of the tests above would never reach the wide one and
+# always take the low one, so they run once more in child processes with each of the two forced and forbidden (the rule takes
+# the wide tile for some of the full-size cases).
+@pytest.mark.parametrize("switch,value", [("TURQ_GEMM_WIDE", "1"), ("TURQ_GEMM_WIDE", "0"), ("TURQ_GEMM_LOW", "1"), ("TURQ_GEMM_LOW", "0")])
+def test_prefill_tile_shapes(switch, value):
     import os
     import subprocess
     import sys
 
-    env = dict(os.environ, TURQ_GEMM_WIDE=wide)
+    env = dict(os.environ, **{switch: value})
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "-k", "(prefill or more_rows) and not tile_shapes",
                           "-p", "no:cacheprovider", os.path.join(root, "tests", "test_gpu_qmatmul.py"),

@@ -94,10 +94,16 @@ template <> struct GFmtWN<TURQ_Q8_0> { static constexpr int value = 1; };
 // weight super-blocks alike) and the weights of a super-block are requested in two halves, at the last boundary of the
 // super-block before the previous one and at the first of the previous one.
 template <int DT, int WGM_> struct Geo {
-    static_assert(WGM_ == 1 || WGM_ == 2 || WGM_ == 3, "wave grid 2 x 2, 1 x 4, or 1 x 4 with the wide tile");
-    static constexpr bool WIDE = WGM_ == 3;
-    static constexpr int WGM = WIDE ? 1 : WGM_, WGN = 4 / WGM, WM = MT / WGM;
-    static constexpr int WN = WGM_ == 2 ? GFmtWN<DT>::value : (WIDE ? 2 : 1);  // 1 x 4 waves: 128 (wide: 256) rows of n
+    // WGM_ = 4 is the LOW form for launches that would leave CUs idle: 64 rows of m (two m-tiles) by 128 of n, four waves of
+    // 64 x 32, i.e. twice the workgroups of the 128 x 128 tile; it uses the wide form's two-deep rings and copy schedule.
+    static_assert(WGM_ >= 1 && WGM_ <= 4, "wave grid 2 x 2, 1 x 4, or 1 x 4 with the wide or the low tile");
+    static constexpr bool LOW = WGM_ == 4;
+    static constexpr bool WIDE = WGM_ == 3 || LOW;                 // (the ring and copy schedule, not the width)
+    static constexpr int GMT = LOW ? 2 : MT;                       // m-tiles per workgroup
+    static constexpr int GBM = GMT * 32;
+    static constexpr int GA_STAGE = GMT * 4 * 1024;
+    static constexpr int WGM = WIDE ? 1 : WGM_, WGN = 4 / WGM, WM = GMT / WGM;
+    static constexpr int WN = WGM_ == 2 ? GFmtWN<DT>::value : (WGM_ == 3 ? 2 : 1);  // 1 x 4 waves: 128 (wide: 256) rows of n
     static constexpr int RA = WIDE ? 2 : NA, RW = WIDE ? 2 : NW;               // ring depths
     static constexpr int BN = WGN * WN * 32;
     static constexpr int NT16 = BN / 16;                           // 16-row weight tiles per workgroup
@@ -106,7 +112,7 @@ template <int DT, int WGM_> struct Geo {
     static constexpr int W_CHUNKS = (W_BYTES + 1023) / 1024;       // copies of 1 KiB; the last may be partial
     static constexpr int W_STRIDE = W_CHUNKS * 1024;               // ring stride: a partial last copy lands in padding
     static constexpr int CPW = 2 * ((W_CHUNKS + 7) / 8);           // wide form: weight copies per wave and super-block (even)
-    static constexpr int A_OFF = 0, W_OFF = RA * A_STAGE, S_OFF = W_OFF + RW * W_STRIDE;
+    static constexpr int A_OFF = 0, W_OFF = RA * GA_STAGE, S_OFF = W_OFF + RW * W_STRIDE;
     static constexpr int OUT_PITCH = WN * 32 + 8;                  // floats per staged result row: rows r and r + 4 land 32 banks apart
     static_assert(WIDE || W_CHUNKS <= 32, "weight copies: two per wave and group");
     static_assert(!WIDE || (CPW % 2 == 0 && CPW <= 24), "wide form: two halves of CPW / 2 copies per wave");
@@ -434,10 +440,15 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
 
     // ---- copy schedule (all wave-uniform except the per-lane weight offsets) ----
     // activations: this wave's m-tile; one past the end re-reads the last valid tile (never stored)
-    int64_t my_mt = (int64_t)mb * MT + wave;
+    // (low form: two waves per m-tile, two of its four steps each; sums block of m-tile wave % 2 into slot `wave`)
+    int64_t my_mt = (int64_t)mb * G::GMT + (G::LOW ? wave >> 1 : wave);
     my_mt = my_mt < mtiles ? my_mt : mtiles - 1;
-    const uint8_t *a_src = uniform_ptr(frags + ((size_t)(my_mt * ntc * 17) << 10));
-    const uint32_t a_dst = lds_base + G::A_OFF + (uint32_t)wave * 4096u;  // + ks * A_STAGE (+ step * 1024 by the offset)
+    int64_t my_mt_s = G::LOW ? (int64_t)mb * G::GMT + (wave & 1) : my_mt;
+    my_mt_s = my_mt_s < mtiles ? my_mt_s : mtiles - 1;
+    const uint32_t a_half = G::LOW ? (uint32_t)(wave & 1) * 2048u : 0u;
+    const uint8_t *a_src = uniform_ptr(frags + ((size_t)(my_mt * ntc * 17) << 10) + a_half);
+    const uint8_t *s_src = uniform_ptr(frags + ((size_t)(my_mt_s * ntc * 17) << 10));
+    const uint32_t a_dst = lds_base + G::A_OFF + (uint32_t)(G::LOW ? wave >> 1 : wave) * 4096u + a_half;  // + ks * A_STAGE (+ step * 1024)
     const uint32_t s_dst = lds_base + G::S_OFF + (uint32_t)wave * 1024u;  // + (b & 1) * S_BYTES
     // weights: copy c of a super-block covers bytes [1024 c, 1024 c + 1024) of the concatenated tiles of the workgroup;
     // group g = 0..3 holds copies 4g + wave and 16 + 4g + wave (clamped to the last copy; lanes past the end of the
@@ -468,10 +479,12 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
 
     auto issue_a = [&](int bb, int ks) {  // stage (bb, ks) -> stage buffer ks (wide form: ks % 2)
         const uint8_t *src = a_src + ((size_t)(bb * 17 + 4 * ks) << 10);
-        dma_set<0>(lane_off, src, a_dst + (uint32_t)(ks % G::RA) * A_STAGE);
+        dma_set<0>(lane_off, src, a_dst + (uint32_t)(ks % G::RA) * G::GA_STAGE);
         dma_more<1024>(lane_off, src);
-        dma_more<2048>(lane_off, src);
-        dma_more<3072>(lane_off, src);
+        if constexpr (!G::LOW) {
+            dma_more<2048>(lane_off, src);
+            dma_more<3072>(lane_off, src);
+        }
     };
     auto issue_w = [&](int bb, int g, uint32_t ring) {  // group g of super-block bb
         const uint8_t *src = w_src + (size_t)bb * TB;
@@ -484,7 +497,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
         }
     };
     auto issue_s = [&](int bb) {
-        if constexpr (SUMS) dma_set<0>(lane_off, a_src + ((size_t)(bb * 17 + 16) << 10), s_dst + (uint32_t)(bb & 1) * S_BYTES);
+        if constexpr (SUMS) dma_set<0>(lane_off, s_src + ((size_t)(bb * 17 + 16) << 10), s_dst + (uint32_t)(bb & 1) * S_BYTES);
     };
 
     // ---- LDS read addresses ----
@@ -558,7 +571,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                     // next step's activation fragments come in while this step computes
                     static_for<WM>([&](auto I) {
                         constexpr int i = decltype(I)::value;
-                        lds_read128<(ks % G::RA) * A_STAGE + i * 4096 + (st + 1) * 1024>(af[pa ^ 1][i], a_rd);
+                        lds_read128<(ks % G::RA) * G::GA_STAGE + i * 4096 + (st + 1) * 1024>(af[pa ^ 1][i], a_rd);
                     });
                     wait_lds<WM>();  // everything but the reads just issued
 #pragma unroll
@@ -619,7 +632,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
                             Fm::template read_hdr<j * 2 * TB>(hd[j], w_rd, wr1);
                         });
                     }
-                    static_for<WM>([&](auto I) { lds_read128<(nks % G::RA) * A_STAGE + decltype(I)::value * 4096>(af[0][decltype(I)::value], a_rd); });
+                    static_for<WM>([&](auto I) { lds_read128<(nks % G::RA) * G::GA_STAGE + decltype(I)::value * 4096>(af[0][decltype(I)::value], a_rd); });
                 }
                 // operand step 4 ks + st of the lane's 128 columns
                 half8v bop[WN];
@@ -672,7 +685,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     // ---- results ----
     // 32x32 result: lane (n32, g32), register e holds row 8 * (e / 4) + 4 * g32 + e % 4 of column n32
     constexpr int OUT_PITCH = G::OUT_PITCH;
-    const int64_t row0 = (int64_t)mb * BM + wm * (WM * 32);
+    const int64_t row0 = (int64_t)mb * G::GBM + wm * (WM * 32);
     const int64_t col0 = (int64_t)nb * G::BN + wn * (WN * 32);
     if (vec_out) {
         float *stage = (float *)lds + (size_t)wave * (WM * 32 * OUT_PITCH);
@@ -749,7 +762,7 @@ hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, i
     static const hipError_t attr =
         hipFuncSetAttribute((const void *)gemm_kq_kernel<DT, WGM_>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (attr != hipSuccess) return attr;
-    const int nbn = (int)((n + G::BN - 1) / G::BN), nbm = (int)((m + BM - 1) / BM);
+    const int nbn = (int)((n + G::BN - 1) / G::BN), nbm = (int)((m + G::GBM - 1) / G::GBM);
     const dim3 grid((unsigned)(nbn * nbm)), block(256);
     const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
     const int vec_out = ((uintptr_t)y % 16 == 0 && ((uint64_t)ldy * es) % 16 == 0 && n % 8 == 0) ? 1 : 0;
@@ -791,6 +804,19 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
         if (wide_env >= 0) return wide_env == 1;
         return 2 * wide_wgs >= cus && fill_wide * gain >= fill(bn_other, nullptr);
     };
+    // The low tile (64 x 128, Geo<.., 4>) for launches whose 128 x 128 tiles would leave at least half of the CUs without a
+    // workgroup: twice the workgroups.  TURQ_GEMM_LOW = 0 / 1 overrides the rule.
+    static const int low_env = [] { const char *e = getenv("TURQ_GEMM_LOW"); return e ? (atoi(e) != 0 ? 1 : 0) : -1; }();
+    const int64_t wgs128 = ((n + 127) / 128) * ((m + BM - 1) / BM);
+    const bool low = low_env >= 0 ? low_env == 1 : (m > 64 && 2 * wgs128 <= cus);
+    if (low && wide_env != 1) {
+        switch (dtype) {
+        case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K, 4>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+        case TURQ_Q5_K: return launch_gemm<TURQ_Q5_K, 4>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+        case TURQ_Q6_K: return launch_gemm<TURQ_Q6_K, 4>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+        default: break;
+        }
+    }
     switch (dtype) {
     case TURQ_Q4_K:
         if (wide_env == 1) return launch_gemm<TURQ_Q4_K, 3>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
