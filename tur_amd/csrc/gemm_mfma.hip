@@ -804,11 +804,12 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
         if (wide_env >= 0) return wide_env == 1;
         return 2 * wide_wgs >= cus && fill_wide * gain >= fill(bn_other, nullptr);
     };
-    // The low tile (64 x 128, Geo<.., 4>) for launches whose 128 x 128 tiles would leave at least half of the CUs without a
-    // workgroup: twice the workgroups.  TURQ_GEMM_LOW = 0 / 1 overrides the rule.
+    // The low tile (64 x 128, Geo<.., 4>) for launches of up to 64 rows, and for those whose 128 x 128 tiles would leave at
+    // least half of the CUs without a workgroup (twice the workgroups).  TURQ_GEMM_LOW = 0 / 1 overrides the rule.
     static const int low_env = [] { const char *e = getenv("TURQ_GEMM_LOW"); return e ? (atoi(e) != 0 ? 1 : 0) : -1; }();
     const int64_t wgs128 = ((n + 127) / 128) * ((m + BM - 1) / BM);
-    const bool low = low_env >= 0 ? low_env == 1 : (m > 64 && 2 * wgs128 <= cus);
+    // (up to 64 rows the low tile is the whole problem's height: half the MFMA work and activation traffic of a 128-row tile)
+    const bool low = low_env >= 0 ? low_env == 1 : (m <= 64 || 2 * wgs128 <= cus);
     if (low && wide_env != 1) {
         switch (dtype) {
         case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K, 4>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
