@@ -462,6 +462,24 @@ def test_two_rows_two_formats(gpu, first):
         gpu.release(w)
 
 
+def test_multi_weight_prefill_shares_the_preparation(gpu):
+    # more than 32 rows with device pointers: the activations are prepared once per fragment order and every weight runs its
+    # GEMM on them; the results are those of the single calls bit for bit (same kernels, same inputs)
+    k, dts, ns = 1024, (Q4_K, Q6_K, Q8_0, Q8_0, Q5_K), [272, 64, 100, 48, 528]
+    raws = [synth.random_weight(dt, n, k, seed=3 * i + n) for i, (dt, n) in enumerate(zip(dts, ns))]
+    ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
+    biases = [None if i == 2 else np.random.default_rng(i).standard_normal(n).astype(np.float32) for i, n in enumerate(ns)]
+    for m in (33, 70, 200):
+        x = synth.random_activation(m, k, seed=m, bf16=True)
+        for x_dtype in (capi.ACT_F32, capi.ACT_BF16):
+            ys = gpu.qmatmul_multi(ws, x, ns, k, x_dtype=x_dtype, biases=biases)
+            for dt, n, raw, w, y, b in zip(dts, ns, raws, ws, ys, biases):
+                assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, k) + (0 if b is None else b)) <= 1e-3, (m, dt, n)
+                assert np.array_equal(y, gpu.qmatmul(w, x, n, k, x_dtype=x_dtype, bias=b)), (m, dt, n)
+    for w in ws:
+        gpu.release(w)
+
+
 def test_multi_weight_falls_back_to_single_calls(gpu):
     # more than 32 rows, or host pointers: the same as the calls one after the other
     k, ns, dts = 512, [48, 80], (Q4_K, Q4_K)

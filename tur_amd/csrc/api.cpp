@@ -447,8 +447,9 @@ int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weigh
     if (count < 0) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_multi: count=%d is negative", count);
     if (count == 0) return TURQ_OK;
     if (!weights || !ys || !ldys) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_multi: null weight, output or stride array");
-    bool one_launch = mem == TURQ_MEM_DEVICE && (algo == TURQ_ALGO_AUTO || algo == TURQ_ALGO_GEMV) && count > 1 && m >= 1 &&
-                      m <= TURQ_GEMV_MAX_M && x != nullptr;
+    const bool many_rows = m > TURQ_GEMV_MAX_M && (algo == TURQ_ALGO_AUTO || algo == TURQ_ALGO_GEMM);
+    bool one_launch = mem == TURQ_MEM_DEVICE && count > 1 && x != nullptr &&
+                      (many_rows || ((algo == TURQ_ALGO_AUTO || algo == TURQ_ALGO_GEMV) && m >= 1 && m <= TURQ_GEMV_MAX_M));
     for (int i = 0; i < count && one_launch; i++) {
         const turq_weight *w = weights[i];
         one_launch = w && ys[i] && w->device == ctx->device && turq_dt_is_quant(w->dtype) && w->layout == TURQ_LAYOUT_TILED &&
@@ -456,6 +457,13 @@ int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weigh
     }
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
     one_launch = one_launch && xb && yb && ldx >= weights[0]->k;
+    if (one_launch && many_rows) {
+        // prefill: one preparation of the activations for all the weights, then a GEMM each
+        bool taken = false;
+        const int rc = turq_qmatmul_multi_gemm(ctx, count, weights, x, xt, m, ldx, ys, yt, ldys, biases, &taken);
+        if (rc != TURQ_OK || taken) return rc;
+        one_launch = false;
+    }
     if (!one_launch) {
         // anything else is the same as the calls one after the other (which also report what is wrong with an argument)
         for (int i = 0; i < count; i++) {

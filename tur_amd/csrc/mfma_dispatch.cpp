@@ -72,7 +72,47 @@ int pick_rows_row1(const turq_ctx *ctx, int64_t row_tiles) {
     return row_tiles >= 16 * cus ? 2 : 1;
 }
 
+// whether the prefill GEMM can take this weight (its largest packed value must fit f16), and the power of two by which the
+// kernel multiplies the block scales
+bool gemm_takes(const turq_weight *w, float *wscale) {
+    const float top = w->dtype == TURQ_Q4_K ? 1039.0f : w->dtype == TURQ_Q5_K ? 1055.0f : w->dtype == TURQ_Q6_K ? 319.0f : 128.0f;
+    const bool ok = turq_dt_is_quant(w->dtype) && w->k % 256 == 0 && w->max_scale * top < 60000.0f;
+    float ws = 1.0f;
+    if (ok && w->max_scale > 0.0f)
+        while (ws < 32768.0f && w->max_scale * top * ws * 2.0f < 40000.0f) ws *= 2.0f;
+    *wscale = ws;
+    return ok;
+}
+
 }  // namespace
+
+// More than 32 rows, several weights that take the same activations: the fragments are prepared once per fragment order
+// (K-quants / Q8_0) and every weight runs its GEMM on them.  *taken = false (nothing launched) if one of the weights cannot
+// go through the GEMM.
+int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m, int64_t ldx,
+                            void *const *y, int yt, const int64_t *ldy, const float *const *bias, bool *taken) {
+    *taken = false;
+    float ws[16];
+    if (count > 16) return TURQ_OK;
+    for (int i = 0; i < count; i++)
+        if (!gemm_takes(w[i], &ws[i])) return TURQ_OK;
+    int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep32_bytes(m, w[0]->k));
+    if (rc != TURQ_OK) return rc;
+    int prepared = 0;  // 1: K-quant order, 2: Q8_0 order
+    for (int i = 0; i < count; i++) {
+        const int order = w[i]->dtype == TURQ_Q8_0 ? 2 : 1;
+        if (order != prepared) {
+            TURQ_HIP(ctx, turq_launch_act_prep32(w[i]->dtype, x, xt, m, w[i]->k, ldx, ctx->act_prep, ctx->stream));
+            prepared = order;
+        }
+        hipEvent_t ev0 = nullptr, ev1 = nullptr;
+        TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+        TURQ_HIP(ctx, turq_launch_gemm_mfma(w[i]->dtype, w[i]->dev, w[i]->n, w[i]->k, ctx->act_prep, m, y[i], yt, ldy[i],
+                                            bias ? bias[i] : nullptr, ws[i], ctx->compute_units, ctx->stream, ev0, ev1));
+    }
+    *taken = true;
+    return TURQ_OK;
+}
 
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
                       int yt, int64_t ldy, const float *bias, int algo) {
@@ -81,11 +121,8 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
     // Q4_K / Q5_K, 256 for the 6-bit values of Q6_K; q * d for Q8_0), the scales multiplied by a power of two that puts the
     // largest of them near 2^15 (small scales would otherwise lose bits in the f16 subnormals); a tensor whose largest value
     // does not fit f16 even unscaled goes through the exact skinny kernel instead
-    const float top = w->dtype == TURQ_Q4_K ? 1039.0f : w->dtype == TURQ_Q5_K ? 1055.0f : w->dtype == TURQ_Q6_K ? 319.0f : 128.0f;
-    const bool gemm_ok = turq_dt_is_quant(w->dtype) && w->k % 256 == 0 && w->max_scale * top < 60000.0f;
     float wscale = 1.0f;
-    if (gemm_ok && w->max_scale > 0.0f)
-        while (wscale < 32768.0f && w->max_scale * top * wscale * 2.0f < 40000.0f) wscale *= 2.0f;
+    const bool gemm_ok = gemm_takes(w, &wscale);
     if (algo == TURQ_ALGO_GEMM && !gemm_ok && m > TURQ_GEMV_MAX_M)
         algo = TURQ_ALGO_GEMV;  // scales too large for f16 operands, ragged Q8_0 columns: walk m in chunks through the skinny kernel
     if (m > TURQ_GEMV_MAX_M && algo == TURQ_ALGO_GEMM) {
