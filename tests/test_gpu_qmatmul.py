@@ -480,6 +480,52 @@ def test_multi_weight_prefill_shares_the_preparation(gpu):
         gpu.release(w)
 
 
+def test_multi_weight_prefill_small_launches_side_by_side(gpu):
+    # q / k / v of a prompt chunk: launches that fill at most half of the machine alternate between the context's stream and
+    # a second one between the shared preparation and the end of the call.  Same kernels, same inputs: bit-equal with the
+    # single calls, eagerly (twice, the buffers reused) and in a captured graph replayed with other activations.
+    L, ctx = gpu.L, gpu.ctx
+    k, dts, ns = 1024, (Q4_K, Q4_K, Q6_K, Q5_K), [512, 128, 128, 80]
+    raws = [synth.random_weight(dt, n, k, seed=7 * i + n) for i, (dt, n) in enumerate(zip(dts, ns))]
+    ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
+    biases = [np.random.default_rng(i).standard_normal(n).astype(np.float32) if i == 1 else None for i, n in enumerate(ns)]
+    for m in (40, 130, 512, 40):
+        x = synth.random_activation(m, k, seed=m, bf16=True)
+        ys = gpu.qmatmul_multi(ws, x, ns, k, biases=biases)
+        for dt, n, raw, w, y, b in zip(dts, ns, raws, ws, ys, biases):
+            assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, k) + (0 if b is None else b)) <= 1e-3, (m, dt, n)
+            assert np.array_equal(y, gpu.qmatmul(w, x, n, k, bias=b)), (m, dt, n)
+
+    def dev(nbytes):
+        p = ctypes.c_void_p()
+        capi.check(L.turq_dev_alloc(ctx, nbytes, ctypes.byref(p)), ctx)
+        return p
+    m = 96
+    xd, yd = dev(m * k * 4), [dev(m * n * 4) for n in ns]
+    warr = (ctypes.c_void_p * 4)(*[w.value for w in ws])
+    yarr = (ctypes.c_void_p * 4)(*[p.value for p in yd])
+    ldys = (ctypes.c_int64 * 4)(*ns)
+    capi.check(L.turq_graph_begin(ctx), ctx)
+    capi.check(L.turq_qmatmul_multi(ctx, 4, warr, xd, capi.ACT_F32, m, k, yarr, capi.ACT_F32, ldys, None, capi.MEM_DEVICE,
+                                    capi.ALGO_AUTO), ctx)
+    graph = ctypes.c_void_p()
+    capi.check(L.turq_graph_end(ctx, ctypes.byref(graph)), ctx)
+    for seed in (1, 2, 3):
+        x = synth.random_activation(m, k, seed=seed, bf16=True)
+        capi.check(L.turq_memcpy_h2d(ctx, xd, capi.ptr(x), x.nbytes), ctx)
+        capi.check(L.turq_graph_launch(ctx, graph), ctx)
+        capi.check(L.turq_sync(ctx), ctx)
+        for w, n, p in zip(ws, ns, yd):
+            y = np.zeros((m, n), np.float32)
+            capi.check(L.turq_memcpy_d2h(ctx, capi.ptr(y), p, y.nbytes), ctx)
+            assert np.array_equal(y, gpu.qmatmul(w, x, n, k)), (seed, n)   # eager work of the same context between the replays
+    L.turq_graph_destroy(graph)
+    for p in [xd] + yd:
+        capi.check(L.turq_dev_free(ctx, p), ctx)
+    for w in ws:
+        gpu.release(w)
+
+
 def test_multi_weight_falls_back_to_single_calls(gpu):
     # more than 32 rows, or host pointers: the same as the calls one after the other
     k, ns, dts = 512, [48, 80], (Q4_K, Q4_K)

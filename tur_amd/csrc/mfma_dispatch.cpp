@@ -89,6 +89,34 @@ bool gemm_takes(const turq_weight *w, float *wscale) {
 // More than 32 rows, several weights that take the same activations: the fragments are prepared once per fragment order
 // (K-quants / Q8_0) and every weight runs its GEMM on them.  *taken = false (nothing launched) if one of the weights cannot
 // go through the GEMM.
+// The second stream and its two events, made on first use.  Not while a graph is being captured (creating a stream is not a
+// call to make in the middle of a capture): the caller then stays on one stream.
+static bool side_ready(turq_ctx *ctx) {
+    if (ctx->side) return true;
+    if (ctx->capturing) return false;
+    hipStream_t s = nullptr;
+    hipEvent_t a = nullptr, b = nullptr;
+    if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) return false;
+    if (hipEventCreateWithFlags(&a, hipEventDisableTiming) != hipSuccess ||
+        hipEventCreateWithFlags(&b, hipEventDisableTiming) != hipSuccess) {
+        if (a) (void)hipEventDestroy(a);
+        (void)hipStreamDestroy(s);
+        return false;
+    }
+    ctx->side = s;
+    ctx->ev_fork = a;
+    ctx->ev_join = b;
+    return true;
+}
+
+// workgroups of the GEMM launch for [m, n] (the launcher's choice between the 64-row and the 128-row tiles, wide tiles counted
+// as two): a launch of at most half as many workgroups as the GPU has CUs leaves room for another one next to it
+static bool gemm_underfills(const turq_ctx *ctx, const turq_weight *w, int64_t m) {
+    const int64_t nt = (w->n + 127) / 128, wgs128 = ((m + 127) / 128) * nt;
+    const int64_t wgs = (m <= 64 || 2 * wgs128 <= ctx->compute_units) ? ((m + 63) / 64) * nt : wgs128;
+    return 2 * wgs <= ctx->compute_units;
+}
+
 int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m, int64_t ldx,
                             void *const *y, int yt, const int64_t *ldy, const float *const *bias, bool *taken) {
     *taken = false;
@@ -98,18 +126,56 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
         if (!gemm_takes(w[i], &ws[i])) return TURQ_OK;
     int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep32_bytes(m, w[0]->k));
     if (rc != TURQ_OK) return rc;
-    int prepared = 0;  // 1: K-quant order, 2: Q8_0 order
+    // k_proj / v_proj of a prompt chunk are launches of a quarter of the machine each: every second one of such launches goes
+    // to the second stream, where it needs nothing but the prepared activations (an event recorded after the preparation, or
+    // later, orders it behind them).  Only when one preparation serves the whole
+    // call (a later preparation would overwrite fragments that the other stream still reads).
+    static const bool no_side = getenv("TURQ_GEMM_NO_SIDE") != nullptr;
+    int n_small = 0;
+    bool one_order = true;
     for (int i = 0; i < count; i++) {
+        n_small += gemm_underfills(ctx, w[i], m);
+        one_order = one_order && (w[i]->dtype == TURQ_Q8_0) == (w[0]->dtype == TURQ_Q8_0);
+    }
+    const bool fork = !no_side && one_order && n_small >= 2 && side_ready(ctx);
+    bool forked = false, pair_open = false;
+    int prepared = 0;  // 1: K-quant order, 2: Q8_0 order
+    int small_seen = 0;
+    hipError_t e = hipSuccess;
+    for (int i = 0; i < count && e == hipSuccess; i++) {
         const int order = w[i]->dtype == TURQ_Q8_0 ? 2 : 1;
         if (order != prepared) {
-            TURQ_HIP(ctx, turq_launch_act_prep32(w[i]->dtype, x, xt, m, w[i]->k, ldx, ctx->act_prep, ctx->stream));
+            e = turq_launch_act_prep32(w[i]->dtype, x, xt, m, w[i]->k, ldx, ctx->act_prep, ctx->stream);
+            if (e != hipSuccess) break;
             prepared = order;
         }
+        hipStream_t st = ctx->stream;
+        if (fork && gemm_underfills(ctx, w[i], m)) {
+            // small launches go in pairs: the second stream starts its one where the first stream starts the other, so the two
+            // share the machine with each other and not with a launch that fills it on its own
+            if (!(small_seen++ & 1)) {
+                e = hipEventRecord(ctx->ev_fork, ctx->stream);
+                pair_open = e == hipSuccess;
+            } else if (pair_open) {
+                e = hipStreamWaitEvent(ctx->side, ctx->ev_fork, 0);
+                pair_open = false;
+                forked = true;
+                st = ctx->side;
+            }
+            if (e != hipSuccess) break;
+        }
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
-        TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
-        TURQ_HIP(ctx, turq_launch_gemm_mfma(w[i]->dtype, w[i]->dev, w[i]->n, w[i]->k, ctx->act_prep, m, y[i], yt, ldy[i],
-                                            bias ? bias[i] : nullptr, ws[i], ctx->compute_units, ctx->stream, ev0, ev1));
+        e = turq_prof_next(ctx, &ev0, &ev1);
+        if (e == hipSuccess)
+            e = turq_launch_gemm_mfma(w[i]->dtype, w[i]->dev, w[i]->n, w[i]->k, ctx->act_prep, m, y[i], yt, ldy[i],
+                                      bias ? bias[i] : nullptr, ws[i], ctx->compute_units, st, ev0, ev1);
     }
+    if (forked) {  // also after an error: nothing may stay behind on the second stream
+        hipError_t j = hipEventRecord(ctx->ev_join, ctx->side);
+        if (j == hipSuccess) j = hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0);
+        if (e == hipSuccess) e = j;
+    }
+    TURQ_HIP(ctx, e);
     *taken = true;
     return TURQ_OK;
 }
