@@ -166,9 +166,9 @@ int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype
  * go out as ONE kernel launch (for more than one row on all but small matrices, or activation rows that are not
  * 16-byte aligned, after one preparation of the activations for all the weights); with more than 32 rows the
  * activations are prepared once for all the weights and each weight runs its GEMM on them (the results of the single
- * calls, bit for bit; GEMMs that leave half of the GPU free, such as k_proj and v_proj of a prompt chunk, run in pairs,
- * one of each pair on a second stream of the context that is joined to the first before the call returns, so the caller
- * still sees one stream); every other case is exactly the turq_qmatmul calls one after the other (including their errors).  `biases` may be NULL, and so may its entries.
+ * calls, bit for bit; GEMMs that leave half of the GPU free, such as k_proj and v_proj of a prompt chunk, run next to each other,
+ * up to three at a time, on further streams of the context that are joined to the first before the call returns, so the
+ * caller still sees one stream); every other case is exactly the turq_qmatmul calls one after the other (including their errors).  `biases` may be NULL, and so may its entries.
  * Replaces: the back-to-back `forward` calls on one input in the reference's decoder layer - q_proj / k_proj /
  * v_proj (src/models/qwen3.rs:272-274) and gate_proj / up_proj (src/models/qwen3.rs:161-167). */
 int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int x_dtype, int64_t m,

@@ -481,8 +481,8 @@ def test_multi_weight_prefill_shares_the_preparation(gpu):
 
 
 def test_multi_weight_prefill_small_launches_side_by_side(gpu):
-    # q / k / v of a prompt chunk: launches that fill at most half of the machine alternate between the context's stream and
-    # a second one between the shared preparation and the end of the call.  Same kernels, same inputs: bit-equal with the
+    # q / k / v of a prompt chunk: launches that leave half of the machine free run in groups of up to three, the first on
+    # the context's stream, the others on further streams, between the shared preparation and the end of the call.  Same kernels, same inputs: bit-equal with the
     # single calls, eagerly (twice, the buffers reused) and in a captured graph replayed with other activations.
     L, ctx = gpu.L, gpu.ctx
     k, dts, ns = 1024, (Q4_K, Q4_K, Q6_K, Q5_K), [512, 128, 128, 80]

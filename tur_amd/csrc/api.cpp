@@ -130,9 +130,11 @@ void turq_ctx_destroy(turq_ctx *ctx) {
     if (ctx->gate_up) (void)hipFree(ctx->gate_up);
     if (ctx->stage_b) (void)hipFree(ctx->stage_b);
     for (auto &p : ctx->prof_events) { (void)hipEventDestroy(p.first); (void)hipEventDestroy(p.second); }
-    if (ctx->side) { (void)hipStreamSynchronize(ctx->side); (void)hipStreamDestroy(ctx->side); }
+    for (int i = 0; i < turq_ctx::kSide; i++) {
+        if (ctx->side[i]) { (void)hipStreamSynchronize(ctx->side[i]); (void)hipStreamDestroy(ctx->side[i]); }
+        if (ctx->ev_join[i]) (void)hipEventDestroy(ctx->ev_join[i]);
+    }
     if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
-    if (ctx->ev_join) (void)hipEventDestroy(ctx->ev_join);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }

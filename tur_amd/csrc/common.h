@@ -73,10 +73,11 @@ struct turq_ctx {
     void *stage_b = nullptr;  size_t stage_b_cap = 0;
     void *act_prep = nullptr; size_t act_prep_cap = 0;
     void *gate_up = nullptr;  size_t gate_up_cap = 0;  // the two f32 products of turq_qmatmul_gate_up's general path
-    // second stream for small prefill GEMMs of one turq_qmatmul_multi call that run next to each other: forked from `stream`
-    // after the shared activation preparation and joined again before the call returns (created on first use)
-    hipStream_t side = nullptr;
-    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+    // further streams for small prefill GEMMs of one turq_qmatmul_multi call that run next to each other: forked from `stream`
+    // where the first launch of a group starts and joined again before the call returns (created on first use)
+    static constexpr int kSide = 2;
+    hipStream_t side[kSide] = {nullptr, nullptr};
+    hipEvent_t ev_fork = nullptr, ev_join[kSide] = {nullptr, nullptr};
     // kernel timing (turq_profile_*): event pairs recorded around matmul kernels
     bool profiling = false;
     bool capturing = false;

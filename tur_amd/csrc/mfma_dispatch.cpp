@@ -89,35 +89,37 @@ bool gemm_takes(const turq_weight *w, float *wscale) {
 // More than 32 rows, several weights that take the same activations: the fragments are prepared once per fragment order
 // (K-quants / Q8_0) and every weight runs its GEMM on them.  *taken = false (nothing launched) if one of the weights cannot
 // go through the GEMM.
-// The second stream and its two events, made on first use.  Not while a graph is being captured (creating a stream is not a
+// The further streams and their events, made on first use.  Not while a graph is being captured (creating a stream is not a
 // call to make in the middle of a capture): the caller then stays on one stream.
 static bool side_ready(turq_ctx *ctx) {
-    if (ctx->side) return true;
+    if (ctx->side[0]) return true;
     if (ctx->capturing) return false;
-    hipStream_t s = nullptr;
-    hipEvent_t a = nullptr, b = nullptr;
-    if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess) return false;
-    if (hipEventCreateWithFlags(&a, hipEventDisableTiming) != hipSuccess ||
-        hipEventCreateWithFlags(&b, hipEventDisableTiming) != hipSuccess) {
-        if (a) (void)hipEventDestroy(a);
-        (void)hipStreamDestroy(s);
+    hipStream_t s[turq_ctx::kSide] = {};
+    hipEvent_t j[turq_ctx::kSide] = {}, f = nullptr;
+    bool ok = hipEventCreateWithFlags(&f, hipEventDisableTiming) == hipSuccess;
+    for (int i = 0; i < turq_ctx::kSide && ok; i++)
+        ok = hipStreamCreateWithFlags(&s[i], hipStreamNonBlocking) == hipSuccess &&
+             hipEventCreateWithFlags(&j[i], hipEventDisableTiming) == hipSuccess;
+    if (!ok) {
+        for (int i = 0; i < turq_ctx::kSide; i++) {
+            if (j[i]) (void)hipEventDestroy(j[i]);
+            if (s[i]) (void)hipStreamDestroy(s[i]);
+        }
+        if (f) (void)hipEventDestroy(f);
         return false;
     }
-    ctx->side = s;
-    ctx->ev_fork = a;
-    ctx->ev_join = b;
+    ctx->ev_fork = f;
+    for (int i = 0; i < turq_ctx::kSide; i++) { ctx->side[i] = s[i]; ctx->ev_join[i] = j[i]; }
     return true;
 }
 
-// Does the GEMM launch for [m, n] leave room for another one next to it?  Its workgroups, by the launcher's choice between the
-// 64-row tile (two of those workgroups share a CU) and the 128-row tiles (one per CU; wide tiles counted as two), against half
-// of the CUs.  Measured on the Q4_K_M layer: pairing launches of 192 workgroups helps with the 64-row tile (m = 128: +4.8 %)
-// and hurts with the 128-row tile (m = 256: -2.7 %).
-static bool gemm_underfills(const turq_ctx *ctx, const turq_weight *w, int64_t m) {
+// CUs that the GEMM launch for [m, n] takes: its workgroups, by the launcher's choice between the 64-row tile (two of those
+// workgroups share a CU) and the 128-row tiles (one per CU; wide tiles counted as two).  Measured on the Q4_K_M layer: launches
+// of 192 workgroups next to each other help with the 64-row tile (m = 128: +4.8 %) and hurt with the 128-row tile (m = 256: -2.7 %).
+static int64_t gemm_cus_taken(const turq_ctx *ctx, const turq_weight *w, int64_t m) {
     const int64_t nt = (w->n + 127) / 128, wgs128 = ((m + 127) / 128) * nt;
     const bool low = m <= 64 || 2 * wgs128 <= ctx->compute_units;
-    const int64_t cus_taken = low ? (((m + 63) / 64) * nt + 1) / 2 : wgs128;
-    return 2 * cus_taken <= ctx->compute_units;
+    return low ? (((m + 63) / 64) * nt + 1) / 2 : wgs128;
 }
 
 int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m, int64_t ldx,
@@ -129,21 +131,24 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
         if (!gemm_takes(w[i], &ws[i])) return TURQ_OK;
     int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep32_bytes(m, w[0]->k));
     if (rc != TURQ_OK) return rc;
-    // k_proj / v_proj of a prompt chunk are launches of a quarter of the machine each: every second one of such launches goes
-    // to the second stream, where it needs nothing but the prepared activations (an event recorded after the preparation, or
-    // later, orders it behind them).  Only when one preparation serves the whole
-    // call (a later preparation would overwrite fragments that the other stream still reads).
+    // k_proj / v_proj of a prompt chunk are launches of a quarter of the machine each.  Launches that leave half of the CUs free
+    // run in groups, as many as fit the machine together (three at most): the first of a group on the context's stream, the
+    // others on further streams that start where it starts (an event recorded there; behind the preparation, the only thing
+    // they need) and are joined before the call returns.  Only when one preparation serves the whole call (a later
+    // preparation would overwrite fragments that another stream still reads).
     static const bool no_side = getenv("TURQ_GEMM_NO_SIDE") != nullptr;
+    const int64_t cus = ctx->compute_units;
     int n_small = 0;
     bool one_order = true;
     for (int i = 0; i < count; i++) {
-        n_small += gemm_underfills(ctx, w[i], m);
+        n_small += 2 * gemm_cus_taken(ctx, w[i], m) <= cus;
         one_order = one_order && (w[i]->dtype == TURQ_Q8_0) == (w[0]->dtype == TURQ_Q8_0);
     }
     const bool fork = !no_side && one_order && n_small >= 2 && side_ready(ctx);
-    bool forked = false, pair_open = false;
-    int prepared = 0;  // 1: K-quant order, 2: Q8_0 order
-    int small_seen = 0;
+    bool used[turq_ctx::kSide] = {};
+    int group_n = 0;        // launches in the open group (0: none open)
+    int64_t group_cus = 0;  // CUs they take together
+    int prepared = 0;       // 1: K-quant order, 2: Q8_0 order
     hipError_t e = hipSuccess;
     for (int i = 0; i < count && e == hipSuccess; i++) {
         const int order = w[i]->dtype == TURQ_Q8_0 ? 2 : 1;
@@ -153,19 +158,22 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
             prepared = order;
         }
         hipStream_t st = ctx->stream;
-        if (fork && gemm_underfills(ctx, w[i], m)) {
-            // small launches go in pairs: the second stream starts its one where the first stream starts the other, so the two
-            // share the machine with each other and not with a launch that fills it on its own
-            if (!(small_seen++ & 1)) {
-                e = hipEventRecord(ctx->ev_fork, ctx->stream);
-                pair_open = e == hipSuccess;
-            } else if (pair_open) {
-                e = hipStreamWaitEvent(ctx->side, ctx->ev_fork, 0);
-                pair_open = false;
-                forked = true;
-                st = ctx->side;
+        const int64_t c = gemm_cus_taken(ctx, w[i], m);
+        if (fork && 2 * c <= cus) {
+            if (group_n == 0 || group_n > turq_ctx::kSide || group_cus + c > cus) {
+                e = hipEventRecord(ctx->ev_fork, ctx->stream);  // opens a group
+                group_n = 1;
+                group_cus = c;
+            } else {
+                st = ctx->side[group_n - 1];
+                e = hipStreamWaitEvent(st, ctx->ev_fork, 0);
+                used[group_n - 1] = true;
+                group_n++;
+                group_cus += c;
             }
             if (e != hipSuccess) break;
+        } else {
+            group_n = 0;  // a launch that fills the machine closes the group
         }
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
         e = turq_prof_next(ctx, &ev0, &ev1);
@@ -173,9 +181,10 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
             e = turq_launch_gemm_mfma(w[i]->dtype, w[i]->dev, w[i]->n, w[i]->k, ctx->act_prep, m, y[i], yt, ldy[i],
                                       bias ? bias[i] : nullptr, ws[i], ctx->compute_units, st, ev0, ev1);
     }
-    if (forked) {  // also after an error: nothing may stay behind on the second stream
-        hipError_t j = hipEventRecord(ctx->ev_join, ctx->side);
-        if (j == hipSuccess) j = hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0);
+    for (int s = 0; s < turq_ctx::kSide; s++) {  // also after an error: nothing may stay behind on the other streams
+        if (!used[s]) continue;
+        hipError_t j = hipEventRecord(ctx->ev_join[s], ctx->side[s]);
+        if (j == hipSuccess) j = hipStreamWaitEvent(ctx->stream, ctx->ev_join[s], 0);
         if (e == hipSuccess) e = j;
     }
     TURQ_HIP(ctx, e);
