@@ -86,13 +86,14 @@ class Bench:
         self.device = name.value.decode()
         self.cus = cus.value
         self.desc, self.mats = WORKLOADS[args.workload]
-        self.m = args.m
         self.xt, self.xbytes, self.xnp = ACT[args.act]
         self.yt, self.ybytes = OUT[args.out]
         self.weights = []      # [layer][matrix] -> handle
         self.host_raw = {}     # label -> raw bytes of the first layer (CPU baseline, checks)
         self.calls = []        # (weight, x_dev, y_dev, n, k)
+        self.x_dev, self.y_dev = {}, []
         self._setup()
+        self.set_m(args.m)
 
     def dev_alloc(self, nbytes):
         p = ctypes.c_void_p()
@@ -118,7 +119,14 @@ class Bench:
                 capi.check(L.turq_weight_upload(ctx, dt, n, k, capi.ptr(raw), raw.size, capi.LAYOUT_TILED, ctypes.byref(w)), ctx)
                 row.append(w)
             self.weights.append(row)
-        # activations: one resident input per distinct k, one output buffer per matrix
+
+    def set_m(self, m):
+        """(re)allocate the activations and outputs for m rows: one resident input per distinct k, one output per matrix"""
+        L, ctx, layers = self.L, self.ctx, self.args.layers
+        for p in list(self.x_dev.values()) + list(self.y_dev):
+            capi.check(L.turq_dev_free(ctx, p), ctx)
+        self.m = m
+        self.calls = []
         self.x_host = {}
         self.x_dev = {}
         for _, _, n, k in self.mats:
@@ -206,7 +214,8 @@ class Bench:
             raise SystemExit(f"bench: output differs from the oracle (rel-L2 {worst:.3e} > {bar})")
         return worst
 
-    def run(self):
+    def measure(self, steps, warmup):
+        """verify against the oracle, time `steps` steps (whole step), then time the matmul kernels alone"""
         a = self.args
         L, ctx = self.L, self.ctx
         rel = self.verify()
@@ -218,20 +227,20 @@ class Bench:
             capi.check(L.turq_graph_end(ctx, ctypes.byref(g)), ctx)
             graph = g
         one = (lambda: capi.check(L.turq_graph_launch(ctx, graph), ctx)) if graph else self.step_eager
-        for _ in range(a.warmup):
+        for _ in range(warmup):
             one()
         self.sync()
         t0 = time.perf_counter()
-        for _ in range(a.steps):
+        for _ in range(steps):
             one()
         self.sync()
         dt_s = time.perf_counter() - t0
-        ms_per_step = dt_s / a.steps * 1e3
-        gbps = self.step_bytes / (dt_s / a.steps) / 1e9
+        ms_per_step = dt_s / steps * 1e3
+        gbps = self.step_bytes / (dt_s / steps) / 1e9
 
         # dominant kernel alone: event pairs around every matmul kernel launch, same steps, untimed pass
         capi.check(L.turq_profile_begin(ctx), ctx)
-        prof_steps = max(1, min(a.steps, 10))
+        prof_steps = max(1, min(steps, 10))
         for _ in range(prof_steps):
             self.step_eager()
         n_launch = ctypes.c_int64()
@@ -243,41 +252,50 @@ class Bench:
         achieved = bytes_per_launch / (avg_us * 1e-6) / 1e9
         if graph:
             L.turq_graph_destroy(graph)
-        gemm = self.m > 32
-        if gemm:
+        traffic = None if a.gate_up else TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls)))
+        if self.m > 32:
             flops_per_launch = self.step_flops * prof_steps / max(1, n_launch.value)
             tfl = flops_per_launch / (avg_us * 1e-6) / 1e12
             roofline = {
                 "bound": "mfma", "achieved": round(tfl, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(tfl / MFMA_F16_PEAK_TFLOPS, 4), "traffic": (None if a.gate_up else TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls)))),
+                "frac": round(tfl / MFMA_F16_PEAK_TFLOPS, 4), "traffic": traffic,
                 "kernel": "gemm_kq_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "flops_per_launch": int(flops_per_launch),
             }
-            what = "Q4_K, Qwen3-8B up_proj" if a.workload == "q4k_prefill_up_8b" else a.workload
-            metric, value, unit = f"quantized prefill GEMM TFLOP/s ({what})", self.step_flops / (dt_s / a.steps) / 1e12, "TFLOP/s"
+            value, unit = self.step_flops / (dt_s / steps) / 1e12, "TFLOP/s"
         else:
             roofline = {
                 "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": (None if a.gate_up else TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls)))),
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                 "kernel": "gemv_row1_kernel" if self.m == 1 else "gemv_multi_frag_kernel / gemv_multi_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "algorithmic_bytes_per_launch": int(bytes_per_launch),
             }
-            metric, value, unit = "quantized GEMV HBM GB/s (Q4_K/Q6_K, Qwen3-8B shapes)", gbps, "GB/s"
+            value, unit = gbps, "GB/s"
+        return {"value": value, "unit": unit, "ms_per_step": ms_per_step, "gbps": gbps, "roofline": roofline, "rel": rel}
+
+    def run(self):
+        a = self.args
+        r = self.measure(a.steps, a.warmup)
+        if self.m > 32:
+            what = "Q4_K, Qwen3-8B up_proj" if a.workload == "q4k_prefill_up_8b" else a.workload
+            metric = f"quantized prefill GEMM TFLOP/s ({what})"
+        else:
+            metric = "quantized GEMV HBM GB/s (Q4_K/Q6_K, Qwen3-8B shapes)"
         out = {
             "metric": metric,
-            "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-            "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+            "value": round(r["value"], 1), "unit": r["unit"], "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+            "ms_per_step": round(r["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": f"{a.workload}: {self.desc}", "m": self.m, "layers": a.layers,
                        "activations": a.act, "outputs": a.out, "launch": "eager" if a.eager else "hip-graph",
                        "calls": "turq_qmatmul" if a.single_calls else ("turq_qmatmul_gate_up + turq_qmatmul_multi" if a.gate_up else "turq_qmatmul_multi"),
                        "step_bytes": int(self.step_bytes), "device": self.device, "compute_units": self.cus,
-                       "max_rel_l2_vs_oracle": float(f"{rel:.3e}")},
-            "whole_step_gbps": round(gbps, 1), "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBPS, 2),
-            "roofline": roofline,
+                       "max_rel_l2_vs_oracle": float(f"{r['rel']:.3e}")},
+            "whole_step_gbps": round(r["gbps"], 1), "pct_of_hbm_peak": round(100 * r["gbps"] / HBM_PEAK_GBPS, 2),
+            "roofline": r["roofline"],
             "cpu_baseline": self.cpu_baseline() if not a.no_cpu else None,
         }
-        print(json.dumps(out), flush=True)
+        return out
 
     def calibrate_copy(self, nelem=64 * 1024 * 1024):
         L, ctx = self.L, self.ctx
@@ -370,6 +388,11 @@ def run_embedding(args):
     L.turq_ctx_destroy(ctx)
 
 
+def default_layers(per_layer):
+    # enough distinct weight copies that a step streams well over the 256 MB Infinity Cache
+    return max(36 if per_layer < 200e6 else 2, -(-768_000_000 // per_layer))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -382,6 +405,8 @@ def main():
     ap.add_argument("--out", default="f32", choices=sorted(OUT), help="output element type")
     ap.add_argument("--eager", action="store_true", help="launch every call from the host instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="default workload only: leave out the prefill GEMM, mixed-layer and LM-head legs of the JSON line")
     ap.add_argument("--single-calls", action="store_true",
                     help="one turq_qmatmul per matrix instead of turq_qmatmul_multi per group of matrices with a common input")
     ap.add_argument("--gate-up", action="store_true",
@@ -397,16 +422,56 @@ def main():
     if args.embedding:
         return run_embedding(args)
     if args.layers is None:
-        # enough distinct weight copies that a step streams well over the 256 MB Infinity Cache
         per_layer = sum(synth.weight_nbytes(dt, n, k) for _, dt, n, k in WORKLOADS[args.workload][1])
-        args.layers = max(36 if per_layer < 200e6 else 2, -(-768_000_000 // per_layer))
+        args.layers = default_layers(per_layer)
+    headline = all(getattr(args, f) == ap.get_default(f) for f in ("workload", "m", "act", "out")) and not (
+        args.eager or args.single_calls or args.gate_up or args.calibrate_copy)
     b = Bench(args)
     try:
         if args.calibrate_copy:
             b.calibrate_copy()
-        b.run()
+        out = b.run()
     finally:
         b.close()
+    if headline and not args.no_extra:
+        out.update(other_halves(args))
+    print(json.dumps(out), flush=True)
+
+
+def side_leg(base, workload, ms, act, outdt, steps, warmup):
+    """the same measurement on another workload of the metric, in this process: one entry per m"""
+    args = argparse.Namespace(**vars(base))
+    args.workload, args.act, args.out, args.m = workload, act, outdt, ms[0]
+    per_layer = sum(synth.weight_nbytes(dt, n, k) for _, dt, n, k in WORKLOADS[workload][1])
+    args.layers = default_layers(per_layer)
+    b = Bench(args)
+    rows = []
+    try:
+        for m in ms:
+            if m != b.m:
+                b.set_m(m)
+            r = b.measure(steps, warmup)
+            rf = r["roofline"]
+            rows.append({"m": m, "value": round(r["value"], 1), "unit": r["unit"], "ms_per_step": round(r["ms_per_step"], 4),
+                         "kernel_achieved": rf["achieved"], "frac": rf["frac"], "avg_launch_us": rf["avg_launch_us"],
+                         "launches_timed": rf["launches_timed"], "max_rel_l2_vs_oracle": float(f"{r['rel']:.3e}")})
+    finally:
+        b.close()
+    return {"workload": f"{workload}: {WORKLOADS[workload][0]}", "layers": args.layers, "activations": act, "outputs": outdt,
+            "bound": "mfma" if ms[0] > 32 else "hbm", "peak": MFMA_F16_PEAK_TFLOPS if ms[0] > 32 else HBM_PEAK_GBPS,
+            "rows": rows}
+
+
+def other_halves(base):
+    """The rest of the headline metric, measured in the same process with the same method (value = whole step, frac = the
+    matmul kernels alone against the peak): the prefill GEMM (BASELINE config 4), the mixed Q4_K / Q6_K decoder layer at
+    its batch sizes (config 3) and the Q6_K LM head (config 5)."""
+    steps, warmup = 20, 3
+    return {
+        "prefill": side_leg(base, "q4k_prefill_up_8b", [512, 2048], "bf16", "bf16", steps, warmup),
+        "q4km_layer": side_leg(base, "q4km_layer_8b", [1, 8, 32], "f32", "f32", steps, warmup),
+        "lm_head_q6k": side_leg(base, "lm_head_q6k_8b", [1], "bf16", "f32", steps, warmup),
+    }
 
 
 if __name__ == "__main__":

@@ -207,11 +207,23 @@ int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void
 /* Capture every TURQ_MEM_DEVICE forward call made on ctx between begin and end into a graph and
  * replay it with one launch.  Run the same calls once eagerly first: scratch buffers must already
  * have their final size, allocation is not allowed while capturing.  The captured calls keep
- * referring to the same x / y / weight pointers. */
+ * referring to the same x / y / weight pointers, and to the context's scratch buffers by address.
+ * Scratch lifetime: while a graph of the context is alive (between turq_graph_end and
+ * turq_graph_destroy), a scratch buffer that a later, larger eager call outgrows is kept allocated
+ * next to its replacement instead of being freed, so the graph stays valid to launch; outgrown
+ * buffers are released once no graph of the context is alive, or with the context.  Destroy the
+ * graphs of a context before the context.
+ * A call that fails between begin and end (bad argument, a scratch buffer that would have to grow)
+ * ends the capture and discards what was recorded: the stream and the context stay usable, and
+ * turq_graph_end then returns TURQ_ERR_INVALID. */
 int turq_graph_begin(turq_ctx *ctx);
 int turq_graph_end(turq_ctx *ctx, turq_graph **out);
 int turq_graph_launch(turq_ctx *ctx, turq_graph *g);
 void turq_graph_destroy(turq_graph *g);
+/* Bookkeeping behind the rule above, for hosts and tests that want to see it: graphs of the context
+ * that are alive, outgrown scratch buffers kept for them, and the size of the activation-fragment
+ * buffer.  Any out pointer may be NULL. */
+int turq_ctx_scratch_info(const turq_ctx *ctx, int *live_graphs, int *retired_buffers, size_t *act_prep_bytes);
 /* Between begin and end every MFMA matmul kernel (not the activation preparation) is launched
  * with a pair of HIP events that the runtime stamps with the dispatch's own begin and end times;
  * end waits for the stream and returns the number of timed launches and the sum of their

@@ -65,6 +65,43 @@ class Gpu:
             y = synth.from_bf16_bits(y).reshape(m, ldy)
         return np.asarray(y, np.float32)[:, :n]
 
+    def dev_buffer(self, arr=None, nbytes=None):
+        """device memory holding a copy of `arr` (or nbytes of uninitialised memory); free with dev_free"""
+        p = ctypes.c_void_p()
+        size = arr.nbytes if arr is not None else nbytes
+        capi.check(self.L.turq_dev_alloc(self.ctx, max(size, 16), ctypes.byref(p)), self.ctx)
+        if arr is not None:
+            capi.check(self.L.turq_memcpy_h2d(self.ctx, p, capi.ptr(arr), arr.nbytes), self.ctx)
+        return p
+
+    def dev_free(self, p):
+        capi.check(self.L.turq_dev_free(self.ctx, p), self.ctx)
+
+    def read_back(self, p, shape, dtype):
+        out = np.empty(shape, dtype)
+        capi.check(self.L.turq_memcpy_d2h(self.ctx, capi.ptr(out), p, out.nbytes), self.ctx)
+        return out
+
+    def qmatmul_device(self, w, x, n, k, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_F32, algo=capi.ALGO_AUTO):
+        """turq_qmatmul on device pointers; x: f32 values [m, k]; returns the output as the call
+        wrote it (f32 values; bf16 outputs widened)"""
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
+        m = x.shape[0]
+        xsend = (synth.to_bf16_bits(x).reshape(m, k) if x_dtype == capi.ACT_BF16 else x.astype(np.float16) if x_dtype == capi.ACT_F16 else x)
+        ydt = {capi.ACT_F32: np.float32, capi.ACT_BF16: np.uint16, capi.ACT_F16: np.float16}[y_dtype]
+        xd = self.dev_buffer(xsend)
+        yd = self.dev_buffer(np.full((m, n), 0, ydt))
+        try:
+            rc = self.L.turq_qmatmul(self.ctx, w, xd, x_dtype, m, k, yd, y_dtype, n, None, capi.MEM_DEVICE, algo)
+            capi.check(rc, self.ctx)
+            y = self.read_back(yd, (m, n), ydt)
+        finally:
+            self.dev_free(xd)
+            self.dev_free(yd)
+        if y_dtype == capi.ACT_BF16:
+            y = synth.from_bf16_bits(y).reshape(m, n)
+        return np.asarray(y, np.float32)
+
     def qmatmul_multi(self, ws, x, ns, k, x_dtype=capi.ACT_F32, biases=None, mem=capi.MEM_DEVICE):
         """several weights against the same activations through turq_qmatmul_multi; f32 outputs.
         With mem = MEM_DEVICE the activations, biases and outputs live in device buffers."""

@@ -23,11 +23,12 @@ def gpu():
 
 CASES = [
     ("q8_0 gate 0.6B", Q8_0, 3072, 1024, [1]),
-    ("q4_k gate/up 8B", Q4_K, 12288, 4096, [1, 4, 16]),
-    ("q4_k down 8B", Q4_K, 4096, 12288, [1, 16]),
+    ("q4_k gate/up 8B", Q4_K, 12288, 4096, [1, 4, 8, 16, 32]),
+    ("q4_k down 8B", Q4_K, 4096, 12288, [1, 4, 16]),
+    ("q4_k q/o_proj 8B", Q4_K, 4096, 4096, [1, 8, 32]),
     ("q4_k k_proj 8B", Q4_K, 1024, 4096, [1, 8, 32]),
     ("q6_k v_proj 8B", Q6_K, 1024, 4096, [1, 8, 32]),
-    ("q6_k down 8B", Q6_K, 4096, 12288, [1, 32]),
+    ("q6_k down 8B", Q6_K, 4096, 12288, [1, 8, 32]),
 ]
 
 
@@ -79,12 +80,54 @@ def test_prefill_up_proj(gpu, m):
     w = gpu.upload(Q4_K, n, k, raw, capi.LAYOUT_TILED)
     x = synth.random_activation(m, k, seed=m, bf16=True)
     y = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    # the configuration's own output type: f32 sums stored as bf16, i.e. the f32 result rounded once (to nearest even)
+    yb = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16)
     gpu.release(w)
     rows = np.arange(5, n, 16)
     sub = raw.reshape(n, -1)[rows].reshape(-1)
     want = orc.matmul_dequant(Q4_K, x, sub, len(rows), k)
     assert np.all(np.isfinite(y))
     assert rel_l2(y[:, rows], want) <= 1e-3
+    assert np.array_equal(synth.to_bf16_bits(y).reshape(m, n), synth.to_bf16_bits(yb).reshape(m, n))
+    assert rel_l2(yb[:, rows], synth.from_bf16_bits(synth.to_bf16_bits(want)).reshape(want.shape)) <= 1.5e-3
+
+
+# BASELINE config 3: one Qwen3-8B decoder layer of a Q4_K_M file
+LAYER = [("q", Q4_K, 4096, 4096), ("k", Q4_K, 1024, 4096), ("v", Q6_K, 1024, 4096), ("o", Q4_K, 4096, 4096),
+         ("gate", Q4_K, 12288, 4096), ("up", Q4_K, 12288, 4096), ("down", Q6_K, 4096, 12288)]
+
+
+@pytest.fixture(scope="module")
+def layer(gpu):
+    raws = {lb: synth.random_weight(dt, n, k, seed=300 + i) for i, (lb, dt, n, k) in enumerate(LAYER)}
+    ws = {lb: gpu.upload(dt, n, k, raws[lb], capi.LAYOUT_TILED) for lb, dt, n, k in LAYER}
+    yield raws, ws
+    for w in ws.values():
+        gpu.release(w)
+
+
+@pytest.mark.parametrize("x_dtype", [capi.ACT_F32, capi.ACT_BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("m", [1, 8, 32])
+def test_q4km_decoder_layer_grouped_calls(gpu, layer, m, x_dtype):
+    # the layer's seven linears driven as the reference's decoder layer drives them (src/models/qwen3.rs:272-274, 161-167):
+    # q / k / v on one tensor through turq_qmatmul_multi (two formats in one launch), o_proj alone, gate / up through
+    # turq_qmatmul_multi, down_proj alone; device pointers, every output against the f32 matmul on the dequantized weights
+    raws, ws = layer
+    bf = x_dtype == capi.ACT_BF16
+    bar = 2e-5 if bf else 1e-3
+    shape = {lb: (dt, n, k) for lb, dt, n, k in LAYER}
+    for gi, group in enumerate((("q", "k", "v"), ("o",), ("gate", "up"), ("down",))):
+        k = shape[group[0]][2]
+        x = synth.random_activation(m, k, seed=17 * m + gi, bf16=bf)
+        ns = [shape[lb][1] for lb in group]
+        if len(group) > 1:
+            outs = gpu.qmatmul_multi([ws[lb] for lb in group], x, ns, k, x_dtype=x_dtype)
+        else:
+            outs = [gpu.qmatmul_device(ws[group[0]], x, ns[0], k, x_dtype=x_dtype)]
+        for lb, y in zip(group, outs):
+            dt, n, _ = shape[lb]
+            assert y.shape == (m, n)
+            assert rel_l2(y, orc.matmul_dequant(dt, x, raws[lb], n, k)) <= bar, (lb, m)
 
 
 def test_mlp_gate_up_and_token_embd(gpu):

@@ -130,3 +130,89 @@ def test_graph_misuse_is_an_error_not_a_crash(gpu):
     capi.check(L.turq_sync(ctx), ctx)
     L.turq_graph_destroy(g)
     L.turq_graph_destroy(None)
+
+
+def scratch_info(gpu):
+    live, retired, cap = ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t()
+    capi.check(gpu.L.turq_ctx_scratch_info(gpu.ctx, ctypes.byref(live), ctypes.byref(retired), ctypes.byref(cap)), gpu.ctx)
+    return live.value, retired.value, cap.value
+
+
+def test_scratch_that_grows_under_a_live_graph_is_kept_for_it():
+    # a graph captured at m = 8 refers to the fragment buffer by address; a later, larger eager call (m = 32 on a wider
+    # matrix) makes that buffer grow.  The old buffer must stay allocated while the graph is alive (the replay below then
+    # reads and writes valid memory and gives the eager result again), and is released once no graph is alive.
+    gpu = Gpu()                           # a context of its own: the bookkeeping starts from zero
+    L, ctx = gpu.L, gpu.ctx
+    st = Step(gpu, 8)
+    big = Step(gpu, 32, k=4096)
+    try:
+        x = synth.random_activation(8, st.k, seed=5)
+        st.set_x(x)
+        st.calls()
+        want = st.outputs()
+        assert scratch_info(gpu)[:2] == (0, 0)
+        cap0 = scratch_info(gpu)[2]
+        capi.check(L.turq_graph_begin(ctx), ctx)
+        st.calls()
+        g = ctypes.c_void_p()
+        capi.check(L.turq_graph_end(ctx, ctypes.byref(g)), ctx)
+        assert scratch_info(gpu)[:2] == (1, 0)
+        big.set_x(synth.random_activation(32, big.k, seed=6))
+        big.calls()                       # needs more scratch than the capture left behind
+        big.outputs()
+        live, retired, cap1 = scratch_info(gpu)
+        assert cap1 > cap0 and (live, retired) == (1, 1)
+        for _ in range(2):
+            st.clear_outputs()
+            capi.check(L.turq_graph_launch(ctx, g), ctx)
+            got = st.outputs()
+            for y, w in zip(got, want):
+                assert np.array_equal(y, w)
+        L.turq_graph_destroy(g)
+        assert scratch_info(gpu)[0] == 0
+        huge = Step(gpu, 32, k=8192)      # the next growth finds no live graph and lets the retired buffer go
+        try:
+            huge.set_x(synth.random_activation(32, huge.k, seed=7))
+            huge.calls()
+            huge.outputs()
+            assert scratch_info(gpu)[:2] == (0, 0)
+        finally:
+            huge.close()
+    finally:
+        st.close()
+        big.close()
+        gpu.close()
+
+
+def test_a_call_that_fails_inside_a_capture_ends_it():
+    gpu = Gpu()
+    L, ctx = gpu.L, gpu.ctx
+    st = Step(gpu, 8)
+    try:
+        x = synth.random_activation(8, st.k, seed=8)
+        st.set_x(x)
+        capi.check(L.turq_graph_begin(ctx), ctx)
+        # first use of the fragment buffer inside a capture: it would have to be allocated, which a capture does not allow
+        rc = L.turq_qmatmul_multi(ctx, 3, st.warr, st.x, capi.ACT_F32, 8, st.k, st.yarr, capi.ACT_F32, st.ldys, None,
+                                  capi.MEM_DEVICE, capi.ALGO_AUTO)
+        assert rc == capi.ERR_INVALID
+        assert "capture" in capi.last_error(ctx)
+        g = ctypes.c_void_p()
+        assert L.turq_graph_end(ctx, ctypes.byref(g)) == capi.ERR_INVALID      # the capture is gone
+        assert not g.value
+        st.calls()                                                             # stream and context are usable again
+        want = st.outputs()
+        for dt, n, raw, y in zip(st.dts, st.ns, st.raws, want):
+            assert rel_l2(y, orc.matmul_dequant(dt, x, raw, n, st.k)) <= 1e-3
+        capi.check(L.turq_graph_begin(ctx), ctx)                               # and so is capturing
+        st.calls()
+        capi.check(L.turq_graph_end(ctx, ctypes.byref(g)), ctx)
+        st.clear_outputs()
+        capi.check(L.turq_graph_launch(ctx, g), ctx)
+        for y, w in zip(st.outputs(), want):
+            assert np.array_equal(y, w)
+        L.turq_graph_destroy(g)
+    finally:
+        st.close()
+        gpu.close()

@@ -55,6 +55,7 @@ _SIGS = {
     "turq_graph_end": (c_int, [c_void_p, POINTER(c_void_p)]),
     "turq_graph_launch": (c_int, [c_void_p, c_void_p]),
     "turq_graph_destroy": (None, [c_void_p]),
+    "turq_ctx_scratch_info": (c_int, [c_void_p, POINTER(c_int), POINTER(c_int), POINTER(c_size_t)]),
     "turq_profile_begin": (c_int, [c_void_p]),
     "turq_profile_end": (c_int, [c_void_p, POINTER(c_int64), POINTER(c_double)]),
     "turq_gguf_open": (c_int, [c_char_p, POINTER(c_void_p)]),

@@ -16,8 +16,22 @@ int turq_ctx_reserve(turq_ctx *ctx, void **buf, size_t *cap, size_t need) {
     if (ctx->capturing)
         return turq_fail(ctx, TURQ_ERR_INVALID, "a scratch buffer would have to grow (%zu > %zu bytes) while a graph is being captured: run the same calls once before turq_graph_begin", need, *cap);
     TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));  // the old buffer may still be in use
+    const bool graphs_alive = ctx->tally && ctx->tally->live.load(std::memory_order_acquire) > 0;
+    if (!graphs_alive) {  // nothing refers to outgrown buffers any more
+        for (void *p : ctx->retired) (void)hipFree(p);
+        ctx->retired.clear();
+    }
     if (*buf) {
-        TURQ_HIP(ctx, hipFree(*buf));
+        // a captured graph holds the addresses it was recorded with: while one is alive the old buffer stays allocated
+        if (graphs_alive) {
+            try {
+                ctx->retired.push_back(*buf);
+            } catch (const std::bad_alloc &) {
+                return turq_fail(ctx, TURQ_ERR_OOM, "turq_ctx_reserve: out of host memory");
+            }
+        } else {
+            TURQ_HIP(ctx, hipFree(*buf));
+        }
         *buf = nullptr;
         *cap = 0;
     }
@@ -114,6 +128,11 @@ int turq_ctx_create(int device, turq_ctx **out) {
     if (e != hipSuccess) return turq_fail(nullptr, TURQ_ERR_HIP, "hipGetDeviceProperties failed: %s", hipGetErrorString(e));
     ctx->compute_units = prop.multiProcessorCount;
     snprintf(ctx->device_name, sizeof ctx->device_name, "%s (%s)", prop.name, prop.gcnArchName);
+    try {
+        ctx->tally = std::make_shared<turq_graph_tally>();
+    } catch (const std::bad_alloc &) {
+        return turq_fail(nullptr, TURQ_ERR_OOM, "turq_ctx_create: out of host memory");
+    }
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e != hipSuccess) return turq_fail(nullptr, TURQ_ERR_HIP, "hipStreamCreate failed: %s", hipGetErrorString(e));
     *out = ctx.release();
@@ -129,6 +148,7 @@ void turq_ctx_destroy(turq_ctx *ctx) {
     if (ctx->act_prep) (void)hipFree(ctx->act_prep);
     if (ctx->gate_up) (void)hipFree(ctx->gate_up);
     if (ctx->stage_b) (void)hipFree(ctx->stage_b);
+    for (void *p : ctx->retired) (void)hipFree(p);  // graphs that still refer to them can no longer be launched: that needs the context
     for (auto &p : ctx->prof_events) { (void)hipEventDestroy(p.first); (void)hipEventDestroy(p.second); }
     for (int i = 0; i < turq_ctx::kSide; i++) {
         if (ctx->side[i]) { (void)hipStreamSynchronize(ctx->side[i]); (void)hipStreamDestroy(ctx->side[i]); }
@@ -325,7 +345,7 @@ int turq_weight_export(turq_ctx *ctx, const turq_weight *w, void *host_bytes, si
 
 // ---- dequantize ----
 
-int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem) {
+static int impl_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem) {
     TURQ_ENTER(ctx);
     if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_dequantize: null weight");
     if (w->device != ctx->device) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_dequantize: weight lives on device %d, context on %d", w->device, ctx->device);
@@ -347,7 +367,7 @@ int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem
     return TURQ_OK;
 }
 
-int turq_embedding_lookup(turq_ctx *ctx, const turq_weight *w, const uint32_t *ids, int64_t count, void *out, int out_dtype,
+static int impl_embedding_lookup(turq_ctx *ctx, const turq_weight *w, const uint32_t *ids, int64_t count, void *out, int out_dtype,
                           int64_t ldo, int mem) {
     TURQ_ENTER(ctx);
     if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_embedding_lookup: null weight");
@@ -406,7 +426,7 @@ static int qmatmul_device(turq_ctx *ctx, const turq_weight *w, const void *x, in
     }
 }
 
-int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y, int yt,
+static int impl_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y, int yt,
                  int64_t ldy, const float *bias, int mem, int algo) {
     TURQ_ENTER(ctx);
     if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: null weight");
@@ -446,7 +466,7 @@ int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int
     return TURQ_OK;
 }
 
-int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int xt, int64_t m,
+static int impl_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int xt, int64_t m,
                        int64_t ldx, void *const *ys, int yt, const int64_t *ldys, const float *const *biases, int mem, int algo) {
     TURQ_ENTER(ctx);
     if (count < 0) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_multi: count=%d is negative", count);
@@ -489,7 +509,7 @@ uint16_t host_bf16(float v) {  // round to nearest even, as the kernels store it
 }
 }  // namespace
 
-int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m, int64_t ldx,
+static int impl_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m, int64_t ldx,
                          void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, int act, int mem) {
     TURQ_ENTER(ctx);
     if (!gate || !up) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_gate_up: null weight");
@@ -565,7 +585,8 @@ int turq_graph_end(turq_ctx *ctx, turq_graph **out) {
     TURQ_ENTER(ctx);
     if (!out) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_end: null out pointer");
     *out = nullptr;
-    if (!ctx->capturing) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_end: no capture is running");
+    if (!ctx->capturing)
+        return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_end: no capture is running (a call that fails inside a capture ends and discards it)");
     ctx->capturing = false;
     std::unique_ptr<turq_graph> g(new (std::nothrow) turq_graph);
     hipGraph_t graph = nullptr;
@@ -581,6 +602,9 @@ int turq_graph_end(turq_ctx *ctx, turq_graph **out) {
         (void)hipGraphDestroy(graph);
         return turq_fail(ctx, TURQ_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
     }
+    // from here on the graph refers to the context's scratch buffers by address (see turq_ctx_reserve)
+    g->tally = ctx->tally;
+    g->tally->live.fetch_add(1, std::memory_order_acq_rel);
     *out = g.release();
     return TURQ_OK;
 }
@@ -598,6 +622,7 @@ void turq_graph_destroy(turq_graph *g) {
     DeviceGuard guard(g->device);
     if (g->exec) (void)hipGraphExecDestroy(g->exec);
     if (g->graph) (void)hipGraphDestroy(g->graph);
+    if (g->tally) g->tally->live.fetch_sub(1, std::memory_order_acq_rel);
     delete g;
 }
 
@@ -659,14 +684,64 @@ static int quantize_common(turq_ctx *ctx, const float *x, int64_t m, int64_t k, 
     return TURQ_OK;
 }
 
-int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
+static int impl_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
     TURQ_ENTER(ctx);
     return quantize_common(ctx, x, m, k, out, mem, false);
 }
 
-int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
+static int impl_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
     TURQ_ENTER(ctx);
     return quantize_common(ctx, x, m, k, out, mem, true);
+}
+
+
+// ---- the entry points a graph capture may hold ----
+// A call that fails while the context's stream is capturing ends the capture and discards what was recorded, so that the stream
+// and the context are usable again (turq_graph_end then reports that no capture is running).
+static int capture_guard(turq_ctx *ctx, int rc) {
+    if (rc != TURQ_OK && ctx && ctx->capturing) {
+        hipGraph_t dead = nullptr;
+        (void)hipStreamEndCapture(ctx->stream, &dead);
+        if (dead) (void)hipGraphDestroy(dead);
+        (void)hipGetLastError();  // ending an invalidated capture reports an error of its own
+        ctx->capturing = false;
+        ctx->err += " (the graph capture in progress was ended and discarded)";
+    }
+    return rc;
+}
+
+int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem) {
+    return capture_guard(ctx, impl_dequantize(ctx, w, out, out_mem));
+}
+int turq_embedding_lookup(turq_ctx *ctx, const turq_weight *w, const uint32_t *ids, int64_t count, void *out, int out_dtype,
+                          int64_t ldo, int mem) {
+    return capture_guard(ctx, impl_embedding_lookup(ctx, w, ids, count, out, out_dtype, ldo, mem));
+}
+int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y, int yt,
+                 int64_t ldy, const float *bias, int mem, int algo) {
+    return capture_guard(ctx, impl_qmatmul(ctx, w, x, xt, m, ldx, y, yt, ldy, bias, mem, algo));
+}
+int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int xt, int64_t m,
+                       int64_t ldx, void *const *ys, int yt, const int64_t *ldys, const float *const *biases, int mem, int algo) {
+    return capture_guard(ctx, impl_qmatmul_multi(ctx, count, weights, x, xt, m, ldx, ys, yt, ldys, biases, mem, algo));
+}
+int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m, int64_t ldx,
+                         void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, int act, int mem) {
+    return capture_guard(ctx, impl_qmatmul_gate_up(ctx, gate, up, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, act, mem));
+}
+int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
+    return capture_guard(ctx, impl_quantize_q8_0(ctx, x, m, k, out, mem));
+}
+int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
+    return capture_guard(ctx, impl_quantize_q8_k(ctx, x, m, k, out, mem));
+}
+
+int turq_ctx_scratch_info(const turq_ctx *ctx, int *live_graphs, int *retired_buffers, size_t *act_prep_bytes) {
+    if (!ctx) return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_ctx_scratch_info: null context");
+    if (live_graphs) *live_graphs = ctx->tally ? ctx->tally->live.load(std::memory_order_acquire) : 0;
+    if (retired_buffers) *retired_buffers = (int)ctx->retired.size();
+    if (act_prep_bytes) *act_prep_bytes = ctx->act_prep_cap;
+    return TURQ_OK;
 }
 
 }  // extern "C"

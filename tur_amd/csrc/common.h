@@ -8,6 +8,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <memory>
 #include <string>
 #include <utility>
 #include <vector>
@@ -61,6 +62,13 @@ inline int turq_act_bytes(int act) {
 }
 
 // ---- objects behind the opaque handles ----
+// Live graphs of a context, shared between the context and its graphs (either may be destroyed first).  While the count is
+// above zero a scratch buffer that has to grow is retired instead of freed: a captured graph keeps the addresses it was
+// recorded with.
+struct turq_graph_tally {
+    std::atomic<int> live{0};
+};
+
 struct turq_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -73,6 +81,10 @@ struct turq_ctx {
     void *stage_b = nullptr;  size_t stage_b_cap = 0;
     void *act_prep = nullptr; size_t act_prep_cap = 0;
     void *gate_up = nullptr;  size_t gate_up_cap = 0;  // the two f32 products of turq_qmatmul_gate_up's general path
+    // scratch buffers that were outgrown while a captured graph still referred to them: freed once no graph of the context is
+    // alive (at the next growth) or with the context
+    std::vector<void *> retired;
+    std::shared_ptr<turq_graph_tally> tally;
     // further streams for small prefill GEMMs of one turq_qmatmul_multi call that run next to each other: forked from `stream`
     // where the first launch of a group starts and joined again before the call returns (created on first use)
     static constexpr int kSide = 2;
@@ -89,6 +101,7 @@ struct turq_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     int device = 0;
+    std::shared_ptr<turq_graph_tally> tally;  // of the context it was captured on
 };
 
 // Kernel timing: hands out the next event pair (both null unless turq_profile_begin is active).
