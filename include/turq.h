@@ -161,6 +161,23 @@ int turq_embedding_lookup(turq_ctx *ctx, const turq_weight *w, const uint32_t *i
 int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype, int64_t m,
                  int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias, int mem, int algo);
 
+/* turq_qmatmul for callers that cannot allocate device memory around the call (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same product, same kernels and bit-identical results as turq_qmatmul with
+ * TURQ_MEM_DEVICE and TURQ_ALGO_AUTO, but the prepared activation fragments of calls with more than
+ * one row live in a static device array of TURQ_NOALLOC_SCRATCH_BYTES (one copy per GPU, held until
+ * the process ends) instead of the context's growable buffer: the call runs no hipMalloc / hipFree
+ * and creates no stream or event.  A call that needs more is refused with TURQ_ERR_SHAPE and a
+ * message that names the bytes needed: fragments take 2.25 * mpad * k bytes for up to 32 rows (mpad
+ * = m rounded up to 1, 2, 4, 8, 16 or 32) and 2.125 * 32 * ceil(m / 32) * k bytes above, so 16 MiB
+ * hold e.g. m = 512 at k = 12288 or m = 1920 at k = 4096.  x, y and bias are device pointers.
+ * All contexts of a GPU share that GPU's array and it keeps the last call's contents (every call
+ * writes all it reads, nothing has to start at zero): calls through this entry point that overlap
+ * on one GPU - two contexts, i.e. two streams - race; serialise them. */
+#define TURQ_NOALLOC_SCRATCH_BYTES (16u << 20)
+int turq_qmatmul_noalloc(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype, int64_t m,
+                         int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias);
+
 /* The same product for `count` weights that take the same activations: ys[i][m, n_i] = x[m, k] * W_i^T (+ biases[i]).
  * All weights must share k.  With device pointers, tiled weights and m <= 32, neighbouring weights of one format
  * go out as ONE kernel launch (for more than one row on all but small matrices, or activation rows that are not

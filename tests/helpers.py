@@ -82,8 +82,8 @@ class Gpu:
         capi.check(self.L.turq_memcpy_d2h(self.ctx, capi.ptr(out), p, out.nbytes), self.ctx)
         return out
 
-    def qmatmul_device(self, w, x, n, k, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_F32, algo=capi.ALGO_AUTO):
-        """turq_qmatmul on device pointers; x: f32 values [m, k]; returns the output as the call
+    def qmatmul_device(self, w, x, n, k, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_F32, noalloc=False, algo=capi.ALGO_AUTO):
+        """turq_qmatmul (or turq_qmatmul_noalloc) on device pointers; x: f32 values [m, k]; returns the output as the call
         wrote it (f32 values; bf16 outputs widened)"""
         x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
         m = x.shape[0]
@@ -92,7 +92,10 @@ class Gpu:
         xd = self.dev_buffer(xsend)
         yd = self.dev_buffer(np.full((m, n), 0, ydt))
         try:
-            rc = self.L.turq_qmatmul(self.ctx, w, xd, x_dtype, m, k, yd, y_dtype, n, None, capi.MEM_DEVICE, algo)
+            if noalloc:
+                rc = self.L.turq_qmatmul_noalloc(self.ctx, w, xd, x_dtype, m, k, yd, y_dtype, n, None)
+            else:
+                rc = self.L.turq_qmatmul(self.ctx, w, xd, x_dtype, m, k, yd, y_dtype, n, None, capi.MEM_DEVICE, algo)
             capi.check(rc, self.ctx)
             y = self.read_back(yd, (m, n), ydt)
         finally:

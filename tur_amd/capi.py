@@ -17,6 +17,7 @@ LAYOUT_NATIVE, LAYOUT_TILED = 0, 1
 MEM_HOST, MEM_DEVICE = 0, 1
 ALGO_AUTO, ALGO_SIMPLE, ALGO_GEMV, ALGO_GEMM = 0, 1, 2, 3
 ACTFN_SILU = 0
+NOALLOC_SCRATCH_BYTES = 16 << 20
 
 # every symbol include/turq.h declares: (restype, argtypes)
 _SIGS = {
@@ -45,6 +46,7 @@ _SIGS = {
     "turq_dequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_int]),
     "turq_embedding_lookup": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int]),
     "turq_qmatmul": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int, c_int]),
+    "turq_qmatmul_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p]),
     "turq_qmatmul_multi": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p, c_void_p,
                                    c_int, c_int]),
     "turq_qmatmul_gate_up": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64,

@@ -13,6 +13,8 @@ std::string &turq_thread_error() {
 
 int turq_ctx_reserve(turq_ctx *ctx, void **buf, size_t *cap, size_t need) {
     if (need <= *cap) return TURQ_OK;
+    if (ctx->fixed_scratch)
+        return turq_fail(ctx, TURQ_ERR_INVALID, "this call needs %zu bytes of scratch memory, the static array it may use holds %zu", need, *cap);
     if (ctx->capturing)
         return turq_fail(ctx, TURQ_ERR_INVALID, "a scratch buffer would have to grow (%zu > %zu bytes) while a graph is being captured: run the same calls once before turq_graph_begin", need, *cap);
     TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));  // the old buffer may still be in use
@@ -46,6 +48,7 @@ hipError_t turq_prof_next(turq_ctx *ctx, hipEvent_t *start, hipEvent_t *stop) {
     *stop = nullptr;
     if (!ctx->profiling) return hipSuccess;
     if (ctx->prof_used == ctx->prof_events.size()) {
+        if (ctx->fixed_scratch) return hipSuccess;  // a call that may not allocate: this launch goes untimed
         hipEvent_t a = nullptr, b = nullptr;
         hipError_t e = hipEventCreate(&a);
         if (e != hipSuccess) return e;
@@ -133,6 +136,9 @@ int turq_ctx_create(int device, turq_ctx **out) {
     } catch (const std::bad_alloc &) {
         return turq_fail(nullptr, TURQ_ERR_OOM, "turq_ctx_create: out of host memory");
     }
+    // the device's copy of the static scratch array of turq_qmatmul_noalloc; a failure is reported by that entry point
+    ctx->static_scratch_err = (int)turq_static_scratch(&ctx->static_scratch, &ctx->static_scratch_cap);
+    if (ctx->static_scratch_err != (int)hipSuccess) { ctx->static_scratch = nullptr; ctx->static_scratch_cap = 0; }
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e != hipSuccess) return turq_fail(nullptr, TURQ_ERR_HIP, "hipStreamCreate failed: %s", hipGetErrorString(e));
     *out = ctx.release();

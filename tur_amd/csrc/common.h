@@ -85,6 +85,12 @@ struct turq_ctx {
     // alive (at the next growth) or with the context
     std::vector<void *> retired;
     std::shared_ptr<turq_graph_tally> tally;
+    // turq_qmatmul_noalloc: for the duration of such a call act_prep points at the device's static scratch array and nothing
+    // may be allocated (turq_ctx_reserve fails instead of growing, no timing events are created)
+    bool fixed_scratch = false;
+    void *static_scratch = nullptr;       // this device's copy of the static array (hipGetSymbolAddress at context creation)
+    size_t static_scratch_cap = 0;
+    int static_scratch_err = 0;           // hipError_t of that lookup
     // further streams for small prefill GEMMs of one turq_qmatmul_multi call that run next to each other: forked from `stream`
     // where the first launch of a group starts and joined again before the call returns (created on first use)
     static constexpr int kSide = 2;
@@ -146,6 +152,8 @@ inline int turq_fail(turq_ctx *ctx, int code, const char *fmt, ...) {
 
 // grow-only scratch on the context's device
 int turq_ctx_reserve(turq_ctx *ctx, void **buf, size_t *cap, size_t need);
+// The static scratch array of the current device (noalloc.hip): its device address and size.  The device must be current.
+hipError_t turq_static_scratch(void **ptr, size_t *cap);
 
 // ---- kernel launchers implemented in the .hip translation units ----
 // All are asynchronous on `stream` and return hipGetLastError() of the launch.
