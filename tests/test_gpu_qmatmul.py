@@ -569,6 +569,24 @@ def test_one_row_launch_shapes(row_tiles, in_flight):
     assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-1000:]
 
 
+# The kernel that keeps a column tile's activation fragments in registers (gemv_cs.hip) is picked for launches of several row
+# tiles per compute unit, which the small matrices here never are: the batch tests run once more in child processes with each of
+# its row-tile group sizes forced (every format, m = 2 .. 32, ragged shapes, strides, biases, all activation and output types).
+@pytest.mark.parametrize("row_tiles", [2, 3, 6])
+def test_rows_in_registers_kernel_shapes(row_tiles):
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, TURQ_CS_RG=str(row_tiles))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    picked = ("test_mfma_gemv_tiled_layout or test_multi_weight_launch or test_activation_and_output_dtypes or test_bias_and_row_strides "
+              "or test_q8_0_ragged_k or test_single_tile_shapes or test_mfma_more_rows_than_one_launch")
+    out = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "-k", picked, "-p", "no:cacheprovider",
+                          os.path.join(root, "tests", "test_gpu_qmatmul.py")], cwd=root, env=env, capture_output=True, text=True, timeout=280)
+    assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-1000:]
+
+
 # The prefill GEMM picks its tile (128 x 128, 128 x 192, the wide 128 x 256 with two-deep rings, or the low 64 x 128 for launches
 # that would leave CUs idle) from the problem size; the small matrices of the tests above would never reach the wide one and
 # always take the low one, so they run once more in child processes with each of the two forced and forbidden (the rule takes

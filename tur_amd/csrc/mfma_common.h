@@ -170,6 +170,10 @@ hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w_tile
                                  int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
                                  const float *const *bias, int waves_per_group, int row_tiles_per_group, hipStream_t stream,
                                  hipEvent_t ev_start, hipEvent_t ev_stop);
+bool turq_gemv_cs_rows_ok(int row_tiles_per_group);
+hipError_t turq_launch_gemv_cs(int dtype, int count, const void *const *w_tiled, const int64_t *n, int64_t k, const void *x, int x_dtype,
+                               int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy, const float *const *bias,
+                               int nwaves, int row_tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
 bool turq_gemv_multi_mixed_supports(int dtype_a, int dtype_b);
 hipError_t turq_launch_gemv_multi_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w_tiled, const int64_t *n,
                                         int64_t k, const void *frags, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,

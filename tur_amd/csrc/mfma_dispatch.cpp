@@ -72,6 +72,27 @@ int pick_rows_row1(const turq_ctx *ctx, int64_t row_tiles) {
     return row_tiles >= 16 * cus ? 2 : 1;
 }
 
+// Row tiles per workgroup of the kernel that keeps a column tile's activation fragments in registers and streams the row tiles
+// past them (gemv_cs.hip), or 0 where it does not apply.  It needs no preparation launch and reads the activations once per
+// workgroup, but runs one eight-wave workgroup per compute unit: measured against preparation + prepared-fragment kernel it
+// wins where the launch is one to two such workgroups per unit (gate + up of an MLP: 5 .. 15 % for 5 <= m <= 16, Q4_K and Q6_K)
+// and loses where there are many (the LM head: - 12 .. - 30 %) or 32 rows (registers).  TURQ_CS = 0 switches it off,
+// TURQ_CS_RG forces the group size (2, 3 or 6).
+int cs_row_tiles(const turq_ctx *ctx, int64_t m, int64_t row_tiles, int dtype, bool aligned) {
+    static const int mode = [] { const char *e = getenv("TURQ_CS"); return e ? atoi(e) : -1; }();
+    static const int forced = [] { const char *e = getenv("TURQ_CS_RG"); return e ? atoi(e) : 0; }();
+    if (mode == 0 || !aligned || m < 2 || m > TURQ_GEMV_MAX_M) return 0;
+    const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+    int rg = (m <= 16 && dtype != TURQ_Q8_0 && row_tiles >= 6 * cus && row_tiles <= 12 * cus) ? 6 : 0;
+    if (forced && turq_gemv_cs_rows_ok(forced)) {
+        rg = forced;
+        // instantiations that do not fit the register file
+        if (rg == 6 && (m > 16 || dtype == TURQ_Q8_0)) rg = 3;
+        if (rg == 3 && dtype == TURQ_Q8_0 && m > 16) rg = 2;
+    }
+    return rg;
+}
+
 // whether the prefill GEMM can take this weight (its largest packed value must fit f16), and the power of two by which the
 // kernel multiplies the block scales
 bool gemm_takes(const turq_weight *w, float *wscale) {
@@ -325,6 +346,28 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
                                                           yt, ldy + i, bias ? bias + i : nullptr, pick_waves_row1(w[i]->k), ctx->stream,
                                                           ev0, ev1));
                 i = j2;
+                continue;
+            }
+        }
+        if (!row1_ok) {
+            // several row tiles per compute unit: fragments in registers, built from the rows themselves, no preparation
+            int64_t tiles = 0;
+            for (int t = i; t < j; t++) tiles += turq_tile_rows(w[t]->n);
+            const int rg = cs_row_tiles(ctx, m, tiles, w[i]->dtype, aligned);
+            if (rg) {
+                const void *wp[4];
+                int64_t nn[4];
+                for (int t = i; t < j; t++) {
+                    wp[t - i] = w[t]->dev;
+                    nn[t - i] = w[t]->n;
+                }
+                static const int cs_waves = [] { const char *e = getenv("TURQ_CS_WAVES"); return e ? atoi(e) : 0; }();
+                const int nw = (int)std::min<int64_t>(cs_waves >= 1 && cs_waves <= 8 ? cs_waves : 8, turq_tile_cols(w[i]->k));
+                hipEvent_t ev0 = nullptr, ev1 = nullptr;
+                TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+                TURQ_HIP(ctx, turq_launch_gemv_cs(w[i]->dtype, j - i, wp, nn, w[i]->k, x, xt, ldx, m, y + i, yt, ldy + i,
+                                                  bias ? bias + i : nullptr, nw, rg, ctx->stream, ev0, ev1));
+                i = j;
                 continue;
             }
         }
