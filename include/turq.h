@@ -145,6 +145,16 @@ int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem
 int turq_embedding_lookup(turq_ctx *ctx, const turq_weight *w, const uint32_t *ids, int64_t count, void *out, int out_dtype,
                           int64_t ldo, int mem);
 
+/* ---- RmsNorm ---- */
+/* y[r][c] = x[r][c] / sqrt(mean_c(x[r][c]^2) + eps) * weight[c] for m rows of k elements, in f32 and in candle's order (sum of
+ * squares, one square root, per element a division and a multiplication).  weight: f32 [k] in the same memory space as x
+ * and y - the `weight` tensor of the GGUF file as turq_dequantize returns it (a Gemma model adds 1 to it at load,
+ * src/models/layers/norm.rs:89).  x, y, strides and `mem` as in turq_qmatmul; y may be x.
+ * Replaces: `NormX::forward` over candle_nn::RmsNorm built by `layers::norm::rms_norm` (src/models/layers/norm.rs:52-94),
+ * which the decoder layers apply in front of the q / k / v and gate / up projections. */
+int turq_rms_norm(turq_ctx *ctx, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, const float *weight,
+                  float eps, void *y, int y_dtype, int64_t ldy, int mem);
+
 /* ---- forward ---- */
 /* y[m, n] = x[m, k] * W^T  (+ bias[n] when bias != NULL).
  *   x: m rows of k elements of `x_dtype`, row stride ldx elements (ldx >= k);

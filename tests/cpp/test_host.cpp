@@ -108,7 +108,32 @@ int main(int argc, char **argv) {
         // dequantize of the norm weight (F32 tensor) is a copy
         std::vector<float> norm = b0.pp("attn_norm").get({k}, "weight").dequantize();
         std::printf("norm %zu %.9g %.9g\n", norm.size(), norm.front(), norm.back());
-        try { turq::QMatMul::from_arc(b0.pp("attn_norm").get({k}, "weight")); return fail("dense tensor accepted by QMatMul"); } catch (const turq::Error &) {}
+        // a dense tensor takes the dense arm of QMatMul::from_arc: a [1, k] weight against one row is the dot product
+        {
+            turq::QMatMul dense = turq::QMatMul::from_arc(b0.pp("attn_norm").get({k}, "weight"));
+            if (!dense.dense()) return fail("dense tensor did not take the dense arm");
+            const std::vector<float> one = dense.forward(std::vector<float>(norm.begin(), norm.end()), 1);
+            double want = 0.0;
+            for (float v : norm) want += (double)v * (double)v;
+            if (one.size() != 1 || std::fabs((double)one[0] - want) > 1e-5 * want) return fail("dense arm: wrong dot product");
+        }
+        // RmsNorm from the same tensor, then checked against the formula
+        {
+            turq::NormX nx = turq::rms_norm(k, 1e-6, b0.pp("attn_norm"));
+            turq::NormX copy = nx;  // NormX is Clone in the reference
+            std::vector<float> xs((size_t)2 * k);
+            for (size_t i = 0; i < xs.size(); i++) xs[i] = std::cos(0.11f * (float)i) * 3.0f;
+            const std::vector<float> ys = copy.forward(xs, 2);
+            for (int r = 0; r < 2; r++) {
+                double ss = 0.0;
+                for (int64_t c = 0; c < k; c++) ss += (double)xs[r * k + c] * (double)xs[r * k + c];
+                const double rms = std::sqrt(ss / (double)k + 1e-6);
+                for (int64_t c = 0; c < k; c++) {
+                    const double w = (double)xs[r * k + c] / rms * (double)norm[c];
+                    if (std::fabs((double)ys[r * k + c] - w) > 1e-5 * (std::fabs(w) + 1e-3)) return fail("rms norm differs from the formula");
+                }
+            }
+        }
     } catch (const std::exception &e) {
         std::fprintf(stderr, "FAIL: exception: %s\n", e.what());
         return 1;

@@ -142,3 +142,76 @@ def test_gguf_v2_and_alignment(tmp_path):
     capi.check(L.turq_gguf_read_tensor(g, b"b.weight", capi.ptr(buf), buf.size))
     assert np.array_equal(buf, raw[::-1])
     L.turq_gguf_close(g)
+
+
+# ---- a GGUF file assembled by hand from the published layout (not by tur_amd.gguf), and hostile variants of it ----
+def _gguf_v3_bytes(tensor_offset_1=None, dup=False, str_len=None, arr_len=None):
+    import struct
+
+    def s(b):
+        return struct.pack("<Q", len(b)) + b
+
+    q8 = bytes(range(34)) * 2                       # one row of two Q8_0 blocks: [1, 64]
+    f32 = struct.pack("<6f", 1.0, 2.0, 3.0, 4.0, 5.0, 6.0)      # [2, 3] row-major
+    head = b"GGUF" + struct.pack("<I", 3) + struct.pack("<QQ", 2, 3)
+    # metadata: one string, one u32, one array of three i32
+    head += s(b"general.architecture") + struct.pack("<I", 8) + (struct.pack("<Q", str_len) + b"qwen3" if str_len is not None else s(b"qwen3"))
+    head += s(b"qwen3.block_count") + struct.pack("<II", 4, 36)
+    head += s(b"some.list") + struct.pack("<IIQ", 9, 5, 3 if arr_len is None else arr_len) + struct.pack("<3i", 7, 8, 9)
+    # tensor infos: name, n_dims, dims innermost first, ggml dtype, offset into the data section
+    head += s(b"blk.0.w") + struct.pack("<I", 2) + struct.pack("<QQ", 64, 1) + struct.pack("<IQ", 8, 0)
+    second = b"blk.0.w" if dup else b"norm.weight"
+    head += s(second) + struct.pack("<I", 2) + struct.pack("<QQ", 3, 2) + struct.pack("<IQ", 0, 96 if tensor_offset_1 is None else tensor_offset_1)
+    pad = (-len(head)) % 32
+    data = q8 + b"\0" * (96 - len(q8)) + f32          # second tensor at the next multiple of 32 after 68 bytes
+    return head + b"\0" * pad + data, len(head) + pad, q8, f32
+
+
+def test_gguf_reader_on_a_hand_assembled_file(tmp_path):
+    L = capi.lib()
+    blob, data_off, q8, f32 = _gguf_v3_bytes()
+    p = tmp_path / "hand.gguf"
+    p.write_bytes(blob)
+    g = ctypes.c_void_p()
+    assert L.turq_gguf_open(str(p).encode(), ctypes.byref(g)) == capi.OK, capi.last_error()
+    assert L.turq_gguf_tensor_count(g) == 2
+    assert [L.turq_gguf_tensor_name(g, i) for i in range(2)] == [b"blk.0.w", b"norm.weight"]
+    dt, nd, off, nb = ctypes.c_int(), ctypes.c_int(), ctypes.c_uint64(), ctypes.c_size_t()
+    dims = (ctypes.c_int64 * 4)()
+    assert L.turq_gguf_tensor_info(g, b"blk.0.w", ctypes.byref(dt), ctypes.byref(nd), dims, ctypes.byref(off), ctypes.byref(nb)) == capi.OK
+    assert (dt.value, nd.value, dims[0], dims[1], off.value, nb.value) == (capi.Q8_0, 2, 1, 64, data_off, 68)      # (n, k): GGUF order reversed
+    assert L.turq_gguf_tensor_info(g, b"norm.weight", ctypes.byref(dt), ctypes.byref(nd), dims, ctypes.byref(off), ctypes.byref(nb)) == capi.OK
+    assert (dt.value, nd.value, dims[0], dims[1], off.value, nb.value) == (capi.F32, 2, 2, 3, data_off + 96, 24)
+    buf = ctypes.create_string_buffer(68)
+    assert L.turq_gguf_read_tensor(g, b"blk.0.w", buf, 68) == capi.OK and buf.raw == q8
+    buf = ctypes.create_string_buffer(24)
+    assert L.turq_gguf_read_tensor(g, b"norm.weight", buf, 24) == capi.OK and buf.raw == f32
+    v = ctypes.c_uint64()
+    assert L.turq_gguf_meta_u64(g, b"qwen3.block_count", ctypes.byref(v)) == capi.OK and v.value == 36
+    assert L.turq_gguf_meta_u64(g, b"some.list", ctypes.byref(v)) == capi.OK and v.value == 3      # arrays report their length
+    name = ctypes.create_string_buffer(32)
+    assert L.turq_gguf_meta_str(g, b"general.architecture", name, 32) == capi.OK and name.value == b"qwen3"
+    L.turq_gguf_close(g)
+
+
+@pytest.mark.parametrize("kwargs,what", [
+    (dict(tensor_offset_1=2**64 - 8), "runs past the end"),        # offset + size wraps around 2^64
+    (dict(tensor_offset_1=10**6), "runs past the end"),
+    (dict(dup=True), "listed twice"),
+    (dict(str_len=2**40), "runs past the end"),                    # a string longer than the file
+    (dict(arr_len=2**62), "runs past the end"),                    # array length * element size wraps
+], ids=["offset-wraps", "offset-beyond", "duplicate-name", "string-length", "array-length"])
+def test_gguf_reader_refuses_hostile_files(tmp_path, kwargs, what):
+    L = capi.lib()
+    blob = _gguf_v3_bytes(**kwargs)[0]
+    p = tmp_path / "bad.gguf"
+    p.write_bytes(blob)
+    g = ctypes.c_void_p()
+    rc = L.turq_gguf_open(str(p).encode(), ctypes.byref(g))
+    if rc == capi.OK:          # the header parses; the tensor whose bytes are not there must be refused on read
+        buf = ctypes.create_string_buffer(24)
+        assert L.turq_gguf_read_tensor(g, b"norm.weight", buf, 24) == capi.ERR_IO
+        assert what in L.turq_gguf_last_error(g).decode()
+        L.turq_gguf_close(g)
+    else:
+        assert rc == capi.ERR_IO and what in capi.last_error()

@@ -168,8 +168,7 @@ def test_forward_argument_errors(model):
         layer.forward(np.zeros((2, 4, HID), np.float32)[:, ::2, :])     # not contiguous
     with pytest.raises(capi.TurqError):
         layer.forward(np.zeros((1, HID), np.float64))                   # unsupported dtype
-    with pytest.raises(capi.TurqError):
-        qlinear.QMatMul.from_arc(vb.pp("blk").pp(0).pp("attn_norm").get(HID, "weight"))   # dense tensor
+    assert qlinear.QMatMul.from_arc(vb.pp("blk").pp(0).pp("attn_norm").get(HID, "weight")).dense   # a dense tensor: the dense arm
     assert layer.forward(np.zeros((0, HID), np.float32)).shape == (0, KV)   # empty batch
 
 
@@ -202,3 +201,64 @@ def test_cpp_host_mirror(model, tmp_path):
     assert rel_l2(y, orc.matmul_dequant(Q4_K, x, gate, n, k)) <= 1e-3
     assert rel_l2(yb, orc.matmul_dequant(Q6_K, x, biased, 96, k) + bias) <= 1e-3
     assert lines[-3].startswith(f"norm {k} ")
+
+
+# ---- the dense arm of QMatMul::from_arc (src/models/layers/linear.rs:69 -> candle: F32 / F16 / BF16 tensors, and every
+# tensor under CANDLE_DEQUANTIZE_ALL, become a dense f32 matmul on the dequantized weights) ----
+def _dense_raw(dt, n, k, seed):
+    w = np.random.default_rng(seed).standard_normal((n, k)).astype(np.float32) * 0.05
+    if dt == capi.F32:
+        return w.view(np.uint8).reshape(-1)
+    if dt == capi.F16:
+        return w.astype(np.float16).view(np.uint8).reshape(-1)
+    return synth.to_bf16_bits(w).view(np.uint8).reshape(-1)
+
+
+@pytest.mark.parametrize("dt", [capi.F32, capi.F16, capi.BF16], ids=["f32", "f16", "bf16"])
+@pytest.mark.parametrize("n,k", [(96, 512), (33, 100), (7, 4099), (1, 5)])
+def test_dense_weights_take_the_dense_matmul(model, dt, n, k):
+    dev = model[0]
+    raw = _dense_raw(dt, n, k, seed=n + k)
+    layer = qlinear.LinearX(qlinear.QMatMul.from_arc(qlinear.QTensor.new(dev, dt, (n, k), raw)))
+    assert layer.qmatmul.dense
+    rng = np.random.default_rng(1)
+    for shape in ((1, 1, k), (2, 5, k), (1, 40, k)):
+        x = (rng.standard_normal(shape) * 3).astype(np.float32)
+        y = layer.forward(x)
+        want = orc.matmul_dequant(dt, x.reshape(-1, k), raw, n, k).reshape(y.shape)
+        assert y.shape == shape[:-1] + (n,)
+        assert rel_l2(y, want) <= 2e-6        # f32 products and sums against the f64 sum: no activation rounding
+
+
+def test_dense_weight_from_a_gguf_file_and_activation_range(model, tmp_path):
+    dev = model[0]
+    n, k = 48, 256
+    raw16 = _dense_raw(capi.F16, n, k, seed=3)
+    bias = np.random.default_rng(4).standard_normal(n).astype("<f4")
+    path = tmp_path / "dense.gguf"
+    write_gguf(str(path), [("output.weight", capi.F16, (n, k), raw16), ("output.bias", 0, (n,), bias.view(np.uint8))])
+    vb = qlinear.QVarBuilder.from_gguf(str(path), dev)
+    layer = qlinear.linear(k, n, vb.pp("output"))
+    assert layer.qmatmul.dense and np.array_equal(layer.bias, bias)
+    # the dense arm computes in f32: activations far outside the f16 range are fine
+    x = (np.random.default_rng(5).standard_normal((3, k)) * 1e6).astype(np.float32)
+    want = orc.matmul_dequant(capi.F16, x, raw16, n, k) + bias
+    assert rel_l2(layer.forward(x), want) <= 2e-6
+
+
+@pytest.mark.parametrize("dt", [Q8_0, Q4_K, Q5_K, Q6_K])
+def test_dequantize_all_switch(model, dt, monkeypatch):
+    # CANDLE_DEQUANTIZE_ALL: the quantized tensor becomes a dense f32 matmul on its dequantized values
+    dev = model[0]
+    n, k = 80, 1024
+    raw = synth.random_weight(dt, n, k, seed=dt)
+    qt = qlinear.QTensor.new(dev, dt, (n, k), raw)              # tiled, as the loader uploads matmul weights
+    x = np.random.default_rng(6).standard_normal((5, k)).astype(np.float32)
+    want = orc.matmul_dequant(dt, x, raw, n, k)
+    quantized = qlinear.QMatMul.from_arc(qt)
+    assert not quantized.dense
+    monkeypatch.setenv("CANDLE_DEQUANTIZE_ALL", "1")
+    dense = qlinear.QMatMul.from_arc(qt)
+    assert dense.dense
+    err_dense, err_quant = rel_l2(dense.forward(x), want), rel_l2(quantized.forward(x), want)
+    assert err_dense <= 2e-6 and err_quant <= 1e-3 and err_dense < err_quant

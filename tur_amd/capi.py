@@ -45,6 +45,7 @@ _SIGS = {
     "turq_untile_host": (c_int, [c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "turq_dequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_int]),
     "turq_embedding_lookup": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int]),
+    "turq_rms_norm": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_int, c_int64, c_int]),
     "turq_qmatmul": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_int, c_int]),
     "turq_qmatmul_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p]),
     "turq_qmatmul_multi": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p, c_void_p,

@@ -408,6 +408,38 @@ static int impl_embedding_lookup(turq_ctx *ctx, const turq_weight *w, const uint
     return TURQ_OK;
 }
 
+// ---- RmsNorm ----
+
+static int impl_rms_norm(turq_ctx *ctx, const void *x, int xt, int64_t m, int64_t k, int64_t ldx, const float *weight, float eps, void *y,
+                         int yt, int64_t ldy, int mem) {
+    TURQ_ENTER(ctx);
+    const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
+    if (!xb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_rms_norm: unsupported activation dtype %d", xt);
+    if (!yb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_rms_norm: unsupported output dtype %d", yt);
+    if (m < 0 || k < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_rms_norm: negative shape (%lld, %lld)", (long long)m, (long long)k);
+    if (ldx < k || ldy < k) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_rms_norm: a row stride (%lld, %lld) is smaller than k=%lld", (long long)ldx, (long long)ldy, (long long)k);
+    if (m == 0 || k == 0) return TURQ_OK;
+    if (!x || !y || !weight) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_rms_norm: null activation, weight or output pointer");
+    if (mem == TURQ_MEM_DEVICE) {
+        TURQ_HIP(ctx, turq_launch_rms_norm(x, xt, m, k, ldx, weight, eps, y, yt, ldy, ctx->stream));
+        return TURQ_OK;
+    }
+    if (mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_rms_norm: bad mem %d", mem);
+    const size_t xrow = (size_t)k * xb, yrow = (size_t)k * yb;
+    int rc = turq_ctx_reserve(ctx, &ctx->stage_x, &ctx->stage_x_cap, xrow * (size_t)m);
+    if (rc != TURQ_OK) return rc;
+    rc = turq_ctx_reserve(ctx, &ctx->stage_y, &ctx->stage_y_cap, yrow * (size_t)m);
+    if (rc != TURQ_OK) return rc;
+    rc = turq_ctx_reserve(ctx, &ctx->stage_b, &ctx->stage_b_cap, (size_t)k * sizeof(float));
+    if (rc != TURQ_OK) return rc;
+    TURQ_HIP(ctx, hipMemcpy2DAsync(ctx->stage_x, xrow, x, (size_t)ldx * xb, xrow, (size_t)m, hipMemcpyHostToDevice, ctx->stream));
+    TURQ_HIP(ctx, hipMemcpyAsync(ctx->stage_b, weight, (size_t)k * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
+    TURQ_HIP(ctx, turq_launch_rms_norm(ctx->stage_x, xt, m, k, k, (const float *)ctx->stage_b, eps, ctx->stage_y, yt, k, ctx->stream));
+    TURQ_HIP(ctx, hipMemcpy2DAsync(y, (size_t)ldy * yb, ctx->stage_y, yrow, yrow, (size_t)m, hipMemcpyDeviceToHost, ctx->stream));
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    return TURQ_OK;
+}
+
 // ---- forward ----
 
 static int qmatmul_device(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
@@ -437,8 +469,8 @@ static int impl_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int 
     TURQ_ENTER(ctx);
     if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: null weight");
     if (w->device != ctx->device) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: weight lives on device %d, context on %d", w->device, ctx->device);
-    if (!turq_dt_is_quant(w->dtype))
-        return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: weight dtype %s is not block-quantized (dequantize it and use a dense matmul)", turq_dt_name(w->dtype));
+    if (!turq_dt_is_quant(w->dtype) && w->dtype != TURQ_F32 && w->dtype != TURQ_F16 && w->dtype != TURQ_BF16)
+        return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: unsupported weight dtype %d", w->dtype);
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
     if (!xb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: unsupported activation dtype %d", xt);
     if (!yb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: unsupported output dtype %d", yt);
@@ -740,6 +772,11 @@ int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void
 }
 int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
     return capture_guard(ctx, impl_quantize_q8_k(ctx, x, m, k, out, mem));
+}
+
+int turq_rms_norm(turq_ctx *ctx, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, const float *weight, float eps, void *y,
+                  int y_dtype, int64_t ldy, int mem) {
+    return capture_guard(ctx, impl_rms_norm(ctx, x, x_dtype, m, k, ldx, weight, eps, y, y_dtype, ldy, mem));
 }
 
 int turq_ctx_scratch_info(const turq_ctx *ctx, int *live_graphs, int *retired_buffers, size_t *act_prep_bytes) {

@@ -161,6 +161,8 @@ hipError_t turq_launch_gather_rows(int dtype, int layout, const void *w, int64_t
                                    void *out, int out_dtype, int64_t ldo, hipStream_t stream);
 hipError_t turq_launch_dequant(int dtype, int layout, const void *w, int64_t n, int64_t k, float *out,
                                hipStream_t stream);
+hipError_t turq_launch_rms_norm(const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, const float *weight, float eps, void *y,
+                                int y_dtype, int64_t ldy, hipStream_t stream);
 hipError_t turq_launch_quantize_q8_0(const float *x, int64_t nblocks, void *out, hipStream_t stream);
 hipError_t turq_launch_quantize_q8_k(const float *x, int64_t nblocks, void *out, hipStream_t stream);
 hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t k, const void *x, int x_dtype,

@@ -2,6 +2,8 @@
 // to f32 in registers (same decode as the dequantize kernel), f32 FMA against the activations, and
 // a wave-wide shuffle reduction.  It is the straightforward statement of y = x * dequant(W)^T for
 // any shape and any m; the MFMA kernels on the tiled layout are the fast path.
+// It is also the dense arm of the layer: F32 / F16 / BF16 weights (candle's `QMatMul::from_arc` turns those GGUF tensors,
+// and every tensor under CANDLE_DEQUANTIZE_ALL, into a dense f32 matmul; src/models/layers/linear.rs:69), any k.
 #include "block_decode.h"
 
 namespace {
@@ -46,8 +48,28 @@ __global__ void __launch_bounds__(256) gemv_simple_kernel(const uint8_t *__restr
         float acc[MT];
 #pragma unroll
         for (int i = 0; i < MT; i++) acc[i] = 0.0f;
+        constexpr bool DENSE = DT == TURQ_F32 || DT == TURQ_F16 || DT == TURQ_BF16;
         for (int64_t e0 = (int64_t)lane * 8; e0 < k; e0 += 64 * 8) {
             float wv[8];
+            if (DENSE && e0 + 8 > k) {  // a dense row may end inside the lane's eight columns
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    if (e0 + j >= k) wv[j] = 0.0f;
+                    else if (DT == TURQ_F32) wv[j] = ((const float *)wr)[e0 + j];
+                    else if (DT == TURQ_F16) wv[j] = turq_h2f(((const uint16_t *)wr)[e0 + j]);
+                    else wv[j] = turq_bf2f(((const uint16_t *)wr)[e0 + j]);
+                }
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    if (m0 + i < m) {
+                        const int64_t base = (m0 + i) * ldx + e0;
+#pragma unroll
+                        for (int j = 0; j < 8; j++)
+                            if (e0 + j < k) acc[i] = fmaf(wv[j], load_act<XT>(x, base + j), acc[i]);
+                    }
+                }
+                continue;
+            }
             Decode8<DT>::run(wr, e0, wv);
 #pragma unroll
             for (int i = 0; i < MT; i++) {
@@ -110,6 +132,9 @@ hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t 
     case TURQ_Q4_K: return launch1<TURQ_Q4_K>(x_dtype, y_dtype, w, n, k, x, m, ldx, y, ldy, bias, stream);
     case TURQ_Q5_K: return launch1<TURQ_Q5_K>(x_dtype, y_dtype, w, n, k, x, m, ldx, y, ldy, bias, stream);
     case TURQ_Q6_K: return launch1<TURQ_Q6_K>(x_dtype, y_dtype, w, n, k, x, m, ldx, y, ldy, bias, stream);
+    case TURQ_F32: return launch1<TURQ_F32>(x_dtype, y_dtype, w, n, k, x, m, ldx, y, ldy, bias, stream);
+    case TURQ_F16: return launch1<TURQ_F16>(x_dtype, y_dtype, w, n, k, x, m, ldx, y, ldy, bias, stream);
+    case TURQ_BF16: return launch1<TURQ_BF16>(x_dtype, y_dtype, w, n, k, x, m, ldx, y, ldy, bias, stream);
     default: return hipErrorInvalidValue;
     }
 }

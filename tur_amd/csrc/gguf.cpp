@@ -55,6 +55,7 @@ namespace {
 struct Reader {
     FILE *fp;
     uint32_t version;
+    uint64_t file_size = 0;  // lengths read from the file are checked against what is left of it
     bool ok = true;
     std::string why;
     void fail(const std::string &m) { if (ok) { ok = false; why = m; } }
@@ -65,17 +66,23 @@ struct Reader {
     }
     template <typename T> T num() { T v{}; raw(&v, sizeof v); return v; }  // little-endian host assumed
     uint64_t count() { return version == 1 ? (uint64_t)num<uint32_t>() : num<uint64_t>(); }
+    uint64_t left() {
+        const off_t at = ftello(fp);
+        return at < 0 || (uint64_t)at > file_size ? 0 : file_size - (uint64_t)at;
+    }
     std::string str() {
         const uint64_t len = count();
         if (!ok) return {};
-        if (len > (1ull << 30)) { fail("string length is implausible"); return {}; }
+        if (len > (1ull << 30) || len > left()) { fail("string length " + std::to_string(len) + " runs past the end of the file"); return {}; }
         std::string s((size_t)len, '\0');
         raw(s.data(), (size_t)len);
         while (!s.empty() && s.back() == '\0') s.pop_back();  // GGUF v1 strings may carry a terminator
         return s;
     }
     void skip(uint64_t n) {
-        if (ok && fseeko(fp, (off_t)n, SEEK_CUR) != 0) fail("seek failed");
+        if (!ok) return;
+        if (n > left()) { fail("a value of " + std::to_string(n) + " bytes runs past the end of the file"); return; }
+        if (fseeko(fp, (off_t)n, SEEK_CUR) != 0) fail("seek failed");
     }
     static size_t scalar_size(uint32_t t) {
         switch (t) {
@@ -113,6 +120,7 @@ struct Reader {
             } else {
                 const size_t sz = scalar_size(v.elem_type);
                 if (!sz) fail("unknown array element type " + std::to_string(v.elem_type));
+                else if (v.u > left() / sz) fail("array of " + std::to_string(v.u) + " elements runs past the end of the file");
                 else skip(v.u * sz);
             }
             break;
@@ -138,10 +146,22 @@ const TensorInfo *find(const turq_gguf *g, const char *name) {
 
 extern "C" {
 
+static int gguf_open_impl(const char *path, turq_gguf **out);
+
 int turq_gguf_open(const char *path, turq_gguf **out) {
     if (!out) return gfail(nullptr, TURQ_ERR_INVALID, "turq_gguf_open: null out pointer");
     *out = nullptr;
     if (!path) return gfail(nullptr, TURQ_ERR_INVALID, "turq_gguf_open: null path");
+    try {  // strings, maps and vectors sized by the file: nothing may unwind through the C boundary
+        return gguf_open_impl(path, out);
+    } catch (const std::bad_alloc &) {
+        return gfail(nullptr, TURQ_ERR_OOM, std::string(path) + ": out of memory while reading the header");
+    } catch (const std::exception &e) {
+        return gfail(nullptr, TURQ_ERR_IO, std::string(path) + ": " + e.what());
+    }
+}
+
+static int gguf_open_impl(const char *path, turq_gguf **out) {
     std::unique_ptr<turq_gguf> g(new (std::nothrow) turq_gguf);
     if (!g) return gfail(nullptr, TURQ_ERR_OOM, "turq_gguf_open: out of memory");
     g->path = path;
@@ -156,7 +176,7 @@ int turq_gguf_open(const char *path, turq_gguf **out) {
     g->file_size = (uint64_t)ftello(g->fp);
     fseeko(g->fp, 0, SEEK_SET);
 
-    Reader rd{g->fp, 0};
+    Reader rd{g->fp, 0, g->file_size};
     const uint32_t magic = rd.num<uint32_t>();
     if (!rd.ok || magic != 0x46554747u) return bail(TURQ_ERR_IO, "not a GGUF file (bad magic)");
     g->version = rd.num<uint32_t>();
@@ -200,6 +220,7 @@ int turq_gguf_open(const char *path, turq_gguf **out) {
             }
             ti.nbytes = (size_t)(nelem / (uint64_t)be) * (size_t)turq_dt_block_bytes(ti.dtype);
         }  // dtypes this library cannot hold stay listed with nbytes == 0 and fail on load
+        if (g->tensors.count(name)) { rd.fail("tensor " + name + " is listed twice"); break; }
         g->names.push_back(name);
         g->tensors.emplace(std::move(name), ti);
     }
@@ -293,8 +314,10 @@ int turq_gguf_read_tensor(turq_gguf *g, const char *name, void *host_bytes, size
         return gfail(g, TURQ_ERR_SHAPE, std::string("tensor ") + name + " has " + std::to_string(ti->nbytes) + " bytes, buffer has " + std::to_string(nbytes));
     if (nbytes == 0) return TURQ_OK;
     if (!host_bytes) return gfail(g, TURQ_ERR_INVALID, "turq_gguf_read_tensor: null buffer");
+    // (checked without forming data_offset + offset + nbytes, which a hostile offset could wrap)
+    if (g->data_offset > g->file_size || ti->offset > g->file_size - g->data_offset || nbytes > g->file_size - g->data_offset - ti->offset)
+        return gfail(g, TURQ_ERR_IO, std::string("tensor ") + name + " runs past the end of " + g->path);
     const uint64_t off = g->data_offset + ti->offset;
-    if (off + nbytes > g->file_size) return gfail(g, TURQ_ERR_IO, std::string("tensor ") + name + " runs past the end of " + g->path);
     std::lock_guard<std::mutex> lock(g->mu);
     if (fseeko(g->fp, (off_t)off, SEEK_SET) != 0) return gfail(g, TURQ_ERR_IO, std::string("seek failed in ") + g->path);
     if (fread(host_bytes, 1, nbytes, g->fp) != nbytes) return gfail(g, TURQ_ERR_IO, std::string("short read in ") + g->path);

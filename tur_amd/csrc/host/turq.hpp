@@ -16,6 +16,7 @@
 #include <cstdint>
 #include <memory>
 #include <mutex>
+#include <cstdlib>
 #include <optional>
 #include <stdexcept>
 #include <string>
@@ -82,6 +83,7 @@ public:
     int dtype() const { return dtype_; }
     int64_t rows() const { return n_; }
     int64_t cols() const { return k_; }
+    int layout() const { return layout_; }
     turq_weight *handle() const { return w_.get(); }
     const Device &device() const { return dev_; }
     // `QTensor::dequantize(device)`: f32 values, bit-exact with candle's to_float
@@ -101,27 +103,42 @@ private:
     size_t device_bytes_ = 0;
 };
 
+// As in candle, a block-quantized tensor gives the quantized matmul (QMatMul::QTensor) and an F32 / F16 / BF16 tensor - or any
+// tensor while CANDLE_DEQUANTIZE_ALL / CANDLE_DEQUANTIZE_ALL_F16 is set - the dense one (QMatMul::Tensor): f32 arithmetic on
+// the dequantized weights, activations not rounded (the plain kernel on the tensor's GGUF bytes; a tiled tensor is uploaded
+// once more in GGUF order for it).
 class QMatMul {
 public:
+    static bool dequantize_all() {
+        const char *a = std::getenv("CANDLE_DEQUANTIZE_ALL"), *b = std::getenv("CANDLE_DEQUANTIZE_ALL_F16");
+        return (a && *a) || (b && *b);
+    }
     static QMatMul from_arc(const QTensor &t) {
         const int dt = t.dtype();
-        if (dt != TURQ_Q8_0 && dt != TURQ_Q4_K && dt != TURQ_Q5_K && dt != TURQ_Q6_K)
-            throw Error(TURQ_ERR_DTYPE, "QMatMul needs a block-quantized tensor");
-        return QMatMul(t);
+        const bool quant = dt == TURQ_Q8_0 || dt == TURQ_Q4_K || dt == TURQ_Q5_K || dt == TURQ_Q6_K;
+        if (!quant && dt != TURQ_F32 && dt != TURQ_F16 && dt != TURQ_BF16) throw Error(TURQ_ERR_DTYPE, "QMatMul: unsupported ggml dtype");
+        const bool dense = !quant || dequantize_all();
+        if (dense && t.layout() != TURQ_LAYOUT_NATIVE) {
+            std::vector<uint8_t> raw(turq_weight_nbytes(dt, t.rows(), t.cols()));
+            t.device().check(turq_weight_export(t.device().ctx(), t.handle(), raw.data(), raw.size()));
+            return QMatMul(QTensor::from_blocks(t.device(), dt, t.rows(), t.cols(), raw.data(), raw.size(), TURQ_LAYOUT_NATIVE), true);
+        }
+        return QMatMul(t, dense);
     }
+    bool dense() const { return dense_; }
     // host tensors: xs is [m, k] row-major f32, returns [m, n]
     std::vector<float> forward(const std::vector<float> &xs, int64_t m, const float *bias = nullptr) const {
         if (m < 0 || (int64_t)xs.size() != m * t_.cols()) throw Error(TURQ_ERR_SHAPE, "shape mismatch in matmul: input is not [m, k]");
         std::vector<float> y((size_t)m * (size_t)t_.rows());
         t_.device().check(turq_qmatmul(t_.device().ctx(), t_.handle(), xs.data(), TURQ_ACT_F32, m, t_.cols(), y.data(), TURQ_ACT_F32,
-                                       t_.rows(), bias, TURQ_MEM_HOST, TURQ_ALGO_AUTO));
+                                       t_.rows(), bias, TURQ_MEM_HOST, dense_ ? TURQ_ALGO_SIMPLE : TURQ_ALGO_AUTO));
         return y;
     }
     // device tensors: asynchronous on the device's stream
     void forward(const void *x_dev, int x_dtype, int64_t m, int64_t ldx, void *y_dev, int y_dtype, int64_t ldy,
                  const float *bias_dev = nullptr) const {
         t_.device().check(turq_qmatmul(t_.device().ctx(), t_.handle(), x_dev, x_dtype, m, ldx, y_dev, y_dtype, ldy, bias_dev,
-                                       TURQ_MEM_DEVICE, TURQ_ALGO_AUTO));
+                                       TURQ_MEM_DEVICE, dense_ ? TURQ_ALGO_SIMPLE : TURQ_ALGO_AUTO));
     }
     // Several projections of one device tensor (q / k / v, gate / up: src/models/qwen3.rs:161-167, 272-274), ys[i] is
     // [m, n_i] with row stride n_i: one kernel launch per run of equal formats for m <= 32, the single calls otherwise.
@@ -150,8 +167,9 @@ public:
     const QTensor &qtensor() const { return t_; }
 
 private:
-    explicit QMatMul(const QTensor &t) : t_(t) {}
+    explicit QMatMul(const QTensor &t, bool dense = false) : t_(t), dense_(dense) {}
     QTensor t_;
+    bool dense_ = false;
 };
 
 // LinearX::Quantized { qmatmul, bias }: forward = qmatmul.forward(x), then broadcast_add(bias)
@@ -168,6 +186,36 @@ public:
 private:
     QMatMul q_;
     std::optional<std::vector<float>> bias_;
+};
+
+// NormX over candle_nn's RmsNorm (src/models/layers/norm.rs:9-41), GGUF arm: f32 weight, f32 arithmetic, output in the input's type
+class NormX {
+public:
+    NormX(const Device &d, std::vector<float> weight, float eps)
+        : dev_(d), w_(std::move(weight)), eps_(eps), wdev_(std::make_shared<DeviceBuffer>(d, w_.size() * sizeof(float))) {
+        wdev_->upload(w_.data(), w_.size() * sizeof(float));
+    }
+    // host tensor [m, k] f32
+    std::vector<float> forward(const std::vector<float> &xs, int64_t m) const {
+        const int64_t k = (int64_t)w_.size();
+        if (m < 0 || (int64_t)xs.size() != m * k) throw Error(TURQ_ERR_SHAPE, "shape mismatch in rms-norm: input is not [m, k]");
+        std::vector<float> y(xs.size());
+        dev_.check(turq_rms_norm(dev_.ctx(), xs.data(), TURQ_ACT_F32, m, k, k, w_.data(), eps_, y.data(), TURQ_ACT_F32, k, TURQ_MEM_HOST));
+        return y;
+    }
+    // device tensors, asynchronous on the device's stream; y may be x
+    void forward(const void *x_dev, int x_dtype, int64_t m, int64_t ldx, void *y_dev, int y_dtype, int64_t ldy) const {
+        dev_.check(turq_rms_norm(dev_.ctx(), x_dev, x_dtype, m, (int64_t)w_.size(), ldx, (const float *)wdev_->ptr(), eps_, y_dev, y_dtype, ldy,
+                                 TURQ_MEM_DEVICE));
+    }
+    const std::vector<float> &weight() const { return w_; }
+    static const char *name() { return "RmsNorm"; }
+
+private:
+    Device dev_;
+    std::vector<float> w_;
+    float eps_;
+    std::shared_ptr<DeviceBuffer> wdev_;  // clones share the device copy of the weight
 };
 
 // candle's Embedding over a table that stays quantized: forward gathers and dequantizes the rows of the given token ids where
@@ -268,18 +316,28 @@ private:
     std::vector<std::string> path_;
 };
 
-// GGUF arm of layers::linear: the weight stays quantized, an optional bias is dequantized at load (`.ok()`)
+// GGUF arm of layers::linear: the weight stays quantized; the bias is looked up with `.ok()` (absent or mis-shaped: none) and
+// dequantized at load, where a failure is an error (`.transpose()?`)
 inline LinearX linear(int64_t in_dim, int64_t out_dim, const QVarBuilder &vb) {
     QTensor qweight = vb.get({out_dim, in_dim}, "weight");
-    std::optional<std::vector<float>> bias;
-    if (vb.contains_key("bias")) {
-        try {
-            bias = vb.get({out_dim}, "bias").dequantize();
-        } catch (const Error &) {
-            bias.reset();
-        }
+    std::optional<QTensor> qbias;
+    try {
+        qbias = vb.get({out_dim}, "bias");
+    } catch (const Error &) {
+        qbias.reset();
     }
+    std::optional<std::vector<float>> bias;
+    if (qbias) bias = qbias->dequantize();
     return LinearX(QMatMul::from_arc(qweight), std::move(bias));
+}
+
+// GGUF arm of layers::norm::rms_norm (src/models/layers/norm.rs:52-94): the `weight` tensor dequantized to f32, plus one for the
+// Gemma family
+inline NormX rms_norm(int64_t size, double eps, const QVarBuilder &vb, bool is_gemma = false) {
+    std::vector<float> w = vb.get({size}, "weight").dequantize();
+    if (is_gemma)
+        for (float &v : w) v += 1.0f;
+    return NormX(vb.device(), std::move(w), (float)eps);
 }
 
 }  // namespace turq

@@ -9,7 +9,8 @@ Same names, argument meaning and error behaviour as the reference so that tests 
 * ``LinearX``         — ``src/models/layers/linear.rs:8-31``: ``Quantized{qmatmul, bias}``, ``forward`` adds the bias;
 * ``QVarBuilder``     — ``src/weights/gguf_varbuilder.rs``: ``from_gguf``, ``pp``, ``get``, ``get_no_shape``,
                         ``contains_key``, ``tensor_shape``, ``all_keys``, with the one-entry last-tensor cache;
-* ``linear(in_dim, out_dim, vb)`` — ``src/models/layers/linear.rs:50-70`` (GGUF arm).
+* ``linear(in_dim, out_dim, vb)`` — ``src/models/layers/linear.rs:50-70`` (GGUF arm);
+* ``NormX`` / ``rms_norm(size, eps, vb)`` — ``src/models/layers/norm.rs:9-94`` (GGUF arm, RmsNorm).
 
 Activations and results are NumPy arrays on the host here (this mirror is for tests and scripting; an engine
 binds the C ABI directly and keeps its tensors on the device).
@@ -106,12 +107,32 @@ class QTensor:
             pass
 
 
-class QMatMul:
-    """``QMatMul::from_arc`` + ``forward``: y = x @ W.T for x of shape [..., k]."""
+def dequantize_all() -> bool:
+    """candle's switch: with CANDLE_DEQUANTIZE_ALL (or CANDLE_DEQUANTIZE_ALL_F16) set, ``QMatMul::from_arc`` turns every
+    tensor into a dense matmul instead of the quantized one"""
+    import os
 
-    def __init__(self, qtensor: QTensor):
-        if qtensor.dtype() not in (capi.Q8_0, capi.Q4_K, capi.Q5_K, capi.Q6_K):
-            raise TurqError(capi.ERR_DTYPE, "QMatMul needs a block-quantized tensor; dequantize F32/F16/BF16 tensors")
+    return bool(os.environ.get("CANDLE_DEQUANTIZE_ALL") or os.environ.get("CANDLE_DEQUANTIZE_ALL_F16"))
+
+
+class QMatMul:
+    """``QMatMul::from_arc`` + ``forward``: y = x @ W.T for x of shape [..., k].
+
+    As in candle, a block-quantized tensor gives the quantized matmul (``QMatMul::QTensor``) and an F32 / F16 / BF16 tensor -
+    or any tensor while ``CANDLE_DEQUANTIZE_ALL`` is set - the dense one (``QMatMul::Tensor``): f32 arithmetic on the
+    dequantized weights, activations not rounded (here: the plain kernel on the tensor's GGUF bytes, which dequantizes on
+    the fly; a tiled tensor is re-uploaded in GGUF order for it)."""
+
+    def __init__(self, qtensor: QTensor, dense: Optional[bool] = None):
+        quant = qtensor.dtype() in (capi.Q8_0, capi.Q4_K, capi.Q5_K, capi.Q6_K)
+        if not quant and qtensor.dtype() not in (capi.F32, capi.F16, capi.BF16):
+            raise TurqError(capi.ERR_DTYPE, f"QMatMul: unsupported ggml dtype {qtensor.dtype()}")
+        self.dense = (not quant) or (dequantize_all() if dense is None else dense)
+        if self.dense and qtensor._layout != capi.LAYOUT_NATIVE:
+            dev = qtensor.device
+            raw = np.empty(synth.weight_nbytes(qtensor.dtype(), qtensor._n, qtensor._k), np.uint8)
+            capi.check(dev.L.turq_weight_export(dev.ctx, qtensor.handle, capi.ptr(raw), raw.size), dev.ctx)
+            qtensor = QTensor.new(dev, qtensor.dtype(), (qtensor._n, qtensor._k), raw, capi.LAYOUT_NATIVE)
         self.qtensor = qtensor
 
     @classmethod
@@ -139,6 +160,8 @@ class QMatMul:
         y = np.empty((m, n), np.float32)
         b = None if bias is None else np.ascontiguousarray(bias, np.float32)
         dev = q.device
+        if self.dense:
+            algo = capi.ALGO_SIMPLE
         capi.check(dev.L.turq_qmatmul(dev.ctx, q.handle, capi.ptr(xs), xt, m, k, capi.ptr(y), capi.ACT_F32, n, capi.ptr(b),
                                       capi.MEM_HOST, algo), dev.ctx)
         return y.reshape(lead + (n,))
@@ -208,7 +231,7 @@ class LinearX:
         return self.qmatmul.forward(x, bias=self.bias)
 
     def __repr__(self) -> str:
-        return "LinearX::Quantized"
+        return "LinearX::Quantized"     # candle keeps dense GGUF tensors inside QMatMul too (QMatMul::Tensor)
 
 
 class QVarBuilder:
@@ -290,12 +313,54 @@ def linear(in_dim: int, out_dim: int, vb: QVarBuilder) -> LinearX:
     bias tensor is dequantized at load."""
     qweight = vb.get((out_dim, in_dim), "weight")
     bias = None
-    if vb.contains_key("bias"):
-        try:
-            bias = vb.get(out_dim, "bias").dequantize(vb.device()).reshape(-1)
-        except TurqError:
-            bias = None     # the reference looks the bias up with `.ok()`
+    try:
+        qbias = vb.get(out_dim, "bias")     # the reference looks the bias up with `.ok()`: absent or mis-shaped means none
+    except TurqError:
+        qbias = None
+    if qbias is not None:
+        bias = qbias.dequantize(vb.device()).reshape(-1)     # ... but a failing dequantize is an error (`.transpose()?`)
     return LinearX(QMatMul.from_arc(qweight), bias)
+
+
+class NormX:
+    """``NormX`` over candle_nn's ``RmsNorm`` (src/models/layers/norm.rs:9-41): the input is taken as it comes (f32 or f16 here),
+    normalised in f32 and returned in the input's type."""
+
+    def __init__(self, device: Device, weight: np.ndarray, eps: float):
+        self.device = device
+        self.weight = np.ascontiguousarray(weight, np.float32).reshape(-1)
+        self.eps = float(eps)
+
+    def forward(self, xs: np.ndarray) -> np.ndarray:
+        xs = np.asarray(xs)
+        k = self.weight.size
+        if xs.ndim < 1 or xs.shape[-1] != k:
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch in rms-norm: last dim {xs.shape[-1] if xs.ndim else None} != {k}")
+        if xs.dtype == np.float32:
+            xt = capi.ACT_F32
+        elif xs.dtype == np.float16:
+            xt = capi.ACT_F16
+        else:
+            raise TurqError(capi.ERR_DTYPE, f"unsupported activation dtype {xs.dtype}")
+        xs = np.ascontiguousarray(xs)
+        m = xs.size // k if k else 0
+        y = np.empty_like(xs)
+        dev = self.device
+        capi.check(dev.L.turq_rms_norm(dev.ctx, capi.ptr(xs), xt, m, k, k, capi.ptr(self.weight), self.eps, capi.ptr(y), xt, k,
+                                       capi.MEM_HOST), dev.ctx)
+        return y
+
+    def __repr__(self) -> str:
+        return "RmsNorm"
+
+
+def rms_norm(size: int, eps: float, vb: QVarBuilder, is_gemma: bool = False) -> NormX:
+    """GGUF arm of ``layers::norm::rms_norm`` (src/models/layers/norm.rs:52-94): the ``weight`` tensor dequantized to f32
+    (plus one for the Gemma family)."""
+    w = vb.get(size, "weight").dequantize(vb.device()).reshape(-1)
+    if is_gemma:
+        w = w + np.float32(1.0)
+    return NormX(vb.device(), w, eps)
 
 
 class Embedding:
