@@ -94,6 +94,17 @@ const char *turq_last_error(const turq_ctx *ctx);
 int turq_sync(turq_ctx *ctx);
 /* the context's hipStream_t, for hosts that time or order their own work on it */
 void *turq_ctx_stream(turq_ctx *ctx);
+/* Activation range of forward calls on device pointers.  The matrix kernels round activations to f16: magnitudes from 65504 on
+ * become infinities and rows whose values all sit far below 6e-5 lose precision, where the reference takes f32 activations of
+ * any magnitude (src/weights/mod.rs:84-99; candle scales every 256-element block of them on its own).  With `on` != 0 every
+ * turq_qmatmul / turq_qmatmul_multi / turq_qmatmul_gate_up on device pointers with f32 or bf16 activations is bracketed by two
+ * small kernels: rows multiplied by the power of two that puts their largest magnitude into [2^9, 2^10) and written as f16,
+ * output rows multiplied back (both exact) - any finite f32 row then stays within the 1e-3 bar, infinities and NaNs
+ * propagate.  It costs two launches per call and the grouped launches of turq_qmatmul_multi / turq_qmatmul_gate_up.  Default:
+ * off, for engines whose activations are known to be bounded (after an RmsNorm, say).  Calls on HOST pointers always take the
+ * wide path: they are the reference's own contract, and the staging copies dominate them anyway.  turq_qmatmul_noalloc never
+ * takes it. */
+int turq_ctx_set_wide_activations(turq_ctx *ctx, int on);
 /* name and compute-unit count of the context's device */
 int turq_ctx_device_info(turq_ctx *ctx, char *name, size_t name_cap, int *compute_units);
 

@@ -42,8 +42,10 @@ class Gpu:
         return out
 
     def qmatmul(self, w, x, n, k, algo=capi.ALGO_AUTO, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_F32, bias=None,
-                ldx=None, ldy=None):
-        """x: f32 [m, k] values; converted to the requested activation dtype before the call."""
+                ldx=None, ldy=None, mem=capi.MEM_DEVICE):
+        """x: f32 [m, k] values; converted to the requested activation dtype before the call.  Device pointers by default (the
+        kernels read the activations as they are); mem=MEM_HOST goes through the staged host path, which always scales the
+        rows into the f16 range first."""
         x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
         m = x.shape[0]
         ldx = ldx or k
@@ -59,8 +61,19 @@ class Gpu:
         ydt = {capi.ACT_F32: np.float32, capi.ACT_BF16: np.uint16, capi.ACT_F16: np.float16}[y_dtype]
         y = np.zeros((m, ldy), ydt)
         b = None if bias is None else np.ascontiguousarray(bias, np.float32)
-        capi.check(self.L.turq_qmatmul(self.ctx, w, capi.ptr(xsend), x_dtype, m, ldx, capi.ptr(y), y_dtype, ldy,
-                                       capi.ptr(b), capi.MEM_HOST, algo), self.ctx)
+        if mem == capi.MEM_DEVICE and m > 0:
+            xd, yd = self.dev_buffer(xsend), self.dev_buffer(y)
+            bd = None if b is None else self.dev_buffer(b)
+            try:
+                capi.check(self.L.turq_qmatmul(self.ctx, w, xd, x_dtype, m, ldx, yd, y_dtype, ldy, bd, capi.MEM_DEVICE, algo), self.ctx)
+                y = self.read_back(yd, (m, ldy), ydt)
+            finally:
+                for p in (xd, yd, bd):
+                    if p is not None:
+                        self.dev_free(p)
+        else:
+            capi.check(self.L.turq_qmatmul(self.ctx, w, capi.ptr(xsend), x_dtype, m, ldx, capi.ptr(y), y_dtype, ldy,
+                                           capi.ptr(b), capi.MEM_HOST, algo), self.ctx)
         if y_dtype == capi.ACT_BF16:
             y = synth.from_bf16_bits(y).reshape(m, ldy)
         return np.asarray(y, np.float32)[:, :n]

@@ -1,0 +1,116 @@
+"""f32 activations of any finite magnitude (the reference's contract, src/weights/mod.rs:84-99: candle's CPU path scales every
+256-element block of the activations on its own): calls on host pointers and, after turq_ctx_set_wide_activations, calls on
+device pointers stay within the 1e-3 bar for rows far outside the f16 range; non-finite inputs propagate."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from oracle import capi as orc
+from tests.helpers import Gpu, rel_l2
+from tur_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+MAGNITUDES = [1e-12, 1e-6, 1.0, 1e5, 1e20]
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    g = Gpu()
+    yield g
+    g.close()
+
+
+def rows_of_mixed_magnitude(m, k, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    scale = np.array([MAGNITUDES[i % len(MAGNITUDES)] for i in range(m)], np.float32)[:, None]
+    return (x * scale).astype(np.float32)
+
+
+def per_row_rel(y, want):
+    y, want = np.asarray(y, np.float64), np.asarray(want, np.float64)
+    return np.linalg.norm(y - want, axis=1) / np.maximum(np.linalg.norm(want, axis=1), 1e-300)
+
+
+@pytest.mark.parametrize("dt", [Q8_0, Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("m", [1, 2, 5, 20, 40, 100])          # one-row kernel, batch kernels, prefill GEMM
+def test_host_calls_take_any_f32_magnitude(gpu, dt, m):
+    n, k = 208, 1024
+    raw = synth.random_weight(dt, n, k, seed=dt + m)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    x = rows_of_mixed_magnitude(m, k, seed=m)
+    bias = np.random.default_rng(1).standard_normal(n).astype(np.float32) * 1e-3
+    y = gpu.qmatmul(w, x, n, k, bias=bias, mem=capi.MEM_HOST)
+    want = orc.matmul_dequant(dt, x, raw, n, k).astype(np.float64) + bias
+    assert np.all(np.isfinite(y))
+    assert per_row_rel(y, want).max() <= 1e-3          # every row on its own: a tiny row must not drown next to a huge one
+    gpu.release(w)
+
+
+@pytest.mark.parametrize("x_dtype", [capi.ACT_F32, capi.ACT_BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("y_dtype", [capi.ACT_F32, capi.ACT_BF16], ids=["to-f32", "to-bf16"])
+def test_device_calls_after_the_switch(x_dtype, y_dtype):
+    g = Gpu()
+    try:
+        L, ctx = g.L, g.ctx
+        dt, n, k = Q4_K, 320, 2048
+        raw = synth.random_weight(dt, n, k, seed=3)
+        w = g.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+        for m in (1, 8, 64):
+            x = rows_of_mixed_magnitude(m, k, seed=10 + m)
+            if x_dtype == capi.ACT_BF16:
+                x = synth.from_bf16_bits(synth.to_bf16_bits(x)).reshape(m, k)
+            want = orc.matmul_dequant(dt, x, raw, n, k)
+            # without the switch rows of 1e5 and more overflow f16: infinities or NaNs, not a crash
+            y = g.qmatmul(w, x, n, k, x_dtype=x_dtype, y_dtype=y_dtype)
+            big = np.abs(x).max(axis=1) >= 65504
+            assert m == 1 or (big.any() and not np.all(np.isfinite(y[big])))
+            capi.check(L.turq_ctx_set_wide_activations(ctx, 1), ctx)
+            y = g.qmatmul(w, x, n, k, x_dtype=x_dtype, y_dtype=y_dtype)
+            assert np.all(np.isfinite(y))
+            assert per_row_rel(y, want).max() <= (1e-3 if y_dtype == capi.ACT_F32 else 4e-3)
+            capi.check(L.turq_ctx_set_wide_activations(ctx, 0), ctx)
+        g.release(w)
+    finally:
+        g.close()
+
+
+def test_grouped_calls_and_gate_up_under_the_switch():
+    from oracle import oracle_np as onp
+    g = Gpu()
+    try:
+        capi.check(g.L.turq_ctx_set_wide_activations(g.ctx, 1), g.ctx)
+        k, ns, dts = 1024, [96, 48, 160], (Q4_K, Q4_K, Q6_K)
+        raws = [synth.random_weight(dt, n, k, seed=n) for dt, n in zip(dts, ns)]
+        ws = [g.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
+        for m in (1, 6, 48):
+            x = rows_of_mixed_magnitude(m, k, seed=m)
+            for y, dt, n, raw in zip(g.qmatmul_multi(ws, x, ns, k), dts, ns, raws):
+                assert per_row_rel(y, orc.matmul_dequant(dt, x, raw, n, k)).max() <= 1e-3
+        # gate / up: SiLU is not homogeneous, so the rows go back to their own scale before it is applied
+        n = 128
+        rg, ru = synth.random_weight(Q4_K, n, k, seed=5), synth.random_weight(Q4_K, n, k, seed=6)
+        wg, wu = g.upload(Q4_K, n, k, rg, capi.LAYOUT_TILED), g.upload(Q4_K, n, k, ru, capi.LAYOUT_TILED)
+        x = rows_of_mixed_magnitude(5, k, seed=2)
+        x[np.abs(x).max(axis=1) > 1e10] *= 1e-12        # keep gate * up inside f32
+        y = g.gate_up(wg, wu, x, n, k)
+        want = onp.silu_mul(orc.matmul_dequant(Q4_K, x, rg, n, k), orc.matmul_dequant(Q4_K, x, ru, n, k))
+        assert per_row_rel(y, want).max() <= 2e-3
+    finally:
+        g.close()
+
+
+def test_non_finite_activations_propagate(gpu):
+    dt, n, k = Q4_K, 64, 512
+    raw = synth.random_weight(dt, n, k, seed=8)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    x = np.random.default_rng(0).standard_normal((4, k)).astype(np.float32)
+    x[1, 7] = np.inf
+    x[2, 300] = np.nan
+    y = gpu.qmatmul(w, x, n, k, mem=capi.MEM_HOST)
+    want = orc.matmul_dequant(dt, x[[0, 3]], raw, n, k)
+    assert rel_l2(y[[0, 3]], want) <= 1e-3                      # the finite rows are untouched
+    assert not np.any(np.isfinite(y[1])) and np.all(np.isnan(y[2]))
+    gpu.release(w)

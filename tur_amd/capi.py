@@ -30,6 +30,7 @@ _SIGS = {
     "turq_last_error": (c_char_p, [c_void_p]),
     "turq_sync": (c_int, [c_void_p]),
     "turq_ctx_stream": (c_void_p, [c_void_p]),
+    "turq_ctx_set_wide_activations": (c_int, [c_void_p, c_int]),
     "turq_ctx_device_info": (c_int, [c_void_p, c_char_p, c_size_t, POINTER(c_int)]),
     "turq_dev_alloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "turq_dev_free": (c_int, [c_void_p, c_void_p]),

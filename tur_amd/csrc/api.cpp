@@ -153,6 +153,9 @@ void turq_ctx_destroy(turq_ctx *ctx) {
     if (ctx->stage_y) (void)hipFree(ctx->stage_y);
     if (ctx->act_prep) (void)hipFree(ctx->act_prep);
     if (ctx->gate_up) (void)hipFree(ctx->gate_up);
+    if (ctx->wide_x) (void)hipFree(ctx->wide_x);
+    if (ctx->wide_s) (void)hipFree(ctx->wide_s);
+    if (ctx->wide_y) (void)hipFree(ctx->wide_y);
     if (ctx->stage_b) (void)hipFree(ctx->stage_b);
     for (void *p : ctx->retired) (void)hipFree(p);  // graphs that still refer to them can no longer be launched: that needs the context
     for (auto &p : ctx->prof_events) { (void)hipEventDestroy(p.first); (void)hipEventDestroy(p.second); }
@@ -442,11 +445,33 @@ static int impl_rms_norm(turq_ctx *ctx, const void *x, int xt, int64_t m, int64_
 
 // ---- forward ----
 
+// wide: activations of any finite f32 magnitude (wide.hip) where the kernel would round them to f16
 static int qmatmul_device(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
-                          int yt, int64_t ldy, const float *bias, int algo) {
+                          int yt, int64_t ldy, const float *bias, int algo, bool wide) {
     if (algo == TURQ_ALGO_AUTO) {
         if (w->layout == TURQ_LAYOUT_NATIVE) algo = TURQ_ALGO_SIMPLE;
         else algo = (m <= TURQ_GEMV_MAX_M) ? TURQ_ALGO_GEMV : TURQ_ALGO_GEMM;
+    }
+    if (wide && !ctx->fixed_scratch && xt != TURQ_ACT_F16 && (algo == TURQ_ALGO_GEMV || algo == TURQ_ALGO_GEMM) &&
+        w->layout == TURQ_LAYOUT_TILED && m <= 65535) {
+        // rows scaled by powers of two into the f16 range, the plain call on the f16 copy, rows scaled back (+ bias)
+        int rc = turq_ctx_reserve(ctx, &ctx->wide_x, &ctx->wide_x_cap, (size_t)m * (size_t)w->k * 2);
+        if (rc != TURQ_OK) return rc;
+        rc = turq_ctx_reserve(ctx, &ctx->wide_s, &ctx->wide_s_cap, (size_t)m * sizeof(float));
+        if (rc != TURQ_OK) return rc;
+        float *y32 = (float *)y;
+        int64_t ld32 = ldy;
+        if (yt != TURQ_ACT_F32) {
+            rc = turq_ctx_reserve(ctx, &ctx->wide_y, &ctx->wide_y_cap, (size_t)m * (size_t)w->n * sizeof(float));
+            if (rc != TURQ_OK) return rc;
+            y32 = (float *)ctx->wide_y;
+            ld32 = w->n;
+        }
+        TURQ_HIP(ctx, turq_launch_wide_scale(x, xt, m, w->k, ldx, ctx->wide_x, (float *)ctx->wide_s, ctx->stream));
+        rc = turq_qmatmul_mfma(ctx, w, ctx->wide_x, TURQ_ACT_F16, m, w->k, y32, TURQ_ACT_F32, ld32, nullptr, algo);
+        if (rc != TURQ_OK) return rc;
+        TURQ_HIP(ctx, turq_launch_wide_rescale(y32, ld32, m, w->n, (const float *)ctx->wide_s, bias, y, yt, ldy, ctx->stream));
+        return TURQ_OK;
     }
     switch (algo) {
     case TURQ_ALGO_SIMPLE:
@@ -481,7 +506,7 @@ static int impl_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int 
     if (!x || !y) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: null activation or output pointer");
     if (w->k == 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul: k=0");
 
-    if (mem == TURQ_MEM_DEVICE) return qmatmul_device(ctx, w, x, xt, m, ldx, y, yt, ldy, bias, algo);
+    if (mem == TURQ_MEM_DEVICE) return qmatmul_device(ctx, w, x, xt, m, ldx, y, yt, ldy, bias, algo, ctx->wide);
     if (mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: bad mem %d", mem);
 
     // host pointers: stage rows densely (ld = k / n on the device side), run, copy back
@@ -497,7 +522,8 @@ static int impl_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int 
         TURQ_HIP(ctx, hipMemcpyAsync(ctx->stage_b, bias, (size_t)w->n * sizeof(float), hipMemcpyHostToDevice, ctx->stream));
         bias = (const float *)ctx->stage_b;
     }
-    rc = qmatmul_device(ctx, w, ctx->stage_x, xt, m, w->k, ctx->stage_y, yt, w->n, bias, algo);
+    // host tensors are the reference's own contract (f32 activations of any magnitude, src/weights/mod.rs:84-99): always wide
+    rc = qmatmul_device(ctx, w, ctx->stage_x, xt, m, w->k, ctx->stage_y, yt, w->n, bias, algo, true);
     if (rc != TURQ_OK) return rc;
     TURQ_HIP(ctx, hipMemcpy2DAsync(y, (size_t)ldy * yb, ctx->stage_y, yrow, yrow, (size_t)m, hipMemcpyDeviceToHost, ctx->stream));
     TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -511,7 +537,7 @@ static int impl_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const
     if (count == 0) return TURQ_OK;
     if (!weights || !ys || !ldys) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_multi: null weight, output or stride array");
     const bool many_rows = m > TURQ_GEMV_MAX_M && (algo == TURQ_ALGO_AUTO || algo == TURQ_ALGO_GEMM);
-    bool one_launch = mem == TURQ_MEM_DEVICE && count > 1 && x != nullptr &&
+    bool one_launch = mem == TURQ_MEM_DEVICE && !(ctx->wide && xt != TURQ_ACT_F16) && count > 1 && x != nullptr &&
                       (many_rows || ((algo == TURQ_ALGO_AUTO || algo == TURQ_ALGO_GEMV) && m >= 1 && m <= TURQ_GEMV_MAX_M));
     for (int i = 0; i < count && one_launch; i++) {
         const turq_weight *w = weights[i];
@@ -589,7 +615,7 @@ static int impl_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const tu
         return TURQ_OK;
     }
     if (m > 0 && n > 0 && x && y && gate->device == ctx->device && up->device == ctx->device && gate->k > 0 && ldx >= gate->k &&
-        turq_act_bytes(xt)) {
+        turq_act_bytes(xt) && !(ctx->wide && xt != TURQ_ACT_F16)) {
         bool taken = false;
         const int rc = turq_qmatmul_gate_up_mfma(ctx, gate, up, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, &taken);
         if (rc != TURQ_OK || taken) return rc;
@@ -777,6 +803,13 @@ int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void
 int turq_rms_norm(turq_ctx *ctx, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, const float *weight, float eps, void *y,
                   int y_dtype, int64_t ldy, int mem) {
     return capture_guard(ctx, impl_rms_norm(ctx, x, x_dtype, m, k, ldx, weight, eps, y, y_dtype, ldy, mem));
+}
+
+int turq_ctx_set_wide_activations(turq_ctx *ctx, int on) {
+    if (!ctx) return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_ctx_set_wide_activations: null context");
+    if (ctx->capturing) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_ctx_set_wide_activations: a graph capture is running");
+    ctx->wide = on != 0;
+    return TURQ_OK;
 }
 
 int turq_ctx_scratch_info(const turq_ctx *ctx, int *live_graphs, int *retired_buffers, size_t *act_prep_bytes) {

@@ -81,6 +81,11 @@ struct turq_ctx {
     void *stage_b = nullptr;  size_t stage_b_cap = 0;
     void *act_prep = nullptr; size_t act_prep_cap = 0;
     void *gate_up = nullptr;  size_t gate_up_cap = 0;  // the two f32 products of turq_qmatmul_gate_up's general path
+    // the wide-activation path (wide.hip): scaled f16 copy of the activations, per-row inverse scales, f32 results before rescaling
+    void *wide_x = nullptr;   size_t wide_x_cap = 0;
+    void *wide_s = nullptr;   size_t wide_s_cap = 0;
+    void *wide_y = nullptr;   size_t wide_y_cap = 0;
+    bool wide = false;  // device-pointer calls take that path too (host-pointer calls always do)
     // scratch buffers that were outgrown while a captured graph still referred to them: freed once no graph of the context is
     // alive (at the next growth) or with the context
     std::vector<void *> retired;
@@ -161,6 +166,9 @@ hipError_t turq_launch_gather_rows(int dtype, int layout, const void *w, int64_t
                                    void *out, int out_dtype, int64_t ldo, hipStream_t stream);
 hipError_t turq_launch_dequant(int dtype, int layout, const void *w, int64_t n, int64_t k, float *out,
                                hipStream_t stream);
+hipError_t turq_launch_wide_scale(const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *x16, float *inv, hipStream_t stream);
+hipError_t turq_launch_wide_rescale(const float *y32, int64_t ld32, int64_t m, int64_t n, const float *inv, const float *bias, void *y,
+                                    int y_dtype, int64_t ldy, hipStream_t stream);
 hipError_t turq_launch_rms_norm(const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, const float *weight, float eps, void *y,
                                 int y_dtype, int64_t ldy, hipStream_t stream);
 hipError_t turq_launch_quantize_q8_0(const float *x, int64_t nblocks, void *out, hipStream_t stream);
