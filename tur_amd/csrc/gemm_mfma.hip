@@ -142,7 +142,10 @@ template <int N> __device__ inline void wait_vmcnt() {
 // wait until at most N of this wave's LDS reads are outstanding
 template <int N> __device__ inline void wait_lds() { asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory"); }
 // a value read by lds_read128 may be used only after a wait; passing it through an (empty) volatile
-// statement placed after that wait keeps its users from being scheduled ahead of the wait
+// statement placed after that wait keeps its users from being scheduled ahead of the wait (the value it yields is a new one
+// to the compiler, so no copy made earlier can stand in for it).  What the compiler could still do is copy or spill the
+// register between the read and the wait; the build walks the device assembly of this file and fails if any instruction
+// touches the destination of an LDS read before the wait that covers it, or if a kernel here spills (check_lds_waits.py).
 template <typename T> __device__ inline void pin(T &v) { asm volatile("" : "+v"(v)); }
 
 template <int OFF, typename T> __device__ inline void lds_read128(T &dst, uint32_t addr) {
