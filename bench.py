@@ -132,6 +132,10 @@ class Bench:
         for _, _, n, k in self.mats:
             if k not in self.x_dev:
                 x = synth.random_activation(self.m, k, seed=k, bf16=(self.args.act == "bf16"))
+                if self.use_mlp():
+                    # the synthetic weights give products of a few hundred at unit activations and act(gate) * up would leave
+                    # the f16 range that down_proj rounds its input to: a power of two keeps the bf16 values exact
+                    x = x * np.float32(2.0 ** -7)
                 self.x_host[k] = x
                 send = synth.to_bf16_bits(x).reshape(self.m, k) if self.args.act == "bf16" else x
                 p = self.dev_alloc(send.nbytes)
@@ -144,9 +148,18 @@ class Bench:
         # neighbouring matrices that take the same input (gate/up, q/k/v) go through turq_qmatmul_multi, as the
         # reference calls them back to back on one tensor (src/models/qwen3.rs:161-167, 272-274)
         self.groups = []       # (count, weight array, x, y array, ldy array, k)
+        labels = [mt[0] for mt in self.mats]
         for layer in self.weights:
             i = 0
             while i < len(self.mats):
+                if self.use_mlp() and labels[i:i + 3] == ["gate", "up", "down"]:
+                    # the whole MLP through turq_mlp (src/models/qwen3.rs:161-167): x -> down_proj's output
+                    warr = (ctypes.c_void_p * 3)(*[w.value for w in layer[i:i + 3]])
+                    yarr = (ctypes.c_void_p * 1)(self.y_dev[i + 2].value)
+                    ldys = (ctypes.c_int64 * 1)(self.mats[i + 2][2])
+                    self.groups.append((3, warr, self.x_dev[self.mats[i][3]], yarr, ldys, self.mats[i][3], "mlp"))
+                    i += 3
+                    continue
                 j = i + 1
                 while j < len(self.mats) and self.mats[j][3] == self.mats[i][3] and shares_input(self.mats[i][0], self.mats[j][0]):
                     j += 1
@@ -161,12 +174,29 @@ class Bench:
         if getattr(self.args, "gate_up", False):
             # turq_qmatmul_gate_up reads the shared activations once and writes one output for the pair
             self.step_bytes -= layers * sum(self.m * (n * self.ybytes + k * self.xbytes) for lb, _, n, k in self.mats if lb == "up")
+        if self.use_mlp():
+            # one input, one output; the f32 intermediate (m * 12288 floats written and read back) is not counted
+            self.step_bytes -= layers * sum(self.m * (n * self.ybytes + (k * self.xbytes if lb == "up" else 0))
+                                            for lb, _, n, k in self.mats if lb in ("gate", "up"))
+            self.step_bytes -= layers * sum(self.m * k * self.xbytes for lb, _, n, k in self.mats if lb == "down")
         self.step_flops = layers * sum(2 * self.m * n * k for _, _, n, k in self.mats)
+
+    def use_mlp(self):
+        """gate / up / down as one turq_mlp call per layer (--mlp), decode rows only"""
+        labels = [mt[0] for mt in self.mats]
+        has = any(labels[i:i + 3] == ["gate", "up", "down"] for i in range(len(labels)))
+        return has and bool(getattr(self.args, "mlp", False)) and not self.args.single_calls and not self.args.gate_up and getattr(self, "m", 1) <= 32
 
     def step_eager(self):
         L, ctx, m, xt = self.L, self.ctx, self.m, self.xt
         if not self.args.single_calls:
             for cnt, warr, x, yarr, ldys, k, fused in self.groups:
+                if fused == "mlp":
+                    rc = L.turq_mlp(ctx, warr[0], warr[1], warr[2], x, xt, m, k, yarr[0], self.yt, ldys[0], None, None, None,
+                                    capi.ACTFN_SILU, capi.MEM_DEVICE)
+                    if rc:
+                        capi.check(rc, ctx)
+                    continue
                 if fused:
                     rc = L.turq_qmatmul_gate_up(ctx, warr[0], warr[1], x, xt, m, k, yarr[0], self.yt, ldys[0], None, None,
                                                 capi.ACTFN_SILU, capi.MEM_DEVICE)
@@ -192,9 +222,13 @@ class Bench:
         self.sync()
         worst = 0.0
         fused = bool(getattr(self.args, "gate_up", False)) and not self.args.single_calls
+        mlp = self.use_mlp()
+        by_label = {mt[0]: mt for mt in self.mats}
         for (label, dt, n, k), y in zip(self.mats, self.y_dev):
             if fused and label == "up":
                 continue      # its product went into the gate's output
+            if mlp and label in ("gate", "up"):
+                continue      # only down_proj's output leaves the call
             got = np.empty((self.m, n), np.float32 if self.yt == capi.ACT_F32 else np.uint16)
             capi.check(self.L.turq_memcpy_d2h(self.ctx, capi.ptr(got), y, got.nbytes), self.ctx)
             if self.yt != capi.ACT_F32:
@@ -202,7 +236,14 @@ class Bench:
             rows = np.arange(0, n, max(1, (n * self.m) // (4096 * 16)))      # bounded CPU time at prefill sizes
             got = got[:, rows]
             sub = self.host_raw[label].reshape(n, -1)[rows].reshape(-1)
-            want = orc.matmul_dequant(dt, self.x_host[k], sub, len(rows), k)
+            if mlp and label == "down":
+                from oracle import oracle_np as onp
+                _, gdt, gn, gk = by_label["gate"]
+                xg = self.x_host[gk].astype(np.float16).astype(np.float32)
+                h = onp.silu_mul(orc.matmul_dequant(gdt, xg, self.host_raw["gate"], gn, gk), orc.matmul_dequant(gdt, xg, self.host_raw["up"], gn, gk))
+                want = orc.matmul_dequant(dt, h, sub, len(rows), k)
+            else:
+                want = orc.matmul_dequant(dt, self.x_host[k], sub, len(rows), k)
             if fused and label == "gate":
                 from oracle import oracle_np as onp
                 sub_up = self.host_raw["up"].reshape(n, -1)[rows].reshape(-1)
@@ -252,7 +293,7 @@ class Bench:
         achieved = bytes_per_launch / (avg_us * 1e-6) / 1e9
         if graph:
             L.turq_graph_destroy(graph)
-        traffic = None if a.gate_up else TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls)))
+        traffic = None if (a.gate_up or self.use_mlp()) else TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls)))
         if self.m > 32:
             flops_per_launch = self.step_flops * prof_steps / max(1, n_launch.value)
             tfl = flops_per_launch / (avg_us * 1e-6) / 1e12
@@ -288,7 +329,7 @@ class Bench:
             "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": f"{a.workload}: {self.desc}", "m": self.m, "layers": a.layers,
                        "activations": a.act, "outputs": a.out, "launch": "eager" if a.eager else "hip-graph",
-                       "calls": "turq_qmatmul" if a.single_calls else ("turq_qmatmul_gate_up + turq_qmatmul_multi" if a.gate_up else "turq_qmatmul_multi"),
+                       "calls": "turq_qmatmul" if a.single_calls else "turq_mlp + turq_qmatmul_multi" if self.use_mlp() else ("turq_qmatmul_gate_up + turq_qmatmul_multi" if a.gate_up else "turq_qmatmul_multi"),
                        "step_bytes": int(self.step_bytes), "device": self.device, "compute_units": self.cus,
                        "max_rel_l2_vs_oracle": float(f"{r['rel']:.3e}")},
             "whole_step_gbps": round(r["gbps"], 1), "pct_of_hbm_peak": round(100 * r["gbps"] / HBM_PEAK_GBPS, 2),
@@ -409,6 +450,9 @@ def main():
                     help="default workload only: leave out the prefill GEMM, mixed-layer and LM-head legs of the JSON line")
     ap.add_argument("--single-calls", action="store_true",
                     help="one turq_qmatmul per matrix instead of turq_qmatmul_multi per group of matrices with a common input")
+    ap.add_argument("--mlp", action="store_true",
+                    help="the whole MLP through turq_mlp (down_proj takes act(gate) * up; the activations are scaled by 2^-7 so that the "
+                         "synthetic intermediate stays in the f16 range) instead of gate / up and down on independent activations")
     ap.add_argument("--gate-up", action="store_true",
                     help="gate_proj / up_proj through turq_qmatmul_gate_up (SiLU and the product applied in the call, one output)")
     ap.add_argument("--embedding", action="store_true",
@@ -425,7 +469,7 @@ def main():
         per_layer = sum(synth.weight_nbytes(dt, n, k) for _, dt, n, k in WORKLOADS[args.workload][1])
         args.layers = default_layers(per_layer)
     headline = all(getattr(args, f) == ap.get_default(f) for f in ("workload", "m", "act", "out")) and not (
-        args.eager or args.single_calls or args.gate_up or args.calibrate_copy)
+        args.eager or args.single_calls or args.gate_up or args.mlp or args.calibrate_copy)
     b = Bench(args)
     try:
         if args.calibrate_copy:

@@ -240,6 +240,24 @@ impl HipQMatMul {
         }
         Tensor::from_vec(y, dims, xs.device())
     }
+
+    /// `down_proj(act_fn(gate_proj(x)) * up_proj(x))`, the whole of `Qwen3MLP::forward` (src/models/qwen3.rs:161-167), SiLU.
+    pub fn forward_mlp(gate: &HipQMatMul, up: &HipQMatMul, down: &HipQMatMul, xs: &Tensor) -> Result<Tensor> {
+        let (k, n_out) = (gate.t.k, down.t.n);
+        let (m, mut dims) = rows_of(xs, k)?;
+        let x: Vec<f32> = xs.flatten_all()?.to_vec1()?;
+        let mut y = vec![0f32; m * n_out];
+        let ctx = gate.t.dev.ctx();
+        // SAFETY: x holds m * k floats, y m * n_out
+        check(ctx, unsafe {
+            turq_mlp(ctx, gate.t.w, up.t.w, down.t.w, x.as_ptr().cast(), TURQ_ACT_F32, m as i64, k as i64, y.as_mut_ptr().cast(),
+                     TURQ_ACT_F32, n_out as i64, ptr::null(), ptr::null(), ptr::null(), TURQ_ACTFN_SILU, TURQ_MEM_HOST)
+        })?;
+        if let Some(last) = dims.last_mut() {
+            *last = n_out;
+        }
+        Tensor::from_vec(y, dims, xs.device())
+    }
 }
 
 /// candle_nn's RmsNorm as `layers::norm::rms_norm` builds it from a GGUF file (src/models/layers/norm.rs:52-94).

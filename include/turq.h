@@ -232,6 +232,21 @@ int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weig
                          int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up, int act,
                          int mem);
 
+/* The reference's whole MLP in one call: y[m, n_out] = (act(x * gate^T + bias_gate) * (x * up^T + bias_up)) * down^T + bias_down.
+ * gate and up are two weights of one shape [n_ff, k], down is [n_out, n_ff]; the intermediate is kept in f32 (scratch memory of
+ * the context, m * n_ff floats, which grows on demand, never inside a graph capture).  The results are those of
+ * turq_qmatmul_gate_up into an f32 buffer followed by turq_qmatmul on it, bit for bit, and so are the errors and the meaning of
+ * x, y, the strides, the biases (NULL: none), `act` and `mem`.
+ * The call is those two calls one after the other on the context's stream.  (A single launch for the whole MLP - one
+ * persistent workgroup per compute unit, down_proj's first tiles requested while the last gate / up tiles are computed, a grid-wide
+ * barrier on device counters before down_proj reads the intermediate - was built, gave the same bits and was slower: 26 us
+ * against 20.4 us for a Qwen3-8B MLP row, the barrier alone 4.7 us; it is not in the library.)
+ * Replaces: `Qwen3MLP::forward` (src/models/qwen3.rs:161-167; the Granite MLP, src/models/granite_41.rs:151-155, has the
+ * same form). */
+int turq_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int x_dtype,
+             int64_t m, int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up,
+             const float *bias_down, int act, int mem);
+
 /* ---- activation quantisation (candle's VecDotType::from_float, bit-exact) ---- */
 /* x f32 [m, k] (row stride k) -> Q8_0 blocks (34 B per 32) / Q8_K blocks (292 B per 256).
  * The GPU forward path does not use them (it keeps activations in f16); they are the device

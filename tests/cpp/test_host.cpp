@@ -91,6 +91,16 @@ int main(int argc, char **argv) {
                 const double v = y[i], want = v / (1.0 + std::exp(-v)) * v;
                 if (std::fabs(y6[i] - want) > 1e-4 * (1.0 + std::fabs(want))) return fail("forward_gate_up differs from silu(forward) * forward");
             }
+            // the whole MLP in one call = down_proj of that product, bit for bit
+            turq::LinearX down = turq::linear(n, 64, b0.pp("ffn_down"));
+            turq::DeviceBuffer z1(dev, (size_t)m * 64 * 4), z2(dev, (size_t)m * 64 * 4);
+            down.qmatmul().forward(yg.ptr(), TURQ_ACT_F32, m, n, z1.ptr(), TURQ_ACT_F32, 64);
+            turq::QMatMul::forward_mlp(copy.qmatmul(), copy.qmatmul(), down.qmatmul(), xd.ptr(), TURQ_ACT_F32, m, k, z2.ptr(), TURQ_ACT_F32, 64);
+            dev.synchronize();
+            std::vector<float> a1((size_t)m * 64), a2((size_t)m * 64);
+            z1.download(a1.data(), a1.size() * 4);
+            z2.download(a2.data(), a2.size() * 4);
+            if (std::memcmp(a1.data(), a2.data(), a1.size() * 4) != 0) return fail("forward_mlp differs from forward_gate_up + forward");
         }
 
         // embedding rows of the quantized table = rows of its full dequantize

@@ -206,6 +206,46 @@ class Gpu:
             y = synth.from_bf16_bits(y).reshape(m, ldy)
         return np.asarray(y, np.float32)[:, :n]
 
+    def mlp(self, wg, wu, wd, x, n_ff, k, n_out, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_F32, biases=(None, None, None),
+            mem=capi.MEM_DEVICE, launches=None):
+        """down(act(gate(x)) * up(x)) through turq_mlp; returns f32 [m, n_out].  launches: a list that receives the number of
+        matmul kernel launches the call made (device pointers only; from the library's kernel timing)."""
+        L, ctx = self.L, self.ctx
+        x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
+        m = x.shape[0]
+        xsend = (synth.to_bf16_bits(x).reshape(m, k) if x_dtype == capi.ACT_BF16 else x.astype(np.float16) if x_dtype == capi.ACT_F16 else x)
+        ydt = {capi.ACT_F32: np.float32, capi.ACT_BF16: np.uint16, capi.ACT_F16: np.float16}[y_dtype]
+        y = np.full((m, n_out), 0, ydt)
+        bs = [None if b is None else np.ascontiguousarray(b, np.float32) for b in biases]
+        freed = []
+        if mem == capi.MEM_DEVICE:
+            def dev(arr):
+                p = self.dev_buffer(arr)
+                freed.append(p)
+                return p
+            xp, yp = dev(xsend), dev(y)
+            bp = [None if b is None else dev(b) for b in bs]
+        else:
+            xp, yp, bp = capi.ptr(xsend), capi.ptr(y), [capi.ptr(b) for b in bs]
+        try:
+            if launches is not None:
+                capi.check(L.turq_profile_begin(ctx), ctx)
+            rc = L.turq_mlp(ctx, wg, wu, wd, xp, x_dtype, m, k, yp, y_dtype, n_out, bp[0], bp[1], bp[2], 0, mem)
+            if launches is not None:
+                cnt, ms = ctypes.c_int64(), ctypes.c_double()
+                capi.check(L.turq_profile_end(ctx, ctypes.byref(cnt), ctypes.byref(ms)), ctx)
+                launches.append(cnt.value)
+            capi.check(rc, ctx)
+            capi.check(L.turq_sync(ctx), ctx)
+            if mem == capi.MEM_DEVICE:
+                y = self.read_back(yp, (m, n_out), ydt)
+        finally:
+            for p in freed:
+                self.dev_free(p)
+        if y_dtype == capi.ACT_BF16:
+            y = synth.from_bf16_bits(y).reshape(m, n_out)
+        return np.asarray(y, np.float32)
+
     def quantize(self, x, kind):
         x = np.ascontiguousarray(x, np.float32)
         m, k = x.shape

@@ -111,6 +111,12 @@ def test_mlp_gate_up_in_one_call(model):
     down = qlinear.linear(FFN, HID, vb.pp("blk").pp(0).pp("ffn_down"))
     with pytest.raises(capi.TurqError):       # gate and up of different shapes
         qlinear.QMatMul.forward_gate_up(gate.qmatmul, down.qmatmul, x)
+    # the whole of Qwen3MLP::forward through one call: down_proj of that product
+    z = qlinear.QMatMul.forward_mlp(gate.qmatmul, up.qmatmul, down.qmatmul, x)
+    assert z.shape == (2, 3, HID)
+    assert rel_l2(z, down.forward(y)) <= 1e-6
+    with pytest.raises(capi.TurqError):       # down_proj must take what gate / up give
+        qlinear.QMatMul.forward_mlp(gate.qmatmul, up.qmatmul, gate.qmatmul, x)
 
 
 def test_embedding_over_the_quantized_table(model):
@@ -185,8 +191,10 @@ def test_cpp_host_mirror(model, tmp_path):
     biased = synth.random_weight(Q6_K, 96, k, seed=2)
     bias = rng.standard_normal(96).astype("<f4")
     norm = rng.standard_normal(k).astype("<f4")
+    down = synth.random_weight(Q8_0, 64, n, seed=3)
     path = tmp_path / "cpp.gguf"
     write_gguf(str(path), [("blk.0.ffn_gate.weight", Q4_K, (n, k), gate), ("blk.0.biased.weight", Q6_K, (96, k), biased),
+                           ("blk.0.ffn_down.weight", Q8_0, (64, n), down),
                            ("blk.0.biased.bias", 0, (96,), bias.view(np.uint8)), ("blk.0.attn_norm.weight", 0, (k,), norm.view(np.uint8))])
     res = subprocess.run([exe, str(path)], capture_output=True, text=True, timeout=120)
     assert res.returncode == 0, res.stderr

@@ -53,6 +53,8 @@ _SIGS = {
                                    c_int, c_int]),
     "turq_qmatmul_gate_up": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64,
                                      c_void_p, c_void_p, c_int, c_int]),
+    "turq_mlp": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64,
+                         c_void_p, c_void_p, c_void_p, c_int, c_int]),
     "turq_quantize_q8_0": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
     "turq_quantize_q8_k": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
     "turq_graph_begin": (c_int, [c_void_p]),

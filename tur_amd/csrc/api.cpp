@@ -153,6 +153,7 @@ void turq_ctx_destroy(turq_ctx *ctx) {
     if (ctx->stage_y) (void)hipFree(ctx->stage_y);
     if (ctx->act_prep) (void)hipFree(ctx->act_prep);
     if (ctx->gate_up) (void)hipFree(ctx->gate_up);
+    if (ctx->mlp_h) (void)hipFree(ctx->mlp_h);
     if (ctx->wide_x) (void)hipFree(ctx->wide_x);
     if (ctx->wide_s) (void)hipFree(ctx->wide_s);
     if (ctx->wide_y) (void)hipFree(ctx->wide_y);
@@ -634,6 +635,36 @@ static int impl_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const tu
     return TURQ_OK;
 }
 
+static int impl_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt, int64_t m,
+                    int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, const float *bias_down, int act,
+                    int mem) {
+    TURQ_ENTER(ctx);
+    if (!gate || !up || !down) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_mlp: null weight");
+    if (act != TURQ_ACTFN_SILU) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_mlp: activation %d is not supported", act);
+    if (gate->n != up->n || gate->k != up->k)
+        return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_mlp: gate is [%lld, %lld], up is [%lld, %lld]", (long long)gate->n, (long long)gate->k,
+                         (long long)up->n, (long long)up->k);
+    if (down->k != gate->n)
+        return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_mlp: down takes %lld columns, gate and up give %lld", (long long)down->k, (long long)gate->n);
+    if (mem != TURQ_MEM_DEVICE && mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_mlp: bad mem %d", mem);
+    if (!turq_act_bytes(yt)) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_mlp: output dtype %d", yt);
+    if (m < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_mlp: m=%lld is negative", (long long)m);
+    const int64_t n_ff = gate->n;
+    const size_t h_elems = (size_t)m * (size_t)n_ff;
+    if (mem == TURQ_MEM_HOST) {
+        std::vector<float> h;
+        try { h.resize(h_elems ? h_elems : 1); } catch (...) { return turq_fail(ctx, TURQ_ERR_OOM, "turq_mlp: host scratch"); }
+        int rc = impl_qmatmul_gate_up(ctx, gate, up, x, xt, m, ldx, h.data(), TURQ_ACT_F32, n_ff, bias_gate, bias_up, act, mem);
+        if (rc != TURQ_OK) return rc;
+        return impl_qmatmul(ctx, down, h.data(), TURQ_ACT_F32, m, n_ff, y, yt, ldy, bias_down, mem, TURQ_ALGO_AUTO);
+    }
+    int rc = turq_ctx_reserve(ctx, &ctx->mlp_h, &ctx->mlp_h_cap, h_elems * sizeof(float) + 16);
+    if (rc != TURQ_OK) return rc;
+    rc = impl_qmatmul_gate_up(ctx, gate, up, x, xt, m, ldx, ctx->mlp_h, TURQ_ACT_F32, n_ff, bias_gate, bias_up, act, mem);
+    if (rc != TURQ_OK) return rc;
+    return impl_qmatmul(ctx, down, ctx->mlp_h, TURQ_ACT_F32, m, n_ff, y, yt, ldy, bias_down, mem, TURQ_ALGO_AUTO);
+}
+
 // ---- graphs and kernel timing ----
 
 int turq_graph_begin(turq_ctx *ctx) {
@@ -792,6 +823,10 @@ int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weigh
 int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m, int64_t ldx,
                          void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, int act, int mem) {
     return capture_guard(ctx, impl_qmatmul_gate_up(ctx, gate, up, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, act, mem));
+}
+int turq_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt, int64_t m,
+             int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, const float *bias_down, int act, int mem) {
+    return capture_guard(ctx, impl_mlp(ctx, gate, up, down, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem));
 }
 int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
     return capture_guard(ctx, impl_quantize_q8_0(ctx, x, m, k, out, mem));

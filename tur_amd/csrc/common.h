@@ -86,6 +86,7 @@ struct turq_ctx {
     void *wide_s = nullptr;   size_t wide_s_cap = 0;
     void *wide_y = nullptr;   size_t wide_y_cap = 0;
     bool wide = false;  // device-pointer calls take that path too (host-pointer calls always do)
+    void *mlp_h = nullptr;    size_t mlp_h_cap = 0;  // turq_mlp: the f32 intermediate act(gate) * up
     // scratch buffers that were outgrown while a captured graph still referred to them: freed once no graph of the context is
     // alive (at the next growth) or with the context
     std::vector<void *> retired;

@@ -164,6 +164,14 @@ public:
         d.check(turq_qmatmul_gate_up(d.ctx(), gate.t_.handle(), up.t_.handle(), x_dev, x_dtype, m, ldx, y_dev, y_dtype, ldy, nullptr,
                                      nullptr, TURQ_ACTFN_SILU, TURQ_MEM_DEVICE));
     }
+    // (silu(x gate^T) * (x up^T)) down^T of a device tensor, the whole of Qwen3MLP::forward (src/models/qwen3.rs:161-167); the
+    // f32 intermediate lives in the context's scratch memory
+    static void forward_mlp(const QMatMul &gate, const QMatMul &up, const QMatMul &down, const void *x_dev, int x_dtype, int64_t m,
+                            int64_t ldx, void *y_dev, int y_dtype, int64_t ldy) {
+        const Device &d = gate.t_.device();
+        d.check(turq_mlp(d.ctx(), gate.t_.handle(), up.t_.handle(), down.t_.handle(), x_dev, x_dtype, m, ldx, y_dev, y_dtype, ldy, nullptr,
+                         nullptr, nullptr, TURQ_ACTFN_SILU, TURQ_MEM_DEVICE));
+    }
     const QTensor &qtensor() const { return t_; }
 
 private:

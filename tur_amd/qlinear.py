@@ -220,6 +220,25 @@ class QMatMul:
         return y.reshape(lead + (n,))
 
 
+    @staticmethod
+    def forward_mlp(gate: "QMatMul", up: "QMatMul", down: "QMatMul", xs: np.ndarray) -> np.ndarray:
+        """``(silu(x @ gate.T) * (x @ up.T)) @ down.T``, the whole of ``Qwen3MLP::forward`` (src/models/qwen3.rs:161-167),
+        through ``turq_mlp``: the intermediate stays in f32 on the library's side."""
+        xs = np.asarray(xs)
+        k, n_out = gate.qtensor._k, down.qtensor._n
+        if xs.ndim < 2 or xs.shape[-1] != k:
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch in matmul: input {xs.shape}, layers need last dim {k}")
+        if xs.dtype != np.float32 or not xs.flags["C_CONTIGUOUS"]:
+            raise TurqError(capi.ERR_INVALID, "forward_mlp needs a contiguous f32 input")
+        lead = xs.shape[:-1]
+        m = int(np.prod(lead)) if lead else 1
+        y = np.empty((m, n_out), np.float32)
+        dev = gate.qtensor.device
+        capi.check(dev.L.turq_mlp(dev.ctx, gate.qtensor.handle, up.qtensor.handle, down.qtensor.handle, capi.ptr(xs), capi.ACT_F32, m, k,
+                                  capi.ptr(y), capi.ACT_F32, n_out, None, None, None, capi.ACTFN_SILU, capi.MEM_HOST), dev.ctx)
+        return y.reshape(lead + (n_out,))
+
+
 class LinearX:
     """``LinearX::Quantized { qmatmul, bias }`` (src/models/layers/linear.rs:8-31)."""
 
