@@ -506,6 +506,53 @@ def side_leg(base, workload, ms, act, outdt, steps, warmup):
             "rows": rows}
 
 
+def read_floor():
+    """What a launch that only READS the bytes of a decode launch takes (turq_read_yardstick: one 16-wave workgroup per compute
+    unit, the shape of the decode kernels), timed like the kernels.  The sizes are those of the launches of the two decode
+    workloads; each launch reads a region of its own of a 2 GiB buffer, so nothing is served from a cache."""
+    L = capi.lib()
+    ctx = ctypes.c_void_p()
+    capi.check(L.turq_ctx_create(0, ctypes.byref(ctx)))
+    total = 2 << 30
+    buf = ctypes.c_void_p()
+    rows = []
+    try:
+        capi.check(L.turq_dev_alloc(ctx, total, ctypes.byref(buf)), ctx)
+        w = ctypes.c_void_p()   # dequantizing a 64 MiB F32 tensor into every part of the buffer touches (and so maps) all of it
+        one = np.zeros(16 << 20, np.float32)
+        capi.check(L.turq_weight_upload(ctx, capi.F32, 1, one.size, capi.ptr(one), one.nbytes, capi.LAYOUT_NATIVE, ctypes.byref(w)), ctx)
+        for part in range(total // one.nbytes):
+            capi.check(L.turq_dequantize(ctx, w, ctypes.c_void_p(buf.value + part * one.nbytes), capi.MEM_DEVICE), ctx)
+        capi.check(L.turq_sync(ctx), ctx)
+        capi.check(L.turq_weight_release(w))
+        sizes = {"o_proj Q4_K 4096x4096": synth.weight_nbytes(synth.Q4_K, 4096, 4096),
+                 "q,k Q4_K + v Q6_K": synth.weight_nbytes(synth.Q4_K, 5120, 4096) + synth.weight_nbytes(synth.Q6_K, 1024, 4096),
+                 "down Q4_K 4096x12288": synth.weight_nbytes(synth.Q4_K, 4096, 12288),
+                 "down Q6_K 4096x12288": synth.weight_nbytes(synth.Q6_K, 4096, 12288),
+                 "gate + up Q4_K 2 x 12288x4096": 2 * synth.weight_nbytes(synth.Q4_K, 12288, 4096)}
+        for label, nbytes in sizes.items():
+            span = (nbytes + 4095) // 4096 * 4096
+            slots = total // span
+            reps = 40
+            for timed in (False, True):
+                if timed:
+                    capi.check(L.turq_profile_begin(ctx), ctx)
+                for i in range(reps):
+                    capi.check(L.turq_read_yardstick(ctx, ctypes.c_void_p(buf.value + (i % slots) * span), nbytes), ctx)
+                if not timed:
+                    capi.check(L.turq_sync(ctx), ctx)
+            n, ms = ctypes.c_int64(), ctypes.c_double()
+            capi.check(L.turq_profile_end(ctx, ctypes.byref(n), ctypes.byref(ms)), ctx)
+            us = ms.value / max(1, n.value) * 1e3
+            rows.append({"launch": label, "bytes": int(nbytes), "read_us": round(us, 2), "read_gbps": round(nbytes / us / 1e3, 1),
+                         "frac_of_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)})
+    finally:
+        if buf:
+            L.turq_dev_free(ctx, buf)
+        L.turq_ctx_destroy(ctx)
+    return {"what": "a launch of the decode kernels' shape that only reads the same bytes (turq_read_yardstick), kernel time", "rows": rows}
+
+
 def other_halves(base):
     """The rest of the headline metric, measured in the same process with the same method (value = whole step, frac = the
     matmul kernels alone against the peak): the prefill GEMM (BASELINE config 4), the mixed Q4_K / Q6_K decoder layer at
@@ -515,6 +562,7 @@ def other_halves(base):
         "prefill": side_leg(base, "q4k_prefill_up_8b", [512, 2048], "bf16", "bf16", steps, warmup),
         "q4km_layer": side_leg(base, "q4km_layer_8b", [1, 8, 32], "f32", "f32", steps, warmup),
         "lm_head_q6k": side_leg(base, "lm_head_q6k_8b", [1], "bf16", "f32", steps, warmup),
+        "read_floor": read_floor(),
     }
 
 

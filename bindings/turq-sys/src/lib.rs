@@ -109,6 +109,7 @@ extern "C" {
     pub fn turq_ctx_scratch_info(ctx: *const turq_ctx, live_graphs: *mut c_int, retired_buffers: *mut c_int, act_prep_bytes: *mut usize) -> c_int;
     pub fn turq_profile_begin(ctx: *mut turq_ctx) -> c_int;
     pub fn turq_profile_end(ctx: *mut turq_ctx, launches: *mut i64, total_ms: *mut f64) -> c_int;
+    pub fn turq_read_yardstick(ctx: *mut turq_ctx, dev_ptr: *const c_void, nbytes: usize) -> c_int;
     pub fn turq_gguf_open(path: *const c_char, out: *mut *mut turq_gguf) -> c_int;
     pub fn turq_gguf_close(g: *mut turq_gguf);
     pub fn turq_gguf_last_error(g: *const turq_gguf) -> *const c_char;

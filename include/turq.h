@@ -283,6 +283,12 @@ int turq_ctx_scratch_info(const turq_ctx *ctx, int *live_graphs, int *retired_bu
  * execution times (launch gaps excluded). */
 int turq_profile_begin(turq_ctx *ctx);
 int turq_profile_end(turq_ctx *ctx, int64_t *launches, double *total_ms);
+/* A yardstick for the numbers above, not part of the path: one launch that only READS nbytes of device memory at dev_ptr
+ * (16-byte aligned; rounded down to whole 4 KiB) with the launch shape of the decode kernels - one 16-wave workgroup per
+ * compute unit, two 4 KiB chunks in flight per wave - on the context's stream, timed like a matmul kernel when kernel timing
+ * is on.  A launch of a few tens of MB is short enough for the launch itself to weigh as much as its bytes (on an MI355X
+ * 28 MB take 5.0 us and 57 MB 9.2 us, where 8 TB/s would mean 3.5 and 7.1): this is what the decode kernels are up against. */
+int turq_read_yardstick(turq_ctx *ctx, const void *dev_ptr, size_t nbytes);
 
 /* ---- GGUF files ---- */
 /* Parse the header (magic, version 1..3, metadata, tensor infos, alignment).

@@ -216,3 +216,23 @@ def test_a_call_that_fails_inside_a_capture_ends_it():
     finally:
         st.close()
         gpu.close()
+
+
+def test_read_yardstick_is_timed_like_a_kernel(gpu):
+    """turq_read_yardstick: a launch that only reads; with kernel timing on it counts as one timed launch, and it refuses
+    pointers the kernel's 16-byte loads could not take"""
+    L, ctx = gpu.L, gpu.ctx
+    nbytes = 8 << 20
+    buf = gpu.dev_buffer(np.zeros(nbytes // 4, np.float32))
+    capi.check(L.turq_read_yardstick(ctx, buf, nbytes), ctx)
+    capi.check(L.turq_profile_begin(ctx), ctx)
+    for _ in range(3):
+        capi.check(L.turq_read_yardstick(ctx, buf, nbytes), ctx)
+    n, ms = ctypes.c_int64(), ctypes.c_double()
+    capi.check(L.turq_profile_end(ctx, ctypes.byref(n), ctypes.byref(ms)), ctx)
+    assert n.value == 3 and 0.0 < ms.value < 50.0
+    assert L.turq_read_yardstick(ctx, ctypes.c_void_p(buf.value + 4), 4096) == capi.ERR_INVALID
+    assert L.turq_read_yardstick(ctx, None, 4096) == capi.ERR_INVALID
+    assert L.turq_read_yardstick(ctx, buf, 100) == capi.OK      # less than one 4 KiB chunk: nothing to launch
+    capi.check(L.turq_sync(ctx), ctx)
+    gpu.dev_free(buf)

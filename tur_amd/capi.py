@@ -57,6 +57,7 @@ _SIGS = {
                          c_void_p, c_void_p, c_void_p, c_int, c_int]),
     "turq_quantize_q8_0": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
     "turq_quantize_q8_k": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
+    "turq_read_yardstick": (c_int, [c_void_p, c_void_p, c_size_t]),
     "turq_graph_begin": (c_int, [c_void_p]),
     "turq_graph_end": (c_int, [c_void_p, POINTER(c_void_p)]),
     "turq_graph_launch": (c_int, [c_void_p, c_void_p]),

@@ -721,6 +721,16 @@ void turq_graph_destroy(turq_graph *g) {
     delete g;
 }
 
+int turq_read_yardstick(turq_ctx *ctx, const void *dev_ptr, size_t nbytes) {
+    TURQ_ENTER(ctx);
+    if (!dev_ptr && nbytes) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_read_yardstick: null pointer");
+    if ((uintptr_t)dev_ptr % 16) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_read_yardstick: the pointer must be 16-byte aligned");
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+    TURQ_HIP(ctx, turq_launch_read_yardstick(dev_ptr, nbytes, ctx->compute_units > 0 ? ctx->compute_units : 256, ctx->stream, ev0, ev1));
+    return TURQ_OK;
+}
+
 int turq_profile_begin(turq_ctx *ctx) {
     TURQ_ENTER(ctx);
     if (ctx->capturing) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_profile_begin: a graph capture is running");

@@ -187,6 +187,8 @@ hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t 
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
                       int yt, int64_t ldy, const float *bias, int algo);
 // act(gate) * up on two f32 matrices [m, n] of row stride n (act_mul.hip)
+hipError_t turq_launch_read_yardstick(const void *buf, size_t nbytes, int workgroups, hipStream_t stream, hipEvent_t ev_start,
+                                      hipEvent_t ev_stop);
 hipError_t turq_launch_silu_mul(const float *gate, const float *up, int64_t m, int64_t n, void *y, int y_dtype, int64_t ldy,
                                 hipStream_t stream);
 // act(gate) * up inside the one-row kernel; *taken = false (and nothing launched) where that kernel does not apply

@@ -1,0 +1,55 @@
+// A plain streaming read of device memory with the launch shape of the decode kernels: one 16-wave workgroup per compute unit,
+// every wave two 4 KiB chunks in flight, nothing done with the data but an xor.  It is the yardstick for what a decode launch
+// of a given size could reach at best on the device at hand: launches of a few tens of MB are short enough for the launch
+// itself (thousands of waves to start, the first loads to return, the last ones to drain) to weigh as much as the bytes.
+#include <hip/hip_ext.h>
+
+#include "mfma_common.h"
+
+namespace {
+
+__global__ void __launch_bounds__(1024) read_kernel(const uint8_t *__restrict__ buf, size_t nchunks, uint32_t *__restrict__ sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const size_t stride = (size_t)gridDim.x * nw;
+    size_t c = (size_t)blockIdx.x * nw + wave;
+    uint4v r[2][4];
+    uint4v acc = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int d = 0; d < 2; d++) {
+        const size_t cc = c + d * stride;
+        const uint8_t *p = buf + (cc < nchunks ? cc : 0) * 4096 + 16 * lane;
+#pragma unroll
+        for (int i = 0; i < 4; i++) r[d][i] = *(const uint4v *)(p + 1024 * i);
+    }
+    while (c < nchunks) {
+#pragma unroll
+        for (int d = 0; d < 2; d++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc ^= r[d][i];
+            const size_t cn = c + 2 * stride;
+            const uint8_t *p = buf + (cn < nchunks ? cn : 0) * 4096 + 16 * lane;
+#pragma unroll
+            for (int i = 0; i < 4; i++) r[d][i] = *(const uint4v *)(p + 1024 * i);
+            c += stride;
+        }
+    }
+    // never true for memory that holds anything but this one pattern: the loads must not be optimised away
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9E3779B9u && sink) sink[blockIdx.x] = acc.x;
+}
+
+}  // namespace
+
+// reads the first nbytes / 4096 * 4096 bytes at buf (16-byte aligned); workgroups: 1 ..
+hipError_t turq_launch_read_yardstick(const void *buf, size_t nbytes, int workgroups, hipStream_t stream, hipEvent_t ev_start,
+                                      hipEvent_t ev_stop) {
+    if (workgroups < 1 || ((uintptr_t)buf & 15) != 0) return hipErrorInvalidValue;
+    const size_t nchunks = nbytes / 4096;
+    if (nchunks == 0) return hipSuccess;
+    if (ev_start) {
+        hipExtLaunchKernelGGL(read_kernel, dim3((unsigned)workgroups), dim3(1024), 0, stream, ev_start, ev_stop, 0, (const uint8_t *)buf,
+                              nchunks, (uint32_t *)nullptr);
+        return hipGetLastError();
+    }
+    read_kernel<<<dim3((unsigned)workgroups), dim3(1024), 0, stream>>>((const uint8_t *)buf, nchunks, (uint32_t *)nullptr);
+    return hipGetLastError();
+}
