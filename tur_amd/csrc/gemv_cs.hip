@@ -93,6 +93,96 @@ __device__ __forceinline__ void cs_body(const uint8_t *__restrict__ w, int64_t n
     }
 }
 
+// The same workgroup, written out for a wave that owns exactly CPW column tiles.  In the loop above the compiler sizes its
+// waits (s_waitcnt vmcnt) for the worst path through the conditions and schedules the header arithmetic of a tile ahead of the
+// tiles before it, so a tile requested D steps ahead is in fact waited for at once, and the activations of a column tile, which
+// are requested after the weights, drain the whole ring before they can be used.  Here every load sits in straight-line code,
+// the tiles are kept apart by scheduling barriers, and the next column tile's activations are requested BEFORE the last D
+// weight tiles of the current one - loads return in order, so waiting for them leaves the ring in flight - and converted after
+// those D tiles, when they have long arrived.  Results are those of cs_body bit for bit.
+template <int DT, int MT, int XT, int RG, int D, int CPW>
+__device__ __forceinline__ void cs_body_unrolled(const uint8_t *__restrict__ w, int64_t n, int64_t k, const void *__restrict__ x, int64_t ldx,
+                                                 int64_t m, void *__restrict__ y, int yt, int64_t ldy, const float *__restrict__ bias,
+                                                 int64_t grp) {
+    static_assert(RG % D == 0 && RG >= D, "the ring of weight tiles repeats per column tile");
+    extern __shared__ uint8_t smem[];
+    constexpr int TB = TiledFmt<DT>::kTileBytes;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nwaves = blockDim.x >> 6;  // ntc == CPW * nwaves
+    const int64_t ntc = turq_tile_cols(k), nrt = turq_tile_rows(n);
+    const int64_t rt0 = grp * RG;
+    float4v acc[RG][MT];
+    const uint8_t *wrow[RG];  // row tiles past the weight's last one re-read it; their results are not stored
+#pragma unroll
+    for (int r = 0; r < RG; r++) {
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[r][mt] = float4v{0.f, 0.f, 0.f, 0.f};
+        wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+    }
+    GOff go = lane_offsets(lane, 16);
+    // the first column tile's activations go out first, the first D weight tiles right behind them
+    RawRows<XT> raw[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) raw[mt] = load_rows_raw<DT, XT>(x, ldx, m, k, wave, lane, mt);
+    WRegs<DT> wr[D];
+#pragma unroll
+    for (int d = 0; d < D; d++) wr[d] = load_tile<DT>(wrow[d] + (int64_t)wave * TB, go);
+    AFrags<DT, MT> f;
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) frags_from_raw<DT, XT>(raw[mt], f.a[mt]);
+#pragma unroll
+    for (int c = 0; c < CPW; c++) {
+        const int64_t b = wave + (int64_t)c * nwaves, bn = b + nwaves;
+#pragma unroll
+        for (int r = 0; r < RG; r++) {
+            if (r == RG - D && c + 1 < CPW) {
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) raw[mt] = load_rows_raw<DT, XT>(x, ldx, m, k, bn, lane, mt);
+            }
+            TileOp<DT, MT, 4>::run(wr[r % D], f, lane, acc[r]);
+            __builtin_amdgcn_sched_barrier(0);
+            // the slot is free: request the tile D steps ahead
+            if (r + D < RG) wr[r % D] = load_tile<DT>(wrow[r + D] + b * TB, go);
+            else if (c + 1 < CPW) wr[r % D] = load_tile<DT>(wrow[r + D - RG] + bn * TB, go);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (c + 1 < CPW) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) frags_from_raw<DT, XT>(raw[mt], f.a[mt]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // the waves' partial tiles meet in the LDS; wave i adds up the i-th (row tile, m-tile) pair in wave order
+    float4v *red = (float4v *)smem;
+#pragma unroll
+    for (int r = 0; r < RG; r++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) red[((r * MT + mt) * nwaves + wave) * 64 + lane] = acc[r][mt];
+    __syncthreads();
+    const int nn = lane & 15, g = lane >> 4;
+    for (int i = wave; i < RG * MT; i += nwaves) {
+        const int r = i / MT, mt = i - r * MT;
+        float4v s = red[(i * nwaves) * 64 + lane];
+        for (int wv = 1; wv < nwaves; wv++) s += red[(i * nwaves + wv) * 64 + lane];
+        const int64_t col = (rt0 + r) * 16 + nn;
+        if (rt0 + r >= nrt || col >= n) continue;
+        const float bv = bias ? bias[col] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int64_t row = 16 * mt + 4 * g + j;
+            if (row < m) turq_store_any(y, yt, row * ldy + col, s[j] + bv);
+        }
+    }
+}
+
+template <int DT, int MT, int XT, int RG, int D, int CPW, int MAXT>
+__global__ void __launch_bounds__(MAXT) gemv_cs_unrolled_kernel(MultiArgs a, int64_t k, const void *__restrict__ x, int64_t ldx, int64_t m,
+                                                                 int yt) {
+    const MultiPick p = multi_pick(a, (int)blockIdx.x);
+    cs_body_unrolled<DT, MT, XT, RG, D, CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
+}
+
 template <int DT, int MT, int XT, int RG, int D, int MAXT>
 __global__ void __launch_bounds__(MAXT) gemv_cs_kernel(MultiArgs a, int64_t k, const void *__restrict__ x, int64_t ldx, int64_t m, int yt) {
     const MultiPick p = multi_pick(a, (int)blockIdx.x);
@@ -120,6 +210,19 @@ hipError_t launch_final(const CsLaunch &l) {
         if (raised != hipSuccess) return raised;
     }
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
+    // a wave that owns exactly two column tiles (K = 4096 with eight waves): the written-out form
+    static const bool generic = [] { const char *e = getenv("TURQ_CS_GENERIC"); return e && atoi(e) != 0; }();
+    if constexpr (MT == 1 && RG == 6) {
+        if (!generic && l.nwaves > 1 && turq_tile_cols(l.k) == 2 * (int64_t)l.nwaves && lds <= (64u << 10)) {
+            if (l.ev0) {
+                hipExtLaunchKernelGGL((gemv_cs_unrolled_kernel<DT, MT, XT, RG, D, 2, MAXT>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0,
+                                      l.a, l.k, l.x, l.ldx, l.m, l.yt);
+                return hipGetLastError();
+            }
+            gemv_cs_unrolled_kernel<DT, MT, XT, RG, D, 2, MAXT><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
+            return hipGetLastError();
+        }
+    }
     if (l.ev0) {
         hipExtLaunchKernelGGL((gemv_cs_kernel<DT, MT, XT, RG, D, MAXT>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k, l.x,
                               l.ldx, l.m, l.yt);

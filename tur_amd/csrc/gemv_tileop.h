@@ -261,14 +261,46 @@ template <int MT, int NV> struct TileOp<TURQ_Q8_0, MT, NV> {
 };
 
 // ---- activation fragments straight from the caller's rows ----
-template <int XT> __device__ inline half8v load_half8(const uint8_t *p) {
+// The raw activations behind the A fragments of one column tile and m-tile: what frags_from_rows loads, kept apart from what it
+// computes, for kernels that request the next column tile's activations while they still work on the current one.
+template <int XT> struct RawRows {
+    uint4v v[XT == TURQ_ACT_F32 ? 16 : 8];
+};
+template <int DT, int XT>
+__device__ inline RawRows<XT> load_rows_raw(const void *__restrict__ x, int64_t ldx, int64_t m, int64_t k, int64_t b, int lane, int mt) {
+    constexpr bool KQ = DT != TURQ_Q8_0;
+    constexpr int ES = XT == TURQ_ACT_F32 ? 4 : 2;
+    const int r = lane & 15, g = lane >> 4;
+    int64_t row = 16 * mt + r;
+    if (row >= m) row = m - 1;
+    const uint8_t *base = (const uint8_t *)x + (row * ldx + b * 256) * ES;
+    RawRows<XT> raw;
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const int col = KQ ? 64 * g + 8 * q : 32 * q + 8 * g;
+        const bool in = KQ || b * 256 + col < k;
+        const uint8_t *p = base + (in ? col : 0) * ES;
+        if constexpr (XT == TURQ_ACT_F32) {
+            const uint4v a = *(const uint4v *)p, c = *(const uint4v *)(p + 16);
+            raw.v[2 * q] = in ? a : uint4v{0u, 0u, 0u, 0u};
+            raw.v[2 * q + 1] = in ? c : uint4v{0u, 0u, 0u, 0u};
+        } else {
+            const uint4v a = *(const uint4v *)p;
+            raw.v[q] = in ? a : uint4v{0u, 0u, 0u, 0u};
+        }
+    }
+    return raw;
+}
+template <int XT> __device__ inline half8v raw_to_half8(const RawRows<XT> &raw, int q) {
     if constexpr (XT == TURQ_ACT_F32) {
-        const float4v a = *(const float4v *)p, b = *(const float4v *)(p + 16);
-        const half2v h0 = __builtin_convertvector(float2v{a.x, a.y}, half2v), h1 = __builtin_convertvector(float2v{a.z, a.w}, half2v);
-        const half2v h2 = __builtin_convertvector(float2v{b.x, b.y}, half2v), h3 = __builtin_convertvector(float2v{b.z, b.w}, half2v);
+        const uint4v a = raw.v[2 * q], b = raw.v[2 * q + 1];
+        const half2v h0 = __builtin_convertvector(float2v{__uint_as_float(a.x), __uint_as_float(a.y)}, half2v);
+        const half2v h1 = __builtin_convertvector(float2v{__uint_as_float(a.z), __uint_as_float(a.w)}, half2v);
+        const half2v h2 = __builtin_convertvector(float2v{__uint_as_float(b.x), __uint_as_float(b.y)}, half2v);
+        const half2v h3 = __builtin_convertvector(float2v{__uint_as_float(b.z), __uint_as_float(b.w)}, half2v);
         return make_half8(h0, h1, h2, h3);
     } else if constexpr (XT == TURQ_ACT_BF16) {
-        const uint4v u = *(const uint4v *)p;
+        const uint4v u = raw.v[q];
         const uint32_t wd[4] = {u.x, u.y, u.z, u.w};
         half2v h[4];
 #pragma unroll
@@ -276,30 +308,14 @@ template <int XT> __device__ inline half8v load_half8(const uint8_t *p) {
             h[j] = __builtin_convertvector(float2v{__uint_as_float(wd[j] << 16), __uint_as_float(wd[j] & 0xFFFF0000u)}, half2v);
         return make_half8(h[0], h[1], h[2], h[3]);
     } else {
-        return *(const half8v *)p;
+        return __builtin_bit_cast(half8v, raw.v[q]);
     }
 }
-
-// The A fragments of column tile b and m-tile mt, from the activation rows themselves.  Lane (r, g) holds row 16 mt + r:
-// K-quants: step q = columns 256 b + 64 g + 8 q .. + 7, step 8 = the (hi, lo) sums of its four 16-column groups;
-// Q8_0: step q = columns 256 b + 32 q + 8 g .. + 7 (zeros past k, which may end inside the tile).
-// Rows past m repeat row m - 1: every output row depends on its own A row only and those rows are not stored.
-template <int DT, int XT>
-__device__ inline void frags_from_rows(const void *__restrict__ x, int64_t ldx, int64_t m, int64_t k, int64_t b, int lane, int mt,
-                                       half8v *__restrict__ out) {
-    constexpr bool KQ = DT != TURQ_Q8_0;
-    constexpr int ES = XT == TURQ_ACT_F32 ? 4 : 2;
-    const int r = lane & 15, g = lane >> 4;
-    int64_t row = 16 * mt + r;
-    if (row >= m) row = m - 1;
-    const uint8_t *base = (const uint8_t *)x + (row * ldx + b * 256) * ES;
+// the fragments of those activations (the conversions and sums of frags_from_rows, value for value)
+template <int DT, int XT> __device__ inline void frags_from_raw(const RawRows<XT> &raw, half8v *__restrict__ out) {
 #pragma unroll
-    for (int q = 0; q < 8; q++) {
-        const int col = KQ ? 64 * g + 8 * q : 32 * q + 8 * g;
-        if (KQ || b * 256 + col < k) out[q] = load_half8<XT>(base + col * ES);
-        else out[q] = half8v{0, 0, 0, 0, 0, 0, 0, 0};
-    }
-    if constexpr (KQ) {
+    for (int q = 0; q < 8; q++) out[q] = raw_to_half8<XT>(raw, q);
+    if constexpr (DT != TURQ_Q8_0) {
         half2v s[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -313,6 +329,17 @@ __device__ inline void frags_from_rows(const void *__restrict__ x, int64_t ldx, 
         }
         out[8] = make_half8(s[0], s[1], s[2], s[3]);
     }
+}
+
+// The A fragments of column tile b and m-tile mt, from the activation rows themselves.  Lane (r, g) holds row 16 mt + r:
+// K-quants: step q = columns 256 b + 64 g + 8 q .. + 7, step 8 = the (hi, lo) sums of its four 16-column groups;
+// Q8_0: step q = columns 256 b + 32 q + 8 g .. + 7 (zeros past k, which may end inside the tile).
+// Rows past m repeat row m - 1: every output row depends on its own A row only and those rows are not stored.
+template <int DT, int XT>
+__device__ inline void frags_from_rows(const void *__restrict__ x, int64_t ldx, int64_t m, int64_t k, int64_t b, int lane, int mt,
+                                       half8v *__restrict__ out) {
+    const RawRows<XT> raw = load_rows_raw<DT, XT>(x, ldx, m, k, b, lane, mt);
+    frags_from_raw<DT, XT>(raw, out);
 }
 
 // Several weights of one format and one k against the same activations in one launch (gate and up, or q and k,
