@@ -124,7 +124,8 @@ int turq_memcpy_d2h(turq_ctx *ctx, void *dst_host, const void *src_dev, size_t n
  * (src/models/layers/linear.rs:69). */
 int turq_weight_upload(turq_ctx *ctx, int ggml_dtype, int64_t n, int64_t k, const void *host_bytes,
                        size_t nbytes, int layout, turq_weight **out);
-/* Arc<QTensor> clone / drop */
+/* Arc<QTensor> clone / drop.  The release that drops the last reference waits for the whole device to go idle before it frees
+ * the memory (a weight may be in use by launches of any context of that device); do it at teardown, not inside a decode loop. */
 int turq_weight_retain(turq_weight *w);
 int turq_weight_release(turq_weight *w);
 /* QTensor::shape / dtype; any out pointer may be NULL */
@@ -224,7 +225,8 @@ enum { TURQ_ACTFN_SILU = 0 };
  * two: for one row (two on 8 MiB of weights and more) that kernel is the one launch of the call, for more rows it follows
  * one preparation of the activations (scratch memory of the context, which grows on demand, never inside a graph
  * capture).  Every other case computes the two products through turq_qmatmul_multi into scratch memory of the context and
- * combines them in one elementwise pass.  Errors as turq_qmatmul; gate and up of different shapes: TURQ_ERR_SHAPE; an activation other
+ * combines them in one elementwise pass (with TURQ_MEM_HOST that pass runs on the host CPU, in the same f32 arithmetic: the
+ * host form is for tests and one-off calls).  Errors as turq_qmatmul; gate and up of different shapes: TURQ_ERR_SHAPE; an activation other
  * than TURQ_ACTFN_SILU: TURQ_ERR_INVALID.
  * Replaces: `x.apply(&self.gate_proj)?.apply(&self.act_fn)?` times `x.apply(&self.up_proj)?` in `Qwen3MLP::forward`
  * (src/models/qwen3.rs:161-167; the Granite MLP, src/models/granite_41.rs:151-155, has the same form). */
