@@ -124,7 +124,7 @@ class Gpu:
         L, ctx = self.L, self.ctx
         x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
         m = x.shape[0]
-        xsend = synth.to_bf16_bits(x).reshape(m, k) if x_dtype == capi.ACT_BF16 else x
+        xsend = synth.to_bf16_bits(x).reshape(m, k) if x_dtype == capi.ACT_BF16 else x.astype(np.float16) if x_dtype == capi.ACT_F16 else x
         count = len(ws)
         outs = [np.zeros((m, n), np.float32) for n in ns]
         bias_host = [None if biases is None or b is None else np.ascontiguousarray(b, np.float32) for b in (biases or [None] * count)]

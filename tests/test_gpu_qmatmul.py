@@ -587,6 +587,62 @@ def test_rows_in_registers_kernel_shapes(row_tiles):
     assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-1000:]
 
 
+# 5 .. 16 rows on a k that splits evenly over the waves go through the form of that kernel that stages the activation rows
+# through the LDS (no preparation launch, no scratch): k = 1024 is two column tiles per wave, k = 4608 six; n = 200 ends inside
+# a row tile and, with several row tiles per workgroup, inside a workgroup.  One format and the two-format launches, every
+# activation type, strides, biases, bf16 output; the rows of a batch are independent, so a batch of 16 equals two of 8.
+@pytest.mark.parametrize("k", [1024, 4608])
+@pytest.mark.parametrize("dts", [(Q4_K,), (Q5_K,), (Q6_K,), (Q8_0,), (Q4_K, Q4_K, Q6_K), (Q5_K, Q6_K, Q6_K), (Q4_K, Q4_K, Q4_K, Q6_K)])
+def test_staged_rows_kernel(dts, k):
+    own = Gpu()
+    try:
+        ns = [200, 48, 33, 16][: len(dts)]
+        raws = [synth.random_weight(dt, n, k, seed=11 * i + n + k) for i, (dt, n) in enumerate(zip(dts, ns))]
+        ws = [own.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
+        biases = [None if i == 0 else np.random.default_rng(i).standard_normal(n).astype(np.float32) for i, n in enumerate(ns)]
+        x16 = synth.random_activation(16, k, seed=k + len(dts), bf16=True)
+        for m in (5, 8, 9, 16):
+            x = x16[:m]
+            for x_dtype in (capi.ACT_F32, capi.ACT_BF16, capi.ACT_F16):
+                xv = f16_round(x) if x_dtype == capi.ACT_F16 else x
+                ys = own.qmatmul_multi(ws, xv, ns, k, x_dtype=x_dtype, biases=biases)
+                for dt, n, raw, y, b in zip(dts, ns, raws, ys, biases):
+                    want = orc.matmul_dequant(dt, f16_round(xv), raw, n, k) + (0 if b is None else b)
+                    assert rel_l2(y, want) <= 2e-5, (dt, n, m, x_dtype)
+        # no fragments were prepared for any of these calls
+        live, retired, cap = ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t()
+        capi.check(own.L.turq_ctx_scratch_info(own.ctx, ctypes.byref(live), ctypes.byref(retired), ctypes.byref(cap)), own.ctx)
+        assert cap.value == 0
+        # single calls: strides, bf16 store, and rows independent of the batch they are in
+        for dt, n, raw, w, b in zip(dts, ns, raws, ws, biases):
+            y = own.qmatmul(w, x16, n, k, bias=b, ldx=k + 8, ldy=n + 3)
+            want = orc.matmul_dequant(dt, f16_round(x16), raw, n, k) + (0 if b is None else b)
+            assert rel_l2(y, want) <= 2e-5
+            y8 = own.qmatmul(w, x16[8:], n, k, bias=b)
+            assert np.array_equal(y8, y[8:])
+            yb = own.qmatmul(w, x16[:7], n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16)
+            assert rel_l2(yb, orc.matmul_dequant(dt, x16[:7], raw, n, k)) <= 4e-3      # bf16 store
+        for w in ws:
+            own.release(w)
+    finally:
+        own.close()
+
+
+# ... and with each of its row-tile group sizes forced (the rule takes one row tile per workgroup for matrices this small)
+@pytest.mark.parametrize("row_tiles", [2, 3, 6])
+def test_staged_rows_kernel_group_sizes(row_tiles):
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, TURQ_CS_RG=str(row_tiles))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "-k", "test_staged_rows_kernel and not group_sizes",
+                          "-p", "no:cacheprovider", os.path.join(root, "tests", "test_gpu_qmatmul.py")],
+                         cwd=root, env=env, capture_output=True, text=True, timeout=280)
+    assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-1000:]
+
+
 # The prefill GEMM picks its tile (128 x 128, 128 x 192, the wide 128 x 256 with two-deep rings, or the low 64 x 128 for launches
 # that would leave CUs idle) from the problem size; the small matrices of the tests above would never reach the wide one and
 # always take the low one, so they run once more in child processes with each of the two forced and forbidden (the rule takes

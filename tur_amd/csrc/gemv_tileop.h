@@ -291,6 +291,15 @@ __device__ inline RawRows<XT> load_rows_raw(const void *__restrict__ x, int64_t 
     }
     return raw;
 }
+// eight bf16 values -> f16 (through f32, round to nearest even)
+__device__ inline half8v bf16x8_to_half8(uint4v u) {
+    const uint32_t wd[4] = {u.x, u.y, u.z, u.w};
+    half2v h[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        h[j] = __builtin_convertvector(float2v{__uint_as_float(wd[j] << 16), __uint_as_float(wd[j] & 0xFFFF0000u)}, half2v);
+    return make_half8(h[0], h[1], h[2], h[3]);
+}
 template <int XT> __device__ inline half8v raw_to_half8(const RawRows<XT> &raw, int q) {
     if constexpr (XT == TURQ_ACT_F32) {
         const uint4v a = raw.v[2 * q], b = raw.v[2 * q + 1];
@@ -300,35 +309,31 @@ template <int XT> __device__ inline half8v raw_to_half8(const RawRows<XT> &raw, 
         const half2v h3 = __builtin_convertvector(float2v{__uint_as_float(b.z), __uint_as_float(b.w)}, half2v);
         return make_half8(h0, h1, h2, h3);
     } else if constexpr (XT == TURQ_ACT_BF16) {
-        const uint4v u = raw.v[q];
-        const uint32_t wd[4] = {u.x, u.y, u.z, u.w};
-        half2v h[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-            h[j] = __builtin_convertvector(float2v{__uint_as_float(wd[j] << 16), __uint_as_float(wd[j] & 0xFFFF0000u)}, half2v);
-        return make_half8(h[0], h[1], h[2], h[3]);
+        return bf16x8_to_half8(raw.v[q]);
     } else {
         return __builtin_bit_cast(half8v, raw.v[q]);
     }
+}
+// step 8 of a K-quant column tile: the (hi, lo) f16 pairs of the sums of the lane's four 16-column groups (steps 2 j, 2 j + 1)
+__device__ inline half8v kq_group_sums(const half8v *__restrict__ out) {
+    half2v s[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum = __builtin_amdgcn_fdot2(half2v{out[2 * j][2 * e], out[2 * j][2 * e + 1]}, splat2((_Float16)1.0f), sum, false);
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum = __builtin_amdgcn_fdot2(half2v{out[2 * j + 1][2 * e], out[2 * j + 1][2 * e + 1]}, splat2((_Float16)1.0f), sum, false);
+        const _Float16 hi = (_Float16)sum;
+        s[j] = half2v{hi, (_Float16)(sum - (float)hi)};
+    }
+    return make_half8(s[0], s[1], s[2], s[3]);
 }
 // the fragments of those activations (the conversions and sums of frags_from_rows, value for value)
 template <int DT, int XT> __device__ inline void frags_from_raw(const RawRows<XT> &raw, half8v *__restrict__ out) {
 #pragma unroll
     for (int q = 0; q < 8; q++) out[q] = raw_to_half8<XT>(raw, q);
-    if constexpr (DT != TURQ_Q8_0) {
-        half2v s[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            float sum = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 4; e++) sum = __builtin_amdgcn_fdot2(half2v{out[2 * j][2 * e], out[2 * j][2 * e + 1]}, splat2((_Float16)1.0f), sum, false);
-#pragma unroll
-            for (int e = 0; e < 4; e++) sum = __builtin_amdgcn_fdot2(half2v{out[2 * j + 1][2 * e], out[2 * j + 1][2 * e + 1]}, splat2((_Float16)1.0f), sum, false);
-            const _Float16 hi = (_Float16)sum;
-            s[j] = half2v{hi, (_Float16)(sum - (float)hi)};
-        }
-        out[8] = make_half8(s[0], s[1], s[2], s[3]);
-    }
+    if constexpr (DT != TURQ_Q8_0) out[8] = kq_group_sums(out);
 }
 
 // The A fragments of column tile b and m-tile mt, from the activation rows themselves.  Lane (r, g) holds row 16 mt + r:

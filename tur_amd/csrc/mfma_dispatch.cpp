@@ -93,6 +93,24 @@ int cs_row_tiles(const turq_ctx *ctx, int64_t m, int64_t row_tiles, int dtype, b
     return rg;
 }
 
+// The staged form of that kernel (activation rows loaded as they lie in memory and turned into fragments through the LDS) also
+// pays for small launches, where it replaces a preparation launch and a kernel that re-reads prepared fragments: row tiles per
+// workgroup so that the launch is about one workgroup per compute unit.  0: not this call.  TURQ_CS_STAGED = 0 switches it off,
+// TURQ_CS_RG forces the group size.
+int staged_row_tiles(const turq_ctx *ctx, int dtype_a, int dtype_b, int64_t k, int64_t m, int64_t row_tiles, bool aligned) {
+    static const int mode = [] { const char *e = getenv("TURQ_CS_STAGED"); return e ? atoi(e) : -1; }();
+    static const int forced = [] { const char *e = getenv("TURQ_CS_RG"); return e ? atoi(e) : 0; }();
+    static const int min_m = [] { const char *e = getenv("TURQ_CS_STAGED_MIN_M"); return e ? atoi(e) : 5; }();
+    if (mode == 0 || !aligned || m < min_m || m > 16) return 0;
+    const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+    if (row_tiles > 12 * cus && !forced) return 0;  // many rounds of workgroups (an LM head): the prepared fragments do better
+    const int64_t per = (row_tiles + cus - 1) / cus;
+    int rg = per <= 3 ? (int)per : per == 4 ? 2 : per == 5 ? 3 : 6;
+    if (forced) rg = forced;
+    while (rg > 1 && !turq_gemv_cs_staged_takes(dtype_a, dtype_b, k, m, rg)) rg = rg == 6 ? 3 : rg - 1;
+    return turq_gemv_cs_staged_takes(dtype_a, dtype_b, k, m, rg) ? rg : 0;
+}
+
 // whether the prefill GEMM can take this weight (its largest packed value must fit f16), and the power of two by which the
 // kernel multiplies the block scales
 bool gemm_takes(const turq_weight *w, float *wscale) {
@@ -326,6 +344,36 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
         while (j < count && j - i < 4 && w[j]->dtype == w[i]->dtype) j++;
         // one activation row: a run of a second format joins the launch where the kernel has that pair (q, k Q4_K + v Q6_K)
         static const bool no_mixed = getenv("TURQ_GEMV_NO_MIXED") != nullptr;
+        // 5 .. 16 rows: fragments made in the kernel from the rows themselves (staged through the LDS), a second format in the
+        // same launch where the kernel has the pair
+        {
+            int j2 = j;
+            if (!no_mixed && j < count) {
+                j2 = j + 1;
+                while (j2 < count && w[j2]->dtype == w[j]->dtype) j2++;
+                if (j2 - i > 4) j2 = j;
+            }
+            for (int end = j2; end >= j; end = (end == j ? -1 : j)) {
+                int64_t tiles = 0;
+                for (int t = i; t < end; t++) tiles += turq_tile_rows(w[t]->n);
+                const int dtb = end > j ? w[j]->dtype : w[i]->dtype;
+                const int rg = staged_row_tiles(ctx, w[i]->dtype, dtb, w[i]->k, m, tiles, aligned);
+                if (!rg) continue;
+                const void *wp[4];
+                int64_t nn[4];
+                for (int t = i; t < end; t++) {
+                    wp[t - i] = w[t]->dev;
+                    nn[t - i] = w[t]->n;
+                }
+                hipEvent_t ev0 = nullptr, ev1 = nullptr;
+                TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+                TURQ_HIP(ctx, turq_launch_gemv_cs_staged(w[i]->dtype, dtb, end - i, end > j ? j - i : end - i, wp, nn, w[i]->k, x, xt, ldx, m,
+                                                         y + i, yt, ldy + i, bias ? bias + i : nullptr, rg, ctx->stream, ev0, ev1));
+                i = end;
+                break;
+            }
+            if (i >= j) continue;
+        }
         // (more than two rows: only a call of one format, which would otherwise lose the launch it shares with a second one)
         const bool row1_ok = aligned && !no_fuse && use_row1(w[i]->dtype) && row1_takes(m, all_bytes, w[i]->dtype) &&
                              (m <= 2 || (i == 0 && j == count));
