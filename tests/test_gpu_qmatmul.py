@@ -587,10 +587,11 @@ def test_rows_in_registers_kernel_shapes(row_tiles):
     assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-1000:]
 
 
-# 5 .. 16 rows on a k that splits evenly over the waves go through the form of that kernel that stages the activation rows
-# through the LDS (no preparation launch, no scratch): k = 1024 is two column tiles per wave, k = 4608 six; n = 200 ends inside
-# a row tile and, with several row tiles per workgroup, inside a workgroup.  One format and the two-format launches, every
-# activation type, strides, biases, bf16 output; the rows of a batch are independent, so a batch of 16 equals two of 8.
+# 3 .. 32 rows on a k that splits evenly over the waves go through the form of that kernel that stages the activation rows
+# through the LDS (no preparation launch, no scratch; more than 16 rows as two passes of 16): k = 1024 is two column tiles per
+# wave, k = 4608 six; n = 200 ends inside a row tile and, with several row tiles per workgroup, inside a workgroup.  One format
+# and the two-format launches, every activation type, strides, biases, bf16 output; the rows of a batch are independent, so a
+# batch of 32 equals four of 8.
 @pytest.mark.parametrize("k", [1024, 4608])
 @pytest.mark.parametrize("dts", [(Q4_K,), (Q5_K,), (Q6_K,), (Q8_0,), (Q4_K, Q4_K, Q6_K), (Q5_K, Q6_K, Q6_K), (Q4_K, Q4_K, Q4_K, Q6_K)])
 def test_staged_rows_kernel(dts, k):
@@ -600,8 +601,8 @@ def test_staged_rows_kernel(dts, k):
         raws = [synth.random_weight(dt, n, k, seed=11 * i + n + k) for i, (dt, n) in enumerate(zip(dts, ns))]
         ws = [own.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
         biases = [None if i == 0 else np.random.default_rng(i).standard_normal(n).astype(np.float32) for i, n in enumerate(ns)]
-        x16 = synth.random_activation(16, k, seed=k + len(dts), bf16=True)
-        for m in (5, 8, 9, 16):
+        x16 = synth.random_activation(32, k, seed=k + len(dts), bf16=True)
+        for m in (3, 5, 8, 9, 16, 17, 24, 32):
             x = x16[:m]
             for x_dtype in (capi.ACT_F32, capi.ACT_BF16, capi.ACT_F16):
                 xv = f16_round(x) if x_dtype == capi.ACT_F16 else x
@@ -618,8 +619,9 @@ def test_staged_rows_kernel(dts, k):
             y = own.qmatmul(w, x16, n, k, bias=b, ldx=k + 8, ldy=n + 3)
             want = orc.matmul_dequant(dt, f16_round(x16), raw, n, k) + (0 if b is None else b)
             assert rel_l2(y, want) <= 2e-5
-            y8 = own.qmatmul(w, x16[8:], n, k, bias=b)
-            assert np.array_equal(y8, y[8:])
+            for r0 in (8, 16, 24):
+                y8 = own.qmatmul(w, x16[r0:r0 + 8], n, k, bias=b)
+                assert np.array_equal(y8, y[r0:r0 + 8])
             yb = own.qmatmul(w, x16[:7], n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16)
             assert rel_l2(yb, orc.matmul_dequant(dt, x16[:7], raw, n, k)) <= 4e-3      # bf16 store
         for w in ws:

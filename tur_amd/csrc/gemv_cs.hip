@@ -11,10 +11,9 @@
 // The tile arithmetic is the one of the other skinny kernels (gemv_tileop.h).
 #include <hip/hip_ext.h>
 
-#include <algorithm>
 #include <cstdlib>
 
-#include "gemv_tileop.h"
+#include "gemv_cs_staged.h"
 
 namespace {
 
@@ -94,149 +93,6 @@ __device__ __forceinline__ void cs_body(const uint8_t *__restrict__ w, int64_t n
     }
 }
 
-// ---- the same workgroup with the activations staged through the LDS, written out for a wave that owns exactly CPW column tiles ----
-//
-// Two things hold the loop above back.  (1) A lane that loads exactly its own A-operand slots reads 16 bytes from each of 32
-// different cache lines per instruction (rows are a row stride apart, lane groups 256 bytes), and half of that twice when there
-// are no more than 8 rows: the address unit of the CU works through four to eight times the lines the data needs, the loads of
-// the second wave of every SIMD queue behind those of the first, and for microseconds half of the waves have no activations and
-// request no weights.  (2) The compiler sizes its waits (s_waitcnt vmcnt) for the worst path through the loop's conditions and
-// schedules the header arithmetic of a tile ahead of the tiles before it, so a tile requested D steps ahead is waited for at once.
-//
-// Here a wave loads the rows of its column tile as they lie in memory (one KiB per instruction: a whole f32 row, or two rows of
-// 16-bit values), converts them to f16, writes them to its own few KiB of the LDS and reads its A-operand slots back from there
-// (LDS operations of one wave complete in order: no barrier).  Every load sits in straight-line code, the tiles are kept apart
-// by scheduling barriers, and the next column tile's rows are requested as soon as the current ones have been written to the
-// LDS, one column tile ahead of their use.  Results are those of cs_body bit for bit (same conversions, sums and tile order).
-constexpr int kXRow = 512 + 16;  // bytes per staged activation row: 256 f16 and a pad that spreads the rows over the banks
-
-template <int XT, int MR> struct XRows {
-    uint4v v[XT == TURQ_ACT_F32 ? MR : MR / 2];
-};
-// rows 0 .. MR - 1 (rows past m repeat row m - 1) of column tile b
-template <int XT, int MR>
-__device__ inline XRows<XT, MR> load_x_rows(const void *__restrict__ x, int64_t ldx, int64_t m, int64_t b, int lane) {
-    XRows<XT, MR> raw;
-    if constexpr (XT == TURQ_ACT_F32) {
-#pragma unroll
-        for (int j = 0; j < MR; j++) {
-            const int64_t row = j < m ? j : m - 1;
-            raw.v[j] = *(const uint4v *)((const uint8_t *)x + (row * ldx + b * 256) * 4 + 16 * lane);
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < MR / 2; i++) {
-            const int64_t j = 2 * i + (lane >> 5), row = j < m ? j : m - 1;
-            raw.v[i] = *(const uint4v *)((const uint8_t *)x + (row * ldx + b * 256) * 2 + 16 * (lane & 31));
-        }
-    }
-    return raw;
-}
-// ... as f16 into the wave's LDS rows
-template <int XT, int MR> __device__ inline void stage_x_rows(const XRows<XT, MR> &raw, uint8_t *__restrict__ rows, int lane) {
-    if constexpr (XT == TURQ_ACT_F32) {
-#pragma unroll
-        for (int j = 0; j < MR; j++) {
-            const uint4v a = raw.v[j];
-            const half2v h0 = __builtin_convertvector(float2v{__uint_as_float(a.x), __uint_as_float(a.y)}, half2v);
-            const half2v h1 = __builtin_convertvector(float2v{__uint_as_float(a.z), __uint_as_float(a.w)}, half2v);
-            *(uint2v *)(rows + j * kXRow + 8 * lane) = uint2v{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1)};
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < MR / 2; i++) {
-            uint8_t *p = rows + (2 * i + (lane >> 5)) * kXRow + 16 * (lane & 31);
-            if constexpr (XT == TURQ_ACT_BF16) *(half8v *)p = bf16x8_to_half8(raw.v[i]);
-            else *(uint4v *)p = raw.v[i];
-        }
-    }
-}
-// the A fragments of the staged column tile: lane (r, g) holds row r (rows past m repeat row m - 1);
-// K-quants: step q = columns 64 g + 8 q .. + 7, step 8 = the (hi, lo) sums of its four 16-column groups; Q8_0: step q = columns 32 q + 8 g .. + 7
-template <int DT> __device__ inline void frags_from_staged(const uint8_t *__restrict__ rows, int m, int lane, half8v *__restrict__ out) {
-    const int r = lane & 15, g = lane >> 4;
-    const uint8_t *p = rows + (r < m ? r : m - 1) * kXRow + (DT != TURQ_Q8_0 ? 128 : 16) * g;
-#pragma unroll
-    for (int q = 0; q < 8; q++) out[q] = *(const half8v *)(p + (DT != TURQ_Q8_0 ? 16 : 64) * q);
-    if constexpr (DT != TURQ_Q8_0) out[8] = kq_group_sums(out);
-}
-
-// m <= MR (8 or 16) rows, k a multiple of 256, CPW * (waves of the workgroup) column tiles
-template <int DT, int XT, int MR, int RG, int D, int CPW>
-__device__ __forceinline__ void cs_body_staged(const uint8_t *__restrict__ w, int64_t n, int64_t k, const void *__restrict__ x, int64_t ldx,
-                                               int64_t m, void *__restrict__ y, int yt, int64_t ldy, const float *__restrict__ bias,
-                                               int64_t grp) {
-    constexpr int T = RG * CPW;  // the wave's tiles, column tile by column tile
-    static_assert(D >= 1 && D <= T, "ring of weight tiles");
-    extern __shared__ uint8_t smem[];
-    constexpr int TB = TiledFmt<DT>::kTileBytes;
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int nwaves = blockDim.x >> 6;  // ntc == CPW * nwaves
-    const int64_t ntc = turq_tile_cols(k), nrt = turq_tile_rows(n);
-    const int64_t rt0 = grp * RG;
-    float4v acc[RG];
-    const uint8_t *wrow[RG];  // row tiles past the weight's last one re-read it; their results are not stored
-#pragma unroll
-    for (int r = 0; r < RG; r++) {
-        acc[r] = float4v{0.f, 0.f, 0.f, 0.f};
-        wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
-    }
-    GOff go = lane_offsets(lane, 16);
-    // the first column tile's rows go out first, the first D weight tiles right behind them
-    XRows<XT, MR> raw = load_x_rows<XT, MR>(x, ldx, m, wave, lane);
-    WRegs<DT> wr[D];
-#pragma unroll
-    for (int d = 0; d < D; d++) wr[d] = load_tile<DT>(wrow[d % RG] + (wave + (int64_t)(d / RG) * nwaves) * TB, go);
-    uint8_t *rows = smem + wave * (MR * kXRow);
-    AFrags<DT, 1> f;
-#pragma unroll
-    for (int c = 0; c < CPW; c++) {
-        stage_x_rows<XT, MR>(raw, rows, lane);
-        __builtin_amdgcn_sched_barrier(0);
-        if (c + 1 < CPW) raw = load_x_rows<XT, MR>(x, ldx, m, wave + (int64_t)(c + 1) * nwaves, lane);
-        __builtin_amdgcn_sched_barrier(0);
-        frags_from_staged<DT>(rows, (int)m, lane, f.a[0]);
-#pragma unroll
-        for (int r = 0; r < RG; r++) {
-            const int t = c * RG + r;
-            TileOp<DT, 1, 4>::run(wr[t % D], f, lane, &acc[r]);
-            __builtin_amdgcn_sched_barrier(0);
-            // the slot is free: request the tile D steps ahead
-            if (t + D < T) wr[t % D] = load_tile<DT>(wrow[(t + D) % RG] + (wave + (int64_t)((t + D) / RG) * nwaves) * TB, go);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    // the waves' partial tiles meet in the LDS (over the staged rows, once every wave is done with its own);
-    // wave i adds up the i-th row tile in wave order
-    __syncthreads();
-    float4v *red = (float4v *)smem;
-#pragma unroll
-    for (int r = 0; r < RG; r++) red[(r * nwaves + wave) * 64 + lane] = acc[r];
-    __syncthreads();
-    const int nn = lane & 15, g = lane >> 4;
-    for (int r = wave; r < RG; r += nwaves) {
-        float4v s = red[(r * nwaves) * 64 + lane];
-        for (int wv = 1; wv < nwaves; wv++) s += red[(r * nwaves + wv) * 64 + lane];
-        const int64_t col = (rt0 + r) * 16 + nn;
-        if (rt0 + r >= nrt || col >= n) continue;
-        const float bv = bias ? bias[col] : 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int64_t row = 4 * g + j;
-            if (row < m) turq_store_any(y, yt, row * ldy + col, s[j] + bv);
-        }
-    }
-}
-
-// weights [0, a.second) are of format DTA, the others of DTB (one format: DTA == DTB)
-template <int DTA, int DTB, int XT, int MR, int RG, int D, int CPW>
-__global__ void __launch_bounds__(512) gemv_cs_staged_kernel(MultiArgs a, int64_t k, const void *__restrict__ x, int64_t ldx, int64_t m, int yt) {
-    const MultiPick p = multi_pick(a, (int)blockIdx.x);
-    if (DTA == DTB || p.index < a.second) cs_body_staged<DTA, XT, MR, RG, D, CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
-    else cs_body_staged<DTB, XT, MR, RG, D, CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
-}
-
 template <int DT, int MT, int XT, int RG, int D, int MAXT>
 __global__ void __launch_bounds__(MAXT) gemv_cs_kernel(MultiArgs a, int64_t k, const void *__restrict__ x, int64_t ldx, int64_t m, int yt) {
     const MultiPick p = multi_pick(a, (int)blockIdx.x);
@@ -298,59 +154,6 @@ hipError_t launch_xt(int xt, int rg, const CsLaunch &l) {
     }
 }
 
-// ---- staged form: launch ----
-template <int DTA, int DTB, int XT, int MR, int RG, int D, int CPW>
-hipError_t staged_final(const CsLaunch &l) {
-    const size_t lds = std::max((size_t)l.nwaves * MR * kXRow, (size_t)l.nwaves * RG * 64 * sizeof(float4v));
-    const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
-    if (l.ev0) {
-        hipExtLaunchKernelGGL((gemv_cs_staged_kernel<DTA, DTB, XT, MR, RG, D, CPW>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k,
-                              l.x, l.ldx, l.m, l.yt);
-        return hipGetLastError();
-    }
-    gemv_cs_staged_kernel<DTA, DTB, XT, MR, RG, D, CPW><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
-    return hipGetLastError();
-}
-
-// (row tiles per workgroup, column tiles per wave) -> ring depth
-template <int DTA, int DTB, int XT, int MR>
-hipError_t staged_shape(int rg, int cpw, const CsLaunch &l) {
-    if (cpw == 2) {
-        switch (rg) {
-        case 1: return staged_final<DTA, DTB, XT, MR, 1, 2, 2>(l);
-        case 2: return staged_final<DTA, DTB, XT, MR, 2, 4, 2>(l);
-        case 3: return staged_final<DTA, DTB, XT, MR, 3, 3, 2>(l);
-        case 6: return staged_final<DTA, DTB, XT, MR, 6, 3, 2>(l);
-        }
-    } else if (cpw == 6) {
-        switch (rg) {
-        case 1: return staged_final<DTA, DTB, XT, MR, 1, 3, 6>(l);
-        case 2: return staged_final<DTA, DTB, XT, MR, 2, 3, 6>(l);
-        }
-    }
-    return hipErrorInvalidValue;
-}
-
-template <int DTA, int DTB>
-hipError_t staged_xt(int xt, int rg, int cpw, const CsLaunch &l) {
-    const bool small = l.m <= 8;
-    switch (xt) {
-    case TURQ_ACT_F32: return small ? staged_shape<DTA, DTB, TURQ_ACT_F32, 8>(rg, cpw, l) : staged_shape<DTA, DTB, TURQ_ACT_F32, 16>(rg, cpw, l);
-    case TURQ_ACT_BF16: return small ? staged_shape<DTA, DTB, TURQ_ACT_BF16, 8>(rg, cpw, l) : staged_shape<DTA, DTB, TURQ_ACT_BF16, 16>(rg, cpw, l);
-    case TURQ_ACT_F16: return small ? staged_shape<DTA, DTB, TURQ_ACT_F16, 8>(rg, cpw, l) : staged_shape<DTA, DTB, TURQ_ACT_F16, 16>(rg, cpw, l);
-    default: return hipErrorInvalidValue;
-    }
-}
-
-// column tiles per wave the staged form is built for with this k (0: none): an even split over at most eight waves
-int staged_cpw(int64_t k) {
-    if (k <= 0 || k % 256 != 0) return 0;
-    const int64_t ntc = k / 256;
-    if (ntc % 2 == 0 && ntc / 2 <= 8) return 2;
-    if (ntc % 6 == 0 && ntc / 6 <= 8) return 6;
-    return 0;
-}
-
 }  // namespace
 
 // row tiles per workgroup this kernel is built for
@@ -390,20 +193,28 @@ hipError_t turq_launch_gemv_cs(int dtype, int count, const void *const *w, const
     }
 }
 
-// ---- activations staged through the LDS (m <= 16, k = 512 .. 4096 in steps of 512, or 1536 .. 12288 in steps of 1536) ----
+// ---- activations staged through the LDS (gemv_cs_staged.h; one translation unit per activation type) ----
+// k = 512 .. 4096 in steps of 512, or 1536 .. 12288 in steps of 1536; up to 32 rows
+hipError_t turq_launch_gemv_cs_staged_f32(TURQ_STAGED_LAUNCH_ARGS);
+hipError_t turq_launch_gemv_cs_staged_bf16(TURQ_STAGED_LAUNCH_ARGS);
+hipError_t turq_launch_gemv_cs_staged_f16(TURQ_STAGED_LAUNCH_ARGS);
+
 // whether the staged form has this case: formats (dtype_b = dtype_a for one format, else a K-quant pair with Q6_K second),
 // k, m and row tiles per workgroup
 bool turq_gemv_cs_staged_takes(int dtype_a, int dtype_b, int64_t k, int64_t m, int row_tiles) {
-    const int cpw = staged_cpw(k);
-    if (cpw == 0 || m < 1 || m > 16) return false;
+    const int cpw = turq_gemv_cs_staged_cpw(k);
+    if (cpw == 0 || m < 1 || m > 32) return false;
     if (dtype_a != dtype_b && !((dtype_a == TURQ_Q4_K || dtype_a == TURQ_Q5_K) && dtype_b == TURQ_Q6_K)) return false;
     if (dtype_a != TURQ_Q4_K && dtype_a != TURQ_Q5_K && dtype_a != TURQ_Q6_K && dtype_a != TURQ_Q8_0) return false;
-    return cpw == 2 ? (row_tiles == 1 || row_tiles == 2 || row_tiles == 3 || row_tiles == 6) : (row_tiles == 1 || row_tiles == 2);
+    if (cpw == 6) return row_tiles == 1 || row_tiles == 2;
+    return row_tiles == 1 || row_tiles == 2 || row_tiles == 3 || (row_tiles == 6 && m <= 16);
 }
 
-// count (1..4) tiled weights of one k against m (1..16) activation rows of stride ldx (rows 16-byte aligned); the first `second`
+int turq_gemv_cs_staged_second_rows(int row_tiles) { return staged_second_rows(row_tiles); }
+
+// count (1..4) tiled weights of one k against m (1..32) activation rows of stride ldx (rows 16-byte aligned); the first `second`
 // weights are of format dtype_a, the others of dtype_b (second = count and dtype_b = dtype_a: one format); row_tiles per
-// workgroup as turq_gemv_cs_staged_takes accepts
+// workgroup as turq_gemv_cs_staged_takes accepts (the weights of a second format: turq_gemv_cs_staged_second_rows of it)
 hipError_t turq_launch_gemv_cs_staged(int dtype_a, int dtype_b, int count, int second, const void *const *w, const int64_t *n, int64_t k,
                                       const void *x, int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
                                       const float *const *bias, int row_tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
@@ -411,31 +222,10 @@ hipError_t turq_launch_gemv_cs_staged(int dtype_a, int dtype_b, int count, int s
         !turq_gemv_cs_staged_takes(dtype_a, dtype_b, k, m, row_tiles))
         return hipErrorInvalidValue;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
-    const int cpw = staged_cpw(k);
-    CsLaunch l{};
-    int64_t blocks = 0;
-    for (int i = 0; i < count; i++) {
-        l.a.w[i] = (const uint8_t *)w[i];
-        l.a.y[i] = y[i];
-        l.a.bias[i] = bias ? bias[i] : nullptr;
-        l.a.n[i] = n[i];
-        l.a.ldy[i] = ldy ? ldy[i] : n[i];
-        l.a.first[i] = (int)blocks;
-        blocks += (turq_tile_rows(n[i]) + row_tiles - 1) / row_tiles;
-    }
-    l.a.count = count;
-    l.a.second = second;
-    if (blocks == 0) return hipSuccess;
-    if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
-    l.blocks = (int)blocks, l.k = k, l.x = x, l.ldx = ldx, l.m = m, l.yt = y_dtype, l.nwaves = (int)(k / 256 / cpw);
-    l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop;
-    if (dtype_a == TURQ_Q4_K && dtype_b == TURQ_Q6_K) return staged_xt<TURQ_Q4_K, TURQ_Q6_K>(x_dtype, row_tiles, cpw, l);
-    if (dtype_a == TURQ_Q5_K && dtype_b == TURQ_Q6_K) return staged_xt<TURQ_Q5_K, TURQ_Q6_K>(x_dtype, row_tiles, cpw, l);
-    switch (dtype_a) {
-    case TURQ_Q4_K: return staged_xt<TURQ_Q4_K, TURQ_Q4_K>(x_dtype, row_tiles, cpw, l);
-    case TURQ_Q5_K: return staged_xt<TURQ_Q5_K, TURQ_Q5_K>(x_dtype, row_tiles, cpw, l);
-    case TURQ_Q6_K: return staged_xt<TURQ_Q6_K, TURQ_Q6_K>(x_dtype, row_tiles, cpw, l);
-    case TURQ_Q8_0: return staged_xt<TURQ_Q8_0, TURQ_Q8_0>(x_dtype, row_tiles, cpw, l);
+    switch (x_dtype) {
+    case TURQ_ACT_F32: return turq_launch_gemv_cs_staged_f32(TURQ_STAGED_LAUNCH_PASS);
+    case TURQ_ACT_BF16: return turq_launch_gemv_cs_staged_bf16(TURQ_STAGED_LAUNCH_PASS);
+    case TURQ_ACT_F16: return turq_launch_gemv_cs_staged_f16(TURQ_STAGED_LAUNCH_PASS);
     default: return hipErrorInvalidValue;
     }
 }

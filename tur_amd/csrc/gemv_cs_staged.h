@@ -1,0 +1,299 @@
+// The skinny kernel that splits the columns over the waves of a workgroup, in the form that stages the activation rows through
+// the LDS (see gemv_cs.hip for the decomposition).  One translation unit per activation type instantiates it (the written-out
+// kernels are many and large), each through staged_launch<XT>.
+#pragma once
+
+#include <hip/hip_ext.h>
+
+#include <algorithm>
+
+#include "gemv_tileop.h"
+
+namespace {
+
+// ---- a workgroup owns RG row tiles and all columns; written out for a wave that owns exactly CPW column tiles ----
+//
+// Against a loop whose lanes load their own A-operand slots from the caller's rows (gemv_cs.hip):
+// Two things hold the loop above back.  (1) A lane that loads exactly its own A-operand slots reads 16 bytes from each of 32
+// different cache lines per instruction (rows are a row stride apart, lane groups 256 bytes), and half of that twice when there
+// are no more than 8 rows: the address unit of the CU works through four to eight times the lines the data needs, the loads of
+// the second wave of every SIMD queue behind those of the first, and for microseconds half of the waves have no activations and
+// request no weights.  (2) The compiler sizes its waits (s_waitcnt vmcnt) for the worst path through the loop's conditions and
+// schedules the header arithmetic of a tile ahead of the tiles before it, so a tile requested D steps ahead is waited for at once.
+//
+// Here a wave loads the rows of its column tile as they lie in memory (one KiB per instruction: a whole f32 row, or two rows of
+// 16-bit values), converts them to f16, writes them to its own few KiB of the LDS and reads its A-operand slots back from there
+// (LDS operations of one wave complete in order: no barrier).  Every load sits in straight-line code, the tiles are kept apart
+// by scheduling barriers, and the next column tile's rows are requested as soon as the current ones have been written to the
+// LDS, one column tile ahead of their use.  Results are those of cs_body bit for bit (same conversions, sums and tile order).
+constexpr int kXRow = 512 + 16;  // bytes per staged activation row: 256 f16 and a pad that spreads the rows over the banks
+
+template <int XT, int MR> struct XRows {
+    uint4v v[XT == TURQ_ACT_F32 ? MR : MR / 2];
+};
+// rows row0 .. row0 + MR - 1 (rows past m repeat row m - 1) of column tile b
+template <int XT, int MR>
+__device__ inline XRows<XT, MR> load_x_rows(const void *__restrict__ x, int64_t ldx, int64_t m, int row0, int64_t b, int lane) {
+    XRows<XT, MR> raw;
+    if constexpr (XT == TURQ_ACT_F32) {
+#pragma unroll
+        for (int j = 0; j < MR; j++) {
+            const int64_t row = row0 + j < m ? row0 + j : m - 1;
+            raw.v[j] = *(const uint4v *)((const uint8_t *)x + (row * ldx + b * 256) * 4 + 16 * lane);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < MR / 2; i++) {
+            const int64_t j = row0 + 2 * i + (lane >> 5), row = j < m ? j : m - 1;
+            raw.v[i] = *(const uint4v *)((const uint8_t *)x + (row * ldx + b * 256) * 2 + 16 * (lane & 31));
+        }
+    }
+    return raw;
+}
+// ... as f16 into the wave's LDS rows
+template <int XT, int MR> __device__ inline void stage_x_rows(const XRows<XT, MR> &raw, uint8_t *__restrict__ rows, int lane) {
+    if constexpr (XT == TURQ_ACT_F32) {
+#pragma unroll
+        for (int j = 0; j < MR; j++) {
+            const uint4v a = raw.v[j];
+            const half2v h0 = __builtin_convertvector(float2v{__uint_as_float(a.x), __uint_as_float(a.y)}, half2v);
+            const half2v h1 = __builtin_convertvector(float2v{__uint_as_float(a.z), __uint_as_float(a.w)}, half2v);
+            *(uint2v *)(rows + j * kXRow + 8 * lane) = uint2v{__builtin_bit_cast(uint32_t, h0), __builtin_bit_cast(uint32_t, h1)};
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < MR / 2; i++) {
+            uint8_t *p = rows + (2 * i + (lane >> 5)) * kXRow + 16 * (lane & 31);
+            if constexpr (XT == TURQ_ACT_BF16) *(half8v *)p = bf16x8_to_half8(raw.v[i]);
+            else *(uint4v *)p = raw.v[i];
+        }
+    }
+}
+// the A fragments of the staged column tile: lane (r, g) holds row r (rows past m repeat row m - 1);
+// K-quants: step q = columns 64 g + 8 q .. + 7, step 8 = the (hi, lo) sums of its four 16-column groups; Q8_0: step q = columns 32 q + 8 g .. + 7
+template <int DT> __device__ inline void frags_from_staged(const uint8_t *__restrict__ rows, int m, int lane, half8v *__restrict__ out) {
+    const int r = lane & 15, g = lane >> 4;
+    const uint8_t *p = rows + (r < m ? r : m - 1) * kXRow + (DT != TURQ_Q8_0 ? 128 : 16) * g;
+#pragma unroll
+    for (int q = 0; q < 8; q++) out[q] = *(const half8v *)(p + (DT != TURQ_Q8_0 ? 16 : 64) * q);
+    if constexpr (DT != TURQ_Q8_0) out[8] = kq_group_sums(out);
+}
+
+// m <= MR rows (8, 16 or 32), k a multiple of 256, CPW * (waves of the workgroup) column tiles.  More than 16 rows are taken as
+// two halves of 16, one after the other against the same weight tiles (HV = 2): the tiles of a column tile stay in their
+// registers for both passes and are unpacked once per pass, which for these launches costs less than what holding the
+// fragments of 32 rows next to the rows in flight would (registers), or a launch that prepares them.
+template <int DT, int XT, int MR, int RG, int D, int CPW>
+__device__ __forceinline__ void cs_body_staged(const uint8_t *__restrict__ w, int64_t n, int64_t k, const void *__restrict__ x, int64_t ldx,
+                                               int64_t m, void *__restrict__ y, int yt, int64_t ldy, const float *__restrict__ bias,
+                                               int64_t grp) {
+    constexpr int HV = MR > 16 ? 2 : 1;  // passes of HR rows each
+    constexpr int HR = MR / HV;
+    constexpr int T = RG * CPW;          // the wave's tiles, column tile by column tile
+    static_assert(D >= 1 && D <= T && (HV == 1 || D >= RG), "ring of weight tiles: a column tile's tiles stay for both passes");
+    extern __shared__ uint8_t smem[];
+    constexpr int TB = TiledFmt<DT>::kTileBytes;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nwaves = blockDim.x >> 6;  // ntc == CPW * nwaves
+    const int64_t ntc = turq_tile_cols(k), nrt = turq_tile_rows(n);
+    const int64_t rt0 = grp * RG;
+    float4v acc[RG][HV];
+    const uint8_t *wrow[RG];  // row tiles past the weight's last one re-read it; their results are not stored
+#pragma unroll
+    for (int r = 0; r < RG; r++) {
+#pragma unroll
+        for (int h = 0; h < HV; h++) acc[r][h] = float4v{0.f, 0.f, 0.f, 0.f};
+        wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+    }
+    GOff go = lane_offsets(lane, 16);
+    // the first column tile's rows go out first, the first D weight tiles right behind them
+    XRows<XT, HR> raw = load_x_rows<XT, HR>(x, ldx, m, 0, wave, lane);
+    WRegs<DT> wr[D];
+#pragma unroll
+    for (int d = 0; d < D; d++) wr[d] = load_tile<DT>(wrow[d % RG] + (wave + (int64_t)(d / RG) * nwaves) * TB, go);
+    uint8_t *rows = smem + wave * (HR * kXRow);
+    AFrags<DT, 1> f;
+#pragma unroll
+    for (int c = 0; c < CPW; c++) {
+#pragma unroll
+        for (int h = 0; h < HV; h++) {
+            stage_x_rows<XT, HR>(raw, rows, lane);
+            __builtin_amdgcn_sched_barrier(0);
+            // the rows of the next pass: the other half of this column tile, or the next column tile
+            if (h + 1 < HV) raw = load_x_rows<XT, HR>(x, ldx, m, HR * (h + 1), wave + (int64_t)c * nwaves, lane);
+            else if (c + 1 < CPW) raw = load_x_rows<XT, HR>(x, ldx, m, 0, wave + (int64_t)(c + 1) * nwaves, lane);
+            __builtin_amdgcn_sched_barrier(0);
+            frags_from_staged<DT>(rows, (int)m - HR * h, lane, f.a[0]);
+#pragma unroll
+            for (int r = 0; r < RG; r++) {
+                const int t = c * RG + r;
+                // (second pass: unpacked again; what the compiler would keep of the first pass's operands does not fit the
+                // registers of more than one row tile)
+                if constexpr (RG > 1) {
+                    if (h > 0) touch(wr[t % D]);
+                }
+                TileOp<DT, 1, 4>::run(wr[t % D], f, lane, &acc[r][h]);
+                __builtin_amdgcn_sched_barrier(0);
+                // after the last pass the slot is free: request the tile D steps ahead
+                if (h == HV - 1 && t + D < T) wr[t % D] = load_tile<DT>(wrow[(t + D) % RG] + (wave + (int64_t)((t + D) / RG) * nwaves) * TB, go);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+    // the waves' partial tiles meet in the LDS (over the staged rows, once every wave is done with its own);
+    // wave i adds up the i-th (row tile, pass) pair in wave order
+    __syncthreads();
+    float4v *red = (float4v *)smem;
+#pragma unroll
+    for (int r = 0; r < RG; r++)
+#pragma unroll
+        for (int h = 0; h < HV; h++) red[((r * HV + h) * nwaves + wave) * 64 + lane] = acc[r][h];
+    __syncthreads();
+    const int nn = lane & 15, g = lane >> 4;
+    for (int i = wave; i < RG * HV; i += nwaves) {
+        const int r = i / HV, h = i - r * HV;
+        float4v s = red[(i * nwaves) * 64 + lane];
+        for (int wv = 1; wv < nwaves; wv++) s += red[(i * nwaves + wv) * 64 + lane];
+        const int64_t col = (rt0 + r) * 16 + nn;
+        if (rt0 + r >= nrt || col >= n) continue;
+        const float bv = bias ? bias[col] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int64_t row = HR * h + 4 * g + j;
+            if (row < m) turq_store_any(y, yt, row * ldy + col, s[j] + bv);
+        }
+    }
+}
+
+// weight tiles in flight per wave for RG row tiles per workgroup and CPW column tiles per wave (measured on 4096- and 12288-column
+// weights: a deeper ring delays the activation rows behind it); with two passes per tile just a column tile's tiles (a slot is
+// requested again a whole pass before its next use; more does not fit the registers next to 16 f32 rows in flight)
+constexpr int staged_ring(int rg, int cpw, int mr) {
+    if (mr > 16) return rg > 1 ? rg : cpw < 3 ? cpw : 3;
+    return rg * cpw <= 2 ? rg * cpw : (rg == 2 && cpw == 2) ? 4 : 3;
+}
+// row tiles per workgroup for the weights of the second format of a two-format launch: Q6_K tiles behind Q4_K / Q5_K ones are
+// half as large again and cost half as much arithmetic again, so their workgroups take fewer of them
+constexpr int staged_second_rows(int rg) { return (rg + 1) / 2; }
+
+// weights [0, a.second) are of format DTA with RG row tiles per workgroup, the others of DTB with staged_second_rows(RG)
+// (one format: DTA == DTB)
+template <int DTA, int DTB, int XT, int MR, int RG, int CPW>
+__global__ void __launch_bounds__(512) gemv_cs_staged_kernel(MultiArgs a, int64_t k, const void *__restrict__ x, int64_t ldx, int64_t m, int yt) {
+    const MultiPick p = multi_pick(a, (int)blockIdx.x);
+    constexpr int RGB = staged_second_rows(RG);
+    if (DTA == DTB || p.index < a.second)
+        cs_body_staged<DTA, XT, MR, RG, staged_ring(RG, CPW, MR), CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
+    else
+        cs_body_staged<DTB, XT, MR, RGB, staged_ring(RGB, CPW, MR), CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
+}
+
+struct StagedLaunch {
+    MultiArgs a;
+    int blocks;
+    int64_t k;
+    const void *x;
+    int64_t ldx, m;
+    int yt, nwaves;
+    hipStream_t s;
+    hipEvent_t ev0, ev1;
+};
+
+template <int DTA, int DTB, int XT, int MR, int RG, int CPW>
+hipError_t staged_final(const StagedLaunch &l) {
+    constexpr int HV = MR > 16 ? 2 : 1;
+    const size_t lds = std::max((size_t)l.nwaves * (MR / HV) * kXRow, (size_t)l.nwaves * RG * HV * 64 * sizeof(float4v));
+    if (lds > (64u << 10)) {
+        static const hipError_t raised = hipFuncSetAttribute((const void *)gemv_cs_staged_kernel<DTA, DTB, XT, MR, RG, CPW>,
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10);
+        if (raised != hipSuccess) return raised;
+    }
+    const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
+    if (l.ev0) {
+        hipExtLaunchKernelGGL((gemv_cs_staged_kernel<DTA, DTB, XT, MR, RG, CPW>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k, l.x,
+                              l.ldx, l.m, l.yt);
+        return hipGetLastError();
+    }
+    gemv_cs_staged_kernel<DTA, DTB, XT, MR, RG, CPW><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
+    return hipGetLastError();
+}
+
+template <int DTA, int DTB, int XT, int MR>
+hipError_t staged_shape(int rg, int cpw, const StagedLaunch &l) {
+    if (cpw == 2) {
+        switch (rg) {
+        case 1: return staged_final<DTA, DTB, XT, MR, 1, 2>(l);
+        case 2: return staged_final<DTA, DTB, XT, MR, 2, 2>(l);
+        case 3: return staged_final<DTA, DTB, XT, MR, 3, 2>(l);
+        case 6:
+            if constexpr (MR <= 16) return staged_final<DTA, DTB, XT, MR, 6, 2>(l);
+            break;
+        }
+    } else if (cpw == 6) {
+        switch (rg) {
+        case 1: return staged_final<DTA, DTB, XT, MR, 1, 6>(l);
+        case 2: return staged_final<DTA, DTB, XT, MR, 2, 6>(l);
+        }
+    }
+    return hipErrorInvalidValue;
+}
+
+template <int DTA, int DTB, int XT>
+hipError_t staged_rows(int rg, int cpw, const StagedLaunch &l) {
+    if (l.m <= 8) return staged_shape<DTA, DTB, XT, 8>(rg, cpw, l);
+    if (l.m <= 16) return staged_shape<DTA, DTB, XT, 16>(rg, cpw, l);
+    return staged_shape<DTA, DTB, XT, 32>(rg, cpw, l);
+}
+
+}  // namespace
+
+// column tiles per wave the staged form is built for with this k (0: none): an even split over at most eight waves
+inline int turq_gemv_cs_staged_cpw(int64_t k) {
+    if (k <= 0 || k % 256 != 0) return 0;
+    const int64_t ntc = k / 256;
+    if (ntc % 2 == 0 && ntc / 2 <= 8) return 2;
+    if (ntc % 6 == 0 && ntc / 6 <= 8) return 6;
+    return 0;
+}
+
+// the launch for activations of type XT; arguments as turq_launch_gemv_cs_staged, which has checked them
+template <int XT>
+hipError_t staged_launch(int dtype_a, int dtype_b, int count, int second, const void *const *w, const int64_t *n, int64_t k, const void *x,
+                         int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy, const float *const *bias, int row_tiles,
+                         hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+    const int cpw = turq_gemv_cs_staged_cpw(k);
+    StagedLaunch l{};
+    int64_t blocks = 0;
+    for (int i = 0; i < count; i++) {
+        l.a.w[i] = (const uint8_t *)w[i];
+        l.a.y[i] = y[i];
+        l.a.bias[i] = bias ? bias[i] : nullptr;
+        l.a.n[i] = n[i];
+        l.a.ldy[i] = ldy ? ldy[i] : n[i];
+        l.a.first[i] = (int)blocks;
+        const int rt = i < second ? row_tiles : staged_second_rows(row_tiles);
+        blocks += (turq_tile_rows(n[i]) + rt - 1) / rt;
+    }
+    l.a.count = count;
+    l.a.second = second;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    l.blocks = (int)blocks, l.k = k, l.x = x, l.ldx = ldx, l.m = m, l.yt = y_dtype, l.nwaves = (int)(k / 256 / cpw);
+    l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop;
+    if (dtype_a == TURQ_Q4_K && dtype_b == TURQ_Q6_K) return staged_rows<TURQ_Q4_K, TURQ_Q6_K, XT>(row_tiles, cpw, l);
+    if (dtype_a == TURQ_Q5_K && dtype_b == TURQ_Q6_K) return staged_rows<TURQ_Q5_K, TURQ_Q6_K, XT>(row_tiles, cpw, l);
+    switch (dtype_a) {
+    case TURQ_Q4_K: return staged_rows<TURQ_Q4_K, TURQ_Q4_K, XT>(row_tiles, cpw, l);
+    case TURQ_Q5_K: return staged_rows<TURQ_Q5_K, TURQ_Q5_K, XT>(row_tiles, cpw, l);
+    case TURQ_Q6_K: return staged_rows<TURQ_Q6_K, TURQ_Q6_K, XT>(row_tiles, cpw, l);
+    case TURQ_Q8_0: return staged_rows<TURQ_Q8_0, TURQ_Q8_0, XT>(row_tiles, cpw, l);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+#define TURQ_STAGED_LAUNCH_ARGS                                                                                                          \
+    int dtype_a, int dtype_b, int count, int second, const void *const *w, const int64_t *n, int64_t k, const void *x, int64_t ldx,      \
+        int64_t m, void *const *y, int y_dtype, const int64_t *ldy, const float *const *bias, int row_tiles, hipStream_t stream,         \
+        hipEvent_t ev_start, hipEvent_t ev_stop
+#define TURQ_STAGED_LAUNCH_PASS dtype_a, dtype_b, count, second, w, n, k, x, ldx, m, y, y_dtype, ldy, bias, row_tiles, stream, ev_start, ev_stop

@@ -1,0 +1,4 @@
+// The staged form of the column-splitting skinny kernel for bf16 activations (gemv_cs_staged.h).
+#include "gemv_cs_staged.h"
+
+hipError_t turq_launch_gemv_cs_staged_bf16(TURQ_STAGED_LAUNCH_ARGS) { return staged_launch<TURQ_ACT_BF16>(TURQ_STAGED_LAUNCH_PASS); }

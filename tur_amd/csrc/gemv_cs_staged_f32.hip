@@ -1,0 +1,4 @@
+// The staged form of the column-splitting skinny kernel for f32 activations (gemv_cs_staged.h).
+#include "gemv_cs_staged.h"
+
+hipError_t turq_launch_gemv_cs_staged_f32(TURQ_STAGED_LAUNCH_ARGS) { return staged_launch<TURQ_ACT_F32>(TURQ_STAGED_LAUNCH_PASS); }

@@ -71,6 +71,18 @@ template <> __device__ inline WRegs<TURQ_Q8_0> load_tile<TURQ_Q8_0>(const uint8_
     w.dd = *(const uint4v *)(tile + F::kD + o.hdr);
     return w;
 }
+// makes the registers of a tile new values for the compiler (no instruction): what it derived from them before is not kept
+__device__ inline void touch(uint4v &v) { asm volatile("" : "+v"(v)); }
+__device__ inline void touch(uint2v &v) { asm volatile("" : "+v"(v)); }
+__device__ inline void touch(uint32_t &v) { asm volatile("" : "+v"(v)); }
+__device__ inline void touch(WRegs<TURQ_Q4_K> &w) { touch(w.qa), touch(w.qb), touch(w.hd); }
+__device__ inline void touch(WRegs<TURQ_Q5_K> &w) { touch(w.qa), touch(w.qb), touch(w.hd), touch(w.hh); }
+__device__ inline void touch(WRegs<TURQ_Q6_K> &w) { touch(w.qla), touch(w.qlb), touch(w.qh), touch(w.scw), touch(w.d16); }
+__device__ inline void touch(WRegs<TURQ_Q8_0> &w) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) touch(w.p[i]);
+    touch(w.dd);
+}
 __device__ inline GOff lane_offsets(int lane, int mpad) {
     const uint32_t l = (uint32_t)lane, r = l & 15u;
     return GOff{16u * l, 8u * l, 4u * l, 16u * r, 2u * r, 16u * ((l >> 4) * (uint32_t)mpad + (r & (uint32_t)(mpad - 1)))};

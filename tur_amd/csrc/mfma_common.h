@@ -175,6 +175,7 @@ hipError_t turq_launch_gemv_cs(int dtype, int count, const void *const *w_tiled,
                                int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy, const float *const *bias,
                                int nwaves, int row_tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
 bool turq_gemv_cs_staged_takes(int dtype_a, int dtype_b, int64_t k, int64_t m, int row_tiles);
+int turq_gemv_cs_staged_second_rows(int row_tiles);
 hipError_t turq_launch_gemv_cs_staged(int dtype_a, int dtype_b, int count, int second, const void *const *w_tiled, const int64_t *n,
                                       int64_t k, const void *x, int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype,
                                       const int64_t *ldy, const float *const *bias, int row_tiles, hipStream_t stream,

@@ -97,15 +97,26 @@ int cs_row_tiles(const turq_ctx *ctx, int64_t m, int64_t row_tiles, int dtype, b
 // pays for small launches, where it replaces a preparation launch and a kernel that re-reads prepared fragments: row tiles per
 // workgroup so that the launch is about one workgroup per compute unit.  0: not this call.  TURQ_CS_STAGED = 0 switches it off,
 // TURQ_CS_RG forces the group size.
-int staged_row_tiles(const turq_ctx *ctx, int dtype_a, int dtype_b, int64_t k, int64_t m, int64_t row_tiles, bool aligned) {
+int staged_row_tiles(const turq_ctx *ctx, int dtype_a, int dtype_b, int64_t k, int64_t m, int64_t row_tiles, int64_t row_tiles_b,
+                     bool aligned) {
     static const int mode = [] { const char *e = getenv("TURQ_CS_STAGED"); return e ? atoi(e) : -1; }();
     static const int forced = [] { const char *e = getenv("TURQ_CS_RG"); return e ? atoi(e) : 0; }();
-    static const int min_m = [] { const char *e = getenv("TURQ_CS_STAGED_MIN_M"); return e ? atoi(e) : 5; }();
-    if (mode == 0 || !aligned || m < min_m || m > 16) return 0;
+    static const int min_m = [] { const char *e = getenv("TURQ_CS_STAGED_MIN_M"); return e ? atoi(e) : 3; }();
+    static const int max_m = [] { const char *e = getenv("TURQ_CS_STAGED_MAX_M"); return e ? atoi(e) : 32; }();
+    if (mode == 0 || !aligned || m < min_m || m > max_m || m > TURQ_GEMV_MAX_M) return 0;
     const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
     if (row_tiles > 12 * cus && !forced) return 0;  // many rounds of workgroups (an LM head): the prepared fragments do better
+    // the smallest group with which the launch is one round of workgroups (the weights of a second format go out in smaller
+    // groups); beyond three row tiles per unit, two rounds of 2 or 3 or groups of 6
     const int64_t per = (row_tiles + cus - 1) / cus;
-    int rg = per <= 3 ? (int)per : per == 4 ? 2 : per == 5 ? 3 : 6;
+    int rg = per == 4 ? 2 : per == 5 ? 3 : 6;
+    for (int g = 3; g >= 1; g--) {
+        const int gb = turq_gemv_cs_staged_second_rows(g);
+        if ((row_tiles - row_tiles_b + g - 1) / g + (row_tiles_b + gb - 1) / gb <= cus) rg = g;
+    }
+    // more than 16 rows (two passes per weight tile, each unpacking it): pays on launches of up to two row tiles per unit of
+    // weights with few columns, where the preparation launch is a third of the time; larger ones are better off with it
+    if (m > 16 && !forced && (rg > 2 || row_tiles > 2 * cus || k > 4096)) return 0;
     if (forced) rg = forced;
     while (rg > 1 && !turq_gemv_cs_staged_takes(dtype_a, dtype_b, k, m, rg)) rg = rg == 6 ? 3 : rg - 1;
     return turq_gemv_cs_staged_takes(dtype_a, dtype_b, k, m, rg) ? rg : 0;
@@ -354,10 +365,11 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
                 if (j2 - i > 4) j2 = j;
             }
             for (int end = j2; end >= j; end = (end == j ? -1 : j)) {
-                int64_t tiles = 0;
+                int64_t tiles = 0, tiles_b = 0;
                 for (int t = i; t < end; t++) tiles += turq_tile_rows(w[t]->n);
+                for (int t = j; t < end; t++) tiles_b += turq_tile_rows(w[t]->n);
                 const int dtb = end > j ? w[j]->dtype : w[i]->dtype;
-                const int rg = staged_row_tiles(ctx, w[i]->dtype, dtb, w[i]->k, m, tiles, aligned);
+                const int rg = staged_row_tiles(ctx, w[i]->dtype, dtb, w[i]->k, m, tiles, tiles_b, aligned);
                 if (!rg) continue;
                 const void *wp[4];
                 int64_t nn[4];
