@@ -139,15 +139,15 @@ def scratch_info(gpu):
 
 
 def test_scratch_that_grows_under_a_live_graph_is_kept_for_it():
-    # a graph captured at m = 20 refers to the fragment buffer by address; a later, larger eager call (m = 32 on a wider
+    # a graph captured at m = 40 refers to the fragment buffer by address; a later, larger eager call (m = 64 on a wider
     # matrix) makes that buffer grow.  The old buffer must stay allocated while the graph is alive (the replay below then
     # reads and writes valid memory and gives the eager result again), and is released once no graph is alive.
     gpu = Gpu()                           # a context of its own: the bookkeeping starts from zero
     L, ctx = gpu.L, gpu.ctx
-    st = Step(gpu, 20)                    # more than 16 rows: the kernels read fragments prepared in the context's scratch
-    big = Step(gpu, 32, k=4096)
+    st = Step(gpu, 40)                    # more than 32 rows: the kernels read fragments prepared in the context's scratch
+    big = Step(gpu, 64, k=4096)
     try:
-        x = synth.random_activation(20, st.k, seed=5)
+        x = synth.random_activation(40, st.k, seed=5)
         st.set_x(x)
         st.calls()
         want = st.outputs()
@@ -158,7 +158,7 @@ def test_scratch_that_grows_under_a_live_graph_is_kept_for_it():
         g = ctypes.c_void_p()
         capi.check(L.turq_graph_end(ctx, ctypes.byref(g)), ctx)
         assert scratch_info(gpu)[:2] == (1, 0)
-        big.set_x(synth.random_activation(32, big.k, seed=6))
+        big.set_x(synth.random_activation(64, big.k, seed=6))
         big.calls()                       # needs more scratch than the capture left behind
         big.outputs()
         live, retired, cap1 = scratch_info(gpu)
@@ -171,9 +171,9 @@ def test_scratch_that_grows_under_a_live_graph_is_kept_for_it():
                 assert np.array_equal(y, w)
         L.turq_graph_destroy(g)
         assert scratch_info(gpu)[0] == 0
-        huge = Step(gpu, 32, k=8192)      # the next growth finds no live graph and lets the retired buffer go
+        huge = Step(gpu, 128, k=8192)      # the next growth finds no live graph and lets the retired buffer go
         try:
-            huge.set_x(synth.random_activation(32, huge.k, seed=7))
+            huge.set_x(synth.random_activation(128, huge.k, seed=7))
             huge.calls()
             huge.outputs()
             assert scratch_info(gpu)[:2] == (0, 0)
@@ -188,13 +188,13 @@ def test_scratch_that_grows_under_a_live_graph_is_kept_for_it():
 def test_a_call_that_fails_inside_a_capture_ends_it():
     gpu = Gpu()
     L, ctx = gpu.L, gpu.ctx
-    st = Step(gpu, 20)
+    st = Step(gpu, 40)
     try:
-        x = synth.random_activation(20, st.k, seed=8)
+        x = synth.random_activation(40, st.k, seed=8)
         st.set_x(x)
         capi.check(L.turq_graph_begin(ctx), ctx)
         # first use of the fragment buffer inside a capture: it would have to be allocated, which a capture does not allow
-        rc = L.turq_qmatmul_multi(ctx, 3, st.warr, st.x, capi.ACT_F32, 20, st.k, st.yarr, capi.ACT_F32, st.ldys, None,
+        rc = L.turq_qmatmul_multi(ctx, 3, st.warr, st.x, capi.ACT_F32, 40, st.k, st.yarr, capi.ACT_F32, st.ldys, None,
                                   capi.MEM_DEVICE, capi.ALGO_AUTO)
         assert rc == capi.ERR_INVALID
         assert "capture" in capi.last_error(ctx)

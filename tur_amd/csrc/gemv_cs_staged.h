@@ -83,10 +83,15 @@ template <int DT> __device__ inline void frags_from_staged(const uint8_t *__rest
 // two halves of 16, one after the other against the same weight tiles (HV = 2): the tiles of a column tile stay in their
 // registers for both passes and are unpacked once per pass, which for these launches costs less than what holding the
 // fragments of 32 rows next to the rows in flight would (registers), or a launch that prepares them.
-template <int DT, int XT, int MR, int RG, int D, int CPW>
+// GU: the workgroup's row tiles are RG / 2 of a gate weight (w) and the same RG / 2 of an up weight (w2) of one shape, and what
+// is stored is silu(gate) * up (src/models/qwen3.rs:161-167).
+template <int DT, int XT, int MR, int RG, int D, int CPW, bool GU = false>
 __device__ __forceinline__ void cs_body_staged(const uint8_t *__restrict__ w, int64_t n, int64_t k, const void *__restrict__ x, int64_t ldx,
                                                int64_t m, void *__restrict__ y, int yt, int64_t ldy, const float *__restrict__ bias,
-                                               int64_t grp) {
+                                               int64_t grp, const uint8_t *__restrict__ w2 = nullptr,
+                                               const float *__restrict__ bias2 = nullptr) {
+    static_assert(!GU || RG % 2 == 0, "gate and up tiles come in pairs");
+    constexpr int RO = GU ? RG / 2 : RG;  // row tiles of the output per workgroup
     constexpr int HV = MR > 16 ? 2 : 1;  // passes of HR rows each
     constexpr int HR = MR / HV;
     constexpr int T = RG * CPW;          // the wave's tiles, column tile by column tile
@@ -97,14 +102,15 @@ __device__ __forceinline__ void cs_body_staged(const uint8_t *__restrict__ w, in
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nwaves = blockDim.x >> 6;  // ntc == CPW * nwaves
     const int64_t ntc = turq_tile_cols(k), nrt = turq_tile_rows(n);
-    const int64_t rt0 = grp * RG;
+    const int64_t rt0 = grp * RO;
     float4v acc[RG][HV];
     const uint8_t *wrow[RG];  // row tiles past the weight's last one re-read it; their results are not stored
 #pragma unroll
     for (int r = 0; r < RG; r++) {
 #pragma unroll
         for (int h = 0; h < HV; h++) acc[r][h] = float4v{0.f, 0.f, 0.f, 0.f};
-        wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+        const int ro = r < RO ? r : r - RO;
+        wrow[r] = (r < RO ? w : w2) + (rt0 + ro < nrt ? rt0 + ro : nrt - 1) * ntc * TB;
     }
     GOff go = lane_offsets(lane, 16);
     // the first column tile's rows go out first, the first D weight tiles right behind them
@@ -151,17 +157,29 @@ __device__ __forceinline__ void cs_body_staged(const uint8_t *__restrict__ w, in
         for (int h = 0; h < HV; h++) red[((r * HV + h) * nwaves + wave) * 64 + lane] = acc[r][h];
     __syncthreads();
     const int nn = lane & 15, g = lane >> 4;
-    for (int i = wave; i < RG * HV; i += nwaves) {
+    for (int i = wave; i < RO * HV; i += nwaves) {
         const int r = i / HV, h = i - r * HV;
         float4v s = red[(i * nwaves) * 64 + lane];
         for (int wv = 1; wv < nwaves; wv++) s += red[(i * nwaves + wv) * 64 + lane];
+        float4v s2 = float4v{0.f, 0.f, 0.f, 0.f};
+        if constexpr (GU) {
+            const int i2 = i + RO * HV;  // the up tile of the pair
+            s2 = red[(i2 * nwaves) * 64 + lane];
+            for (int wv = 1; wv < nwaves; wv++) s2 += red[(i2 * nwaves + wv) * 64 + lane];
+        }
         const int64_t col = (rt0 + r) * 16 + nn;
         if (rt0 + r >= nrt || col >= n) continue;
-        const float bv = bias ? bias[col] : 0.0f;
+        const float bv = bias ? bias[col] : 0.0f, bv2 = (GU && bias2) ? bias2[col] : 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int64_t row = HR * h + 4 * g + j;
-            if (row < m) turq_store_any(y, yt, row * ldy + col, s[j] + bv);
+            if (row >= m) continue;
+            if constexpr (GU) {
+                const float gate = s[j] + bv, up = s2[j] + bv2;
+                turq_store_any(y, yt, row * ldy + col, gate / (1.0f + expf(-gate)) * up);
+            } else {
+                turq_store_any(y, yt, row * ldy + col, s[j] + bv);
+            }
         }
     }
 }
@@ -187,6 +205,14 @@ __global__ void __launch_bounds__(512) gemv_cs_staged_kernel(MultiArgs a, int64_
         cs_body_staged<DTA, XT, MR, RG, staged_ring(RG, CPW, MR), CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
     else
         cs_body_staged<DTB, XT, MR, RGB, staged_ring(RGB, CPW, MR), CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
+}
+
+// gate (a.w[0]) and up (a.w[1]) of one MLP, RG / 2 row tiles of each per workgroup, silu(gate) * up stored to a.y[0]
+template <int DT, int XT, int MR, int RG, int CPW>
+__global__ void __launch_bounds__(512) gemv_cs_staged_gateup_kernel(MultiArgs a, int64_t k, const void *__restrict__ x, int64_t ldx, int64_t m,
+                                                                     int yt) {
+    cs_body_staged<DT, XT, MR, RG, staged_ring(RG, CPW, MR), CPW, true>(a.w[0], a.n[0], k, x, ldx, m, a.y[0], yt, a.ldy[0], a.bias[0],
+                                                                         (int64_t)blockIdx.x, a.w[1], a.bias[1]);
 }
 
 struct StagedLaunch {
@@ -236,6 +262,33 @@ hipError_t staged_shape(int rg, int cpw, const StagedLaunch &l) {
         case 2: return staged_final<DTA, DTB, XT, MR, 2, 6>(l);
         }
     }
+    return hipErrorInvalidValue;
+}
+
+template <int DT, int XT, int MR, int RG, int CPW>
+hipError_t staged_gateup_final(const StagedLaunch &l) {
+    const size_t lds = std::max((size_t)l.nwaves * MR * kXRow, (size_t)l.nwaves * RG * 64 * sizeof(float4v));
+    if (lds > (64u << 10)) {
+        static const hipError_t raised = hipFuncSetAttribute((const void *)gemv_cs_staged_gateup_kernel<DT, XT, MR, RG, CPW>,
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10);
+        if (raised != hipSuccess) return raised;
+    }
+    const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
+    if (l.ev0) {
+        hipExtLaunchKernelGGL((gemv_cs_staged_gateup_kernel<DT, XT, MR, RG, CPW>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k, l.x,
+                              l.ldx, l.m, l.yt);
+        return hipGetLastError();
+    }
+    gemv_cs_staged_gateup_kernel<DT, XT, MR, RG, CPW><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
+    return hipGetLastError();
+}
+
+// tiles per workgroup (both weights together): 2 or 6 with two column tiles per wave, 2 with six
+template <int DT, int XT>
+hipError_t staged_gateup_shape(int rg, int cpw, const StagedLaunch &l) {
+    if (cpw == 2 && rg == 2) return l.m <= 8 ? staged_gateup_final<DT, XT, 8, 2, 2>(l) : staged_gateup_final<DT, XT, 16, 2, 2>(l);
+    if (cpw == 2 && rg == 6) return l.m <= 8 ? staged_gateup_final<DT, XT, 8, 6, 2>(l) : staged_gateup_final<DT, XT, 16, 6, 2>(l);
+    if (cpw == 6 && rg == 2) return l.m <= 8 ? staged_gateup_final<DT, XT, 8, 2, 6>(l) : staged_gateup_final<DT, XT, 16, 2, 6>(l);
     return hipErrorInvalidValue;
 }
 
@@ -291,6 +344,35 @@ hipError_t staged_launch(int dtype_a, int dtype_b, int count, int second, const 
     default: return hipErrorInvalidValue;
     }
 }
+
+// gate and up of one MLP (same format, n and k) with silu(gate) * up stored: tiles per workgroup = 2 * (row tiles of the output)
+template <int XT>
+hipError_t staged_gateup_launch(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x, int64_t ldx, int64_t m,
+                                void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up, int tiles,
+                                hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+    const int cpw = turq_gemv_cs_staged_cpw(k);
+    StagedLaunch l{};
+    l.a.w[0] = (const uint8_t *)w_gate, l.a.w[1] = (const uint8_t *)w_up;
+    l.a.bias[0] = bias_gate, l.a.bias[1] = bias_up;
+    l.a.y[0] = y, l.a.n[0] = l.a.n[1] = n, l.a.ldy[0] = ldy, l.a.count = 2, l.a.second = 2;
+    const int64_t blocks = (turq_tile_rows(n) + tiles / 2 - 1) / (tiles / 2);
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
+    l.blocks = (int)blocks, l.k = k, l.x = x, l.ldx = ldx, l.m = m, l.yt = y_dtype, l.nwaves = (int)(k / 256 / cpw);
+    l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop;
+    switch (dtype) {
+    case TURQ_Q4_K: return staged_gateup_shape<TURQ_Q4_K, XT>(tiles, cpw, l);
+    case TURQ_Q5_K: return staged_gateup_shape<TURQ_Q5_K, XT>(tiles, cpw, l);
+    case TURQ_Q6_K: return staged_gateup_shape<TURQ_Q6_K, XT>(tiles, cpw, l);
+    case TURQ_Q8_0: return staged_gateup_shape<TURQ_Q8_0, XT>(tiles, cpw, l);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+#define TURQ_STAGED_GATEUP_ARGS                                                                                                          \
+    int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x, int64_t ldx, int64_t m, void *y, int y_dtype,  \
+        int64_t ldy, const float *bias_gate, const float *bias_up, int tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop
+#define TURQ_STAGED_GATEUP_PASS dtype, w_gate, w_up, n, k, x, ldx, m, y, y_dtype, ldy, bias_gate, bias_up, tiles, stream, ev_start, ev_stop
 
 #define TURQ_STAGED_LAUNCH_ARGS                                                                                                          \
     int dtype_a, int dtype_b, int count, int second, const void *const *w, const int64_t *n, int64_t k, const void *x, int64_t ldx,      \

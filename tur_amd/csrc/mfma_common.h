@@ -180,6 +180,11 @@ hipError_t turq_launch_gemv_cs_staged(int dtype_a, int dtype_b, int count, int s
                                       int64_t k, const void *x, int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype,
                                       const int64_t *ldy, const float *const *bias, int row_tiles, hipStream_t stream,
                                       hipEvent_t ev_start, hipEvent_t ev_stop);
+int turq_gemv_cs_staged_gateup_tiles(int dtype, int64_t n, int64_t k, int64_t m, int64_t units);
+hipError_t turq_launch_gemv_cs_staged_gateup(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x,
+                                             int x_dtype, int64_t ldx, int64_t m, void *y, int y_dtype, int64_t ldy,
+                                             const float *bias_gate, const float *bias_up, int tiles, hipStream_t stream,
+                                             hipEvent_t ev_start, hipEvent_t ev_stop);
 bool turq_gemv_multi_mixed_supports(int dtype_a, int dtype_b);
 hipError_t turq_launch_gemv_multi_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w_tiled, const int64_t *n,
                                         int64_t k, const void *frags, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,

@@ -306,6 +306,20 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
         up->layout != TURQ_LAYOUT_TILED)
         return TURQ_OK;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // 3 .. 16 rows: the kernel that makes its fragments from the rows themselves (no preparation launch), activation in its epilogue
+    {
+        static const int staged = [] { const char *e = getenv("TURQ_CS_STAGED"); return e ? atoi(e) : -1; }();
+        const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+        const int tiles = (staged != 0 && aligned && m >= 3 && gate->n == up->n && gate->k == up->k)
+                              ? turq_gemv_cs_staged_gateup_tiles(gate->dtype, gate->n, gate->k, m, cus) : 0;
+        if (tiles) {
+            TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+            TURQ_HIP(ctx, turq_launch_gemv_cs_staged_gateup(gate->dtype, gate->dev, up->dev, gate->n, gate->k, x, xt, ldx, m, y, yt, ldy,
+                                                            bias_gate, bias_up, tiles, ctx->stream, ev0, ev1));
+            *taken = true;
+            return TURQ_OK;
+        }
+    }
     if (no_fuse || !aligned || m > 2 || !use_row1(gate->dtype) || !row1_takes(m, gate->dev_bytes + up->dev_bytes, gate->dtype)) {
         // up to 32 rows: fragments prepared once, then one launch whose workgroups take row tile b of both weights (the shape
         // of the two-row-tile kernel: at most four waves) and store the product
