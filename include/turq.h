@@ -186,8 +186,8 @@ int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype
 /* turq_qmatmul for callers that cannot allocate device memory around the call (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
  * reference.  Same product, same kernels and bit-identical results as turq_qmatmul with
- * TURQ_MEM_DEVICE and TURQ_ALGO_AUTO, but the prepared activation fragments of calls with more than
- * one row live in a static device array of TURQ_NOALLOC_SCRATCH_BYTES (one copy per GPU, held until
+ * TURQ_MEM_DEVICE and TURQ_ALGO_AUTO, but the prepared activation fragments of the calls that use them
+ * (more than 32 rows, and 17 - 32 rows on all but small weights) live in a static device array of TURQ_NOALLOC_SCRATCH_BYTES (one copy per GPU, held until
  * the process ends) instead of the context's growable buffer: the call runs no hipMalloc / hipFree
  * and creates no stream or event.  A call that needs more is refused with TURQ_ERR_SHAPE and a
  * message that names the bytes needed: fragments take 2.25 * mpad * k bytes for up to 32 rows (mpad
@@ -202,8 +202,10 @@ int turq_qmatmul_noalloc(turq_ctx *ctx, const turq_weight *w, const void *x, int
 
 /* The same product for `count` weights that take the same activations: ys[i][m, n_i] = x[m, k] * W_i^T (+ biases[i]).
  * All weights must share k.  With device pointers, tiled weights and m <= 32, neighbouring weights of one format
- * go out as ONE kernel launch (for more than one row on all but small matrices, or activation rows that are not
- * 16-byte aligned, after one preparation of the activations for all the weights); with more than 32 rows the
+ * go out as ONE kernel launch, and so do Q4_K or Q5_K weights followed by Q6_K ones (q, k and v of a Q4_K_M file); up to
+ * 16 rows that launch is all there is (the kernel makes its MFMA operands from the activation rows themselves), with 17 - 32
+ * rows on all but small weights, with activation rows that are not 16-byte aligned, and with k outside 512 .. 4096 in steps
+ * of 512 and 1536 .. 12288 in steps of 1536, one preparation of the activations for all the weights comes first; with more than 32 rows the
  * activations are prepared once for all the weights and each weight runs its GEMM on them (the results of the single
  * calls, bit for bit; GEMMs that leave half of the GPU free, such as k_proj and v_proj of a prompt chunk, run next to each other,
  * up to three at a time, on further streams of the context that are joined to the first before the call returns, so the
@@ -222,9 +224,9 @@ enum { TURQ_ACTFN_SILU = 0 };
  * act = SiLU, v / (1 + exp(-v)), computed in f32.  gate and up are two weights of one shape [n, k]; x, y, the strides, the
  * biases (NULL: none) and `mem` as in turq_qmatmul.  With device pointers, tiled weights of one format and up to 32
  * activation rows the activation and the product are applied inside the matmul kernel, which writes one output instead of
- * two: for one row (two on 8 MiB of weights and more) that kernel is the one launch of the call, for more rows it follows
- * one preparation of the activations (scratch memory of the context, which grows on demand, never inside a graph
- * capture).  Every other case computes the two products through turq_qmatmul_multi into scratch memory of the context and
+ * two: up to 16 rows that kernel is the one launch of the call, for more rows (and for the k and alignments named at
+ * turq_qmatmul_multi) it follows one preparation of the activations (scratch memory of the context, which grows on demand,
+ * never inside a graph capture).  Every other case computes the two products through turq_qmatmul_multi into scratch memory of the context and
  * combines them in one elementwise pass (with TURQ_MEM_HOST that pass runs on the host CPU, in the same f32 arithmetic: the
  * host form is for tests and one-off calls).  Errors as turq_qmatmul; gate and up of different shapes: TURQ_ERR_SHAPE; an activation other
  * than TURQ_ACTFN_SILU: TURQ_ERR_INVALID.
