@@ -206,6 +206,7 @@ bool turq_gemv_cs_staged_takes(int dtype_a, int dtype_b, int64_t k, int64_t m, i
     if (cpw == 0 || m < 1 || m > 32) return false;
     if (dtype_a != dtype_b && !((dtype_a == TURQ_Q4_K || dtype_a == TURQ_Q5_K) && dtype_b == TURQ_Q6_K)) return false;
     if (dtype_a != TURQ_Q4_K && dtype_a != TURQ_Q5_K && dtype_a != TURQ_Q6_K && dtype_a != TURQ_Q8_0) return false;
+    if (turq_gemv_cs_staged_two_cpw(k, m, row_tiles)) return true;  // 17 .. 32 rows, four waves, both 16-row tiles per unpack
     if (cpw == 6) return row_tiles == 1 || row_tiles == 2;
     return row_tiles == 1 || row_tiles == 2 || row_tiles == 3 || (row_tiles == 6 && m <= 16);
 }

@@ -215,6 +215,100 @@ __global__ void __launch_bounds__(512) gemv_cs_staged_gateup_kernel(MultiArgs a,
                                                                          (int64_t)blockIdx.x, a.w[1], a.bias[1]);
 }
 
+// ---- 17 .. 32 rows, both 16-row tiles against ONE unpack of a weight tile ----
+// The fragments of 32 rows (72 registers) next to 32 f32 rows in flight (128) and the accumulators of six row tiles (48) do not
+// fit 256 registers, which is what a wave gets with two waves per SIMD; with FOUR waves per workgroup (one per SIMD) a wave may
+// use 512, and a weight tile is unpacked once for both 16-row tiles instead of once per pass.  That wins where there are several
+// row tiles per set of fragments (gate / up at 32 rows: 25.3 us against 32.8 in two passes and 26.1 + 3.9 with prepared
+// fragments); with one row tile per workgroup the two passes with eight waves are as fast, and with two row tiles of Q4_K next to
+// one of Q6_K (q / k / v) faster (13.7 against 15.0 us), so only groups of six are built.
+template <int DT, int XT, int RG, int D, int CPW>
+__device__ __forceinline__ void cs_body_staged_two(const uint8_t *__restrict__ w, int64_t n, int64_t k, const void *__restrict__ x, int64_t ldx,
+                                                   int64_t m, void *__restrict__ y, int yt, int64_t ldy, const float *__restrict__ bias,
+                                                   int64_t grp) {
+    constexpr int T = RG * CPW;
+    static_assert(D >= 1 && D <= T, "ring of weight tiles");
+    extern __shared__ uint8_t smem[];
+    constexpr int TB = TiledFmt<DT>::kTileBytes;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int nwaves = blockDim.x >> 6;  // ntc == CPW * nwaves
+    const int64_t ntc = turq_tile_cols(k), nrt = turq_tile_rows(n);
+    const int64_t rt0 = grp * RG;
+    float4v acc[RG][2];
+    const uint8_t *wrow[RG];  // row tiles past the weight's last one re-read it; their results are not stored
+#pragma unroll
+    for (int r = 0; r < RG; r++) {
+        acc[r][0] = acc[r][1] = float4v{0.f, 0.f, 0.f, 0.f};
+        wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+    }
+    GOff go = lane_offsets(lane, 16);
+    XRows<XT, 16> raw[2];
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) raw[mt] = load_x_rows<XT, 16>(x, ldx, m, 16 * mt, wave, lane);
+    WRegs<DT> wr[D];
+#pragma unroll
+    for (int d = 0; d < D; d++) wr[d] = load_tile<DT>(wrow[d % RG] + (wave + (int64_t)(d / RG) * nwaves) * TB, go);
+    uint8_t *rows = smem + wave * (32 * kXRow);
+    AFrags<DT, 2> f;
+#pragma unroll
+    for (int c = 0; c < CPW; c++) {
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) stage_x_rows<XT, 16>(raw[mt], rows + mt * 16 * kXRow, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        if (c + 1 < CPW) {
+#pragma unroll
+            for (int mt = 0; mt < 2; mt++) raw[mt] = load_x_rows<XT, 16>(x, ldx, m, 16 * mt, wave + (int64_t)(c + 1) * nwaves, lane);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) frags_from_staged<DT>(rows + mt * 16 * kXRow, (int)m - 16 * mt, lane, f.a[mt]);
+#pragma unroll
+        for (int r = 0; r < RG; r++) {
+            const int t = c * RG + r;
+            TileOp<DT, 2, 4>::run(wr[t % D], f, lane, acc[r]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (t + D < T) wr[t % D] = load_tile<DT>(wrow[(t + D) % RG] + (wave + (int64_t)((t + D) / RG) * nwaves) * TB, go);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    __syncthreads();
+    float4v *red = (float4v *)smem;
+#pragma unroll
+    for (int r = 0; r < RG; r++)
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++) red[((r * 2 + mt) * nwaves + wave) * 64 + lane] = acc[r][mt];
+    __syncthreads();
+    const int nn = lane & 15, g = lane >> 4;
+    for (int i = wave; i < RG * 2; i += nwaves) {
+        const int r = i / 2, mt = i - 2 * r;
+        float4v s = red[(i * nwaves) * 64 + lane];
+        for (int wv = 1; wv < nwaves; wv++) s += red[(i * nwaves + wv) * 64 + lane];
+        const int64_t col = (rt0 + r) * 16 + nn;
+        if (rt0 + r >= nrt || col >= n) continue;
+        const float bv = bias ? bias[col] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int64_t row = 16 * mt + 4 * g + j;
+            if (row < m) turq_store_any(y, yt, row * ldy + col, s[j] + bv);
+        }
+    }
+}
+
+constexpr int staged_two_ring(int rg, int cpw) { return rg * cpw < 3 ? rg * cpw : 3; }
+
+// four waves; weights [0, a.second) of format DTA with RG row tiles per workgroup, the others of DTB with staged_second_rows(RG)
+template <int DTA, int DTB, int XT, int RG, int CPW>
+__global__ void __launch_bounds__(256) gemv_cs_staged_two_kernel(MultiArgs a, int64_t k, const void *__restrict__ x, int64_t ldx, int64_t m,
+                                                                  int yt) {
+    const MultiPick p = multi_pick(a, (int)blockIdx.x);
+    constexpr int RGB = staged_second_rows(RG);
+    if (DTA == DTB || p.index < a.second)
+        cs_body_staged_two<DTA, XT, RG, staged_two_ring(RG, CPW), CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
+    else
+        cs_body_staged_two<DTB, XT, RGB, staged_two_ring(RGB, CPW), CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
+}
+
 struct StagedLaunch {
     MultiArgs a;
     int blocks;
@@ -224,6 +318,7 @@ struct StagedLaunch {
     int yt, nwaves;
     hipStream_t s;
     hipEvent_t ev0, ev1;
+    bool two;  // the four-wave form for 17 .. 32 rows
 };
 
 template <int DTA, int DTB, int XT, int MR, int RG, int CPW>
@@ -292,8 +387,34 @@ hipError_t staged_gateup_shape(int rg, int cpw, const StagedLaunch &l) {
     return hipErrorInvalidValue;
 }
 
+template <int DTA, int DTB, int XT, int RG, int CPW>
+hipError_t staged_two_final(const StagedLaunch &l) {
+    const size_t lds = std::max((size_t)l.nwaves * 32 * kXRow, (size_t)l.nwaves * RG * 2 * 64 * sizeof(float4v));
+    if (lds > (64u << 10)) {
+        static const hipError_t raised = hipFuncSetAttribute((const void *)gemv_cs_staged_two_kernel<DTA, DTB, XT, RG, CPW>,
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10);
+        if (raised != hipSuccess) return raised;
+    }
+    const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
+    if (l.ev0) {
+        hipExtLaunchKernelGGL((gemv_cs_staged_two_kernel<DTA, DTB, XT, RG, CPW>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k, l.x,
+                              l.ldx, l.m, l.yt);
+        return hipGetLastError();
+    }
+    gemv_cs_staged_two_kernel<DTA, DTB, XT, RG, CPW><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
+    return hipGetLastError();
+}
+
+template <int DTA, int DTB, int XT>
+hipError_t staged_two_shape(int rg, int cpw, const StagedLaunch &l) {
+    if (cpw == 4 && rg == 6) return staged_two_final<DTA, DTB, XT, 6, 4>(l);
+    if (cpw == 2 && rg == 6) return staged_two_final<DTA, DTB, XT, 6, 2>(l);
+    return hipErrorInvalidValue;
+}
+
 template <int DTA, int DTB, int XT>
 hipError_t staged_rows(int rg, int cpw, const StagedLaunch &l) {
+    if (l.two) return staged_two_shape<DTA, DTB, XT>(rg, cpw, l);
     if (l.m <= 8) return staged_shape<DTA, DTB, XT, 8>(rg, cpw, l);
     if (l.m <= 16) return staged_shape<DTA, DTB, XT, 16>(rg, cpw, l);
     return staged_shape<DTA, DTB, XT, 32>(rg, cpw, l);
@@ -310,13 +431,22 @@ inline int turq_gemv_cs_staged_cpw(int64_t k) {
     return 0;
 }
 
+// column tiles per wave of the four-wave form for 17 .. 32 rows (0: it does not take this k or this group size)
+inline int turq_gemv_cs_staged_two_cpw(int64_t k, int64_t m, int row_tiles) {
+    if (k <= 0 || k % 1024 != 0 || m <= 16 || row_tiles != 6) return 0;
+    const int64_t cpw = k / 1024;
+    return cpw == 2 || cpw == 4 ? (int)cpw : 0;
+}
+
 // the launch for activations of type XT; arguments as turq_launch_gemv_cs_staged, which has checked them
 template <int XT>
 hipError_t staged_launch(int dtype_a, int dtype_b, int count, int second, const void *const *w, const int64_t *n, int64_t k, const void *x,
                          int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy, const float *const *bias, int row_tiles,
                          hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
-    const int cpw = turq_gemv_cs_staged_cpw(k);
+    const int two = turq_gemv_cs_staged_two_cpw(k, m, row_tiles);
+    const int cpw = two ? two : turq_gemv_cs_staged_cpw(k);
     StagedLaunch l{};
+    l.two = two != 0;
     int64_t blocks = 0;
     for (int i = 0; i < count; i++) {
         l.a.w[i] = (const uint8_t *)w[i];

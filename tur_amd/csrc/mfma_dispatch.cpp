@@ -114,9 +114,12 @@ int staged_row_tiles(const turq_ctx *ctx, int dtype_a, int dtype_b, int64_t k, i
         const int gb = turq_gemv_cs_staged_second_rows(g);
         if ((row_tiles - row_tiles_b + g - 1) / g + (row_tiles_b + gb - 1) / gb <= cus) rg = g;
     }
-    // more than 16 rows (two passes per weight tile, each unpacking it): pays on launches of up to two row tiles per unit of
-    // weights with few columns, where the preparation launch is a third of the time; larger ones are better off with it
-    if (m > 16 && !forced && (rg > 2 || row_tiles > 2 * cus || k > 4096)) return 0;
+    // more than 16 rows: on weights of up to 4096 columns (beyond, the f32 rows that every unit reads outweigh the preparation
+    // launch); up to two row tiles per unit as two passes of 16 rows, more in the four-wave form with groups of six
+    if (m > 16 && !forced) {
+        if (k > 4096) return 0;
+        if (row_tiles > 2 * cus) rg = 6;  // the four-wave form
+    }
     if (forced) rg = forced;
     while (rg > 1 && !turq_gemv_cs_staged_takes(dtype_a, dtype_b, k, m, rg)) rg = rg == 6 ? 3 : rg - 1;
     return turq_gemv_cs_staged_takes(dtype_a, dtype_b, k, m, rg) ? rg : 0;
