@@ -131,15 +131,16 @@ def test_q4km_decoder_layer_grouped_calls(gpu, layer, m, x_dtype):
 
 
 def test_mlp_gate_up_and_token_embd(gpu):
-    # the two calls that widen the path, at Qwen3-8B sizes: gate / up with SiLU (12288 x 4096 Q4_K, one launch for one row, the two
-    # products plus an elementwise pass for sixteen) and token_embd rows (151936 x 4096 Q6_K) against the full dequantize
+    # the two calls that widen the path, at Qwen3-8B sizes: gate / up with SiLU (12288 x 4096 Q4_K: one launch at every row count
+    # here - the one-row kernel, the staged rows kernel with six tiles per workgroup, its four-wave form from 17 rows on) and
+    # token_embd rows (151936 x 4096 Q6_K) against the full dequantize
     from oracle import oracle_np as onp
     n, k = 12288, 4096
     raw_g = synth.random_weight(Q4_K, n, k, seed=1)
     raw_u = synth.random_weight(Q4_K, n, k, seed=2)
     wg = gpu.upload(Q4_K, n, k, raw_g, capi.LAYOUT_TILED)
     wu = gpu.upload(Q4_K, n, k, raw_u, capi.LAYOUT_TILED)
-    for m in (1, 2, 16):
+    for m in (1, 2, 5, 16, 17, 32):
         x = synth.random_activation(m, k, seed=40 + m, bf16=True)
         y = gpu.gate_up(wg, wu, x, n, k, x_dtype=capi.ACT_BF16)
         want = onp.silu_mul(orc.matmul_dequant(Q4_K, x, raw_g, n, k), orc.matmul_dequant(Q4_K, x, raw_u, n, k))

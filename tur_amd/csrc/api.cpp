@@ -658,11 +658,17 @@ static int impl_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *u
         if (rc != TURQ_OK) return rc;
         return impl_qmatmul(ctx, down, h.data(), TURQ_ACT_F32, m, n_ff, y, yt, ldy, bias_down, mem, TURQ_ALGO_AUTO);
     }
-    int rc = turq_ctx_reserve(ctx, &ctx->mlp_h, &ctx->mlp_h_cap, h_elems * sizeof(float) + 16);
+    // The MFMA kernels round their activations to f16 first thing, so where down_proj goes through them the intermediate is
+    // kept as f16 to begin with: the same values reach the same multiplications, and the rows that every compute unit reads
+    // for down_proj are half as long.  (Not with wide activations, which scale f32 rows before that rounding, and not for a
+    // dense or native-layout down_proj, which multiplies in f32.)
+    const bool h16 = !ctx->wide && turq_dt_is_quant(down->dtype) && down->layout == TURQ_LAYOUT_TILED && n_ff % 8 == 0;
+    const int ht = h16 ? TURQ_ACT_F16 : TURQ_ACT_F32;
+    int rc = turq_ctx_reserve(ctx, &ctx->mlp_h, &ctx->mlp_h_cap, h_elems * (h16 ? sizeof(uint16_t) : sizeof(float)) + 16);
     if (rc != TURQ_OK) return rc;
-    rc = impl_qmatmul_gate_up(ctx, gate, up, x, xt, m, ldx, ctx->mlp_h, TURQ_ACT_F32, n_ff, bias_gate, bias_up, act, mem);
+    rc = impl_qmatmul_gate_up(ctx, gate, up, x, xt, m, ldx, ctx->mlp_h, ht, n_ff, bias_gate, bias_up, act, mem);
     if (rc != TURQ_OK) return rc;
-    return impl_qmatmul(ctx, down, ctx->mlp_h, TURQ_ACT_F32, m, n_ff, y, yt, ldy, bias_down, mem, TURQ_ALGO_AUTO);
+    return impl_qmatmul(ctx, down, ctx->mlp_h, ht, m, n_ff, y, yt, ldy, bias_down, mem, TURQ_ALGO_AUTO);
 }
 
 // ---- graphs and kernel timing ----

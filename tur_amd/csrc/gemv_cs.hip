@@ -237,20 +237,23 @@ hipError_t turq_launch_gemv_cs_staged_gateup_bf16(TURQ_STAGED_GATEUP_ARGS);
 hipError_t turq_launch_gemv_cs_staged_gateup_f16(TURQ_STAGED_GATEUP_ARGS);
 
 // tiles per workgroup (gate and up together: 2 or 6) for n output columns on `units` compute units, 0: not this case
+// (17 .. 32 rows: the four-wave form, which has groups of 6 for k = 2048 and 4096)
 int turq_gemv_cs_staged_gateup_tiles(int dtype, int64_t n, int64_t k, int64_t m, int64_t units) {
-    const int cpw = turq_gemv_cs_staged_cpw(k);
-    if (cpw == 0 || m < 1 || m > 16) return 0;
     if (dtype != TURQ_Q4_K && dtype != TURQ_Q5_K && dtype != TURQ_Q6_K && dtype != TURQ_Q8_0) return 0;
+    if (m > 16) return (m <= 32 && turq_tile_rows(n) > 2 * units && turq_gemv_cs_staged_two_cpw(k, m, 6)) ? 6 : 0;
+    const int cpw = turq_gemv_cs_staged_cpw(k);
+    if (cpw == 0 || m < 1) return 0;
     return (cpw == 2 && turq_tile_rows(n) > 2 * units) ? 6 : 2;
 }
 
-// y[r][c] = silu(x[r] . gate[c] + bias_gate[c]) * (x[r] . up[c] + bias_up[c]); tiled weights of one format, n and k; m (1..16)
+// y[r][c] = silu(x[r] . gate[c] + bias_gate[c]) * (x[r] . up[c] + bias_up[c]); tiled weights of one format, n and k; m (1..32)
 // activation rows of stride ldx (rows 16-byte aligned); tiles as turq_gemv_cs_staged_gateup_tiles says
 hipError_t turq_launch_gemv_cs_staged_gateup(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x, int x_dtype,
                                              int64_t ldx, int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate,
                                              const float *bias_up, int tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
     const int cpw = turq_gemv_cs_staged_cpw(k);
-    if (cpw == 0 || m < 1 || m > 16 || !(tiles == 2 || (tiles == 6 && cpw == 2))) return hipErrorInvalidValue;
+    if (m > 16 ? (m > 32 || !turq_gemv_cs_staged_two_cpw(k, m, tiles)) : (cpw == 0 || m < 1 || !(tiles == 2 || (tiles == 6 && cpw == 2))))
+        return hipErrorInvalidValue;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
     switch (x_dtype) {
     case TURQ_ACT_F32: return turq_launch_gemv_cs_staged_gateup_f32(TURQ_STAGED_GATEUP_PASS);

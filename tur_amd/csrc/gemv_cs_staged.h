@@ -222,10 +222,13 @@ __global__ void __launch_bounds__(512) gemv_cs_staged_gateup_kernel(MultiArgs a,
 // row tiles per set of fragments (gate / up at 32 rows: 25.3 us against 32.8 in two passes and 26.1 + 3.9 with prepared
 // fragments); with one row tile per workgroup the two passes with eight waves are as fast, and with two row tiles of Q4_K next to
 // one of Q6_K (q / k / v) faster (13.7 against 15.0 us), so only groups of six are built.
-template <int DT, int XT, int RG, int D, int CPW>
+template <int DT, int XT, int RG, int D, int CPW, bool GU = false>
 __device__ __forceinline__ void cs_body_staged_two(const uint8_t *__restrict__ w, int64_t n, int64_t k, const void *__restrict__ x, int64_t ldx,
                                                    int64_t m, void *__restrict__ y, int yt, int64_t ldy, const float *__restrict__ bias,
-                                                   int64_t grp) {
+                                                   int64_t grp, const uint8_t *__restrict__ w2 = nullptr,
+                                                   const float *__restrict__ bias2 = nullptr) {
+    static_assert(!GU || RG % 2 == 0, "gate and up tiles come in pairs");
+    constexpr int RO = GU ? RG / 2 : RG;  // row tiles of the output per workgroup
     constexpr int T = RG * CPW;
     static_assert(D >= 1 && D <= T, "ring of weight tiles");
     extern __shared__ uint8_t smem[];
@@ -234,13 +237,14 @@ __device__ __forceinline__ void cs_body_staged_two(const uint8_t *__restrict__ w
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nwaves = blockDim.x >> 6;  // ntc == CPW * nwaves
     const int64_t ntc = turq_tile_cols(k), nrt = turq_tile_rows(n);
-    const int64_t rt0 = grp * RG;
+    const int64_t rt0 = grp * RO;
     float4v acc[RG][2];
     const uint8_t *wrow[RG];  // row tiles past the weight's last one re-read it; their results are not stored
 #pragma unroll
     for (int r = 0; r < RG; r++) {
         acc[r][0] = acc[r][1] = float4v{0.f, 0.f, 0.f, 0.f};
-        wrow[r] = w + (rt0 + r < nrt ? rt0 + r : nrt - 1) * ntc * TB;
+        const int ro = r < RO ? r : r - RO;
+        wrow[r] = (r < RO ? w : w2) + (rt0 + ro < nrt ? rt0 + ro : nrt - 1) * ntc * TB;
     }
     GOff go = lane_offsets(lane, 16);
     XRows<XT, 16> raw[2];
@@ -280,17 +284,29 @@ __device__ __forceinline__ void cs_body_staged_two(const uint8_t *__restrict__ w
         for (int mt = 0; mt < 2; mt++) red[((r * 2 + mt) * nwaves + wave) * 64 + lane] = acc[r][mt];
     __syncthreads();
     const int nn = lane & 15, g = lane >> 4;
-    for (int i = wave; i < RG * 2; i += nwaves) {
+    for (int i = wave; i < RO * 2; i += nwaves) {
         const int r = i / 2, mt = i - 2 * r;
         float4v s = red[(i * nwaves) * 64 + lane];
         for (int wv = 1; wv < nwaves; wv++) s += red[(i * nwaves + wv) * 64 + lane];
+        float4v s2 = float4v{0.f, 0.f, 0.f, 0.f};
+        if constexpr (GU) {
+            const int i2 = i + RO * 2;  // the up tile of the pair
+            s2 = red[(i2 * nwaves) * 64 + lane];
+            for (int wv = 1; wv < nwaves; wv++) s2 += red[(i2 * nwaves + wv) * 64 + lane];
+        }
         const int64_t col = (rt0 + r) * 16 + nn;
         if (rt0 + r >= nrt || col >= n) continue;
-        const float bv = bias ? bias[col] : 0.0f;
+        const float bv = bias ? bias[col] : 0.0f, bv2 = (GU && bias2) ? bias2[col] : 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int64_t row = 16 * mt + 4 * g + j;
-            if (row < m) turq_store_any(y, yt, row * ldy + col, s[j] + bv);
+            if (row >= m) continue;
+            if constexpr (GU) {
+                const float gate = s[j] + bv, up = s2[j] + bv2;
+                turq_store_any(y, yt, row * ldy + col, gate / (1.0f + expf(-gate)) * up);
+            } else {
+                turq_store_any(y, yt, row * ldy + col, s[j] + bv);
+            }
         }
     }
 }
@@ -307,6 +323,14 @@ __global__ void __launch_bounds__(256) gemv_cs_staged_two_kernel(MultiArgs a, in
         cs_body_staged_two<DTA, XT, RG, staged_two_ring(RG, CPW), CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
     else
         cs_body_staged_two<DTB, XT, RGB, staged_two_ring(RGB, CPW), CPW>(p.w, p.n, k, x, ldx, m, p.y, yt, p.ldy, p.bias, (int64_t)p.block);
+}
+
+// ... gate (a.w[0]) and up (a.w[1]) of one MLP, three row tiles of each per workgroup, silu(gate) * up stored to a.y[0]
+template <int DT, int XT, int CPW>
+__global__ void __launch_bounds__(256) gemv_cs_staged_two_gateup_kernel(MultiArgs a, int64_t k, const void *__restrict__ x, int64_t ldx,
+                                                                         int64_t m, int yt) {
+    cs_body_staged_two<DT, XT, 6, staged_two_ring(6, CPW), CPW, true>(a.w[0], a.n[0], k, x, ldx, m, a.y[0], yt, a.ldy[0], a.bias[0],
+                                                                      (int64_t)blockIdx.x, a.w[1], a.bias[1]);
 }
 
 struct StagedLaunch {
@@ -378,9 +402,28 @@ hipError_t staged_gateup_final(const StagedLaunch &l) {
     return hipGetLastError();
 }
 
-// tiles per workgroup (both weights together): 2 or 6 with two column tiles per wave, 2 with six
+template <int DT, int XT, int CPW>
+hipError_t staged_two_gateup_final(const StagedLaunch &l) {
+    const size_t lds = std::max((size_t)l.nwaves * 32 * kXRow, (size_t)l.nwaves * 6 * 2 * 64 * sizeof(float4v));
+    if (lds > (64u << 10)) {
+        static const hipError_t raised = hipFuncSetAttribute((const void *)gemv_cs_staged_two_gateup_kernel<DT, XT, CPW>,
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10);
+        if (raised != hipSuccess) return raised;
+    }
+    const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
+    if (l.ev0) {
+        hipExtLaunchKernelGGL((gemv_cs_staged_two_gateup_kernel<DT, XT, CPW>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k, l.x,
+                              l.ldx, l.m, l.yt);
+        return hipGetLastError();
+    }
+    gemv_cs_staged_two_gateup_kernel<DT, XT, CPW><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
+    return hipGetLastError();
+}
+
+// tiles per workgroup (both weights together): 2 or 6 with two column tiles per wave, 2 with six; 17 .. 32 rows: 6, four waves
 template <int DT, int XT>
 hipError_t staged_gateup_shape(int rg, int cpw, const StagedLaunch &l) {
+    if (l.two) return cpw == 4 ? staged_two_gateup_final<DT, XT, 4>(l) : cpw == 2 ? staged_two_gateup_final<DT, XT, 2>(l) : hipErrorInvalidValue;
     if (cpw == 2 && rg == 2) return l.m <= 8 ? staged_gateup_final<DT, XT, 8, 2, 2>(l) : staged_gateup_final<DT, XT, 16, 2, 2>(l);
     if (cpw == 2 && rg == 6) return l.m <= 8 ? staged_gateup_final<DT, XT, 8, 6, 2>(l) : staged_gateup_final<DT, XT, 16, 6, 2>(l);
     if (cpw == 6 && rg == 2) return l.m <= 8 ? staged_gateup_final<DT, XT, 8, 2, 6>(l) : staged_gateup_final<DT, XT, 16, 2, 6>(l);
@@ -480,8 +523,10 @@ template <int XT>
 hipError_t staged_gateup_launch(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x, int64_t ldx, int64_t m,
                                 void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up, int tiles,
                                 hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
-    const int cpw = turq_gemv_cs_staged_cpw(k);
+    const int two = turq_gemv_cs_staged_two_cpw(k, m, tiles);
+    const int cpw = two ? two : turq_gemv_cs_staged_cpw(k);
     StagedLaunch l{};
+    l.two = two != 0;
     l.a.w[0] = (const uint8_t *)w_gate, l.a.w[1] = (const uint8_t *)w_up;
     l.a.bias[0] = bias_gate, l.a.bias[1] = bias_up;
     l.a.y[0] = y, l.a.n[0] = l.a.n[1] = n, l.a.ldy[0] = ldy, l.a.count = 2, l.a.second = 2;
