@@ -237,10 +237,12 @@ int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weig
                          int mem);
 
 /* The reference's whole MLP in one call: y[m, n_out] = (act(x * gate^T + bias_gate) * (x * up^T + bias_up)) * down^T + bias_down.
- * gate and up are two weights of one shape [n_ff, k], down is [n_out, n_ff]; the intermediate is kept in f32 (scratch memory of
- * the context, m * n_ff floats, which grows on demand, never inside a graph capture).  The results are those of
+ * gate and up are two weights of one shape [n_ff, k], down is [n_out, n_ff]; the intermediate lives in scratch memory of the
+ * context (m * n_ff values, which grows on demand, never inside a graph capture).  The results are those of
  * turq_qmatmul_gate_up into an f32 buffer followed by turq_qmatmul on it, bit for bit, and so are the errors and the meaning of
- * x, y, the strides, the biases (NULL: none), `act` and `mem`.
+ * x, y, the strides, the biases (NULL: none), `act` and `mem`.  (Where down_proj runs on the matrix cores - a tiled
+ * quantized weight, wide activations off - its kernels round the activations to f16 first thing, so the intermediate is
+ * stored as f16 to begin with: the same values, half the bytes that every compute unit reads for down_proj.)
  * The call is those two calls one after the other on the context's stream.  (A single launch for the whole MLP - one
  * persistent workgroup per compute unit, down_proj's first tiles requested while the last gate / up tiles are computed, a grid-wide
  * barrier on device counters before down_proj reads the intermediate - was built, gave the same bits and was slower: 26 us
