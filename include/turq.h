@@ -204,8 +204,8 @@ int turq_qmatmul_noalloc(turq_ctx *ctx, const turq_weight *w, const void *x, int
  * All weights must share k.  With device pointers, tiled weights and m <= 32, neighbouring weights of one format
  * go out as ONE kernel launch, and so do Q4_K or Q5_K weights followed by Q6_K ones (q, k and v of a Q4_K_M file); up to
  * 16 rows that launch is all there is (the kernel makes its MFMA operands from the activation rows themselves), with 17 - 32
- * rows on all but small weights, with activation rows that are not 16-byte aligned, and with k outside 512 .. 4096 in steps
- * of 512 and 1536 .. 12288 in steps of 1536, one preparation of the activations for all the weights comes first; with more than 32 rows the
+ * rows on all but small weights, with activation rows that are not 16-byte aligned, and with k that is not a multiple of 512,
+ * one preparation of the activations for all the weights comes first; with more than 32 rows the
  * activations are prepared once for all the weights and each weight runs its GEMM on them (the results of the single
  * calls, bit for bit; GEMMs that leave half of the GPU free, such as k_proj and v_proj of a prompt chunk, run next to each other,
  * up to three at a time, on further streams of the context that are joined to the first before the call returns, so the

@@ -589,11 +589,12 @@ def test_rows_in_registers_kernel_shapes(row_tiles):
 
 # 3 .. 32 rows on a k that splits evenly over the waves go through the form of that kernel that stages the activation rows
 # through the LDS (no preparation launch, no scratch; more than 16 rows as two passes of 16 or, with several row tiles per
-# workgroup and k = 2048, in the four-wave form that takes both 16-row tiles per unpack): k = 1024 and 2048 are two column tiles
-# per wave, k = 4608 six; n = 200 ends inside a row tile and, with several row tiles per workgroup, inside a workgroup.  One format
+# workgroup and up to 4096 columns, in the four-wave form that takes both 16-row tiles per unpack).  A wave walks its column
+# tiles in pairs: k = 512 is one pair for one wave, 1024 and 2048 one pair per wave, 4608 nine pairs for eight waves, 9728
+# nineteen (waves with three and with two: the loop over pairs runs a different number of times per wave); n = 200 ends inside a row tile and, with several row tiles per workgroup, inside a workgroup.  One format
 # and the two-format launches, every activation type, strides, biases, bf16 output; the rows of a batch are independent, so a
 # batch of 32 equals four of 8.
-@pytest.mark.parametrize("k", [1024, 2048, 4608])
+@pytest.mark.parametrize("k", [512, 1024, 2048, 4608, 9728])
 @pytest.mark.parametrize("dts", [(Q4_K,), (Q5_K,), (Q6_K,), (Q8_0,), (Q4_K, Q4_K, Q6_K), (Q5_K, Q6_K, Q6_K), (Q4_K, Q4_K, Q4_K, Q6_K)])
 def test_staged_rows_kernel(dts, k):
     own = Gpu()

@@ -194,21 +194,19 @@ hipError_t turq_launch_gemv_cs(int dtype, int count, const void *const *w, const
 }
 
 // ---- activations staged through the LDS (gemv_cs_staged.h; one translation unit per activation type) ----
-// k = 512 .. 4096 in steps of 512, or 1536 .. 12288 in steps of 1536; up to 32 rows
+// k a multiple of 512; up to 32 rows
 hipError_t turq_launch_gemv_cs_staged_f32(TURQ_STAGED_LAUNCH_ARGS);
 hipError_t turq_launch_gemv_cs_staged_bf16(TURQ_STAGED_LAUNCH_ARGS);
 hipError_t turq_launch_gemv_cs_staged_f16(TURQ_STAGED_LAUNCH_ARGS);
 
 // whether the staged form has this case: formats (dtype_b = dtype_a for one format, else a K-quant pair with Q6_K second),
-// k, m and row tiles per workgroup
+// k, m and row tiles per workgroup (1, 2; 3 up to 16 rows; 6 up to 16 rows and, in the four-wave form, from 17)
 bool turq_gemv_cs_staged_takes(int dtype_a, int dtype_b, int64_t k, int64_t m, int row_tiles) {
-    const int cpw = turq_gemv_cs_staged_cpw(k);
-    if (cpw == 0 || m < 1 || m > 32) return false;
+    if (!turq_gemv_cs_staged_waves(k) || m < 1 || m > 32) return false;
     if (dtype_a != dtype_b && !((dtype_a == TURQ_Q4_K || dtype_a == TURQ_Q5_K) && dtype_b == TURQ_Q6_K)) return false;
     if (dtype_a != TURQ_Q4_K && dtype_a != TURQ_Q5_K && dtype_a != TURQ_Q6_K && dtype_a != TURQ_Q8_0) return false;
-    if (turq_gemv_cs_staged_two_cpw(k, m, row_tiles)) return true;  // 17 .. 32 rows, four waves, both 16-row tiles per unpack
-    if (cpw == 6) return row_tiles == 1 || row_tiles == 2;
-    return row_tiles == 1 || row_tiles == 2 || row_tiles == 3 || (row_tiles == 6 && m <= 16);
+    if (m > 16 && row_tiles != 6 && k > 4096) return false;  // the two passes of 16 rows are only built with one pair per wave
+    return row_tiles == 1 || row_tiles == 2 || (row_tiles == 3 && m <= 16) || row_tiles == 6;
 }
 
 int turq_gemv_cs_staged_second_rows(int row_tiles) { return staged_second_rows(row_tiles); }
@@ -237,13 +235,12 @@ hipError_t turq_launch_gemv_cs_staged_gateup_bf16(TURQ_STAGED_GATEUP_ARGS);
 hipError_t turq_launch_gemv_cs_staged_gateup_f16(TURQ_STAGED_GATEUP_ARGS);
 
 // tiles per workgroup (gate and up together: 2 or 6) for n output columns on `units` compute units, 0: not this case
-// (17 .. 32 rows: the four-wave form, which has groups of 6 for k = 2048 and 4096)
+// (17 .. 32 rows: the four-wave form, which has groups of 6, on up to 4096 columns)
 int turq_gemv_cs_staged_gateup_tiles(int dtype, int64_t n, int64_t k, int64_t m, int64_t units) {
     if (dtype != TURQ_Q4_K && dtype != TURQ_Q5_K && dtype != TURQ_Q6_K && dtype != TURQ_Q8_0) return 0;
-    if (m > 16) return (m <= 32 && turq_tile_rows(n) > 2 * units && turq_gemv_cs_staged_two_cpw(k, m, 6)) ? 6 : 0;
-    const int cpw = turq_gemv_cs_staged_cpw(k);
-    if (cpw == 0 || m < 1) return 0;
-    return (cpw == 2 && turq_tile_rows(n) > 2 * units) ? 6 : 2;
+    if (!turq_gemv_cs_staged_waves(k) || m < 1 || m > 32) return 0;
+    if (m > 16) return (turq_tile_rows(n) > 2 * units && k <= 4096) ? 6 : 0;
+    return turq_tile_rows(n) > 2 * units ? 6 : 2;
 }
 
 // y[r][c] = silu(x[r] . gate[c] + bias_gate[c]) * (x[r] . up[c] + bias_up[c]); tiled weights of one format, n and k; m (1..32)
@@ -251,9 +248,7 @@ int turq_gemv_cs_staged_gateup_tiles(int dtype, int64_t n, int64_t k, int64_t m,
 hipError_t turq_launch_gemv_cs_staged_gateup(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x, int x_dtype,
                                              int64_t ldx, int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate,
                                              const float *bias_up, int tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
-    const int cpw = turq_gemv_cs_staged_cpw(k);
-    if (m > 16 ? (m > 32 || !turq_gemv_cs_staged_two_cpw(k, m, tiles)) : (cpw == 0 || m < 1 || !(tiles == 2 || (tiles == 6 && cpw == 2))))
-        return hipErrorInvalidValue;
+    if (!turq_gemv_cs_staged_waves(k) || m < 1 || m > 32 || (tiles != 2 && tiles != 6) || (m > 16 && tiles != 6)) return hipErrorInvalidValue;
     if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
     switch (x_dtype) {
     case TURQ_ACT_F32: return turq_launch_gemv_cs_staged_gateup_f32(TURQ_STAGED_GATEUP_PASS);
