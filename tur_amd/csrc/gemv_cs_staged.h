@@ -84,7 +84,7 @@ template <int DT> __device__ inline void frags_from_staged(const uint8_t *__rest
     if constexpr (DT != TURQ_Q8_0) out[8] = kq_group_sums(out);
 }
 
-// m <= MR rows (8, 16 or 32), k a multiple of 512.  More than 16 rows are taken as two halves of 16, one after the other against
+// m <= MR rows (4, 8, 16 or 32), k a multiple of 512.  More than 16 rows are taken as two halves of 16, one after the other against
 // the same weight tiles (HV = 2): the tiles of a column tile stay in their registers for both passes and are unpacked once per
 // pass, which for these launches costs less than what holding the fragments of 32 rows next to the rows in flight would
 // (registers), or a launch that prepares them.  D: weight tiles in flight; a ring slot holds the same tile of every pair, so D
@@ -444,6 +444,7 @@ hipError_t staged_rows(int rg, const StagedLaunch &l) {
         if (rg != 6) return hipErrorInvalidValue;
         return l.cnt == 2 ? staged_go<gemv_cs_staged_two_kernel<DTA, DTB, XT, 2>>(lds, l) : staged_go<gemv_cs_staged_two_kernel<DTA, DTB, XT, 0>>(lds, l);
     }
+    if (l.m <= 4) return staged_shape<DTA, DTB, XT, 4>(rg, l);
     if (l.m <= 8) return staged_shape<DTA, DTB, XT, 8>(rg, l);
     if (l.m <= 16) return staged_shape<DTA, DTB, XT, 16>(rg, l);
     return staged_shape<DTA, DTB, XT, 32>(rg, l);
@@ -463,8 +464,8 @@ hipError_t staged_gateup_shape(int rg, const StagedLaunch &l) {
         if (rg != 6) return hipErrorInvalidValue;
         return l.cnt == 2 ? staged_go<gemv_cs_staged_two_gateup_kernel<DT, XT, 2>>(lds, l) : staged_go<gemv_cs_staged_two_gateup_kernel<DT, XT, 0>>(lds, l);
     }
-    if (rg == 2) return l.m <= 8 ? staged_gateup_count<DT, XT, 8, 2>(l) : staged_gateup_count<DT, XT, 16, 2>(l);
-    if (rg == 6) return l.m <= 8 ? staged_gateup_count<DT, XT, 8, 6>(l) : staged_gateup_count<DT, XT, 16, 6>(l);
+    if (rg == 2) return l.m <= 4 ? staged_gateup_count<DT, XT, 4, 2>(l) : l.m <= 8 ? staged_gateup_count<DT, XT, 8, 2>(l) : staged_gateup_count<DT, XT, 16, 2>(l);
+    if (rg == 6) return l.m <= 4 ? staged_gateup_count<DT, XT, 4, 6>(l) : l.m <= 8 ? staged_gateup_count<DT, XT, 8, 6>(l) : staged_gateup_count<DT, XT, 16, 6>(l);
     return hipErrorInvalidValue;
 }
 
