@@ -107,7 +107,7 @@ def layer(gpu):
 
 
 @pytest.mark.parametrize("x_dtype", [capi.ACT_F32, capi.ACT_BF16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("m", [1, 8, 32])
+@pytest.mark.parametrize("m", [1, 4, 8, 16, 32])
 def test_q4km_decoder_layer_grouped_calls(gpu, layer, m, x_dtype):
     # the layer's seven linears driven as the reference's decoder layer drives them (src/models/qwen3.rs:272-274, 161-167):
     # q / k / v on one tensor through turq_qmatmul_multi (two formats in one launch), o_proj alone, gate / up through
