@@ -762,8 +762,7 @@ hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, i
     static_assert(LDS_BYTES <= 160 * 1024, "LDS of one workgroup: the rings, or the staged results after the main loop");
     // per-lane weight offsets are 32-bit
     if ((uint64_t)G::NT16 * (uint64_t)(k / 256) * G::TB >= (1ull << 32)) return hipErrorInvalidValue;
-    static const hipError_t attr =
-        hipFuncSetAttribute((const void *)gemm_kq_kernel<DT, WGM_>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    const hipError_t attr = turq_raise_lds_limit((const void *)gemm_kq_kernel<DT, WGM_>, LDS_BYTES);
     if (attr != hipSuccess) return attr;
     const int nbn = (int)((n + G::BN - 1) / G::BN), nbm = (int)((m + G::GBM - 1) / G::GBM);
     const dim3 grid((unsigned)(nbn * nbm)), block(256);

@@ -115,8 +115,7 @@ hipError_t launch_final(const CsLaunch &l) {
     constexpr int MAXT = 512;
     const size_t lds = l.nwaves > 1 ? (size_t)l.nwaves * RG * MT * 64 * sizeof(float4v) : 0;
     if (lds > (64u << 10)) {
-        static const hipError_t raised = hipFuncSetAttribute((const void *)gemv_cs_kernel<DT, MT, XT, RG, D, MAXT>,
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10);
+        const hipError_t raised = turq_raise_lds_limit((const void *)gemv_cs_kernel<DT, MT, XT, RG, D, MAXT>, 128 << 10);
         if (raised != hipSuccess) return raised;
     }
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));

@@ -396,7 +396,7 @@ struct StagedLaunch {
 template <auto kernel>
 hipError_t staged_go(size_t lds, const StagedLaunch &l) {
     if (lds > (64u << 10)) {
-        static const hipError_t raised = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 144 << 10);
+        const hipError_t raised = turq_raise_lds_limit((const void *)kernel, 144 << 10);
         if (raised != hipSuccess) return raised;
     }
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));

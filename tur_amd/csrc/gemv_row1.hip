@@ -603,8 +603,7 @@ hipError_t launch_final(const Row1Launch &l) {
     const size_t lds = row1_lds<DT, P, R, M>(l.nwaves);
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
     if (lds > (64u << 10)) {  // 16 waves x two tiles in flight x two pairs of rows: 94 KiB
-        static const hipError_t raised = hipFuncSetAttribute((const void *)gemv_row1_kernel<DT, XT, P, R, M, 1024>,
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, 128 << 10);
+        const hipError_t raised = turq_raise_lds_limit((const void *)gemv_row1_kernel<DT, XT, P, R, M, 1024>, 128 << 10);
         if (raised != hipSuccess) return raised;
     }
     if (l.ev0) {

@@ -24,6 +24,10 @@
 // mpad is the m-tile height rounded up to 1, 2, 4, 8 or 16; rows beyond m are zero.
 #pragma once
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 #include "common.h"
 
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
@@ -162,6 +166,21 @@ int turq_gemv_row1_rows(int dtype);
 hipError_t turq_launch_gemv_gateup_frag(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *frags,
                                         int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up,
                                         int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
+// Raises a kernel's dynamic-LDS limit once per (kernel, device): the attribute belongs to the device that is current when it is
+// set, and a process may hold contexts on several.
+inline hipError_t turq_raise_lds_limit(const void *kernel, int bytes) {
+    static std::mutex mu;
+    static std::set<std::pair<const void *, int>> done;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    std::lock_guard<std::mutex> lock(mu);
+    if (done.count({kernel, dev})) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) done.insert({kernel, dev});
+    return e;
+}
+
 bool turq_gemv_row1_supports(int dtype);
 hipError_t turq_launch_gemv_row1_gateup(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x,
                                         int x_dtype, int64_t ldx, int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate,
