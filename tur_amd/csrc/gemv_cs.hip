@@ -8,6 +8,9 @@
 // never drains.  Every weight byte is read once and every activation once per workgroup.  The partial 16 x 16 results of the
 // waves meet in the LDS at the end, in a fixed order.
 //
+// This file holds that form as a loop over single column tiles (any k), and the entry points of the faster form that stages the
+// activation rows through the LDS (gemv_cs_staged.h: k a multiple of 512), which the dispatcher prefers wherever it applies.
+//
 // The tile arithmetic is the one of the other skinny kernels (gemv_tileop.h).
 #include <hip/hip_ext.h>
 

@@ -14,8 +14,8 @@ namespace {
 
 // ---- a workgroup owns RG row tiles and all columns; a wave walks its column tiles in PAIRS ----
 //
-// Against a loop whose lanes load their own A-operand slots from the caller's rows (gemv_cs.hip):
-// Two things hold the loop above back.  (1) A lane that loads exactly its own A-operand slots reads 16 bytes from each of 32
+// Two things hold back the form of this decomposition whose lanes load their own A-operand slots from the caller's rows in a loop
+// over single column tiles (gemv_cs.hip).  (1) A lane that loads exactly its own A-operand slots reads 16 bytes from each of 32
 // different cache lines per instruction (rows are a row stride apart, lane groups 256 bytes), and half of that twice when there
 // are no more than 8 rows: the address unit of the CU works through four to eight times the lines the data needs, the loads of
 // the second wave of every SIMD queue behind those of the first, and for microseconds half of the waves have no activations and
