@@ -178,6 +178,10 @@ int turq_rms_norm(turq_ctx *ctx, const void *x, int x_dtype, int64_t m, int64_t 
  *        synchronous);
  *   algo: TURQ_ALGO_*.
  * Errors instead of panics for m < 0, ld too small, unsupported dtypes.  m == 0 is a no-op.
+ * Device calls of more than 32 rows (prompt chunks) whose workgroup tiles would leave most compute units idle - the tall
+ * down_proj of a model up to about 256 rows, every matrix of a layer up to 64 - split the columns of every tile over several
+ * workgroups, which meet in a scratch buffer of the context (partial tiles, at most 256 MiB; grown like the other scratch
+ * buffers: not during a graph capture).  The sums of a result are the same numbers in the same order on every call.
  * Replaces: `LinearX::forward` -> `QMatMul::forward(&Tensor)` (src/models/layers/linear.rs:19-31)
  * -> candle `CustomOp1::cpu_fwd` -> `k_quants::matmul`. */
 int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype, int64_t m,
@@ -186,7 +190,9 @@ int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype
 /* turq_qmatmul for callers that cannot allocate device memory around the call (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
  * reference.  Same product, same kernels and bit-identical results as turq_qmatmul with
- * TURQ_MEM_DEVICE and TURQ_ALGO_AUTO, but the prepared activation fragments of the calls that use them
+ * TURQ_MEM_DEVICE and TURQ_ALGO_AUTO (one exception: where turq_qmatmul gives the columns of every workgroup tile to several
+ * workgroups - see there - this call runs the same kernel unsplit, the same products added in another order: within 2e-6
+ * relative L2 of each other), but the prepared activation fragments of the calls that use them
  * (more than 32 rows, and 17 - 32 rows on all but small weights) live in a static device array of TURQ_NOALLOC_SCRATCH_BYTES (one copy per GPU, held until
  * the process ends) instead of the context's growable buffer: the call runs no hipMalloc / hipFree
  * and creates no stream or event.  A call that needs more is refused with TURQ_ERR_SHAPE and a

@@ -92,6 +92,28 @@ def test_prefill_up_proj(gpu, m):
     assert rel_l2(yb[:, rows], synth.from_bf16_bits(synth.to_bf16_bits(want)).reshape(want.shape)) <= 1.5e-3
 
 
+@pytest.mark.parametrize("m", [64, 128, 256])
+def test_prefill_down_proj_split_columns(gpu, m):
+    # the tall matrix of the layer (Q6_K down_proj 4096 x 12288) at prompt-chunk sizes: few workgroup tiles, so every tile's
+    # columns go to several workgroups whose partial sums meet in device memory (low tile up to 128 rows, wide tile at 256);
+    # the oracle checks every 16th weight row
+    n, k = 4096, 12288
+    raw = synth.random_weight(Q6_K, n, k, seed=45)
+    w = gpu.upload(Q6_K, n, k, raw, capi.LAYOUT_TILED)
+    x = synth.random_activation(m, k, seed=m, bf16=True)
+    y = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    y2 = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    yb = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16)
+    gpu.release(w)
+    rows = np.arange(3, n, 16)
+    sub = raw.reshape(n, -1)[rows].reshape(-1)
+    want = orc.matmul_dequant(Q6_K, x, sub, len(rows), k)
+    assert np.all(np.isfinite(y))
+    assert rel_l2(y[:, rows], want) <= 1e-3
+    assert np.array_equal(y, y2)
+    assert np.array_equal(synth.to_bf16_bits(y).reshape(m, n), synth.to_bf16_bits(yb).reshape(m, n))
+
+
 # BASELINE config 3: one Qwen3-8B decoder layer of a Q4_K_M file
 LAYER = [("q", Q4_K, 4096, 4096), ("k", Q4_K, 1024, 4096), ("v", Q6_K, 1024, 4096), ("o", Q4_K, 4096, 4096),
          ("gate", Q4_K, 12288, 4096), ("up", Q4_K, 12288, 4096), ("down", Q6_K, 4096, 12288)]

@@ -228,6 +228,32 @@ def test_prefill_gemm(gpu, dt, n, k, m):
     gpu.release(w)
 
 
+# Tall-k matrices at prefill chunk sizes (down_proj: 4096 x 12288) make few workgroup tiles, so the launcher gives every tile
+# to several workgroups that each take a part of the columns and meet in device memory.  Shapes that split on a 256-CU device
+# (few tiles, many super-blocks): results against the oracle, twice in a row (the tiles' counters must be back at zero), with
+# bias, row strides, a ragged n and m, and every output type.
+@pytest.mark.parametrize("dt", [Q4_K, Q5_K, Q6_K])
+@pytest.mark.parametrize("n,k,m", [(512, 8192, 128), (200, 6144, 70), (1024, 12288, 300), (256, 4096, 512)])
+def test_prefill_gemm_split_columns(gpu, dt, n, k, m):
+    raw = synth.random_weight(dt, n, k, seed=n + m)
+    x = synth.random_activation(m, k, seed=m, bf16=True)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    dense = orc.matmul_dequant(dt, x, raw, n, k)
+    y = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    assert rel_l2(y, dense) <= 4e-4, rel_l2(y, dense)
+    y2 = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    assert np.array_equal(y, y2)                                # same sums in the same order on every launch
+    bias = np.random.default_rng(2).standard_normal(n).astype(np.float32)
+    yb = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16, bias=bias, ldx=k + 8, ldy=n + 3)
+    assert rel_l2(yb, dense + bias) <= 4e-3
+    ya = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_F16, bias=bias, ldy=n + (-n) % 8 + 8)
+    assert rel_l2(ya, dense + bias) <= 1.2e-3
+    # fewer rows right after: other tiles, other counters
+    y3 = gpu.qmatmul(w, x[: m // 2 + 1], n, k, x_dtype=capi.ACT_BF16)
+    assert rel_l2(y3, dense[: m // 2 + 1]) <= 4e-4
+    gpu.release(w)
+
+
 @pytest.mark.parametrize("dt", [Q4_K, Q5_K, Q6_K, Q8_0])
 def test_prefill_gemm_large_scales_fall_back(gpu, dt):
     # (base + q) * d * sc would overflow f16 inside the GEMM: the dispatcher must take the exact skinny kernel instead
@@ -655,14 +681,17 @@ def test_staged_rows_kernel_group_sizes(row_tiles):
 # The prefill GEMM picks its tile (128 x 128, 128 x 192, the wide 128 x 256 with two-deep rings, or the low 64 x 128 for launches
 # that would leave CUs idle) from the problem size; the small matrices of the tests above would never reach the wide one and
 # always take the low one, so they run once more in child processes with each of the two forced and forbidden (the rule takes
-# the wide tile for some of the full-size cases).
-@pytest.mark.parametrize("switch,value", [("TURQ_GEMM_WIDE", "1"), ("TURQ_GEMM_WIDE", "0"), ("TURQ_GEMM_LOW", "1"), ("TURQ_GEMM_LOW", "0")])
+# the wide tile for some of the full-size cases), and with the columns of every tile split over 2, 4 or 8 workgroups wherever
+# that number divides the super-blocks (on the wide or the low tile), or never.
+@pytest.mark.parametrize("switch,value", [("TURQ_GEMM_WIDE", "1"), ("TURQ_GEMM_WIDE", "0"), ("TURQ_GEMM_LOW", "1"), ("TURQ_GEMM_LOW", "0"),
+                                          ("TURQ_GEMM_SPLIT", "0"), ("TURQ_GEMM_SPLIT+TURQ_GEMM_SPLIT_FORM", "2+3"),
+                                          ("TURQ_GEMM_SPLIT+TURQ_GEMM_SPLIT_FORM", "4+4"), ("TURQ_GEMM_SPLIT", "8")])
 def test_prefill_tile_shapes(switch, value):
     import os
     import subprocess
     import sys
 
-    env = dict(os.environ, **{switch: value})
+    env = dict(os.environ, **dict(zip(switch.split("+"), value.split("+"))))
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "-k", "(prefill or more_rows) and not tile_shapes",
                           "-p", "no:cacheprovider", os.path.join(root, "tests", "test_gpu_qmatmul.py"),

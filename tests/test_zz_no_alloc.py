@@ -3,6 +3,10 @@
 Both run the same kernels, so the outputs must be bit-identical; the only difference is where the prepared activation
 fragments live (a static device array instead of the context's growable buffer).  Two calls in a row, the second with a
 smaller input, per launch kind: prepared fragments (2 <= m <= 32), the prefill GEMM (m > 32), and one row (no scratch).
+One exception: prefill launches whose columns turq_qmatmul splits over several workgroups (few tiles: small or tall matrices
+at prompt-chunk sizes) need a second scratch buffer for the partial tiles, which the call that allocates nothing does not
+have; it runs the same kernel unsplit, i.e. the same products added up in another order, and is held to 2e-6 relative L2
+against turq_qmatmul there (the bar of both against the oracle is 1e-3).
 """
 from __future__ import annotations
 
@@ -46,7 +50,11 @@ def test_noalloc_equals_qmatmul_twice_in_a_row(gpu, dt, n, k, ms):
         for i, m in enumerate(ms):
             x = synth.random_activation(m, k, seed=100 * i + m, bf16=True)
             got, want = both(gpu, w, x, n, k, capi.ACT_BF16, capi.ACT_F32)
-            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (m, "differs from turq_qmatmul")
+            if m > 32 and not np.array_equal(got.view(np.uint32), want.view(np.uint32)):
+                assert (dt, n, k, m) in ((capi.Q4_K, 1024, 4096, 64), (capi.Q5_K, 512, 2048, 33)), "turq_qmatmul splits only these"
+                assert rel_l2(got, want) <= 2e-6, (m, rel_l2(got, want))
+            else:
+                assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (m, "differs from turq_qmatmul")
             rows = np.arange(0, n, max(1, n * m // (1024 * 64)))
             sub = raw.reshape(n, -1)[rows].reshape(-1)
             assert rel_l2(got[:, rows], orc.matmul_dequant(dt, x, sub, len(rows), k)) <= 1e-3, m

@@ -154,6 +154,7 @@ void turq_ctx_destroy(turq_ctx *ctx) {
     if (ctx->act_prep) (void)hipFree(ctx->act_prep);
     if (ctx->gate_up) (void)hipFree(ctx->gate_up);
     if (ctx->mlp_h) (void)hipFree(ctx->mlp_h);
+    if (ctx->gemm_split) (void)hipFree(ctx->gemm_split);
     if (ctx->wide_x) (void)hipFree(ctx->wide_x);
     if (ctx->wide_s) (void)hipFree(ctx->wide_s);
     if (ctx->wide_y) (void)hipFree(ctx->wide_y);

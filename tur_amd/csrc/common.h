@@ -87,6 +87,10 @@ struct turq_ctx {
     void *wide_y = nullptr;   size_t wide_y_cap = 0;
     bool wide = false;  // device-pointer calls take that path too (host-pointer calls always do)
     void *mlp_h = nullptr;    size_t mlp_h_cap = 0;  // turq_mlp: the f32 intermediate act(gate) * up
+    // prefill GEMM launches that split their columns over several workgroups: kSplitSlots counter blocks (zero between
+    // launches; launch i of a call uses block i), then the partial tiles of the call's launches one after the other
+    static constexpr int kSplitSlots = 16;
+    void *gemm_split = nullptr; size_t gemm_split_cap = 0;
     // scratch buffers that were outgrown while a captured graph still referred to them: freed once no graph of the context is
     // alive (at the next growth) or with the context
     std::vector<void *> retired;

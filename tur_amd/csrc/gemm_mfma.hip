@@ -69,6 +69,7 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 constexpr uint32_t kMagic1024 = 0x64006400u;  // 1024.0: a nibble in mantissa bits 0..3 reads as 1024 + n
 constexpr uint32_t kMagic64 = 0x54005400u;    // 64.0:   a nibble in mantissa bits 4..7 reads as 64 + n
 constexpr uint32_t kMagic256 = 0x5C005C00u;   // 256.0:  a 6-bit value in mantissa bits 2..7 reads as 256 + q
+constexpr int kCoherent = 16;                 // cache policy of buffer loads and stores that other XCDs must see: sc1, as device-scope atomics carry
 // A workgroup is 4 waves and covers 128 rows of m (4 m-tiles of 32): as 2 x 2 waves with 2 m-tiles each (WGM = 2), or as
 // 1 x 4 waves that all take the 4 m-tiles (WGM = 1: every weight is unpacked by ONE wave instead of two, at twice the
 // activation reads per wave; for the formats whose unpack is long)
@@ -409,11 +410,22 @@ template <> struct GFmt<TURQ_Q8_0> {
 
 // frags: 32-row fragments, 1 KiB block index (mt * ntc + b) * 17 + q
 // vec_out: rows of y can be written as aligned 16-byte pieces
-template <int DT, int WGM_>
+// SK: the columns (k) of every workgroup tile are split over `split` workgroups (split divides the number of super-blocks).
+// Each of them - wave by wave, a wave meets only the same wave of the others - writes its partial accumulators to `partials`
+// and counts itself in on the tile's counter; the wave that finds all the others counted adds the partial tiles up in part
+// order, stores the results and puts the counter back to zero for the next launch.  Nobody waits
+// for anybody, and the sums of a result are the same numbers in the same order on every run.  The partial tiles are written
+// and read with the cache policy of device-scope atomics (the L2 caches of the XCDs are not coherent with each other), each
+// wave's stores have completed before its increment goes out and the last wave reads only after its own has returned.
+//   partials: [tile][part][wave] blocks of WM * WN KiB x 4 (a wave's accumulators as its lanes hold them), counters: [tile][wave],
+//   zero before the first launch; launches that share them must not overlap.
+template <int DT, int WGM_, bool SK = false>
 __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
                                                       const uint8_t *__restrict__ frags, int64_t m, void *__restrict__ y,
                                                       int yt, int64_t ldy, const float *__restrict__ bias, int nblocks_n,
-                                                      int nblocks_m, int vec_out, float wscale, float inv_ws) {
+                                                      int nblocks_m, int vec_out, float wscale, float inv_ws, int split = 1,
+                                                      uint8_t *__restrict__ partials = nullptr, uint32_t partial_bytes = 0,
+                                                      uint32_t *__restrict__ counters = nullptr) {
     using Fm = GFmt<DT>;
     using G = Geo<DT, WGM_>;
     constexpr int WGN = G::WGN, WM = G::WM, WN = G::WN, TB = G::TB;
@@ -431,11 +443,14 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     const int r16 = n32 & 15, tsel = n32 >> 4;
     // Workgroups of one XCD (blockIdx % 8) get consecutive logical ids and the m-blocks of one n-block are
     // consecutive in that order: the packed weights they share stay in that XCD's L2.
-    const int nwg = nblocks_n * nblocks_m;
+    const int nwg = nblocks_n * nblocks_m * (SK ? split : 1);
     int lid = blockIdx.x;
     if ((nwg & 7) == 0) lid = (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3);
-    const int nb = lid / nblocks_m, mb = lid - nb * nblocks_m;
-    const int ntc = (int)turq_tile_cols(k);
+    // (split: the m-blocks of one n-block and one part are consecutive, they share the part's packed weights)
+    const int mb = lid % nblocks_m, part = SK ? (lid / nblocks_m) % split : 0, nb = lid / (nblocks_m * (SK ? split : 1));
+    const int ntc = (int)turq_tile_cols(k);         // super-blocks of a row: the strides of the weights and of the fragments
+    const int nloc = SK ? ntc / split : ntc;        // ... of this workgroup: kb0 .. kb0 + nloc - 1
+    const int kb0 = part * nloc;
     const int64_t mtiles = (m + 31) / 32;
     const int nrt = (int)turq_tile_rows(n);
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
@@ -449,15 +464,15 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     int64_t my_mt_s = G::LOW ? (int64_t)mb * G::GMT + (wave & 1) : my_mt;
     my_mt_s = my_mt_s < mtiles ? my_mt_s : mtiles - 1;
     const uint32_t a_half = G::LOW ? (uint32_t)(wave & 1) * 2048u : 0u;
-    const uint8_t *a_src = uniform_ptr(frags + ((size_t)(my_mt * ntc * 17) << 10) + a_half);
-    const uint8_t *s_src = uniform_ptr(frags + ((size_t)(my_mt_s * ntc * 17) << 10));
+    const uint8_t *a_src = uniform_ptr(frags + ((size_t)((my_mt * ntc + kb0) * 17) << 10) + a_half);
+    const uint8_t *s_src = uniform_ptr(frags + ((size_t)((my_mt_s * ntc + kb0) * 17) << 10));
     const uint32_t a_dst = lds_base + G::A_OFF + (uint32_t)(G::LOW ? wave >> 1 : wave) * 4096u + a_half;  // + ks * A_STAGE (+ step * 1024)
     const uint32_t s_dst = lds_base + G::S_OFF + (uint32_t)wave * 1024u;  // + (b & 1) * S_BYTES
     // weights: copy c of a super-block covers bytes [1024 c, 1024 c + 1024) of the concatenated tiles of the workgroup;
     // group g = 0..3 holds copies 4g + wave and 16 + 4g + wave (clamped to the last copy; lanes past the end of the
     // tiles re-read the last 16 bytes into the padding of the ring entry)
     const int tile0 = nb * G::NT16;
-    const uint8_t *w_src = uniform_ptr(w + (size_t)tile0 * ntc * TB);  // + b * TB
+    const uint8_t *w_src = uniform_ptr(w + ((size_t)tile0 * ntc + kb0) * TB);  // + b * TB
     // (wide form: copies wave, wave + 4, ... of the super-block, CPW per wave, in two halves)
     constexpr int NG = G::WIDE ? G::CPW : 4, NI = G::WIDE ? 1 : 2;
     uint32_t w_voff[NG][NI];
@@ -519,7 +534,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
     // ---- prologue: super-block 0 complete, weights of 1 and the first group of 2 on their way ----
-    const int last = ntc - 1;
+    const int last = nloc - 1;
     if constexpr (G::WIDE) {
         // stages 0 and 1 and the weights of super-block 0 complete, the first half of super-block 1 on its way
         issue_a(0, 0);
@@ -560,7 +575,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
         cs[j] = Fm::consts(hd[j], g32, ws);
     }
 
-    for (int b = 0; b < ntc; b++) {
+    for (int b = 0; b < nloc; b++) {
         const uint32_t s_cur = s_rd + (uint32_t)(b & 1) * S_BYTES;
         const int b1 = b + 1 < last ? b + 1 : last, b2 = b + 2 < last ? b + 2 : last, b3 = b + 3 < last ? b + 3 : last;
         static_for<4>([&](auto KS) {  // the four stages of the super-block: ks selects registers, buffers and offsets
@@ -685,6 +700,79 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
+    if constexpr (SK) {
+        // ---- the parts of a tile meet (no workgroup barrier from here on: a wave may leave alone) ----
+        constexpr int NB = WM * WN * 4;                 // 1 KiB blocks of a wave's partial tile (16 bytes per lane each)
+        constexpr uint32_t WAVE_BYTES = NB * 1024u;
+        constexpr int PB = NB >= 32 ? 1 : 32 / NB;      // parts read together: 128 registers of loads in flight per lane
+        const int tile = nb * nblocks_m + mb;
+        uint32_t *cnt = counters + tile * 4 + wave;
+        const __amdgpu_buffer_rsrc_t prs = __builtin_amdgcn_make_buffer_rsrc(partials, 0, (int)partial_bytes, 0x00020000);
+        const uint32_t tile_base = (uint32_t)(tile * split) * (4u * WAVE_BYTES) + (uint32_t)wave * WAVE_BYTES + lane_off;
+        const uint32_t mine = tile_base + (uint32_t)part * (4u * WAVE_BYTES);
+#pragma unroll
+        for (int i = 0; i < WM; i++)
+#pragma unroll
+            for (int j = 0; j < WN; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4v v = float4v{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uint4v, v), prs, mine + (uint32_t)((i * WN + j) * 4 + q) * 1024u, 0,
+                                                           kCoherent);
+                }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        uint32_t ticket = 0;
+        if (lane == 0) ticket = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        if (__builtin_amdgcn_readfirstlane(ticket) != (uint32_t)(split - 1)) return;
+        // the last one in: every part's tile, its own from its registers, added in part order
+        float16v sum[WM][WN];
+#pragma unroll
+        for (int i = 0; i < WM; i++)
+#pragma unroll
+            for (int j = 0; j < WN; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) sum[i][j][e] = 0.0f;
+        for (int p0 = 0; p0 < split; p0 += PB) {
+            if (PB == 1 && p0 == part) {
+#pragma unroll
+                for (int i = 0; i < WM; i++)
+#pragma unroll
+                    for (int j = 0; j < WN; j++) sum[i][j] += acc[i][j];
+                continue;
+            }
+            // (several parts at once: the wave's own among them, as it has just written it; parts past the last: the last
+            // one again, not added)
+            uint4v v[PB][NB];
+#pragma unroll
+            for (int b = 0; b < PB; b++) {
+                const uint32_t from = tile_base + (uint32_t)(p0 + b < split ? p0 + b : split - 1) * (4u * WAVE_BYTES);
+#pragma unroll
+                for (int t = 0; t < NB; t++) v[b][t] = __builtin_amdgcn_raw_buffer_load_b128(prs, from + (uint32_t)t * 1024u, 0, kCoherent);
+            }
+#pragma unroll
+            for (int b = 0; b < PB; b++) {
+                if (p0 + b >= split) break;
+#pragma unroll
+                for (int i = 0; i < WM; i++)
+#pragma unroll
+                    for (int j = 0; j < WN; j++)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) {
+                            const float4v f = __builtin_bit_cast(float4v, v[b][(i * WN + j) * 4 + q]);
+                            sum[i][j][4 * q] += f.x;
+                            sum[i][j][4 * q + 1] += f.y;
+                            sum[i][j][4 * q + 2] += f.z;
+                            sum[i][j][4 * q + 3] += f.w;
+                        }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < WM; i++)
+#pragma unroll
+            for (int j = 0; j < WN; j++) acc[i][j] = sum[i][j];
+        if (lane == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
     // ---- results ----
     // 32x32 result: lane (n32, g32), register e holds row 8 * (e / 4) + 4 * g32 + e % 4 of column n32
     constexpr int OUT_PITCH = G::OUT_PITCH;
@@ -753,41 +841,52 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     }
 }
 
-template <int DT, int WGM_>
+// split > 1: the columns of every tile over `split` workgroups that meet in `partials`, counted on `counters`
+// (kSplitCounterBytes, zero between launches)
+constexpr size_t kSplitCounterBytes = TURQ_GEMM_SPLIT_COUNTER_BYTES;
+template <int DT, int WGM_, bool SK = false>
 hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y, int y_dtype, int64_t ldy,
-                       const float *bias, float wscale, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+                       const float *bias, float wscale, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop, int split = 1,
+                       void *counters = nullptr, void *partials = nullptr, size_t partials_cap = 0) {
     using G = Geo<DT, WGM_>;
     constexpr int RING_BYTES = G::S_OFF + (GFmt<DT>::SUMS ? NS * S_BYTES : 0), STAGING_BYTES = 4 * G::WM * 32 * G::OUT_PITCH * 4;
     constexpr int LDS_BYTES = RING_BYTES > STAGING_BYTES ? RING_BYTES : STAGING_BYTES;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS of one workgroup: the rings, or the staged results after the main loop");
     // per-lane weight offsets are 32-bit
     if ((uint64_t)G::NT16 * (uint64_t)(k / 256) * G::TB >= (1ull << 32)) return hipErrorInvalidValue;
-    const hipError_t attr = turq_raise_lds_limit((const void *)gemm_kq_kernel<DT, WGM_>, LDS_BYTES);
+    const hipError_t attr = turq_raise_lds_limit((const void *)gemm_kq_kernel<DT, WGM_, SK>, LDS_BYTES);
     if (attr != hipSuccess) return attr;
     const int nbn = (int)((n + G::BN - 1) / G::BN), nbm = (int)((m + G::GBM - 1) / G::GBM);
-    const dim3 grid((unsigned)(nbn * nbm)), block(256);
+    size_t partial_bytes = 0;
+    if constexpr (SK) {
+        partial_bytes = (size_t)nbn * nbm * split * (size_t)(G::WM * G::WN * 4 * 4096);
+        if (split < 2 || (k / 256) % split != 0 || !counters || !partials || (size_t)nbn * nbm * 16 > kSplitCounterBytes ||
+            partial_bytes >= (1ull << 31) || partial_bytes > partials_cap)
+            return hipErrorInvalidValue;
+    } else {
+        split = 1;
+    }
+    const dim3 grid((unsigned)(nbn * nbm * split)), block(256);
     const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
     const int vec_out = ((uintptr_t)y % 16 == 0 && ((uint64_t)ldy * es) % 16 == 0 && n % 8 == 0) ? 1 : 0;
     if (ev_start) {
-        hipExtLaunchKernelGGL((gemm_kq_kernel<DT, WGM_>), grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
-                              (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale);
+        hipExtLaunchKernelGGL((gemm_kq_kernel<DT, WGM_, SK>), grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
+                              (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale, split,
+                              (uint8_t *)partials, (uint32_t)partial_bytes, (uint32_t *)counters);
     } else {
-        gemm_kq_kernel<DT, WGM_><<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype,
-                                                                      ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale);
+        gemm_kq_kernel<DT, WGM_, SK><<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype,
+                                                                          ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale, split,
+                                                                          (uint8_t *)partials, (uint32_t)partial_bytes, (uint32_t *)counters);
     }
     return hipGetLastError();
 }
 
 }  // namespace
 
-// frags: activations prepared by turq_launch_act_prep32 (in the order of the same dtype) for all m rows
-// wscale: a power of two in [2^-14, 2^15] by which the kernel multiplies every block scale; compute_units: CUs of the device
-// (0: unknown), for the choice of the tile shape
-hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
-                                 int y_dtype, int64_t ldy, const float *bias, float wscale, int compute_units, hipStream_t stream,
-                                 hipEvent_t ev_start, hipEvent_t ev_stop) {
-    if (n == 0 || m == 0) return hipSuccess;
-    if (k <= 0 || k % 256 != 0 || !(wscale >= 6.103515625e-5f && wscale <= 32768.0f)) return hipErrorInvalidValue;
+// The workgroup tile of a launch: 1: 128 x 128 (1 x 4 waves), 2: 2 x 2 waves (Q4_K 128 x 192, Q8_0 128 x 64), 3: wide 128 x 256,
+// 4: low 64 x 128; 0: no kernel for this format.  compute_units: CUs of the device (0: unknown).
+int turq_gemm_form(int dtype, int64_t n, int64_t k, int64_t m, int compute_units) {
+    (void)k;
     static const bool tall = getenv("TURQ_GEMM_GRID_2X2") == nullptr;  // Q5_K / Q6_K: 1 x 4 waves unless told otherwise
     // The wide tile (128 x 256, Geo<.., 3>) pulls fewer activation bytes through the L2 per flop (Q4_K: + 12 % at m = 2048 and
     // 4096; LM head Q5_K / Q6_K: + 4 .. 21 % from m = 64 to 512) but makes fewer, larger workgroups: it is taken where its
@@ -812,32 +911,116 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
     const int64_t wgs128 = ((n + 127) / 128) * ((m + BM - 1) / BM);
     // (up to 64 rows the low tile is the whole problem's height: half the MFMA work and activation traffic of a 128-row tile)
     const bool low = low_env >= 0 ? low_env == 1 : (m <= 64 || 2 * wgs128 <= cus);
-    if (low && wide_env != 1) {
-        switch (dtype) {
-        case TURQ_Q4_K: return launch_gemm<TURQ_Q4_K, 4>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-        case TURQ_Q5_K: return launch_gemm<TURQ_Q5_K, 4>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-        case TURQ_Q6_K: return launch_gemm<TURQ_Q6_K, 4>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-        default: break;
-        }
-    }
+    const bool kq = dtype == TURQ_Q4_K || dtype == TURQ_Q5_K || dtype == TURQ_Q6_K;
+    if (low && wide_env != 1 && kq) return 4;
     switch (dtype) {
     case TURQ_Q4_K:
-        if (wide_env == 1) return launch_gemm<TURQ_Q4_K, 3>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+        if (wide_env == 1) return 3;
         // 128 x 192 tiles of 2 x 2 waves, unless the 128 x 128 tiles of the 1 x 4 grid still fit the machine in one round:
         // then there are half as many again to spread (m = 128: 96 workgroups instead of 64, 34 us instead of 45)
-        if (compute_units > 0 && ((n + 127) / 128) * ((m + BM - 1) / BM) <= compute_units)
-            return launch_gemm<TURQ_Q4_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-        if (pick_wide(192, 1.10)) return launch_gemm<TURQ_Q4_K, 3>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-        return launch_gemm<TURQ_Q4_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+        if (compute_units > 0 && wgs128 <= compute_units) return 1;
+        return pick_wide(192, 1.10) ? 3 : 2;
     case TURQ_Q5_K:
-        if (pick_wide(128, 1.25)) return launch_gemm<TURQ_Q5_K, 3>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-        if (tall) return launch_gemm<TURQ_Q5_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-        return launch_gemm<TURQ_Q5_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-    case TURQ_Q6_K:
-        if (pick_wide(128, 1.25)) return launch_gemm<TURQ_Q6_K, 3>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-        if (tall) return launch_gemm<TURQ_Q6_K, 1>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-        return launch_gemm<TURQ_Q6_K, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
-    case TURQ_Q8_0: return launch_gemm<TURQ_Q8_0, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop);
+    case TURQ_Q6_K: return pick_wide(128, 1.25) ? 3 : tall ? 1 : 2;
+    case TURQ_Q8_0: return 2;
+    default: return 0;
+    }
+}
+
+// ---- which launches split their columns ----
+// A launch whose tiles leave most CUs idle - the tall-k matrices of a model at prefill chunk sizes (down_proj 4096 x 12288 makes
+// 32 low tiles at 64 rows, 64 wide ones at 512), and every matrix of the layer at 64 rows - gives every tile to `split`
+// workgroups.  What the parts' meeting costs grows with the partial tiles the launch writes and reads back (m x n x 4 bytes
+// x (2 split - 1)), so the rule takes the low tile for few rows and the wide one above, and only as many parts as leave a
+// quarter of the CUs free (low tiles; half of them when k is short, and then only up to 128 rows: less to win) or fill them
+// once (wide tiles, up to an eighth of the CUs).  Measured on MI355X, Q6_K 4096 x 12288, no split -> split: 64 rows 75 -> 35 us
+// (low, 6 parts), 128: 78 -> 47 (low, 3), 256: 82 -> 66 (wide, 6), 512: 97 -> 92 (wide, 4: within what a whole layer's step
+// varies by, not taken), 1024: none helps; Q4_K 4096 x 4096: 64 rows 28 -> 22 us (low, 4), 128: 28 -> 27 (low, 2), from 256
+// rows on none helps; 12288 x 4096: none helps.  TURQ_GEMM_SPLIT = 0: never, s > 1: by s wherever s divides (with
+// TURQ_GEMM_SPLIT_FORM = 3 / 4: on the wide / low tile).
+size_t turq_gemm_split_scratch(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int *form_out, int *split_out) {
+    if (form_out) *form_out = 0;
+    if (split_out) *split_out = 1;
+    static const int env = [] { const char *e = getenv("TURQ_GEMM_SPLIT"); return e ? atoi(e) : -1; }();
+    static const int env_form = [] { const char *e = getenv("TURQ_GEMM_SPLIT_FORM"); return e ? atoi(e) : 0; }();
+    if (env == 0 || compute_units <= 0 || (dtype != TURQ_Q4_K && dtype != TURQ_Q5_K && dtype != TURQ_Q6_K)) return 0;
+    const int64_t cus = compute_units, ntc = k / 256;
+    const int64_t low_tiles = ((n + 127) / 128) * ((m + 63) / 64), wide_tiles = ((n + 255) / 256) * ((m + 127) / 128);
+    // the most parts that divide the super-blocks, leave each part at least min_sb of them and make at most max_wgs workgroups
+    auto parts = [&](int64_t tiles, int64_t max_wgs, int64_t min_sb) {
+        int best = 1;
+        for (int s = 2; s <= 8; s++)
+            if (ntc % s == 0 && ntc / s >= min_sb && tiles * s <= max_wgs) best = s;
+        return best;
+    };
+    int form = 0, split = 1;
+    if (env > 1) {
+        form = env_form == 3 || env_form == 4 ? env_form : (m <= 128 ? 4 : 3);
+        split = ntc % env == 0 ? env : 1;
+    } else {
+        const bool tall = ntc >= 32;
+        split = tall || m <= 128 ? parts(low_tiles, tall ? 3 * cus / 4 : cus / 2, 4) : 1;
+        form = 4;
+        if (split == 1 && tall && 8 * wide_tiles <= cus) {
+            split = parts(wide_tiles, cus, 8);
+            form = 3;
+        }
+    }
+    if (split < 2) return 0;
+    const int64_t bm = form == 4 ? 64 : 128, bn = form == 4 ? 128 : 256;
+    const size_t tiles = (size_t)(form == 4 ? low_tiles : wide_tiles), bytes = tiles * (size_t)split * (size_t)(bm * bn * 4);
+    if (tiles * 16 > kSplitCounterBytes || bytes > (256u << 20)) return 0;
+    if (form_out) *form_out = form;
+    if (split_out) *split_out = split;
+    return bytes;
+}
+
+// frags: activations prepared by turq_launch_act_prep32 (in the order of the same dtype) for all m rows
+// wscale: a power of two in [2^-14, 2^15] by which the kernel multiplies every block scale; compute_units: CUs of the device
+// (0: unknown), for the choice of the tile shape
+hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
+                                 int y_dtype, int64_t ldy, const float *bias, float wscale, int compute_units, hipStream_t stream,
+                                 hipEvent_t ev_start, hipEvent_t ev_stop, void *split_counters, void *split_partials,
+                                 size_t split_partial_bytes) {
+    if (n == 0 || m == 0) return hipSuccess;
+    if (k <= 0 || k % 256 != 0 || !(wscale >= 6.103515625e-5f && wscale <= 32768.0f)) return hipErrorInvalidValue;
+    const int form = turq_gemm_form(dtype, n, k, m, compute_units);
+    if (form == 0) return hipErrorInvalidValue;
+    if (split_counters && split_partials) {
+        int sform = 0, split = 1;
+        const size_t need = turq_gemm_split_scratch(dtype, n, k, m, compute_units, &sform, &split);
+        if (need != 0 && need <= split_partial_bytes) {
+#define TURQ_GEMM_SK(DT, F)                                                                                                           \
+    return launch_gemm<DT, F, true>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop, split, split_counters, \
+                                    split_partials, split_partial_bytes)
+            switch (dtype * 8 + sform) {
+            case TURQ_Q4_K * 8 + 3: TURQ_GEMM_SK(TURQ_Q4_K, 3);
+            case TURQ_Q4_K * 8 + 4: TURQ_GEMM_SK(TURQ_Q4_K, 4);
+            case TURQ_Q5_K * 8 + 3: TURQ_GEMM_SK(TURQ_Q5_K, 3);
+            case TURQ_Q5_K * 8 + 4: TURQ_GEMM_SK(TURQ_Q5_K, 4);
+            case TURQ_Q6_K * 8 + 3: TURQ_GEMM_SK(TURQ_Q6_K, 3);
+            case TURQ_Q6_K * 8 + 4: TURQ_GEMM_SK(TURQ_Q6_K, 4);
+            default: break;
+            }
+#undef TURQ_GEMM_SK
+        }
+    }
+#define TURQ_GEMM(DT, F) return launch_gemm<DT, F>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop)
+    switch (dtype * 8 + form) {
+    case TURQ_Q4_K * 8 + 1: TURQ_GEMM(TURQ_Q4_K, 1);
+    case TURQ_Q4_K * 8 + 2: TURQ_GEMM(TURQ_Q4_K, 2);
+    case TURQ_Q4_K * 8 + 3: TURQ_GEMM(TURQ_Q4_K, 3);
+    case TURQ_Q4_K * 8 + 4: TURQ_GEMM(TURQ_Q4_K, 4);
+    case TURQ_Q5_K * 8 + 1: TURQ_GEMM(TURQ_Q5_K, 1);
+    case TURQ_Q5_K * 8 + 2: TURQ_GEMM(TURQ_Q5_K, 2);
+    case TURQ_Q5_K * 8 + 3: TURQ_GEMM(TURQ_Q5_K, 3);
+    case TURQ_Q5_K * 8 + 4: TURQ_GEMM(TURQ_Q5_K, 4);
+    case TURQ_Q6_K * 8 + 1: TURQ_GEMM(TURQ_Q6_K, 1);
+    case TURQ_Q6_K * 8 + 2: TURQ_GEMM(TURQ_Q6_K, 2);
+    case TURQ_Q6_K * 8 + 3: TURQ_GEMM(TURQ_Q6_K, 3);
+    case TURQ_Q6_K * 8 + 4: TURQ_GEMM(TURQ_Q6_K, 4);
+    case TURQ_Q8_0 * 8 + 2: TURQ_GEMM(TURQ_Q8_0, 2);
     default: return hipErrorInvalidValue;
     }
+#undef TURQ_GEMM
 }

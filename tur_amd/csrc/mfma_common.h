@@ -214,6 +214,16 @@ hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int 
                                        int64_t k, const void *x, int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype,
                                        const int64_t *ldy, const float *const *bias, int waves_per_group, hipStream_t stream,
                                        hipEvent_t ev_start, hipEvent_t ev_stop);
+// split_counters, split_partials (may be null: no launch splits its columns): TURQ_GEMM_SPLIT_COUNTER_BYTES of counters that were
+// zero before the first launch that used them (every launch leaves them at zero), and turq_gemm_split_scratch(...) bytes for the
+// partial tiles; launches that share either must not overlap
 hipError_t turq_launch_gemm_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *frags, int64_t m, void *y,
                                  int y_dtype, int64_t ldy, const float *bias, float wscale, int compute_units, hipStream_t stream,
-                                 hipEvent_t ev_start, hipEvent_t ev_stop);
+                                 hipEvent_t ev_start, hipEvent_t ev_stop, void *split_counters = nullptr, void *split_partials = nullptr,
+                                 size_t split_partial_bytes = 0);
+constexpr size_t TURQ_GEMM_SPLIT_COUNTER_BYTES = 64 << 10;
+// the workgroup tile the launch rules pick (0: no kernel for the format)
+int turq_gemm_form(int dtype, int64_t n, int64_t k, int64_t m, int compute_units);
+// bytes of partial tiles a launch of this shape wants for splitting its columns, 0 if it does not split; form_out / split_out
+// (may be null): the tile (3: wide, 4: low) and the number of parts
+size_t turq_gemm_split_scratch(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int *form_out, int *split_out);

@@ -166,10 +166,50 @@ static bool side_ready(turq_ctx *ctx) {
     return true;
 }
 
+// Scratch for the prefill GEMM launches of one call that split their columns over several workgroups: launch i gets counter
+// block i and its own stretch of partial tiles (launches of one call may run next to each other), counters[i] null where
+// launch i does not split or the call may not allocate.  The counter blocks are cleared when the buffer is allocated and
+// left at zero by every launch; calls on the context's stream follow each other, so they share the buffer.
+struct GemmSplit {
+    void *counters[turq_ctx::kSplitSlots] = {};
+    void *partials[turq_ctx::kSplitSlots] = {};
+    size_t bytes[turq_ctx::kSplitSlots] = {};
+};
+static int gemm_split_reserve(turq_ctx *ctx, int count, const turq_weight *const *w, int64_t m, GemmSplit *out) {
+    *out = GemmSplit{};
+    if (ctx->fixed_scratch || count > turq_ctx::kSplitSlots) return TURQ_OK;
+    constexpr size_t kCounters = (size_t)turq_ctx::kSplitSlots * TURQ_GEMM_SPLIT_COUNTER_BYTES;
+    size_t off[turq_ctx::kSplitSlots], total = kCounters;
+    bool any = false;
+    for (int i = 0; i < count; i++) {
+        out->bytes[i] = turq_gemm_split_scratch(w[i]->dtype, w[i]->n, w[i]->k, m, ctx->compute_units, nullptr, nullptr);
+        off[i] = total;
+        total += (out->bytes[i] + 255) & ~(size_t)255;
+        any = any || out->bytes[i] != 0;
+    }
+    if (!any) return TURQ_OK;
+    if (total > ctx->gemm_split_cap) {
+        int rc = turq_ctx_reserve(ctx, &ctx->gemm_split, &ctx->gemm_split_cap, total);
+        if (rc != TURQ_OK) return rc;
+        TURQ_HIP(ctx, hipMemsetAsync(ctx->gemm_split, 0, kCounters, ctx->stream));  // (never inside a capture: growing is refused there)
+    }
+    for (int i = 0; i < count; i++) {
+        if (out->bytes[i] == 0) continue;
+        out->counters[i] = (uint8_t *)ctx->gemm_split + (size_t)i * TURQ_GEMM_SPLIT_COUNTER_BYTES;
+        out->partials[i] = (uint8_t *)ctx->gemm_split + off[i];
+    }
+    return TURQ_OK;
+}
+
 // CUs that the GEMM launch for [m, n] takes: its workgroups, by the launcher's choice between the 64-row tile (two of those
 // workgroups share a CU) and the 128-row tiles (one per CU; wide tiles counted as two).  Measured on the Q4_K_M layer: launches
 // of 192 workgroups next to each other help with the 64-row tile (m = 128: +4.8 %) and hurt with the 128-row tile (m = 256: -2.7 %).
-static int64_t gemm_cus_taken(const turq_ctx *ctx, const turq_weight *w, int64_t m) {
+static int64_t gemm_cus_taken(const turq_ctx *ctx, const turq_weight *w, int64_t m, bool may_split) {
+    int form = 0, split = 1;
+    if (may_split && turq_gemm_split_scratch(w->dtype, w->n, w->k, m, ctx->compute_units, &form, &split) != 0) {
+        const int64_t tiles = form == 4 ? ((w->n + 127) / 128) * ((m + 63) / 64) : ((w->n + 255) / 256) * ((m + 127) / 128);
+        return form == 4 ? (tiles * split + 1) / 2 : tiles * split;
+    }
     const int64_t nt = (w->n + 127) / 128, wgs128 = ((m + 127) / 128) * nt;
     const bool low = m <= 64 || 2 * wgs128 <= ctx->compute_units;
     return low ? (((m + 63) / 64) * nt + 1) / 2 : wgs128;
@@ -184,6 +224,9 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
         if (!gemm_takes(w[i], &ws[i])) return TURQ_OK;
     int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep32_bytes(m, w[0]->k));
     if (rc != TURQ_OK) return rc;
+    GemmSplit sp;
+    rc = gemm_split_reserve(ctx, count, w, m, &sp);
+    if (rc != TURQ_OK) return rc;
     // k_proj / v_proj of a prompt chunk are launches of a quarter of the machine each.  Launches that leave half of the CUs free
     // run in groups, as many as fit the machine together (three at most): the first of a group on the context's stream, the
     // others on further streams that start where it starts (an event recorded there; behind the preparation, the only thing
@@ -194,7 +237,7 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
     int n_small = 0;
     bool one_order = true;
     for (int i = 0; i < count; i++) {
-        n_small += 2 * gemm_cus_taken(ctx, w[i], m) <= cus;
+        n_small += 2 * gemm_cus_taken(ctx, w[i], m, sp.counters[i] != nullptr) <= cus;
         one_order = one_order && (w[i]->dtype == TURQ_Q8_0) == (w[0]->dtype == TURQ_Q8_0);
     }
     const bool fork = !no_side && one_order && n_small >= 2 && side_ready(ctx);
@@ -211,7 +254,7 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
             prepared = order;
         }
         hipStream_t st = ctx->stream;
-        const int64_t c = gemm_cus_taken(ctx, w[i], m);
+        const int64_t c = gemm_cus_taken(ctx, w[i], m, sp.counters[i] != nullptr);
         if (fork && 2 * c <= cus) {
             if (group_n == 0 || group_n > turq_ctx::kSide || group_cus + c > cus) {
                 e = hipEventRecord(ctx->ev_fork, ctx->stream);  // opens a group
@@ -232,7 +275,8 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
         e = turq_prof_next(ctx, &ev0, &ev1);
         if (e == hipSuccess)
             e = turq_launch_gemm_mfma(w[i]->dtype, w[i]->dev, w[i]->n, w[i]->k, ctx->act_prep, m, y[i], yt, ldy[i],
-                                      bias ? bias[i] : nullptr, ws[i], ctx->compute_units, st, ev0, ev1);
+                                      bias ? bias[i] : nullptr, ws[i], ctx->compute_units, st, ev0, ev1, sp.counters[i], sp.partials[i],
+                                      sp.bytes[i]);
     }
     for (int s = 0; s < turq_ctx::kSide; s++) {  // also after an error: nothing may stay behind on the other streams
         if (!used[s]) continue;
@@ -259,10 +303,14 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
     if (m > TURQ_GEMV_MAX_M && algo == TURQ_ALGO_GEMM) {
         int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep32_bytes(m, w->k));
         if (rc != TURQ_OK) return rc;
+        GemmSplit sp;
+        rc = gemm_split_reserve(ctx, 1, &w, m, &sp);
+        if (rc != TURQ_OK) return rc;
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
         TURQ_HIP(ctx, turq_launch_act_prep32(w->dtype, x, xt, m, w->k, ldx, ctx->act_prep, ctx->stream));
         TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
-        TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, wscale, ctx->compute_units, ctx->stream, ev0, ev1));
+        TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, wscale, ctx->compute_units,
+                                            ctx->stream, ev0, ev1, sp.counters[0], sp.partials[0], sp.bytes[0]));
         return TURQ_OK;
     }
     const int nwaves = pick_waves(ctx, w->n, w->k);
