@@ -308,7 +308,7 @@ class Bench:
             roofline = {
                 "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                "kernel": "gemv_row1_kernel" if self.m == 1 else "gemv_multi_frag_kernel / gemv_multi_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
+                "kernel": "gemv_row1_kernel" if self.m == 1 else "gemv_cs_staged_kernel / gemv_multi_frag_kernel" if self.m > 2 else "gemv_row1_kernel / gemv_multi_kernel", "avg_launch_us": round(avg_us, 3), "launches_timed": n_launch.value,
                 "algorithmic_bytes_per_launch": int(bytes_per_launch),
             }
             value, unit = gbps, "GB/s"
