@@ -129,14 +129,16 @@ def layer(gpu):
 
 
 @pytest.mark.parametrize("x_dtype", [capi.ACT_F32, capi.ACT_BF16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("m", [1, 4, 8, 16, 32])
+@pytest.mark.parametrize("m", [1, 4, 8, 16, 32, 40, 64])
 def test_q4km_decoder_layer_grouped_calls(gpu, layer, m, x_dtype):
     # the layer's seven linears driven as the reference's decoder layer drives them (src/models/qwen3.rs:272-274, 161-167):
     # q / k / v on one tensor through turq_qmatmul_multi (two formats in one launch), o_proj alone, gate / up through
     # turq_qmatmul_multi, down_proj alone; device pointers, every output against the f32 matmul on the dequantized weights
     raws, ws = layer
+    # (40 and 64 rows: gate / up in two chunks through the kernels of up to 32 rows, the others through the prefill GEMM, whose
+    # folded f16 scales cost about 3e-4; down_proj, o_proj and q / k / v with their columns split over several workgroups)
     bf = x_dtype == capi.ACT_BF16
-    bar = 2e-5 if bf else 1e-3
+    bar = 2e-5 if bf and m <= 32 else 1e-3
     shape = {lb: (dt, n, k) for lb, dt, n, k in LAYER}
     for gi, group in enumerate((("q", "k", "v"), ("o",), ("gate", "up"), ("down",))):
         k = shape[group[0]][2]
@@ -149,7 +151,7 @@ def test_q4km_decoder_layer_grouped_calls(gpu, layer, m, x_dtype):
         for lb, y in zip(group, outs):
             dt, n, _ = shape[lb]
             assert y.shape == (m, n)
-            assert rel_l2(y, orc.matmul_dequant(dt, x, raws[lb], n, k)) <= bar, (lb, m)
+            assert rel_l2(y, orc.matmul_dequant(dt, x, raws[lb], n, k)) <= (2e-5 if bf and lb in ("gate", "up") else bar), (lb, m)
 
 
 def test_mlp_gate_up_and_token_embd(gpu):
@@ -162,7 +164,7 @@ def test_mlp_gate_up_and_token_embd(gpu):
     raw_u = synth.random_weight(Q4_K, n, k, seed=2)
     wg = gpu.upload(Q4_K, n, k, raw_g, capi.LAYOUT_TILED)
     wu = gpu.upload(Q4_K, n, k, raw_u, capi.LAYOUT_TILED)
-    for m in (1, 2, 5, 16, 17, 32):
+    for m in (1, 2, 5, 16, 17, 32, 33, 64):      # (33, 64: two chunks of up to 32 rows)
         x = synth.random_activation(m, k, seed=40 + m, bf16=True)
         y = gpu.gate_up(wg, wu, x, n, k, x_dtype=capi.ACT_BF16)
         want = onp.silu_mul(orc.matmul_dequant(Q4_K, x, raw_g, n, k), orc.matmul_dequant(Q4_K, x, raw_u, n, k))

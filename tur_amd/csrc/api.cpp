@@ -1,4 +1,5 @@
 // C ABI of libturq: contexts, device memory helpers, weight upload/export, dequantize, forward.
+#include <algorithm>
 #include <cmath>
 #include <memory>
 #include <new>
@@ -452,7 +453,7 @@ static int qmatmul_device(turq_ctx *ctx, const turq_weight *w, const void *x, in
                           int yt, int64_t ldy, const float *bias, int algo, bool wide) {
     if (algo == TURQ_ALGO_AUTO) {
         if (w->layout == TURQ_LAYOUT_NATIVE) algo = TURQ_ALGO_SIMPLE;
-        else algo = (m <= TURQ_GEMV_MAX_M) ? TURQ_ALGO_GEMV : TURQ_ALGO_GEMM;
+        else algo = (m <= TURQ_GEMV_MAX_M || turq_rows_in_chunks(ctx, 1, &w, x, xt, ldx, m)) ? TURQ_ALGO_GEMV : TURQ_ALGO_GEMM;
     }
     if (wide && !ctx->fixed_scratch && xt != TURQ_ACT_F16 && (algo == TURQ_ALGO_GEMV || algo == TURQ_ALGO_GEMM) &&
         w->layout == TURQ_LAYOUT_TILED && m <= 65535) {
@@ -548,6 +549,16 @@ static int impl_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const
     }
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
     one_launch = one_launch && xb && yb && ldx >= weights[0]->k;
+    if (one_launch && many_rows && turq_rows_in_chunks(ctx, count, weights, x, xt, ldx, m)) {
+        void *yc[4];
+        for (int64_t m0 = 0; m0 < m; m0 += TURQ_GEMV_MAX_M) {
+            for (int i = 0; i < count; i++) yc[i] = (uint8_t *)ys[i] + (size_t)m0 * (size_t)ldys[i] * yb;
+            const int rc = turq_qmatmul_multi_mfma(ctx, count, weights, (const uint8_t *)x + (size_t)m0 * (size_t)ldx * xb, xt,
+                                                   std::min<int64_t>(TURQ_GEMV_MAX_M, m - m0), ldx, yc, yt, ldys, biases);
+            if (rc != TURQ_OK) return rc;
+        }
+        return TURQ_OK;
+    }
     if (one_launch && many_rows) {
         // prefill: one preparation of the activations for all the weights, then a GEMM each
         bool taken = false;

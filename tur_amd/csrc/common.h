@@ -198,6 +198,8 @@ hipError_t turq_launch_silu_mul(const float *gate, const float *up, int64_t m, i
 // act(gate) * up inside the one-row kernel; *taken = false (and nothing launched) where that kernel does not apply
 int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m,
                               int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, bool *taken);
+// whether a call of 33 .. 64 rows on these weights goes through the kernels of up to 32 rows in two chunks
+bool turq_rows_in_chunks(const turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t ldx, int64_t m);
 int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m, int64_t ldx,
                             void *const *y, int yt, const int64_t *ldy, const float *const *bias, bool *taken);
 int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m,

@@ -348,10 +348,48 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
 
 // gate_proj and up_proj of an MLP with the activation and the product in the kernel: one or two activation rows (two: on
 // weights large enough for the one-row kernel, as in row1_takes), tiled weights of one format, 16-byte aligned rows
+// 33 .. 64 rows against weights of more than two row tiles per compute unit and up to 4096 columns (gate / up of an 8B model):
+// two passes of the four-wave staged kernel (up to 32 rows each) stream the weights twice and still beat the prefill GEMM,
+// which at these row counts makes few, half-empty tiles (gate + up 12288 x 4096 at 64 rows: 2 x 24 us against 62 us for
+// two GEMM launches, plus the preparation launch and, fused, the elementwise pass that the staged kernel has in its epilogue).
+// TURQ_ROWS_IN_CHUNKS = 0 switches it off.
+bool turq_rows_in_chunks(const turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t ldx, int64_t m) {
+    static const bool off = [] { const char *e = getenv("TURQ_ROWS_IN_CHUNKS"); return e && atoi(e) == 0; }();
+    if (off || m <= TURQ_GEMV_MAX_M || m > 2 * TURQ_GEMV_MAX_M || count < 1 || count > 4) return false;
+    const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
+    const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
+    int64_t row_tiles = 0;
+    for (int i = 0; i < count; i++) {
+        if (!turq_dt_is_quant(w[i]->dtype) || w[i]->dtype == TURQ_Q8_0 || w[i]->dtype != w[0]->dtype || w[i]->layout != TURQ_LAYOUT_TILED ||
+            w[i]->k != w[0]->k)
+            return false;
+        row_tiles += turq_tile_rows(w[i]->n);
+    }
+    if (row_tiles <= 2 * cus) return false;
+    return staged_row_tiles(ctx, w[0]->dtype, w[0]->dtype, w[0]->k, TURQ_GEMV_MAX_M, row_tiles, 0, aligned) == 6;
+}
+
 int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m,
                               int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, bool *taken) {
     static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
     *taken = false;
+    {
+        const turq_weight *pair[2] = {gate, up};
+        if (m > TURQ_GEMV_MAX_M && gate->n == up->n && turq_rows_in_chunks(ctx, 2, pair, x, xt, ldx, m) &&
+            turq_gemv_cs_staged_gateup_tiles(gate->dtype, gate->n, gate->k, TURQ_GEMV_MAX_M, ctx->compute_units > 0 ? ctx->compute_units : 256) == 6) {
+            const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
+            for (int64_t m0 = 0; m0 < m; m0 += TURQ_GEMV_MAX_M) {
+                bool part = false;
+                const int rc = turq_qmatmul_gate_up_mfma(ctx, gate, up, (const uint8_t *)x + (size_t)m0 * (size_t)ldx * xb, xt,
+                                                         std::min<int64_t>(TURQ_GEMV_MAX_M, m - m0), ldx,
+                                                         (uint8_t *)y + (size_t)m0 * (size_t)ldy * yb, yt, ldy, bias_gate, bias_up, &part);
+                if (rc != TURQ_OK) return rc;
+                if (!part) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_gate_up: a chunk of rows was not taken by the kernel its call was planned for");
+            }
+            *taken = true;
+            return TURQ_OK;
+        }
+    }
     const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
     if (m < 1 || m > TURQ_GEMV_MAX_M || gate->dtype != up->dtype || !turq_dt_is_quant(gate->dtype) || gate->layout != TURQ_LAYOUT_TILED ||
         up->layout != TURQ_LAYOUT_TILED)
