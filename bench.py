@@ -556,11 +556,12 @@ def read_floor():
 def other_halves(base):
     """The rest of the headline metric, measured in the same process with the same method (value = whole step, frac = the
     matmul kernels alone against the peak): the prefill GEMM (BASELINE config 4), the mixed Q4_K / Q6_K decoder layer at
-    its batch sizes (config 3) and the Q6_K LM head (config 5)."""
+    its batch sizes (config 3) and on prompt chunks of 128 and 512 rows, and the Q6_K LM head (config 5)."""
     steps, warmup = 20, 3
     return {
         "prefill": side_leg(base, "q4k_prefill_up_8b", [512, 2048], "bf16", "bf16", steps, warmup),
         "q4km_layer": side_leg(base, "q4km_layer_8b", [1, 8, 32], "f32", "f32", steps, warmup),
+        "q4km_layer_prefill": side_leg(base, "q4km_layer_8b", [128, 512], "bf16", "bf16", 10, 2),
         "lm_head_q6k": side_leg(base, "lm_head_q6k_8b", [1], "bf16", "f32", steps, warmup),
         "read_floor": read_floor(),
     }
