@@ -682,10 +682,13 @@ def test_staged_rows_kernel_group_sizes(row_tiles):
 # that would leave CUs idle) from the problem size; the small matrices of the tests above would never reach the wide one and
 # always take the low one, so they run once more in child processes with each of the two forced and forbidden (the rule takes
 # the wide tile for some of the full-size cases), and with the columns of every tile split over 2, 4 or 8 workgroups wherever
-# that number divides the super-blocks (on the wide or the low tile), or never.
+# that number divides the super-blocks (on the wide or the low tile), or never; and with the low tile's eight-wave form (two
+# groups of waves on alternate super-blocks) forbidden, and forced on every low-tile launch with an even share of super-blocks.
 @pytest.mark.parametrize("switch,value", [("TURQ_GEMM_WIDE", "1"), ("TURQ_GEMM_WIDE", "0"), ("TURQ_GEMM_LOW", "1"), ("TURQ_GEMM_LOW", "0"),
                                           ("TURQ_GEMM_SPLIT", "0"), ("TURQ_GEMM_SPLIT+TURQ_GEMM_SPLIT_FORM", "2+3"),
-                                          ("TURQ_GEMM_SPLIT+TURQ_GEMM_SPLIT_FORM", "4+4"), ("TURQ_GEMM_SPLIT", "8")])
+                                          ("TURQ_GEMM_SPLIT+TURQ_GEMM_SPLIT_FORM", "4+4"), ("TURQ_GEMM_SPLIT", "8"),
+                                          ("TURQ_GEMM_KGROUPS", "1"), ("TURQ_GEMM_KGROUPS+TURQ_GEMM_LOW", "2+1"),
+                                          ("TURQ_GEMM_KGROUPS+TURQ_GEMM_SPLIT+TURQ_GEMM_SPLIT_FORM", "2+2+4")])
 def test_prefill_tile_shapes(switch, value):
     import os
     import subprocess

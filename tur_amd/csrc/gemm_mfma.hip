@@ -419,8 +419,12 @@ template <> struct GFmt<TURQ_Q8_0> {
 // wave's stores have completed before its increment goes out and the last wave reads only after its own has returned.
 //   partials: [tile][part][wave] blocks of WM * WN KiB x 4 (a wave's accumulators as its lanes hold them), counters: [tile][wave],
 //   zero before the first launch; launches that share them must not overlap.
-template <int DT, int WGM_, bool SK = false>
-__global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
+// KG = 2 (low tile): eight waves as two groups of four.  Group g walks the super-blocks g, g + 2, ... of the workgroup's share
+// through rings of its own with the copy schedule, the waits and the barriers of the four-wave form (all eight waves pass the
+// same barriers, so the share must be an even number of super-blocks), which puts two waves on every SIMD; after the loop the
+// second group hands its accumulators to the first through the LDS.
+template <int DT, int WGM_, bool SK = false, int KG = 1>
+__global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
                                                       const uint8_t *__restrict__ frags, int64_t m, void *__restrict__ y,
                                                       int yt, int64_t ldy, const float *__restrict__ bias, int nblocks_n,
                                                       int nblocks_m, int vec_out, float wscale, float inv_ws, int split = 1,
@@ -437,7 +441,10 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    static_assert(KG == 1 || (KG == 2 && G::LOW), "two groups of waves: the low tile only");
+    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int kg = KG > 1 ? wave_all >> 2 : 0;             // the wave's group and its place in it
+    const int wave = KG > 1 ? (wave_all & 3) : wave_all;
     const int wm = wave / WGN, wn = wave % WGN;
     const int n32 = lane & 31, g32 = lane >> 5;
     const int r16 = n32 & 15, tsel = n32 >> 4;
@@ -449,11 +456,12 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     // (split: the m-blocks of one n-block and one part are consecutive, they share the part's packed weights)
     const int mb = lid % nblocks_m, part = SK ? (lid / nblocks_m) % split : 0, nb = lid / (nblocks_m * (SK ? split : 1));
     const int ntc = (int)turq_tile_cols(k);         // super-blocks of a row: the strides of the weights and of the fragments
-    const int nloc = SK ? ntc / split : ntc;        // ... of this workgroup: kb0 .. kb0 + nloc - 1
-    const int kb0 = part * nloc;
+    const int nloc = (SK ? ntc / split : ntc) / KG;  // ... of this group of waves: kb0, kb0 + KG, ... (nloc of them)
+    const int kb0 = part * nloc * KG + kg;
     const int64_t mtiles = (m + 31) / 32;
     const int nrt = (int)turq_tile_rows(n);
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+    constexpr uint32_t GROUP_BYTES = (uint32_t)(G::S_OFF + (SUMS ? NS * S_BYTES : 0) + 1023) & ~1023u;  // rings of one group of waves
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds + (uint32_t)kg * GROUP_BYTES;
     const uint32_t lane_off = 16u * (uint32_t)lane;
 
     // ---- copy schedule (all wave-uniform except the per-lane weight offsets) ----
@@ -496,7 +504,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     uint32_t wr0 = 0, wr1 = G::W_STRIDE, wr2 = 2 * G::W_STRIDE;
 
     auto issue_a = [&](int bb, int ks) {  // stage (bb, ks) -> stage buffer ks (wide form: ks % 2)
-        const uint8_t *src = a_src + ((size_t)(bb * 17 + 4 * ks) << 10);
+        const uint8_t *src = a_src + ((size_t)(bb * (KG * 17) + 4 * ks) << 10);
         dma_set<0>(lane_off, src, a_dst + (uint32_t)(ks % G::RA) * G::GA_STAGE);
         dma_more<1024>(lane_off, src);
         if constexpr (!G::LOW) {
@@ -505,7 +513,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
         }
     };
     auto issue_w = [&](int bb, int g, uint32_t ring) {  // group g of super-block bb
-        const uint8_t *src = w_src + (size_t)bb * TB;
+        const uint8_t *src = w_src + (size_t)bb * (KG * TB);
         if constexpr (G::WIDE) {  // half g of the wave's copies
 #pragma unroll
             for (int i = 0; i < G::CPW / 2; i++) dma_set<0>(w_voff[g * (G::CPW / 2) + i][0], src, w_dst[g * (G::CPW / 2) + i][0] + ring);
@@ -515,7 +523,7 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
         }
     };
     auto issue_s = [&](int bb) {
-        if constexpr (SUMS) dma_set<0>(lane_off, s_src + ((size_t)(bb * 17 + 16) << 10), s_dst + (uint32_t)(bb & 1) * S_BYTES);
+        if constexpr (SUMS) dma_set<0>(lane_off, s_src + ((size_t)(bb * (KG * 17) + 16) << 10), s_dst + (uint32_t)(bb & 1) * S_BYTES);
     };
 
     // ---- LDS read addresses ----
@@ -700,6 +708,35 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
 
+    if constexpr (KG > 1) {
+        // ---- the second group of waves hands its sums to the first (behind the staged results' part of the LDS) ----
+        constexpr int NQ = WM * WN * 4;
+        float4v *red = (float4v *)(lds + 4 * WM * 32 * G::OUT_PITCH * 4) + (size_t)wave * (NQ * 64) + lane;
+        if (kg == 1) {
+#pragma unroll
+            for (int i = 0; i < WM; i++)
+#pragma unroll
+                for (int j = 0; j < WN; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        red[((i * WN + j) * 4 + q) * 64] = float4v{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+        }
+        __syncthreads();
+        if (kg == 1) return;
+#pragma unroll
+        for (int i = 0; i < WM; i++)
+#pragma unroll
+            for (int j = 0; j < WN; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4v f = red[((i * WN + j) * 4 + q) * 64];
+                    acc[i][j][4 * q] += f.x;
+                    acc[i][j][4 * q + 1] += f.y;
+                    acc[i][j][4 * q + 2] += f.z;
+                    acc[i][j][4 * q + 3] += f.w;
+                }
+    }
+
     if constexpr (SK) {
         // ---- the parts of a tile meet (no workgroup barrier from here on: a wave may leave alone) ----
         constexpr int NB = WM * WN * 4;                 // 1 KiB blocks of a wave's partial tile (16 bytes per lane each)
@@ -844,17 +881,20 @@ __global__ void __launch_bounds__(256) gemm_kq_kernel(const uint8_t *__restrict_
 // split > 1: the columns of every tile over `split` workgroups that meet in `partials`, counted on `counters`
 // (kSplitCounterBytes, zero between launches)
 constexpr size_t kSplitCounterBytes = TURQ_GEMM_SPLIT_COUNTER_BYTES;
-template <int DT, int WGM_, bool SK = false>
+template <int DT, int WGM_, bool SK = false, int KG = 1>
 hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y, int y_dtype, int64_t ldy,
                        const float *bias, float wscale, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop, int split = 1,
                        void *counters = nullptr, void *partials = nullptr, size_t partials_cap = 0) {
     using G = Geo<DT, WGM_>;
-    constexpr int RING_BYTES = G::S_OFF + (GFmt<DT>::SUMS ? NS * S_BYTES : 0), STAGING_BYTES = 4 * G::WM * 32 * G::OUT_PITCH * 4;
+    constexpr int RING_BYTES = KG * ((G::S_OFF + (GFmt<DT>::SUMS ? NS * S_BYTES : 0) + 1023) & ~1023);
+    // (after the main loop: the staged results, behind them the sums that a second group of waves hands over)
+    constexpr int STAGING_BYTES = 4 * G::WM * 32 * G::OUT_PITCH * 4 + (KG > 1 ? 4 * G::WM * G::WN * 4096 : 0);
     constexpr int LDS_BYTES = RING_BYTES > STAGING_BYTES ? RING_BYTES : STAGING_BYTES;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS of one workgroup: the rings, or the staged results after the main loop");
     // per-lane weight offsets are 32-bit
     if ((uint64_t)G::NT16 * (uint64_t)(k / 256) * G::TB >= (1ull << 32)) return hipErrorInvalidValue;
-    const hipError_t attr = turq_raise_lds_limit((const void *)gemm_kq_kernel<DT, WGM_, SK>, LDS_BYTES);
+    if ((k / 256 / (SK ? split : 1)) % KG != 0) return hipErrorInvalidValue;
+    const hipError_t attr = turq_raise_lds_limit((const void *)gemm_kq_kernel<DT, WGM_, SK, KG>, LDS_BYTES);
     if (attr != hipSuccess) return attr;
     const int nbn = (int)((n + G::BN - 1) / G::BN), nbm = (int)((m + G::GBM - 1) / G::GBM);
     size_t partial_bytes = 0;
@@ -866,15 +906,15 @@ hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, i
     } else {
         split = 1;
     }
-    const dim3 grid((unsigned)(nbn * nbm * split)), block(256);
+    const dim3 grid((unsigned)(nbn * nbm * split)), block(256 * KG);
     const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
     const int vec_out = ((uintptr_t)y % 16 == 0 && ((uint64_t)ldy * es) % 16 == 0 && n % 8 == 0) ? 1 : 0;
     if (ev_start) {
-        hipExtLaunchKernelGGL((gemm_kq_kernel<DT, WGM_, SK>), grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
+        hipExtLaunchKernelGGL((gemm_kq_kernel<DT, WGM_, SK, KG>), grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
                               (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale, split,
                               (uint8_t *)partials, (uint32_t)partial_bytes, (uint32_t *)counters);
     } else {
-        gemm_kq_kernel<DT, WGM_, SK><<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype,
+        gemm_kq_kernel<DT, WGM_, SK, KG><<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype,
                                                                           ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale, split,
                                                                           (uint8_t *)partials, (uint32_t)partial_bytes, (uint32_t *)counters);
     }
@@ -986,10 +1026,31 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
     if (k <= 0 || k % 256 != 0 || !(wscale >= 6.103515625e-5f && wscale <= 32768.0f)) return hipErrorInvalidValue;
     const int form = turq_gemm_form(dtype, n, k, m, compute_units);
     if (form == 0) return hipErrorInvalidValue;
+    // The low tile with two groups of waves where a workgroup's share of the super-blocks is even and the launch is at most one
+    // workgroup per CU: the second group then fills SIMD time that nothing else would (Q4_K 4096 x 4096 at 256 / 512 rows
+    // 29.4 -> 23.4 / 32.6 -> 26.9 us, 12288 x 4096 at 128 rows 29.9 -> 25.2, 1024 x 4096 at 512 rows 30.4 -> 23.1, Q6_K
+    // 4096 x 12288 at 512 rows 105 -> 97); with more workgroups than CUs two four-wave workgroups share a CU anyway and the
+    // eight-wave one is slower (LM head at 64 rows 178 -> 196 us).  TURQ_GEMM_KGROUPS = 1: never, 2: wherever the share is even.
+    static const int kgroups = [] { const char *e = getenv("TURQ_GEMM_KGROUPS"); return e ? atoi(e) : 0; }();
+    const int64_t low_wgs = ((n + 127) / 128) * ((m + 63) / 64);
+    const int64_t cus_known = compute_units > 0 ? compute_units : 256;
+    auto two_groups_for = [&](int64_t wgs) { return kgroups == 2 || (kgroups != 1 && wgs <= cus_known); };
     if (split_counters && split_partials) {
         int sform = 0, split = 1;
         const size_t need = turq_gemm_split_scratch(dtype, n, k, m, compute_units, &sform, &split);
         if (need != 0 && need <= split_partial_bytes) {
+            if (sform == 4 && two_groups_for(low_wgs * split) && (k / 256 / split) % 2 == 0) {
+#define TURQ_GEMM_SK2(DT)                                                                                                               \
+    return launch_gemm<DT, 4, true, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop, split, split_counters, \
+                                       split_partials, split_partial_bytes)
+                switch (dtype) {
+                case TURQ_Q4_K: TURQ_GEMM_SK2(TURQ_Q4_K);
+                case TURQ_Q5_K: TURQ_GEMM_SK2(TURQ_Q5_K);
+                case TURQ_Q6_K: TURQ_GEMM_SK2(TURQ_Q6_K);
+                default: break;
+                }
+#undef TURQ_GEMM_SK2
+            }
 #define TURQ_GEMM_SK(DT, F)                                                                                                           \
     return launch_gemm<DT, F, true>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop, split, split_counters, \
                                     split_partials, split_partial_bytes)
@@ -1004,6 +1065,16 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
             }
 #undef TURQ_GEMM_SK
         }
+    }
+    if (form == 4 && two_groups_for(low_wgs) && (k / 256) % 2 == 0) {
+#define TURQ_GEMM_2(DT) return launch_gemm<DT, 4, false, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop)
+        switch (dtype) {
+        case TURQ_Q4_K: TURQ_GEMM_2(TURQ_Q4_K);
+        case TURQ_Q5_K: TURQ_GEMM_2(TURQ_Q5_K);
+        case TURQ_Q6_K: TURQ_GEMM_2(TURQ_Q6_K);
+        default: break;
+        }
+#undef TURQ_GEMM_2
     }
 #define TURQ_GEMM(DT, F) return launch_gemm<DT, F>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop)
     switch (dtype * 8 + form) {
