@@ -1015,6 +1015,15 @@ size_t turq_gemm_split_scratch(int dtype, int64_t n, int64_t k, int64_t m, int c
     return bytes;
 }
 
+// whether a low-tile launch whose tiles are split over `split` workgroups each takes the eight-wave form (one such workgroup
+// fills a CU's LDS; two of the four-wave form share one)
+bool turq_gemm_low_two_groups(int64_t n, int64_t k, int64_t m, int split, int compute_units) {
+    static const int kgroups = [] { const char *e = getenv("TURQ_GEMM_KGROUPS"); return e ? atoi(e) : 0; }();
+    if (split < 1 || (k / 256) % split != 0 || (k / 256 / split) % 2 != 0 || kgroups == 1) return false;
+    const int64_t wgs = ((n + 127) / 128) * ((m + 63) / 64) * split;
+    return kgroups == 2 || wgs <= (compute_units > 0 ? compute_units : 256);
+}
+
 // frags: activations prepared by turq_launch_act_prep32 (in the order of the same dtype) for all m rows
 // wscale: a power of two in [2^-14, 2^15] by which the kernel multiplies every block scale; compute_units: CUs of the device
 // (0: unknown), for the choice of the tile shape
@@ -1031,15 +1040,12 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
     // 29.4 -> 23.4 / 32.6 -> 26.9 us, 12288 x 4096 at 128 rows 29.9 -> 25.2, 1024 x 4096 at 512 rows 30.4 -> 23.1, Q6_K
     // 4096 x 12288 at 512 rows 105 -> 97); with more workgroups than CUs two four-wave workgroups share a CU anyway and the
     // eight-wave one is slower (LM head at 64 rows 178 -> 196 us).  TURQ_GEMM_KGROUPS = 1: never, 2: wherever the share is even.
-    static const int kgroups = [] { const char *e = getenv("TURQ_GEMM_KGROUPS"); return e ? atoi(e) : 0; }();
-    const int64_t low_wgs = ((n + 127) / 128) * ((m + 63) / 64);
-    const int64_t cus_known = compute_units > 0 ? compute_units : 256;
-    auto two_groups_for = [&](int64_t wgs) { return kgroups == 2 || (kgroups != 1 && wgs <= cus_known); };
+    auto two_groups_for = [&](int split) { return turq_gemm_low_two_groups(n, k, m, split, compute_units); };
     if (split_counters && split_partials) {
         int sform = 0, split = 1;
         const size_t need = turq_gemm_split_scratch(dtype, n, k, m, compute_units, &sform, &split);
         if (need != 0 && need <= split_partial_bytes) {
-            if (sform == 4 && two_groups_for(low_wgs * split) && (k / 256 / split) % 2 == 0) {
+            if (sform == 4 && two_groups_for(split)) {
 #define TURQ_GEMM_SK2(DT)                                                                                                               \
     return launch_gemm<DT, 4, true, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop, split, split_counters, \
                                        split_partials, split_partial_bytes)
@@ -1066,7 +1072,7 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
 #undef TURQ_GEMM_SK
         }
     }
-    if (form == 4 && two_groups_for(low_wgs) && (k / 256) % 2 == 0) {
+    if (form == 4 && two_groups_for(1)) {
 #define TURQ_GEMM_2(DT) return launch_gemm<DT, 4, false, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop)
         switch (dtype) {
         case TURQ_Q4_K: TURQ_GEMM_2(TURQ_Q4_K);

@@ -224,6 +224,7 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w_tiled, int64_t n, int6
 constexpr size_t TURQ_GEMM_SPLIT_COUNTER_BYTES = 64 << 10;
 // the workgroup tile the launch rules pick (0: no kernel for the format)
 int turq_gemm_form(int dtype, int64_t n, int64_t k, int64_t m, int compute_units);
+bool turq_gemm_low_two_groups(int64_t n, int64_t k, int64_t m, int split, int compute_units);
 // bytes of partial tiles a launch of this shape wants for splitting its columns, 0 if it does not split; form_out / split_out
 // (may be null): the tile (3: wide, 4: low) and the number of parts
 size_t turq_gemm_split_scratch(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int *form_out, int *split_out);

@@ -208,11 +208,14 @@ static int64_t gemm_cus_taken(const turq_ctx *ctx, const turq_weight *w, int64_t
     int form = 0, split = 1;
     if (may_split && turq_gemm_split_scratch(w->dtype, w->n, w->k, m, ctx->compute_units, &form, &split) != 0) {
         const int64_t tiles = form == 4 ? ((w->n + 127) / 128) * ((m + 63) / 64) : ((w->n + 255) / 256) * ((m + 127) / 128);
-        return form == 4 ? (tiles * split + 1) / 2 : tiles * split;
+        const bool whole = form != 4 || turq_gemm_low_two_groups(w->n, w->k, m, split, ctx->compute_units);
+        return whole ? tiles * split : (tiles * split + 1) / 2;
     }
     const int64_t nt = (w->n + 127) / 128, wgs128 = ((m + 127) / 128) * nt;
     const bool low = m <= 64 || 2 * wgs128 <= ctx->compute_units;
-    return low ? (((m + 63) / 64) * nt + 1) / 2 : wgs128;
+    if (!low) return wgs128;
+    const int64_t tiles = ((m + 63) / 64) * nt;
+    return turq_gemm_low_two_groups(w->n, w->k, m, 1, ctx->compute_units) ? tiles : (tiles + 1) / 2;
 }
 
 int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m, int64_t ldx,
