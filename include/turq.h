@@ -216,7 +216,9 @@ int turq_qmatmul_noalloc(turq_ctx *ctx, const turq_weight *w, const void *x, int
  * activations are prepared once for all the weights and each weight runs its GEMM on them (the results of the single
  * calls, bit for bit; GEMMs that leave half of the GPU free, such as k_proj and v_proj of a prompt chunk, run next to each other,
  * up to three at a time, on further streams of the context that are joined to the first before the call returns, so the
- * caller still sees one stream); every other case is exactly the turq_qmatmul calls one after the other (including their errors).  `biases` may be NULL, and so may its entries.
+ * caller still sees one stream; neighbouring large weights of one format and shape - gate_proj and up_proj - go out as ONE
+ * GEMM launch over the rows of all of them where that fills the GPU better, with the tile chosen for all the rows: the same
+ * products, in another order of the f32 sums where the tile's waves split k, within 2e-6 relative L2 of the single calls); every other case is exactly the turq_qmatmul calls one after the other (including their errors).  `biases` may be NULL, and so may its entries.
  * Replaces: the back-to-back `forward` calls on one input in the reference's decoder layer - q_proj / k_proj /
  * v_proj (src/models/qwen3.rs:272-274) and gate_proj / up_proj (src/models/qwen3.rs:161-167). */
 int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int x_dtype, int64_t m,

@@ -119,6 +119,20 @@ template <int DT, int WGM_> struct Geo {
     static_assert(!WIDE || (CPW % 2 == 0 && CPW <= 24), "wide form: two halves of CPW / 2 copies per wave");
 };
 
+// Up to kMaxGroup weights of one format and one k against the same activation fragments in ONE launch (gate and up of an MLP):
+// the n-blocks [first[i], first[i + 1]) of the launch belong to weight i.  One launch over the rows of both fills the rounds
+// over the CUs better than two (and picks its tile for the rows of both).
+constexpr int kMaxGroup = 4;
+struct GemmGroup {
+    const uint8_t *w[kMaxGroup];
+    void *y[kMaxGroup];
+    const float *bias[kMaxGroup];
+    int64_t n[kMaxGroup], ldy[kMaxGroup];
+    float wscale[kMaxGroup];  // per tensor: see the kernel
+    int first[kMaxGroup];
+    int count;
+};
+
 template <int... I, typename F> __device__ inline void static_for_impl(std::integer_sequence<int, I...>, F &&f) {
     (f(std::integral_constant<int, I>{}), ...);
 }
@@ -424,20 +438,44 @@ template <> struct GFmt<TURQ_Q8_0> {
 // same barriers, so the share must be an even number of super-blocks), which puts two waves on every SIMD; after the loop the
 // second group hands its accumulators to the first through the LDS.
 template <int DT, int WGM_, bool SK = false, int KG = 1>
-__global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
-                                                      const uint8_t *__restrict__ frags, int64_t m, void *__restrict__ y,
-                                                      int yt, int64_t ldy, const float *__restrict__ bias, int nblocks_n,
-                                                      int nblocks_m, int vec_out, float wscale, float inv_ws, int split = 1,
-                                                      uint8_t *__restrict__ partials = nullptr, uint32_t partial_bytes = 0,
-                                                      uint32_t *__restrict__ counters = nullptr) {
+__global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_t k, const uint8_t *__restrict__ frags, int64_t m, int yt,
+                                                           int nblocks_n, int nblocks_m, int vec_out, int split = 1,
+                                                           uint8_t *__restrict__ partials = nullptr, uint32_t partial_bytes = 0,
+                                                           uint32_t *__restrict__ counters = nullptr) {
     using Fm = GFmt<DT>;
     using G = Geo<DT, WGM_>;
     constexpr int WGN = G::WGN, WM = G::WM, WN = G::WN, TB = G::TB;
     constexpr bool SUMS = Fm::SUMS;
+    // Workgroups of one XCD (blockIdx % 8) get consecutive logical ids and the m-blocks of one n-block are
+    // consecutive in that order: the packed weights they share stay in that XCD's L2.
+    const int nwg = nblocks_n * nblocks_m * (SK ? split : 1);
+    int lid = blockIdx.x;
+    if ((nwg & 7) == 0) lid = (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3);
+    // (split: the m-blocks of one n-block and one part are consecutive, they share the part's packed weights)
+    const int mb = lid % nblocks_m, part = SK ? (lid / nblocks_m) % split : 0, nb_all = lid / (nblocks_m * (SK ? split : 1));
+    // the weight this n-block belongs to
+    const uint8_t *__restrict__ w = grp.w[0];
+    void *__restrict__ y = grp.y[0];
+    const float *__restrict__ bias = grp.bias[0];
+    int64_t n = grp.n[0], ldy = grp.ldy[0];
+    float wscale = grp.wscale[0];
+    int nb = nb_all;
+#pragma unroll
+    for (int i = 1; i < kMaxGroup; i++)
+        if (i < grp.count && nb_all >= grp.first[i]) {
+            w = grp.w[i];
+            y = grp.y[i];
+            bias = grp.bias[i];
+            n = grp.n[i];
+            ldy = grp.ldy[i];
+            wscale = grp.wscale[i];
+            nb = nb_all - grp.first[i];
+        }
     // every block scale is multiplied by wscale (a power of two chosen per tensor so that the largest packed-f16 weight
     // lands near 2^15) and the results by its inverse: small scales keep their precision instead of dropping into the
     // f16 subnormals (d * sc / 16 of Q5_K does so from d around 1e-4)
-    const _Float16 ws = (_Float16)wscale;  // inv_ws = 1 / wscale comes from the host
+    const _Float16 ws = (_Float16)wscale;
+    const float inv_ws = 1.0f / wscale;  // (a power of two: exact)
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -448,13 +486,6 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(const uint8_t *__rest
     const int wm = wave / WGN, wn = wave % WGN;
     const int n32 = lane & 31, g32 = lane >> 5;
     const int r16 = n32 & 15, tsel = n32 >> 4;
-    // Workgroups of one XCD (blockIdx % 8) get consecutive logical ids and the m-blocks of one n-block are
-    // consecutive in that order: the packed weights they share stay in that XCD's L2.
-    const int nwg = nblocks_n * nblocks_m * (SK ? split : 1);
-    int lid = blockIdx.x;
-    if ((nwg & 7) == 0) lid = (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3);
-    // (split: the m-blocks of one n-block and one part are consecutive, they share the part's packed weights)
-    const int mb = lid % nblocks_m, part = SK ? (lid / nblocks_m) % split : 0, nb = lid / (nblocks_m * (SK ? split : 1));
     const int ntc = (int)turq_tile_cols(k);         // super-blocks of a row: the strides of the weights and of the fragments
     const int nloc = (SK ? ntc / split : ntc) / KG;  // ... of this group of waves: kb0, kb0 + KG, ... (nloc of them)
     const int kb0 = part * nloc * KG + kg;
@@ -742,7 +773,7 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(const uint8_t *__rest
         constexpr int NB = WM * WN * 4;                 // 1 KiB blocks of a wave's partial tile (16 bytes per lane each)
         constexpr uint32_t WAVE_BYTES = NB * 1024u;
         constexpr int PB = NB >= 32 ? 1 : 32 / NB;      // parts read together: 128 registers of loads in flight per lane
-        const int tile = nb * nblocks_m + mb;
+        const int tile = nb_all * nblocks_m + mb;
         uint32_t *cnt = counters + tile * 4 + wave;
         const __amdgpu_buffer_rsrc_t prs = __builtin_amdgcn_make_buffer_rsrc(partials, 0, (int)partial_bytes, 0x00020000);
         const uint32_t tile_base = (uint32_t)(tile * split) * (4u * WAVE_BYTES) + (uint32_t)wave * WAVE_BYTES + lane_off;
@@ -882,9 +913,9 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(const uint8_t *__rest
 // (kSplitCounterBytes, zero between launches)
 constexpr size_t kSplitCounterBytes = TURQ_GEMM_SPLIT_COUNTER_BYTES;
 template <int DT, int WGM_, bool SK = false, int KG = 1>
-hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, int64_t m, void *y, int y_dtype, int64_t ldy,
-                       const float *bias, float wscale, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop, int split = 1,
-                       void *counters = nullptr, void *partials = nullptr, size_t partials_cap = 0) {
+hipError_t launch_gemm(const TurqGemmWeights &ws, int64_t k, const void *frags, int64_t m, int y_dtype, hipStream_t stream,
+                       hipEvent_t ev_start, hipEvent_t ev_stop, int split = 1, void *counters = nullptr, void *partials = nullptr,
+                       size_t partials_cap = 0) {
     using G = Geo<DT, WGM_>;
     constexpr int RING_BYTES = KG * ((G::S_OFF + (GFmt<DT>::SUMS ? NS * S_BYTES : 0) + 1023) & ~1023);
     // (after the main loop: the staged results, behind them the sums that a second group of waves hands over)
@@ -894,9 +925,26 @@ hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, i
     // per-lane weight offsets are 32-bit
     if ((uint64_t)G::NT16 * (uint64_t)(k / 256) * G::TB >= (1ull << 32)) return hipErrorInvalidValue;
     if ((k / 256 / (SK ? split : 1)) % KG != 0) return hipErrorInvalidValue;
+    if (ws.count < 1 || ws.count > kMaxGroup) return hipErrorInvalidValue;
     const hipError_t attr = turq_raise_lds_limit((const void *)gemm_kq_kernel<DT, WGM_, SK, KG>, LDS_BYTES);
     if (attr != hipSuccess) return attr;
-    const int nbn = (int)((n + G::BN - 1) / G::BN), nbm = (int)((m + G::GBM - 1) / G::GBM);
+    GemmGroup grp{};
+    grp.count = ws.count;
+    const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
+    int nbn = 0, vec_out = 1;
+    for (int i = 0; i < ws.count; i++) {
+        grp.w[i] = (const uint8_t *)ws.w[i];
+        grp.y[i] = ws.y[i];
+        grp.bias[i] = ws.bias[i];
+        grp.n[i] = ws.n[i];
+        grp.ldy[i] = ws.ldy[i];
+        grp.wscale[i] = ws.wscale[i];
+        grp.first[i] = nbn;
+        nbn += (int)((ws.n[i] + G::BN - 1) / G::BN);
+        // rows of y can be written as aligned 16-byte pieces (every weight of the launch, or none)
+        vec_out = vec_out && (uintptr_t)ws.y[i] % 16 == 0 && ((uint64_t)ws.ldy[i] * es) % 16 == 0 && ws.n[i] % 8 == 0;
+    }
+    const int nbm = (int)((m + G::GBM - 1) / G::GBM);
     size_t partial_bytes = 0;
     if constexpr (SK) {
         partial_bytes = (size_t)nbn * nbm * split * (size_t)(G::WM * G::WN * 4 * 4096);
@@ -907,15 +955,12 @@ hipError_t launch_gemm(const void *w, int64_t n, int64_t k, const void *frags, i
         split = 1;
     }
     const dim3 grid((unsigned)(nbn * nbm * split)), block(256 * KG);
-    const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
-    const int vec_out = ((uintptr_t)y % 16 == 0 && ((uint64_t)ldy * es) % 16 == 0 && n % 8 == 0) ? 1 : 0;
     if (ev_start) {
-        hipExtLaunchKernelGGL((gemm_kq_kernel<DT, WGM_, SK, KG>), grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, (const uint8_t *)w, n, k,
-                              (const uint8_t *)frags, m, y, y_dtype, ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale, split,
-                              (uint8_t *)partials, (uint32_t)partial_bytes, (uint32_t *)counters);
+        hipExtLaunchKernelGGL((gemm_kq_kernel<DT, WGM_, SK, KG>), grid, block, LDS_BYTES, stream, ev_start, ev_stop, 0, grp, k,
+                              (const uint8_t *)frags, m, y_dtype, nbn, nbm, vec_out, split, (uint8_t *)partials, (uint32_t)partial_bytes,
+                              (uint32_t *)counters);
     } else {
-        gemm_kq_kernel<DT, WGM_, SK, KG><<<grid, block, LDS_BYTES, stream>>>((const uint8_t *)w, n, k, (const uint8_t *)frags, m, y, y_dtype,
-                                                                          ldy, bias, nbn, nbm, vec_out, wscale, 1.0f / wscale, split,
+        gemm_kq_kernel<DT, WGM_, SK, KG><<<grid, block, LDS_BYTES, stream>>>(grp, k, (const uint8_t *)frags, m, y_dtype, nbn, nbm, vec_out, split,
                                                                           (uint8_t *)partials, (uint32_t)partial_bytes, (uint32_t *)counters);
     }
     return hipGetLastError();
@@ -1015,6 +1060,19 @@ size_t turq_gemm_split_scratch(int dtype, int64_t n, int64_t k, int64_t m, int c
     return bytes;
 }
 
+// The launch the rules above would make for these rows: its workgroups, and the share of its rounds over the CUs that it keeps
+// busy, weighted by the wide tile's measured gain.
+double turq_gemm_fill(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int64_t *wgs_out) {
+    const int form = turq_gemm_form(dtype, n, k, m, compute_units);
+    const int64_t cus = compute_units > 0 ? compute_units : 256;
+    const int64_t bm = form == 4 ? 64 : 128;
+    const int64_t bn = form == 3 ? 256 : form == 2 ? (dtype == TURQ_Q4_K ? 192 : dtype == TURQ_Q8_0 ? 64 : 128) : 128;
+    const int64_t wgs = ((n + bn - 1) / bn) * ((m + bm - 1) / bm), rounds = (wgs + cus - 1) / cus;
+    if (wgs_out) *wgs_out = wgs;
+    const double gain = form == 3 ? (dtype == TURQ_Q4_K ? 1.10 : 1.25) : 1.0;
+    return rounds > 0 ? (double)wgs / (double)(rounds * cus) * gain : 0.0;
+}
+
 // whether a low-tile launch whose tiles are split over `split` workgroups each takes the eight-wave form (one such workgroup
 // fills a CU's LDS; two of the four-wave form share one)
 bool turq_gemm_low_two_groups(int64_t n, int64_t k, int64_t m, int split, int compute_units) {
@@ -1031,8 +1089,32 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
                                  int y_dtype, int64_t ldy, const float *bias, float wscale, int compute_units, hipStream_t stream,
                                  hipEvent_t ev_start, hipEvent_t ev_stop, void *split_counters, void *split_partials,
                                  size_t split_partial_bytes) {
-    if (n == 0 || m == 0) return hipSuccess;
-    if (k <= 0 || k % 256 != 0 || !(wscale >= 6.103515625e-5f && wscale <= 32768.0f)) return hipErrorInvalidValue;
+    TurqGemmWeights ws{};
+    ws.count = 1;
+    ws.w[0] = w;
+    ws.y[0] = y;
+    ws.bias[0] = bias;
+    ws.n[0] = n;
+    ws.ldy[0] = ldy;
+    ws.wscale[0] = wscale;
+    return turq_launch_gemm_mfma_group(dtype, ws, k, frags, m, y_dtype, compute_units, stream, ev_start, ev_stop, split_counters,
+                                       split_partials, split_partial_bytes);
+}
+
+// ... for up to four weights of one format in one launch: the tile, the split and the wave groups are chosen for the rows of all
+// of them together (every n a multiple of 256, so that no tile of any form straddles two weights)
+hipError_t turq_launch_gemm_mfma_group(int dtype, const TurqGemmWeights &ws, int64_t k, const void *frags, int64_t m, int y_dtype,
+                                       int compute_units, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop,
+                                       void *split_counters, void *split_partials, size_t split_partial_bytes) {
+    if (ws.count < 1 || ws.count > 4) return hipErrorInvalidValue;
+    int64_t n = 0;
+    for (int i = 0; i < ws.count; i++) {
+        if (ws.n[i] <= 0 || (ws.count > 1 && ws.n[i] % 256 != 0)) return ws.n[i] == 0 && ws.count == 1 ? hipSuccess : hipErrorInvalidValue;
+        if (!(ws.wscale[i] >= 6.103515625e-5f && ws.wscale[i] <= 32768.0f)) return hipErrorInvalidValue;
+        n += ws.n[i];
+    }
+    if (m == 0) return hipSuccess;
+    if (k <= 0 || k % 256 != 0) return hipErrorInvalidValue;
     const int form = turq_gemm_form(dtype, n, k, m, compute_units);
     if (form == 0) return hipErrorInvalidValue;
     // The low tile with two groups of waves where a workgroup's share of the super-blocks is even and the launch is at most one
@@ -1047,8 +1129,8 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
         if (need != 0 && need <= split_partial_bytes) {
             if (sform == 4 && two_groups_for(split)) {
 #define TURQ_GEMM_SK2(DT)                                                                                                               \
-    return launch_gemm<DT, 4, true, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop, split, split_counters, \
-                                       split_partials, split_partial_bytes)
+    return launch_gemm<DT, 4, true, 2>(ws, k, frags, m, y_dtype, stream, ev_start, ev_stop, split, split_counters, split_partials, \
+                                       split_partial_bytes)
                 switch (dtype) {
                 case TURQ_Q4_K: TURQ_GEMM_SK2(TURQ_Q4_K);
                 case TURQ_Q5_K: TURQ_GEMM_SK2(TURQ_Q5_K);
@@ -1058,8 +1140,8 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
 #undef TURQ_GEMM_SK2
             }
 #define TURQ_GEMM_SK(DT, F)                                                                                                           \
-    return launch_gemm<DT, F, true>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop, split, split_counters, \
-                                    split_partials, split_partial_bytes)
+    return launch_gemm<DT, F, true>(ws, k, frags, m, y_dtype, stream, ev_start, ev_stop, split, split_counters, split_partials, \
+                                    split_partial_bytes)
             switch (dtype * 8 + sform) {
             case TURQ_Q4_K * 8 + 3: TURQ_GEMM_SK(TURQ_Q4_K, 3);
             case TURQ_Q4_K * 8 + 4: TURQ_GEMM_SK(TURQ_Q4_K, 4);
@@ -1073,7 +1155,7 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
         }
     }
     if (form == 4 && two_groups_for(1)) {
-#define TURQ_GEMM_2(DT) return launch_gemm<DT, 4, false, 2>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop)
+#define TURQ_GEMM_2(DT) return launch_gemm<DT, 4, false, 2>(ws, k, frags, m, y_dtype, stream, ev_start, ev_stop)
         switch (dtype) {
         case TURQ_Q4_K: TURQ_GEMM_2(TURQ_Q4_K);
         case TURQ_Q5_K: TURQ_GEMM_2(TURQ_Q5_K);
@@ -1082,7 +1164,7 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w, int64_t n, int64_t k,
         }
 #undef TURQ_GEMM_2
     }
-#define TURQ_GEMM(DT, F) return launch_gemm<DT, F>(w, n, k, frags, m, y, y_dtype, ldy, bias, wscale, stream, ev_start, ev_stop)
+#define TURQ_GEMM(DT, F) return launch_gemm<DT, F>(ws, k, frags, m, y_dtype, stream, ev_start, ev_stop)
     switch (dtype * 8 + form) {
     case TURQ_Q4_K * 8 + 1: TURQ_GEMM(TURQ_Q4_K, 1);
     case TURQ_Q4_K * 8 + 2: TURQ_GEMM(TURQ_Q4_K, 2);

@@ -222,8 +222,23 @@ hipError_t turq_launch_gemm_mfma(int dtype, const void *w_tiled, int64_t n, int6
                                  hipEvent_t ev_start, hipEvent_t ev_stop, void *split_counters = nullptr, void *split_partials = nullptr,
                                  size_t split_partial_bytes = 0);
 constexpr size_t TURQ_GEMM_SPLIT_COUNTER_BYTES = 64 << 10;
+// up to four weights of one format and one k in one launch of the prefill GEMM
+struct TurqGemmWeights {
+    const void *w[4];
+    void *y[4];
+    const float *bias[4];
+    int64_t n[4], ldy[4];
+    float wscale[4];
+    int count;
+};
+hipError_t turq_launch_gemm_mfma_group(int dtype, const TurqGemmWeights &ws, int64_t k, const void *frags, int64_t m, int y_dtype,
+                                       int compute_units, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop,
+                                       void *split_counters = nullptr, void *split_partials = nullptr, size_t split_partial_bytes = 0);
 // the workgroup tile the launch rules pick (0: no kernel for the format)
 int turq_gemm_form(int dtype, int64_t n, int64_t k, int64_t m, int compute_units);
+// the launch the tile rules would make for these rows: its workgroups and the share of its CU rounds it keeps busy (x the wide
+// tile's gain)
+double turq_gemm_fill(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int64_t *wgs_out);
 bool turq_gemm_low_two_groups(int64_t n, int64_t k, int64_t m, int split, int compute_units);
 // bytes of partial tiles a launch of this shape wants for splitting its columns, 0 if it does not split; form_out / split_out
 // (may be null): the tile (3: wide, 4: low) and the number of parts
