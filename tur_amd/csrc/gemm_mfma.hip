@@ -49,6 +49,11 @@
 // the mantissa of 256.0 (low nibble at bits 2..5, high field rotated onto bits 6..7) and needs no sums term.  Their
 // tiles are larger (2816 / 3360 bytes), so their workgroup is 128 x 128 to keep three super-blocks of weights in the LDS.  Q8_0 (4352-byte tiles, f16 block scales, no sums term): 128 x 64, wave tile 2 x 1.
 //
+// Launches that would leave CUs idle.  Three further forms of the same loop, chosen per launch by the rules at the end of this
+// file: every tile's super-blocks shared out over several workgroups that meet in device memory (SK); the low tile with eight
+// waves as two groups on alternate super-blocks that meet in the LDS (KG = 2); and up to four weights of one format in one
+// launch (GemmGroup), the n-blocks dealt out to them in order.
+//
 // Results leave through the LDS (free after the main loop): each wave transposes its 64 x 96 tile so
 // that a lane stores 16 contiguous bytes and a row segment is 192 (bf16, f16) or 384 (f32) bytes.
 #include <hip/hip_ext.h>
