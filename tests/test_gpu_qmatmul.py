@@ -506,6 +506,41 @@ def test_multi_weight_prefill_shares_the_preparation(gpu):
         gpu.release(w)
 
 
+def test_multi_weight_prefill_runs_of_one_format(gpu):
+    # neighbouring weights of one K-quant format and shape (rows a multiple of 256) may go out as ONE launch of the prefill GEMM
+    # whose n-blocks are dealt out to the weights; the rule only does that for weights that fill half the machine, so this test
+    # also runs in a child process with every such run merged (test_prefill_merged_runs_forced).  Against the single calls
+    # (other tiles, another order of the f32 sums where waves split k) and the oracle; biases, ragged m.
+    k = 2048
+    dts, ns = (Q5_K, Q5_K, Q5_K, Q6_K, Q6_K, Q6_K, Q6_K, Q4_K, Q4_K, Q8_0), [256, 256, 256, 512, 512, 512, 512, 256, 256, 64]
+    raws = [synth.random_weight(dt, n, k, seed=5 * i + n) for i, (dt, n) in enumerate(zip(dts, ns))]
+    ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for dt, n, raw in zip(dts, ns, raws)]
+    biases = [None if i % 3 == 0 else np.random.default_rng(i).standard_normal(n).astype(np.float32) for i, n in enumerate(ns)]
+    for m in (40, 130, 300):
+        x = synth.random_activation(m, k, seed=m, bf16=True)
+        ys = gpu.qmatmul_multi(ws, x, ns, k, x_dtype=capi.ACT_BF16, biases=biases)
+        for i, (dt, n, raw, w, y, b) in enumerate(zip(dts, ns, raws, ws, ys, biases)):
+            want = orc.matmul_dequant(dt, x, raw, n, k) + (0 if b is None else b)
+            assert rel_l2(y, want) <= 1e-3, (m, i, dt)
+            single = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, bias=b)
+            assert rel_l2(y, single) <= 2e-6, (m, i, dt, rel_l2(y, single))
+    for w in ws:
+        gpu.release(w)
+
+
+def test_prefill_merged_runs_forced():
+    import os
+    import subprocess
+    import sys
+
+    env = dict(os.environ, TURQ_GEMM_MERGE="2")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "-k", "runs_of_one_format",
+                          "-p", "no:cacheprovider", os.path.join(root, "tests", "test_gpu_qmatmul.py")],
+                         cwd=root, env=env, capture_output=True, text=True, timeout=280)
+    assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-1000:]
+
+
 def test_multi_weight_prefill_small_launches_side_by_side(gpu):
     # q / k / v of a prompt chunk: launches that leave half of the machine free run in groups of up to three, the first on
     # the context's stream, the others on further streams, between the shared preparation and the end of the call.  Same kernels, same inputs: bit-equal with the

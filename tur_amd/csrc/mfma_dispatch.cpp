@@ -249,7 +249,8 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
     int64_t group_cus = 0;  // CUs they take together
     int prepared = 0;       // 1: K-quant order, 2: Q8_0 order
     hipError_t e = hipSuccess;
-    static const bool no_merge = [] { const char *v = getenv("TURQ_GEMM_MERGE"); return v && atoi(v) == 0; }();
+    static const int merge_env = [] { const char *v = getenv("TURQ_GEMM_MERGE"); return v ? atoi(v) : -1; }();  // 0: never, 2: every run
+    const bool no_merge = merge_env == 0, merge_all = merge_env == 2;
     for (int i = 0; i < count && e == hipSuccess; i++) {
         const int order = w[i]->dtype == TURQ_Q8_0 ? 2 : 1;
         if (order != prepared) {
@@ -263,15 +264,16 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
         // go out as ONE launch over the rows of all of them where that fills the rounds over the CUs better: where each alone
         // leaves CUs idle and all together still fit one round, or where the tile chosen for all the rows keeps a larger share
         // of its rounds busy (Q4_K 2 x 12288 x 4096, two launches -> one: 128 rows 50 -> 42 us, 256 rows 80 -> 67, 1024 rows
-        // 257 -> 220; at 384 and 512 rows one launch is 3 % slower and the rule keeps two).  TURQ_GEMM_MERGE = 0: never.
-        if (!no_merge && 2 * c > cus && turq_dt_is_quant(w[i]->dtype) && w[i]->dtype != TURQ_Q8_0 && w[i]->n % 256 == 0) {
+        // 257 -> 220; at 384 and 512 rows one launch is 3 % slower and the rule keeps two).  TURQ_GEMM_MERGE = 0: never, 2: every
+        // such run whatever its size.
+        if (!no_merge && (2 * c > cus || merge_all) && turq_dt_is_quant(w[i]->dtype) && w[i]->dtype != TURQ_Q8_0 && w[i]->n % 256 == 0) {
             int j = i + 1;
             while (j < count && j - i < 4 && w[j]->dtype == w[i]->dtype && w[j]->n == w[i]->n) j++;
             if (j - i >= 2) {
                 int64_t wgs_one = 0, wgs_all = 0;
                 const double fill_one = turq_gemm_fill(w[i]->dtype, w[i]->n, w[i]->k, m, ctx->compute_units, &wgs_one);
                 const double fill_all = turq_gemm_fill(w[i]->dtype, w[i]->n * (j - i), w[i]->k, m, ctx->compute_units, &wgs_all);
-                if ((wgs_one < cus && wgs_all <= cus) || fill_all > 1.05 * fill_one) {
+                if (merge_all || (wgs_one < cus && wgs_all <= cus) || fill_all > 1.05 * fill_one) {
                     TurqGemmWeights g{};
                     g.count = j - i;
                     for (int t = i; t < j; t++) {
