@@ -110,6 +110,16 @@ extern "C" {
     pub fn turq_profile_begin(ctx: *mut turq_ctx) -> c_int;
     pub fn turq_profile_end(ctx: *mut turq_ctx, launches: *mut i64, total_ms: *mut f64) -> c_int;
     pub fn turq_read_yardstick(ctx: *mut turq_ctx, dev_ptr: *const c_void, nbytes: usize) -> c_int;
+    pub fn turq_prefill_plan(
+        dtype: c_int,
+        n: i64,
+        k: i64,
+        m: i64,
+        compute_units: c_int,
+        tile: *mut c_int,
+        split: *mut c_int,
+        wave_groups: *mut c_int,
+    ) -> c_int;
     pub fn turq_gguf_open(path: *const c_char, out: *mut *mut turq_gguf) -> c_int;
     pub fn turq_gguf_close(g: *mut turq_gguf);
     pub fn turq_gguf_last_error(g: *const turq_gguf) -> *const c_char;

@@ -304,6 +304,12 @@ int turq_profile_end(turq_ctx *ctx, int64_t *launches, double *total_ms);
  * is on.  A launch of a few tens of MB is short enough for the launch itself to weigh as much as its bytes (on an MI355X
  * 28 MB take 5.0 us and 57 MB 9.2 us, where 8 TB/s would mean 3.5 and 7.1): this is what the decode kernels are up against. */
 int turq_read_yardstick(turq_ctx *ctx, const void *dev_ptr, size_t nbytes);
+/* Which launch the rules for prompt chunks (more than 32 rows, K-quant or Q8_0 weights in the tiled layout) make for a weight of
+ * n rows and k columns on a device with `compute_units` CUs; no GPU is needed and nothing is launched.  tile: 1 = 128 x 128,
+ * 2 = 128 x 192 (Q8_0: 128 x 64), 3 = 128 x 256, 4 = 64 x 128; split: workgroups that share the columns of every tile (1: none);
+ * wave_groups: 2 where the 64 x 128 tile runs eight waves as two groups on alternate super-blocks.  Not part of the path, no
+ * counterpart in the reference: for tests of the rules and for tuning them on another device. */
+int turq_prefill_plan(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int *tile, int *split, int *wave_groups);
 
 /* ---- GGUF files ---- */
 /* Parse the header (magic, version 1..3, metadata, tensor infos, alignment).

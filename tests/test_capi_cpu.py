@@ -215,3 +215,42 @@ def test_gguf_reader_refuses_hostile_files(tmp_path, kwargs, what):
         L.turq_gguf_close(g)
     else:
         assert rc == capi.ERR_IO and what in capi.last_error()
+
+
+def test_prefill_launch_rules_on_a_256_cu_device():
+    # the launches the rules make for the matrices of a Qwen3-8B Q4_K_M layer on prompt chunks, as measured and documented:
+    # (tile, workgroups per tile, wave groups); tiles: 1 = 128 x 128, 2 = 128 x 192, 3 = 128 x 256, 4 = 64 x 128
+    L = capi.lib()
+    Q4_K, Q6_K = capi.Q4_K, capi.Q6_K
+
+    def plan(dt, n, k, m):
+        t, s, g = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        capi.check(L.turq_prefill_plan(dt, n, k, m, 256, ctypes.byref(t), ctypes.byref(s), ctypes.byref(g)))
+        return t.value, s.value, g.value
+
+    # down_proj 4096 x 12288: low tile in 6 / 3 parts up to 128 rows, wide tile in 6 parts at 256, unsplit from 512 on
+    assert plan(Q6_K, 4096, 12288, 64) == (4, 6, 2)
+    assert plan(Q6_K, 4096, 12288, 128) == (4, 3, 2)
+    assert plan(Q6_K, 4096, 12288, 256) == (3, 6, 1)
+    assert plan(Q6_K, 4096, 12288, 512) == (4, 1, 2)
+    assert plan(Q6_K, 4096, 12288, 1024) == (1, 1, 1)
+    # o_proj / q_proj 4096 x 4096: parts only up to 128 rows; eight waves while there is at most one workgroup per CU
+    assert plan(Q4_K, 4096, 4096, 64) == (4, 4, 2)
+    assert plan(Q4_K, 4096, 4096, 128) == (4, 2, 2)
+    assert plan(Q4_K, 4096, 4096, 256) == (4, 1, 2)
+    assert plan(Q4_K, 4096, 4096, 512) == (4, 1, 2)
+    # up_proj 12288 x 4096 alone, and gate + up as one launch (24576 rows)
+    assert plan(Q4_K, 12288, 4096, 128) == (4, 1, 2)
+    assert plan(Q4_K, 12288, 4096, 256) == (1, 1, 1)
+    assert plan(Q4_K, 12288, 4096, 512) == (2, 1, 1)
+    assert plan(Q4_K, 12288, 4096, 2048) == (3, 1, 1)
+    assert plan(Q4_K, 24576, 4096, 128) == (1, 1, 1)
+    assert plan(Q4_K, 24576, 4096, 256) == (2, 1, 1)
+    assert plan(Q4_K, 24576, 4096, 1024) == (3, 1, 1)
+    # the LM head: more workgroups than CUs, four waves
+    assert plan(Q6_K, 151936, 4096, 64) == (4, 1, 1)
+    # arguments
+    t = ctypes.c_int()
+    assert L.turq_prefill_plan(Q4_K, 4096, 4096, 8, 256, ctypes.byref(t), None, None) == capi.ERR_SHAPE
+    assert L.turq_prefill_plan(capi.F32, 4096, 4096, 64, 256, ctypes.byref(t), None, None) == capi.ERR_DTYPE
+

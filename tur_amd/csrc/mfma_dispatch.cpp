@@ -647,3 +647,22 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
     }
     return TURQ_OK;
 }
+
+// which launch the rules above and in gemm_mfma.hip make for a prompt chunk (no GPU needed)
+extern "C" int turq_prefill_plan(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int *tile, int *split, int *wave_groups) {
+    if (tile) *tile = 0;
+    if (split) *split = 1;
+    if (wave_groups) *wave_groups = 1;
+    if (!turq_dt_is_quant(dtype)) return turq_fail(nullptr, TURQ_ERR_DTYPE, "turq_prefill_plan: dtype %d has no prefill kernel", dtype);
+    if (n <= 0 || k <= 0 || k % 256 != 0 || m <= TURQ_GEMV_MAX_M || compute_units <= 0)
+        return turq_fail(nullptr, TURQ_ERR_SHAPE, "turq_prefill_plan: n=%lld k=%lld m=%lld on %d compute units", (long long)n, (long long)k,
+                         (long long)m, compute_units);
+    int form = turq_gemm_form(dtype, n, k, m, compute_units), parts = 1, sform = 0;
+    if (turq_gemm_split_scratch(dtype, n, k, m, compute_units, &sform, &parts) != 0) form = sform;
+    else parts = 1;
+    if (tile) *tile = form;
+    if (split) *split = parts;
+    if (wave_groups) *wave_groups = form == 4 && turq_gemm_low_two_groups(n, k, m, parts, compute_units) ? 2 : 1;
+    return TURQ_OK;
+}
+
