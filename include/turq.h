@@ -181,7 +181,7 @@ int turq_rms_norm(turq_ctx *ctx, const void *x, int x_dtype, int64_t m, int64_t 
  * Device calls of 33 - 64 rows on large weights of up to 4096 columns (gate / up of an 8B model) go through the kernels of up
  * to 32 rows in two chunks.  Device calls of more than 32 rows (prompt chunks) whose workgroup tiles would leave most compute units idle - the tall
  * down_proj of a model up to about 256 rows, every matrix of a layer up to 64 - split the columns of every tile over several
- * workgroups, which meet in a scratch buffer of the context (partial tiles, at most 256 MiB; grown like the other scratch
+ * workgroups, which meet in a scratch buffer of the context (partial tiles, at most 256 MiB per launch and 512 MiB per call; grown like the other scratch
  * buffers: not during a graph capture).  The sums of a result are the same numbers in the same order on every call.
  * Replaces: `LinearX::forward` -> `QMatMul::forward(&Tensor)` (src/models/layers/linear.rs:19-31)
  * -> candle `CustomOp1::cpu_fwd` -> `k_quants::matmul`. */

@@ -188,6 +188,10 @@ static int gemm_split_reserve(turq_ctx *ctx, int count, const turq_weight *const
         any = any || out->bytes[i] != 0;
     }
     if (!any) return TURQ_OK;
+    if (total > ((size_t)512 << 20)) {  // (a call whose launches together want more than this runs them unsplit)
+        *out = GemmSplit{};
+        return TURQ_OK;
+    }
     if (total > ctx->gemm_split_cap) {
         int rc = turq_ctx_reserve(ctx, &ctx->gemm_split, &ctx->gemm_split_cap, total);
         if (rc != TURQ_OK) return rc;
