@@ -234,9 +234,11 @@ def test_prefill_launch_rules_on_a_256_cu_device():
     assert plan(Q6_K, 4096, 12288, 256) == (3, 6, 1)
     assert plan(Q6_K, 4096, 12288, 512) == (4, 1, 2)
     assert plan(Q6_K, 4096, 12288, 1024) == (1, 1, 1)
-    # o_proj / q_proj 4096 x 4096: parts only up to 128 rows; eight waves while there is at most one workgroup per CU
-    assert plan(Q4_K, 4096, 4096, 64) == (4, 4, 2)
-    assert plan(Q4_K, 4096, 4096, 128) == (4, 2, 2)
+    # o_proj / q_proj 4096 x 4096 and k_proj 1024 x 4096: parts only while they take at most a quarter of the CUs; eight waves
+    # while there is at most one workgroup per CU
+    assert plan(Q4_K, 4096, 4096, 64) == (4, 2, 2)
+    assert plan(Q4_K, 4096, 4096, 128) == (4, 1, 2)
+    assert plan(Q4_K, 1024, 4096, 128) == (4, 4, 2)
     assert plan(Q4_K, 4096, 4096, 256) == (4, 1, 2)
     assert plan(Q4_K, 4096, 4096, 512) == (4, 1, 2)
     # up_proj 12288 x 4096 alone, and gate + up as one launch (24576 rows)

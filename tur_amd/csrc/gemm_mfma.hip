@@ -1022,11 +1022,12 @@ int turq_gemm_form(int dtype, int64_t n, int64_t k, int64_t m, int compute_units
 // 32 low tiles at 64 rows, 64 wide ones at 512), and every matrix of the layer at 64 rows - gives every tile to `split`
 // workgroups.  What the parts' meeting costs grows with the partial tiles the launch writes and reads back (m x n x 4 bytes
 // x (2 split - 1)), so the rule takes the low tile for few rows and the wide one above, and only as many parts as leave a
-// quarter of the CUs free (low tiles; half of them when k is short, and then only up to 128 rows: less to win) or fill them
-// once (wide tiles, up to an eighth of the CUs).  Measured on MI355X, Q6_K 4096 x 12288, no split -> split: 64 rows 75 -> 35 us
+// quarter of the CUs free (low tiles; a quarter of the CUs taken when k is short, and then only up to 128 rows: since the
+// low tile runs eight waves there is less to win) or fill them once (wide tiles, up to an eighth of the CUs).  Measured on MI355X, Q6_K 4096 x 12288, no split -> split: 64 rows 75 -> 35 us
 // (low, 6 parts), 128: 78 -> 47 (low, 3), 256: 82 -> 66 (wide, 6), 512: 97 -> 92 (wide, 4: within what a whole layer's step
 // varies by, not taken), 1024: none helps; Q4_K 4096 x 4096: 64 rows 28 -> 22 us (low, 4), 128: 28 -> 27 (low, 2), from 256
-// rows on none helps; 12288 x 4096: none helps.  TURQ_GEMM_SPLIT = 0: never, s > 1: by s wherever s divides (with
+// rows on none helps; 12288 x 4096: none helps; with the eight-wave low tile since: 4096 x 4096 unsplit 21.8 / 22.3 us at 64 /
+// 128 rows against 21.1 / 24.2 in 4 / 2 parts, 1024 x 4096 21.6 / 21.8 against 15.3 / 16.9 in 4 parts.  TURQ_GEMM_SPLIT = 0: never, s > 1: by s wherever s divides (with
 // TURQ_GEMM_SPLIT_FORM = 3 / 4: on the wide / low tile).
 size_t turq_gemm_split_scratch(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int *form_out, int *split_out) {
     if (form_out) *form_out = 0;
@@ -1049,7 +1050,7 @@ size_t turq_gemm_split_scratch(int dtype, int64_t n, int64_t k, int64_t m, int c
         split = ntc % env == 0 ? env : 1;
     } else {
         const bool tall = ntc >= 32;
-        split = tall || m <= 128 ? parts(low_tiles, tall ? 3 * cus / 4 : cus / 2, 4) : 1;
+        split = tall || m <= 128 ? parts(low_tiles, tall ? 3 * cus / 4 : cus / 4, 4) : 1;
         form = 4;
         if (split == 1 && tall && 8 * wide_tiles <= cus) {
             split = parts(wide_tiles, cus, 8);
