@@ -189,8 +189,17 @@ class Bench:
 
     def step_eager(self):
         L, ctx, m, xt = self.L, self.ctx, self.m, self.xt
+        ahead = int(getattr(self.args, "prefetch", 0) or 0)
         if not self.args.single_calls:
-            for cnt, warr, x, yarr, ldys, k, fused in self.groups:
+            for gi, (cnt, warr, x, yarr, ldys, k, fused) in enumerate(self.groups):
+                if ahead:
+                    # the weights of the call `ahead` calls further on (the next step's first ones after the last call): read
+                    # next to this call's launch, in the reference's order of calls
+                    ncnt, nwarr = self.groups[(gi + ahead) % len(self.groups)][:2]
+                    for t in range(ncnt):
+                        rc = L.turq_weight_prefetch(ctx, nwarr[t])
+                        if rc:
+                            capi.check(rc, ctx)
                 if fused == "mlp":
                     rc = L.turq_mlp(ctx, warr[0], warr[1], warr[2], x, xt, m, k, yarr[0], self.yt, ldys[0], None, None, None,
                                     capi.ACTFN_SILU, capi.MEM_DEVICE)
@@ -448,6 +457,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true",
                     help="default workload only: leave out the prefill GEMM, mixed-layer and LM-head legs of the JSON line")
+    ap.add_argument("--prefetch", type=int, default=0,
+                    help="turq_weight_prefetch on the weights of the call this many calls ahead, issued in front of every call")
     ap.add_argument("--single-calls", action="store_true",
                     help="one turq_qmatmul per matrix instead of turq_qmatmul_multi per group of matrices with a common input")
     ap.add_argument("--mlp", action="store_true",

@@ -100,6 +100,7 @@ extern "C" {
     pub fn turq_qmatmul_multi(ctx: *mut turq_ctx, count: c_int, weights: *const *const turq_weight, x: *const c_void, x_dtype: c_int, m: i64, ldx: i64, ys: *const *mut c_void, y_dtype: c_int, ldys: *const i64, biases: *const *const f32, mem: c_int, algo: c_int) -> c_int;
     pub fn turq_qmatmul_gate_up(ctx: *mut turq_ctx, gate: *const turq_weight, up: *const turq_weight, x: *const c_void, x_dtype: c_int, m: i64, ldx: i64, y: *mut c_void, y_dtype: c_int, ldy: i64, bias_gate: *const f32, bias_up: *const f32, act: c_int, mem: c_int) -> c_int;
     pub fn turq_mlp(ctx: *mut turq_ctx, gate: *const turq_weight, up: *const turq_weight, down: *const turq_weight, x: *const c_void, x_dtype: c_int, m: i64, ldx: i64, y: *mut c_void, y_dtype: c_int, ldy: i64, bias_gate: *const f32, bias_up: *const f32, bias_down: *const f32, act: c_int, mem: c_int) -> c_int;
+    pub fn turq_weight_prefetch(ctx: *mut turq_ctx, w: *const turq_weight) -> c_int;
     pub fn turq_quantize_q8_0(ctx: *mut turq_ctx, x: *const f32, m: i64, k: i64, out: *mut c_void, mem: c_int) -> c_int;
     pub fn turq_quantize_q8_k(ctx: *mut turq_ctx, x: *const f32, m: i64, k: i64, out: *mut c_void, mem: c_int) -> c_int;
     pub fn turq_graph_begin(ctx: *mut turq_ctx) -> c_int;

@@ -262,6 +262,18 @@ int turq_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, cons
              int64_t m, int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up,
              const float *bias_down, int act, int mem);
 
+/* A hint that `w` is the weight of one of the next forward calls: one read-only pass over its bytes on a stream of the
+ * context's own, which starts where the context's stream stands when the call is made (so it runs next to whatever is queued
+ * after it) and which nothing waits for.  A decode launch of a few tens of MB spends a third of its time before its first
+ * bytes arrive and after its last request has left, and cannot start before the launch that makes its activations has ended;
+ * its weights depend on nothing, so the memory system can fetch them during those gaps, and the forward call then finds
+ * them in the GPU's memory-side cache (256 MB on an MI355X: hint one or two launches ahead, not a whole model).  Results
+ * are unaffected.  Inside a graph capture the pass becomes a parallel branch of the graph that turq_graph_end joins.
+ * Replaces nothing in the reference, whose CPU path has no launches; the order it serves is the reference's: gate / up then
+ * down in `Qwen3MLP::forward` (src/models/qwen3.rs:161-167), q / k / v, o, gate / up, down per decoder layer
+ * (src/models/qwen3.rs:633-640), one layer after the other. */
+int turq_weight_prefetch(turq_ctx *ctx, const turq_weight *w);
+
 /* ---- activation quantisation (candle's VecDotType::from_float, bit-exact) ---- */
 /* x f32 [m, k] (row stride k) -> Q8_0 blocks (34 B per 32) / Q8_K blocks (292 B per 256).
  * The GPU forward path does not use them (it keeps activations in f16); they are the device

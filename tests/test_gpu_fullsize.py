@@ -63,11 +63,14 @@ def test_lm_head(gpu, dt):
     rows = np.arange(0, n, n // 4096)[:4096]
     sub = raw.reshape(n, -1)[rows].reshape(-1)
     assert rel_l2(y16[:, rows], orc.matmul_dequant(dt, x16, sub, len(rows), k)) <= 2e-5
-    # m = 128 (BASELINE config 5): the prefill GEMM of this format, same spot check, bf16 result
+    # m = 128 (BASELINE config 5): the prefill GEMM of this format (the wide 128 x 256 tile at this shape), same spot check on the
+    # f32 result; the configuration's bf16 output is that result rounded once, bit for bit
     x128 = synth.random_activation(128, k, seed=11, bf16=True)
-    y128 = gpu.qmatmul(w, x128, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16)
+    y128 = gpu.qmatmul(w, x128, n, k, x_dtype=capi.ACT_BF16)
+    yb128 = gpu.qmatmul(w, x128, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16)
     assert np.all(np.isfinite(y128))
-    assert rel_l2(y128[:, rows], orc.matmul_dequant(dt, x128, sub, len(rows), k)) <= 4e-3     # bf16 store: 1.6e-3 alone
+    assert rel_l2(y128[:, rows], orc.matmul_dequant(dt, x128, sub, len(rows), k)) <= 1e-3
+    assert np.array_equal(synth.to_bf16_bits(y128).reshape(128, n), synth.to_bf16_bits(yb128).reshape(128, n))
     gpu.release(w)
 
 

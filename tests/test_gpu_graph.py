@@ -238,3 +238,53 @@ def test_read_yardstick_is_timed_like_a_kernel(gpu):
     assert L.turq_read_yardstick(ctx, buf, 100) == capi.OK      # less than one 4 KiB chunk: nothing to launch
     capi.check(L.turq_sync(ctx), ctx)
     gpu.dev_free(buf)
+
+
+def test_weight_prefetch_changes_no_result_eager_or_captured():
+    """turq_weight_prefetch is a hint: a read-only pass on a stream of the context's own.  The calls around it give the same
+    bits with and without it, eagerly and as a parallel branch of a captured graph (replayed with eager work in between), and a
+    capture that holds such a branch ends cleanly."""
+    gpu = Gpu()
+    L, ctx = gpu.L, gpu.ctx
+    st = Step(gpu, 1, k=2048)
+    other = Step(gpu, 3, k=512)
+    other.set_x(synth.random_activation(3, 512, seed=98))
+
+    def hinted():
+        capi.check(L.turq_weight_prefetch(ctx, st.ws[3]), ctx)     # the weight of the second call, next to the first
+        capi.check(L.turq_qmatmul_multi(ctx, 3, st.warr, st.x, capi.ACT_F32, st.m, st.k, st.yarr, capi.ACT_F32, st.ldys, None,
+                                        capi.MEM_DEVICE, capi.ALGO_AUTO), ctx)
+        for w in st.ws[:3]:                                         # the next step's first weights, next to the second
+            capi.check(L.turq_weight_prefetch(ctx, w), ctx)
+        capi.check(L.turq_qmatmul(ctx, st.ws[3], st.x, capi.ACT_F32, st.m, st.k, st.ys[3], capi.ACT_F32, st.ns[3], None,
+                                  capi.MEM_DEVICE, capi.ALGO_AUTO), ctx)
+
+    try:
+        assert L.turq_weight_prefetch(ctx, None) == capi.ERR_INVALID
+        st.set_x(synth.random_activation(1, st.k, seed=21))
+        st.calls()
+        want = st.outputs()
+        st.clear_outputs()
+        hinted()
+        for y, w in zip(st.outputs(), want):
+            assert np.array_equal(y, w)
+        capi.check(L.turq_graph_begin(ctx), ctx)
+        hinted()
+        g = ctypes.c_void_p()
+        capi.check(L.turq_graph_end(ctx, ctypes.byref(g)), ctx)
+        for rep in range(3):
+            st.set_x(synth.random_activation(1, st.k, seed=30 + rep))
+            st.clear_outputs()
+            st.calls()
+            want = st.outputs()
+            other.calls()
+            other.outputs()
+            st.clear_outputs()
+            capi.check(L.turq_graph_launch(ctx, g), ctx)
+            for y, w in zip(st.outputs(), want):
+                assert np.array_equal(y, w), rep
+        L.turq_graph_destroy(g)
+    finally:
+        st.close()
+        other.close()
+        gpu.close()

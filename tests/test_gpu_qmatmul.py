@@ -228,6 +228,26 @@ def test_prefill_gemm(gpu, dt, n, k, m):
     gpu.release(w)
 
 
+@pytest.mark.parametrize("dt", [Q6_K, Q5_K])
+def test_prefill_tall_weight_f32_and_bf16(gpu, dt):
+    # a vocabulary-like weight (many rows, ragged) at 128 rows: the 128 x 128 tile of the 1 x 4 wave grid by the rule, the wide
+    # 128 x 256 tile when test_prefill_tile_shapes forces it; f32 result against the oracle on every 8th row, and the bf16
+    # output is that result rounded once, bit for bit
+    n, k, m = 20000, 4096, 128
+    raw = synth.random_weight(dt, n, k, seed=dt + 70)
+    w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+    x = synth.random_activation(m, k, seed=71, bf16=True)
+    y = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16)
+    yb = gpu.qmatmul(w, x, n, k, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16)
+    gpu.release(w)
+    rows = np.arange(1, n, 8)
+    sub = raw.reshape(n, -1)[rows].reshape(-1)
+    assert np.all(np.isfinite(y))
+    assert rel_l2(y[:, rows], orc.matmul_dequant(dt, x, sub, len(rows), k)) <= 1e-3
+    assert np.array_equal(synth.to_bf16_bits(y).reshape(m, n), synth.to_bf16_bits(yb).reshape(m, n))
+
+
+
 # Tall-k matrices at prefill chunk sizes (down_proj: 4096 x 12288) make few workgroup tiles, so the launcher gives every tile
 # to several workgroups that each take a part of the columns and meet in device memory.  Shapes that split on a 256-CU device
 # (few tiles, many super-blocks): results against the oracle, twice in a row (the tiles' counters must be back at zero), with

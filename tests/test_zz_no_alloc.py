@@ -2,7 +2,8 @@
 
 Both run the same kernels, so the outputs must be bit-identical; the only difference is where the prepared activation
 fragments live (a static device array instead of the context's growable buffer).  Two calls in a row, the second with a
-smaller input, per launch kind: prepared fragments (2 <= m <= 32), the prefill GEMM (m > 32), and one row (no scratch).
+smaller input, per launch kind: prepared fragments in the static array (17 .. 32 rows of a wide weight, a k that is not a
+multiple of 512), the prefill GEMM (m > 32), and the kernels that use no scratch (one row; rows staged in the kernel).
 One exception: prefill launches whose columns turq_qmatmul splits over several workgroups (few tiles: small or tall matrices
 at prompt-chunk sizes) need a second scratch buffer for the partial tiles, which the call that allocates nothing does not
 have; it runs the same kernel unsplit, i.e. the same products added up in another order, and is held to 2e-6 relative L2
@@ -36,13 +37,15 @@ def both(gpu, w, x, n, k, x_dtype, y_dtype):
 
 
 @pytest.mark.parametrize("dt,n,k,ms", [
-    (capi.Q4_K, 4096, 4096, (32, 8)),       # prepared fragments, then fewer rows
+    (capi.Q4_K, 4096, 4096, (32, 8)),       # up to 4096 columns: fragments made in the kernel from the rows themselves, no scratch
     (capi.Q6_K, 1024, 4096, (16, 3)),
+    (capi.Q6_K, 4096, 12288, (32, 20)),     # 17 .. 32 rows of 12288 columns: fragments prepared in the static array, then fewer rows
+    (capi.Q4_K, 2048, 4352, (24, 17)),      # k not a multiple of 512 (17 column tiles): prepared fragments again
     (capi.Q4_K, 1024, 4096, (512, 64)),     # the prefill GEMM, then a smaller chunk
     (capi.Q5_K, 512, 2048, (200, 33)),
     (capi.Q8_0, 3072, 1024, (48, 2)),
     (capi.Q4_K, 12288, 4096, (1, 1)),       # one row: no scratch at all
-], ids=["q4k-frag", "q6k-frag", "q4k-gemm", "q5k-gemm", "q8_0", "q4k-row1"])
+], ids=["q4k-staged", "q6k-staged", "q6k-frag-k12288", "q4k-frag-odd-k", "q4k-gemm", "q5k-gemm", "q8_0", "q4k-row1"])
 def test_noalloc_equals_qmatmul_twice_in_a_row(gpu, dt, n, k, ms):
     raw = synth.random_weight(dt, n, k, seed=n + k)
     w = gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED)

@@ -55,6 +55,7 @@ _SIGS = {
                                      c_void_p, c_void_p, c_int, c_int]),
     "turq_mlp": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64,
                          c_void_p, c_void_p, c_void_p, c_int, c_int]),
+    "turq_weight_prefetch": (c_int, [c_void_p, c_void_p]),
     "turq_quantize_q8_0": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
     "turq_quantize_q8_k": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
     "turq_read_yardstick": (c_int, [c_void_p, c_void_p, c_size_t]),

@@ -142,6 +142,18 @@ int turq_ctx_create(int device, turq_ctx **out) {
     if (ctx->static_scratch_err != (int)hipSuccess) { ctx->static_scratch = nullptr; ctx->static_scratch_cap = 0; }
     e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
     if (e != hipSuccess) return turq_fail(nullptr, TURQ_ERR_HIP, "hipStreamCreate failed: %s", hipGetErrorString(e));
+    // the prefetch stream and its events exist from the start: nothing can be created while a graph is being captured
+    e = hipStreamCreateWithFlags(&ctx->pf_stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ctx->ev_pf_fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ctx->ev_pf_join, hipEventDisableTiming);
+    if (e != hipSuccess) {
+        turq_ctx *dead = ctx.release();
+        turq_ctx_destroy(dead);
+        return turq_fail(nullptr, TURQ_ERR_HIP, "turq_ctx_create: the prefetch stream could not be made: %s", hipGetErrorString(e));
+    }
+    ctx->pf_workgroups = ctx->compute_units > 0 ? ctx->compute_units : 256;
+    if (const char *v = getenv("TURQ_PREFETCH_WGS")) { const int x = atoi(v); if (x >= 1 && x <= 4096) ctx->pf_workgroups = x; }
+    if (const char *v = getenv("TURQ_PREFETCH_DEPTH")) { const int x = atoi(v); if (x >= 1 && x <= 4) ctx->pf_depth = x; }
     *out = ctx.release();
     return TURQ_OK;
 }
@@ -167,6 +179,9 @@ void turq_ctx_destroy(turq_ctx *ctx) {
         if (ctx->ev_join[i]) (void)hipEventDestroy(ctx->ev_join[i]);
     }
     if (ctx->ev_fork) (void)hipEventDestroy(ctx->ev_fork);
+    if (ctx->pf_stream) { (void)hipStreamSynchronize(ctx->pf_stream); (void)hipStreamDestroy(ctx->pf_stream); }
+    if (ctx->ev_pf_fork) (void)hipEventDestroy(ctx->ev_pf_fork);
+    if (ctx->ev_pf_join) (void)hipEventDestroy(ctx->ev_pf_join);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
 }
@@ -176,6 +191,7 @@ const char *turq_last_error(const turq_ctx *ctx) { return ctx ? ctx->err.c_str()
 int turq_sync(turq_ctx *ctx) {
     TURQ_ENTER(ctx);
     TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (!ctx->capturing) TURQ_HIP(ctx, hipStreamSynchronize(ctx->pf_stream));
     return TURQ_OK;
 }
 
@@ -689,8 +705,10 @@ int turq_graph_begin(turq_ctx *ctx) {
     TURQ_ENTER(ctx);
     if (ctx->capturing) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_begin: a capture is already running");
     if (ctx->profiling) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_begin: kernel timing is on; events cannot be captured");
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->pf_stream));  // eager prefetch work stays outside the capture
     TURQ_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
     ctx->capturing = true;
+    ctx->pf_in_capture = false;
     return TURQ_OK;
 }
 
@@ -700,10 +718,17 @@ int turq_graph_end(turq_ctx *ctx, turq_graph **out) {
     *out = nullptr;
     if (!ctx->capturing)
         return turq_fail(ctx, TURQ_ERR_INVALID, "turq_graph_end: no capture is running (a call that fails inside a capture ends and discards it)");
+    hipError_t e = hipSuccess;
+    if (ctx->pf_in_capture) {  // the prefetch branch joins the captured stream, or the capture could not end
+        e = hipEventRecord(ctx->ev_pf_join, ctx->pf_stream);
+        if (e == hipSuccess) e = hipStreamWaitEvent(ctx->stream, ctx->ev_pf_join, 0);
+        ctx->pf_in_capture = false;
+    }
     ctx->capturing = false;
     std::unique_ptr<turq_graph> g(new (std::nothrow) turq_graph);
     hipGraph_t graph = nullptr;
-    hipError_t e = hipStreamEndCapture(ctx->stream, &graph);
+    const hipError_t e_end = hipStreamEndCapture(ctx->stream, &graph);
+    if (e == hipSuccess) e = e_end;
     if (e != hipSuccess || !g) {
         if (graph) (void)hipGraphDestroy(graph);
         return turq_fail(ctx, g ? TURQ_ERR_HIP : TURQ_ERR_OOM, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
@@ -737,6 +762,19 @@ void turq_graph_destroy(turq_graph *g) {
     if (g->graph) (void)hipGraphDestroy(g->graph);
     if (g->tally) g->tally->live.fetch_sub(1, std::memory_order_acq_rel);
     delete g;
+}
+
+static int impl_weight_prefetch(turq_ctx *ctx, const turq_weight *w) {
+    TURQ_ENTER(ctx);
+    if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_weight_prefetch: null weight");
+    if (w->device != ctx->device) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_weight_prefetch: weight lives on device %d, context on %d", w->device, ctx->device);
+    if (!w->dev || w->dev_bytes < 4096) return TURQ_OK;
+    // starts where the context's stream stands now, i.e. next to whatever is queued on it after this call
+    TURQ_HIP(ctx, hipEventRecord(ctx->ev_pf_fork, ctx->stream));
+    TURQ_HIP(ctx, hipStreamWaitEvent(ctx->pf_stream, ctx->ev_pf_fork, 0));
+    if (ctx->capturing) ctx->pf_in_capture = true;
+    TURQ_HIP(ctx, turq_launch_weight_prefetch(w->dev, w->dev_bytes, ctx->pf_workgroups, ctx->pf_depth, ctx->pf_stream, nullptr, nullptr));
+    return TURQ_OK;
 }
 
 int turq_read_yardstick(turq_ctx *ctx, const void *dev_ptr, size_t nbytes) {
@@ -862,6 +900,8 @@ int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void
 int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
     return capture_guard(ctx, impl_quantize_q8_k(ctx, x, m, k, out, mem));
 }
+
+int turq_weight_prefetch(turq_ctx *ctx, const turq_weight *w) { return capture_guard(ctx, impl_weight_prefetch(ctx, w)); }
 
 int turq_rms_norm(turq_ctx *ctx, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, const float *weight, float eps, void *y,
                   int y_dtype, int64_t ldy, int mem) {

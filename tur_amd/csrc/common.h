@@ -106,6 +106,12 @@ struct turq_ctx {
     static constexpr int kSide = 2;
     hipStream_t side[kSide] = {nullptr, nullptr};
     hipEvent_t ev_fork = nullptr, ev_join[kSide] = {nullptr, nullptr};
+    // turq_weight_prefetch: a stream of its own for the read-only passes, forked from `stream` where the call is made (ev_pf_fork)
+    // and, inside a graph capture, joined to it again before the capture ends (ev_pf_join)
+    hipStream_t pf_stream = nullptr;
+    hipEvent_t ev_pf_fork = nullptr, ev_pf_join = nullptr;
+    bool pf_in_capture = false;  // the running capture holds prefetch work that is not joined yet
+    int pf_workgroups = 0, pf_depth = 4;
     // kernel timing (turq_profile_*): event pairs recorded around matmul kernels
     bool profiling = false;
     bool capturing = false;
@@ -193,6 +199,8 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
 // act(gate) * up on two f32 matrices [m, n] of row stride n (act_mul.hip)
 hipError_t turq_launch_read_yardstick(const void *buf, size_t nbytes, int workgroups, hipStream_t stream, hipEvent_t ev_start,
                                       hipEvent_t ev_stop);
+hipError_t turq_launch_weight_prefetch(const void *buf, size_t nbytes, int workgroups, int depth, hipStream_t stream, hipEvent_t ev_start,
+                                       hipEvent_t ev_stop);
 hipError_t turq_launch_silu_mul(const float *gate, const float *up, int64_t m, int64_t n, void *y, int y_dtype, int64_t ldy,
                                 hipStream_t stream);
 // act(gate) * up inside the one-row kernel; *taken = false (and nothing launched) where that kernel does not apply
