@@ -182,10 +182,10 @@ class Bench:
         self.step_flops = layers * sum(2 * self.m * n * k for _, _, n, k in self.mats)
 
     def use_mlp(self):
-        """gate / up / down as one turq_mlp call per layer (--mlp), decode rows only"""
+        """gate / up / down as one turq_mlp call per layer (--mlp)"""
         labels = [mt[0] for mt in self.mats]
         has = any(labels[i:i + 3] == ["gate", "up", "down"] for i in range(len(labels)))
-        return has and bool(getattr(self.args, "mlp", False)) and not self.args.single_calls and not self.args.gate_up and getattr(self, "m", 1) <= 32
+        return has and bool(getattr(self.args, "mlp", False)) and not self.args.single_calls and not self.args.gate_up
 
     def step_eager(self):
         L, ctx, m, xt = self.L, self.ctx, self.m, self.xt
@@ -248,7 +248,9 @@ class Bench:
             if mlp and label == "down":
                 from oracle import oracle_np as onp
                 _, gdt, gn, gk = by_label["gate"]
-                xg = self.x_host[gk].astype(np.float16).astype(np.float32)
+                keep = min(self.m, 16)      # the chain needs every column of the intermediate: bounded by checking the first rows only
+                got = got[:keep]
+                xg = self.x_host[gk][:keep].astype(np.float16).astype(np.float32)
                 h = onp.silu_mul(orc.matmul_dequant(gdt, xg, self.host_raw["gate"], gn, gk), orc.matmul_dequant(gdt, xg, self.host_raw["up"], gn, gk))
                 want = orc.matmul_dequant(dt, h, sub, len(rows), k)
             else:

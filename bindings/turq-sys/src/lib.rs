@@ -79,6 +79,7 @@ extern "C" {
     pub fn turq_sync(ctx: *mut turq_ctx) -> c_int;
     pub fn turq_ctx_stream(ctx: *mut turq_ctx) -> *mut c_void;
     pub fn turq_ctx_set_wide_activations(ctx: *mut turq_ctx, on: c_int) -> c_int;
+    pub fn turq_ctx_nonfinite_count(ctx: *mut turq_ctx, count: *mut u64, reset: c_int) -> c_int;
     pub fn turq_ctx_device_info(ctx: *mut turq_ctx, name: *mut c_char, name_cap: usize, compute_units: *mut c_int) -> c_int;
     pub fn turq_dev_alloc(ctx: *mut turq_ctx, nbytes: usize, out: *mut *mut c_void) -> c_int;
     pub fn turq_dev_free(ctx: *mut turq_ctx, ptr: *mut c_void) -> c_int;

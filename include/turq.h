@@ -105,6 +105,16 @@ void *turq_ctx_stream(turq_ctx *ctx);
  * wide path: they are the reference's own contract, and the staging copies dominate them anyway.  turq_qmatmul_noalloc never
  * takes it. */
 int turq_ctx_set_wide_activations(turq_ctx *ctx, int on);
+/* Whether a forward call left the number range of its kernels.  Every kernel that stores results (the matmuls, turq_rms_norm,
+ * the fragment preparation of calls with more than 32 rows, the f16 intermediate of turq_mlp) counts the elements it stores
+ * that are no finite numbers: the output of a row that held a finite value of magnitude 65520 or more while wide activations
+ * were off (f16 turns it into an infinity), or of a row that held an infinity or a NaN to begin with.  The call waits for the
+ * context's stream and returns the count since the last reset (it stops at about 2^20; the counters live in device memory of
+ * the context's GPU and are shared by all contexts on it); reset != 0 clears it.  A host that sees a non-zero count re-runs
+ * the step after turq_ctx_set_wide_activations(ctx, 1), with which finite inputs of any magnitude give finite results.  Not
+ * inside a graph capture.
+ * Stands in for: the reference's f32 activations of any magnitude (src/weights/mod.rs:84-99), which never overflow. */
+int turq_ctx_nonfinite_count(turq_ctx *ctx, uint64_t *count, int reset);
 /* name and compute-unit count of the context's device */
 int turq_ctx_device_info(turq_ctx *ctx, char *name, size_t name_cap, int *compute_units);
 

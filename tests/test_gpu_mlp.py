@@ -180,3 +180,29 @@ def test_inside_a_graph(gpu):
         gpu.dev_free(b)
     for w in ws:
         gpu.release(w)
+
+
+@pytest.mark.parametrize("dt_gu,dt_dn", [(Q4_K, Q6_K), (Q5_K, Q4_K)])
+@pytest.mark.parametrize("m", [72, 128, 512])
+def test_prompt_chunks(gpu, dt_gu, dt_dn, m):
+    """More than 32 rows: gate / up GEMMs into f32 scratch, ONE kernel from the two products to down_proj's fragments (no f16 copy
+    of the intermediate, no separate preparation), down_proj's GEMM.  Bit-equal to the two calls, within 1e-3 of the oracle's
+    chain; bf16 in and out as a prompt chunk has them, and with biases."""
+    n_ff, k, n_out = 3072, 2048, 1536
+    raws, ws = weights(gpu, dt_gu, dt_dn, n_ff, k, n_out, seed=23 + m)
+    rng = np.random.default_rng(m)
+    biases = tuple(rng.standard_normal(n).astype(np.float32) * 0.1 for n in (n_ff, n_ff, n_out))
+    x = synth.random_activation(m, k, seed=m, bf16=True) * XS
+    x = synth.from_bf16_bits(synth.to_bf16_bits(x)).reshape(m, k)
+    for bs in ((None, None, None), biases):
+        launches = []
+        y = gpu.mlp(*ws, x, n_ff, k, n_out, x_dtype=capi.ACT_BF16, biases=bs, launches=launches)
+        assert np.array_equal(y, two_calls(gpu, ws, x, n_ff, k, n_out, x_dtype=capi.ACT_BF16, biases=bs))
+        g = orc.matmul_dequant(dt_gu, x, raws[0], n_ff, k) + (0 if bs[0] is None else bs[0])
+        u = orc.matmul_dequant(dt_gu, x, raws[1], n_ff, k) + (0 if bs[1] is None else bs[1])
+        want = orc.matmul_dequant(dt_dn, onp.silu_mul(g, u).astype(np.float32), raws[2], n_out, n_ff) + (0 if bs[2] is None else bs[2])
+        assert rel_l2(y, want) <= 1e-3, rel_l2(y, want)
+    yb = gpu.mlp(*ws, x, n_ff, k, n_out, x_dtype=capi.ACT_BF16, y_dtype=capi.ACT_BF16, biases=biases)
+    assert np.array_equal(synth.to_bf16_bits(yb).reshape(m, n_out), synth.to_bf16_bits(y).reshape(m, n_out))
+    for w in ws:
+        gpu.release(w)

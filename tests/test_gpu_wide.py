@@ -114,3 +114,75 @@ def test_non_finite_activations_propagate(gpu):
     assert rel_l2(y[[0, 3]], want) <= 1e-3                      # the finite rows are untouched
     assert not np.any(np.isfinite(y[1])) and np.all(np.isnan(y[2]))
     gpu.release(w)
+
+
+def nonfinite(g, reset=1):
+    n = ctypes.c_uint64(12345)
+    capi.check(g.L.turq_ctx_nonfinite_count(g.ctx, ctypes.byref(n), reset), g.ctx)
+    return n.value
+
+
+@pytest.mark.parametrize("m", [1, 2, 8, 24, 40, 100])     # one-row kernel, two rows, staged rows, prepared fragments, prefill GEMM
+@pytest.mark.parametrize("dt", [Q4_K, Q6_K, Q8_0])
+def test_overflow_on_device_pointers_is_counted(dt, m):
+    """Wide activations off, device pointers, a finite row of magnitude 1e5: the call returns TURQ_OK and every kernel exits
+    normally, the row comes out as infinities / NaNs, and turq_ctx_nonfinite_count sees it; rows inside the f16 range leave the
+    count at zero, and so does the same input with wide activations on."""
+    g = Gpu()
+    try:
+        L, ctx = g.L, g.ctx
+        n, k = 208, 1024
+        raw = synth.random_weight(dt, n, k, seed=dt + m)
+        w = g.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+        nonfinite(g)                                   # whatever earlier tests of this process left behind
+        x = np.random.default_rng(m).standard_normal((m, k)).astype(np.float32)
+        y = g.qmatmul_device(w, x, n, k)
+        assert np.all(np.isfinite(y)) and nonfinite(g, reset=0) == 0
+        x[m // 2] *= np.float32(1e5)
+        y = g.qmatmul_device(w, x, n, k)
+        assert not np.all(np.isfinite(y[m // 2]))
+        assert nonfinite(g, reset=0) > 0
+        assert nonfinite(g, reset=1) > 0 and nonfinite(g) == 0          # sticky until it is reset
+        capi.check(L.turq_ctx_set_wide_activations(ctx, 1), ctx)
+        y = g.qmatmul_device(w, x, n, k)
+        assert np.all(np.isfinite(y)) and per_row_rel(y, orc.matmul_dequant(dt, x, raw, n, k)).max() <= 1e-3
+        assert nonfinite(g) == 0
+        g.release(w)
+    finally:
+        g.close()
+
+
+@pytest.mark.parametrize("m", [1, 8, 32, 48, 160])
+def test_mlp_intermediate_outside_f16_is_counted_and_wide_handles_it(m):
+    """turq_mlp keeps act(gate) * up as f16 where down_proj's kernels would round it to f16 anyway: an intermediate of magnitude
+    65520 and more is an infinity there.  With wide activations off the call still returns TURQ_OK and the count says so; with
+    wide activations on the intermediate stays f32, its rows are scaled for down_proj, and the result is finite and within the
+    bar of the oracle's chain."""
+    from oracle import oracle_np as onp
+    g = Gpu()
+    try:
+        L, ctx = g.L, g.ctx
+        n_ff, k, n_out = 1024, 512, 192
+        rg, ru = synth.random_weight(Q4_K, n_ff, k, seed=1), synth.random_weight(Q4_K, n_ff, k, seed=2)
+        rd = synth.random_weight(Q6_K, n_out, n_ff, seed=3)
+        ws = [g.upload(Q4_K, n_ff, k, rg, capi.LAYOUT_TILED), g.upload(Q4_K, n_ff, k, ru, capi.LAYOUT_TILED),
+              g.upload(Q6_K, n_out, n_ff, rd, capi.LAYOUT_TILED)]
+        x = synth.random_activation(m, k, seed=m, bf16=True) * np.float32(16.0)
+        h = onp.silu_mul(orc.matmul_dequant(Q4_K, x, rg, n_ff, k), orc.matmul_dequant(Q4_K, x, ru, n_ff, k))
+        assert np.abs(h).max() > 65520 and np.all(np.isfinite(h.astype(np.float32)))      # the case this test is about
+        want = orc.matmul_dequant(Q6_K, h.astype(np.float32), rd, n_out, n_ff)
+        nonfinite(g)
+        y = g.mlp(*ws, x, n_ff, k, n_out)
+        assert not np.all(np.isfinite(y))
+        assert nonfinite(g) > 0
+        capi.check(L.turq_ctx_set_wide_activations(ctx, 1), ctx)
+        y = g.mlp(*ws, x, n_ff, k, n_out)
+        assert np.all(np.isfinite(y))
+        # (two matmuls in a row, each inside its own 1e-3: more than 32 rows go through the prefill GEMM, about 3e-4 a stage,
+        # on an intermediate of six orders of magnitude)
+        assert per_row_rel(y, want).max() <= (1e-3 if m <= 32 else 2e-3)
+        assert nonfinite(g) == 0
+        for w in ws:
+            g.release(w)
+    finally:
+        g.close()

@@ -31,6 +31,7 @@ _SIGS = {
     "turq_sync": (c_int, [c_void_p]),
     "turq_ctx_stream": (c_void_p, [c_void_p]),
     "turq_ctx_set_wide_activations": (c_int, [c_void_p, c_int]),
+    "turq_ctx_nonfinite_count": (c_int, [c_void_p, POINTER(c_uint64), c_int]),
     "turq_ctx_device_info": (c_int, [c_void_p, c_char_p, c_size_t, POINTER(c_int)]),
     "turq_dev_alloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "turq_dev_free": (c_int, [c_void_p, c_void_p]),

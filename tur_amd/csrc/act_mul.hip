@@ -29,3 +29,5 @@ hipError_t turq_launch_silu_mul(const float *gate, const float *up, int64_t m, i
     silu_mul_kernel<<<(unsigned)blocks, 256, 0, stream>>>(gate, up, m, n, y, y_dtype, ldy);
     return hipGetLastError();
 }
+
+TURQ_NONFINITE_READER(turq_nonfinite_act_mul)

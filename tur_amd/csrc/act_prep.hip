@@ -61,6 +61,8 @@ __global__ void __launch_bounds__(256) act_prep_kernel(const void *__restrict__ 
     half8v h0, h1;
     float sum = 0.0f;
 #pragma unroll
+    for (int j = 0; j < 16; j++) turq_note_result<TURQ_ACT_F16>(v[j]);
+#pragma unroll
     for (int j = 0; j < 8; j++) {
         h0[j] = (_Float16)v[j];
         h1[j] = (_Float16)v[8 + j];
@@ -111,9 +113,11 @@ hipError_t launch(int dtype, const void *x, int64_t m, int64_t k, int64_t ldx, v
 // are added up between the four neighbouring lanes that hold a sub-block.  No LDS and no barrier: the kernel is a chain of
 // load -> store latencies, and four times as many, smaller workgroups keep four times as many of them in flight per CU
 // (6.3 -> 5.1 us at m = 512, K = 4096).
-template <int XT, bool Q8>
+// GU: the rows are SiLU(x) * up of two f32 matrices (the MLP's intermediate, src/models/qwen3.rs:161-167), evaluated and
+// rounded to f16 exactly as silu_mul_kernel stores it, so that down_proj's fragments come out of the two products directly.
+template <int XT, bool Q8, bool GU = false>
 __global__ void __launch_bounds__(256) act_prep32_kernel(const void *__restrict__ x, int64_t m, int64_t k, int64_t ldx,
-                                                         int64_t ntc, half8v *__restrict__ frags) {
+                                                         int64_t ntc, half8v *__restrict__ frags, const float *__restrict__ up = nullptr) {
     const int tid = threadIdx.x;
     const int64_t wg = blockIdx.x;  // (mt * ntc + b) * 4 + quarter
     const int quarter = (int)(wg & 3);
@@ -147,10 +151,25 @@ __global__ void __launch_bounds__(256) act_prep32_kernel(const void *__restrict_
 #pragma unroll
         for (int j = 0; j < 8; j++) v[j] = (row < m && col0 + j < k) ? ld_act<XT>(x, row * ldx + col0 + j) : 0.0f;
     }
+    if constexpr (GU) {
+        static_assert(XT == TURQ_ACT_F32, "the two products are f32");
+        float u[8];
+        const float *us = up + row * ldx + col0;
+        if (row < m && col0 + 8 <= k && ((uintptr_t)us & 15) == 0) {
+            const float4v lo = ((const float4v *)us)[0], hi = ((const float4v *)us)[1];
+            u[0] = lo.x, u[1] = lo.y, u[2] = lo.z, u[3] = lo.w, u[4] = hi.x, u[5] = hi.y, u[6] = hi.z, u[7] = hi.w;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) u[j] = (row < m && col0 + j < k) ? us[j] : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = v[j] / (1.0f + expf(-v[j])) * u[j];
+    }
     half8v h;
     float sum = 0.0f;
 #pragma unroll
     for (int j = 0; j < 8; j++) {
+        turq_note_result<TURQ_ACT_F16>(v[j]);
         h[j] = (_Float16)v[j];
         sum += (float)h[j];
     }
@@ -203,3 +222,17 @@ hipError_t turq_launch_act_prep32(int dtype, const void *x, int x_dtype, int64_t
 #undef TURQ_PREP32
     return hipGetLastError();
 }
+
+// fragments of SiLU(gate) * up for the prefill GEMM of down_proj, from the two f32 products [m, n] (row stride n) that the
+// gate / up GEMMs left in scratch memory: what silu_mul_kernel (f16 output) followed by turq_launch_act_prep32 would write
+hipError_t turq_launch_silu_mul_prep32(int dtype, const float *gate, const float *up, int64_t m, int64_t n, void *frags,
+                                       hipStream_t stream) {
+    if (m == 0 || n == 0) return hipSuccess;
+    const int64_t ntc = (n + 255) / 256;
+    const unsigned grid = (unsigned)(((m + 31) / 32) * ntc * 4);
+    if (dtype == TURQ_Q8_0) act_prep32_kernel<TURQ_ACT_F32, true, true><<<grid, 256, 0, stream>>>(gate, m, n, n, ntc, (half8v *)frags, up);
+    else act_prep32_kernel<TURQ_ACT_F32, false, true><<<grid, 256, 0, stream>>>(gate, m, n, n, ntc, (half8v *)frags, up);
+    return hipGetLastError();
+}
+
+TURQ_NONFINITE_READER(turq_nonfinite_act_prep)

@@ -690,6 +690,12 @@ static int impl_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *u
     // kept as f16 to begin with: the same values reach the same multiplications, and the rows that every compute unit reads
     // for down_proj are half as long.  (Not with wide activations, which scale f32 rows before that rounding, and not for a
     // dense or native-layout down_proj, which multiplies in f32.)
+    if (m > TURQ_GEMV_MAX_M && !ctx->wide && x && y && turq_dt_is_quant(gate->dtype) && turq_dt_is_quant(up->dtype) && turq_dt_is_quant(down->dtype)) {
+        // a prompt chunk: the two products, one kernel from them to down_proj's fragments, down_proj's GEMM
+        bool taken = false;
+        const int rc = turq_mlp_prefill(ctx, gate, up, down, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, bias_down, &taken);
+        if (rc != TURQ_OK || taken) return rc;
+    }
     const bool h16 = !ctx->wide && turq_dt_is_quant(down->dtype) && down->layout == TURQ_LAYOUT_TILED && n_ff % 8 == 0;
     const int ht = h16 ? TURQ_ACT_F16 : TURQ_ACT_F32;
     int rc = turq_ctx_reserve(ctx, &ctx->mlp_h, &ctx->mlp_h_cap, h_elems * (h16 ? sizeof(uint16_t) : sizeof(float)) + 16);
@@ -912,6 +918,18 @@ int turq_ctx_set_wide_activations(turq_ctx *ctx, int on) {
     if (!ctx) return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_ctx_set_wide_activations: null context");
     if (ctx->capturing) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_ctx_set_wide_activations: a graph capture is running");
     ctx->wide = on != 0;
+    return TURQ_OK;
+}
+
+int turq_ctx_nonfinite_count(turq_ctx *ctx, uint64_t *count, int reset) {
+    TURQ_ENTER(ctx);
+    if (ctx->capturing) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_ctx_nonfinite_count: a graph capture is running");
+    TURQ_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    unsigned long long sum = 0;
+#define TURQ_READ_NONFINITE(fn) TURQ_HIP(ctx, fn(&sum, reset));
+    TURQ_NONFINITE_UNITS(TURQ_READ_NONFINITE)
+#undef TURQ_READ_NONFINITE
+    if (count) *count = (uint64_t)sum;
     return TURQ_OK;
 }
 

@@ -188,6 +188,15 @@ hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t 
                                    int64_t m, int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias,
                                    hipStream_t stream);
 
+// per translation unit whose kernels store results: adds the current device's count of non-finite results to *sum (mfma_common.h)
+#define TURQ_NONFINITE_UNITS(X)                                                                                                   \
+    X(turq_nonfinite_gemv_mfma) X(turq_nonfinite_gemv_row1) X(turq_nonfinite_gemv_cs) X(turq_nonfinite_gemv_cs_staged_f32)         \
+    X(turq_nonfinite_gemv_cs_staged_bf16) X(turq_nonfinite_gemv_cs_staged_f16) X(turq_nonfinite_gemm_mfma)                        \
+    X(turq_nonfinite_gemv_simple) X(turq_nonfinite_act_mul) X(turq_nonfinite_wide) X(turq_nonfinite_norm) X(turq_nonfinite_act_prep)
+#define TURQ_DECLARE_NONFINITE(fn) hipError_t fn(unsigned long long *sum, int reset);
+TURQ_NONFINITE_UNITS(TURQ_DECLARE_NONFINITE)
+#undef TURQ_DECLARE_NONFINITE
+
 // largest m the skinny MFMA kernel takes; above it the LDS-tiled GEMM runs
 #define TURQ_GEMV_MAX_M 32
 // largest m for which the skinny kernel can prepare the activations itself (no separate launch);
@@ -210,5 +219,10 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
 bool turq_rows_in_chunks(const turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t ldx, int64_t m);
 int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m, int64_t ldx,
                             void *const *y, int yt, const int64_t *ldy, const float *const *bias, bool *taken);
+// The whole MLP of a prompt chunk (more than 32 rows): gate / up GEMMs into f32 scratch, one kernel that turns the two products
+// into down_proj's fragments, down_proj's GEMM on them; *taken = false (nothing launched) where that route does not apply
+int turq_mlp_prefill(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt,
+                     int64_t m, int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up,
+                     const float *bias_down, bool *taken);
 int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m,
                             int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias);

@@ -867,6 +867,8 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        uint32_t bad = 0;  // results that are no finite numbers, or do not fit an f16 output (turq_ctx_nonfinite_count)
+        const float lim = yt == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
         if (yt == TURQ_ACT_F32) {
             constexpr int CPR = WN * 32 / 4;  // 16-byte pieces per row
 #pragma unroll 4
@@ -874,7 +876,10 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                 const int c = it * 64 + lane;
                 const int r = c / CPR, cc = c - r * CPR;
                 const float4v v = *(const float4v *)(stage + r * OUT_PITCH + 4 * cc);
-                if (row0 + r < m && col0 + 4 * cc < n) *(float4v *)((float *)y + (row0 + r) * ldy + col0 + 4 * cc) = v;
+                if (row0 + r < m && col0 + 4 * cc < n) {
+                    turq_note_accum(v.x, lim, bad), turq_note_accum(v.y, lim, bad), turq_note_accum(v.z, lim, bad), turq_note_accum(v.w, lim, bad);
+                    *(float4v *)((float *)y + (row0 + r) * ldy + col0 + 4 * cc) = v;
+                }
             }
         } else {
             constexpr int CPR = WN * 32 / 8;
@@ -889,10 +894,18 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                     o = uint4v{pack_bf16x2(v0.x, v0.y), pack_bf16x2(v0.z, v0.w), pack_bf16x2(v1.x, v1.y), pack_bf16x2(v1.z, v1.w)};
                 else
                     o = uint4v{pack_f16x2(v0.x, v0.y), pack_f16x2(v0.z, v0.w), pack_f16x2(v1.x, v1.y), pack_f16x2(v1.z, v1.w)};
-                if (row0 + r < m && col0 + 8 * cc < n) *(uint4v *)((uint16_t *)y + (row0 + r) * ldy + col0 + 8 * cc) = o;
+                if (row0 + r < m && col0 + 8 * cc < n) {
+                    const float vs[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+                    for (int e = 0; e < 8; e++) turq_note_accum(vs[e], lim, bad);
+                    *(uint4v *)((uint16_t *)y + (row0 + r) * ldy + col0 + 8 * cc) = o;
+                }
             }
         }
+        turq_note_flush(bad);
     } else {
+        uint32_t bad = 0;
+        const float lim = yt == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
 #pragma unroll
         for (int j = 0; j < WN; j++) {
             const int64_t col = col0 + 32 * j + n32;
@@ -905,12 +918,14 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                     const int64_t row = row0 + 32 * i + 8 * (e >> 2) + 4 * g32 + (e & 3);
                     if (row < m) {
                         const float v = acc[i][j][e] * inv_ws + bv;
-                        if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, row * ldy + col, v);
-                        else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, row * ldy + col, v);
-                        else turq_store_out<TURQ_ACT_F16>(y, row * ldy + col, v);
+                        turq_note_accum(v, lim, bad);
+                        if (yt == TURQ_ACT_F32) turq_store_out_raw<TURQ_ACT_F32>(y, row * ldy + col, v);
+                        else if (yt == TURQ_ACT_BF16) turq_store_out_raw<TURQ_ACT_BF16>(y, row * ldy + col, v);
+                        else turq_store_out_raw<TURQ_ACT_F16>(y, row * ldy + col, v);
                     }
                 }
         }
+        turq_note_flush(bad);
     }
 }
 
@@ -1189,3 +1204,5 @@ hipError_t turq_launch_gemm_mfma_group(int dtype, const TurqGemmWeights &ws, int
     }
 #undef TURQ_GEMM
 }
+
+TURQ_NONFINITE_READER(turq_nonfinite_gemm_mfma)

@@ -259,3 +259,5 @@ hipError_t turq_launch_gemv_cs_staged_gateup(int dtype, const void *w_gate, cons
     default: return hipErrorInvalidValue;
     }
 }
+
+TURQ_NONFINITE_READER(turq_nonfinite_gemv_cs)

@@ -3,3 +3,5 @@
 
 hipError_t turq_launch_gemv_cs_staged_f32(TURQ_STAGED_LAUNCH_ARGS) { return staged_launch<TURQ_ACT_F32>(TURQ_STAGED_LAUNCH_PASS); }
 hipError_t turq_launch_gemv_cs_staged_gateup_f32(TURQ_STAGED_GATEUP_ARGS) { return staged_gateup_launch<TURQ_ACT_F32>(TURQ_STAGED_GATEUP_PASS); }
+
+TURQ_NONFINITE_READER(turq_nonfinite_gemv_cs_staged_f32)

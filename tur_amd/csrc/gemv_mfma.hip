@@ -706,3 +706,5 @@ hipError_t turq_launch_gemv_gateup_frag(int dtype, const void *w_gate, const voi
     default: return hipErrorInvalidValue;
     }
 }
+
+TURQ_NONFINITE_READER(turq_nonfinite_gemv_mfma)

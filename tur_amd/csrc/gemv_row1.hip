@@ -830,3 +830,5 @@ hipError_t turq_launch_gemv_row1_gateup(int dtype, const void *w_gate, const voi
     default: return hipErrorInvalidValue;
     }
 }
+
+TURQ_NONFINITE_READER(turq_nonfinite_gemv_row1)

@@ -5,6 +5,7 @@
 // It is also the dense arm of the layer: F32 / F16 / BF16 weights (candle's `QMatMul::from_arc` turns those GGUF tensors,
 // and every tensor under CANDLE_DEQUANTIZE_ALL, into a dense f32 matmul; src/models/layers/linear.rs:69), any k.
 #include "block_decode.h"
+#include "mfma_common.h"
 
 namespace {
 
@@ -22,6 +23,7 @@ __device__ inline uint16_t f2bf(float f) {  // round to nearest even, NaN kept q
 }
 
 template <int YT> __device__ inline void store_out(void *y, int64_t i, float v) {
+    turq_note_result<YT>(v);
     if (YT == TURQ_ACT_F32) ((float *)y)[i] = v;
     else if (YT == TURQ_ACT_BF16) ((uint16_t *)y)[i] = f2bf(v);
     else {
@@ -138,3 +140,5 @@ hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t 
     default: return hipErrorInvalidValue;
     }
 }
+
+TURQ_NONFINITE_READER(turq_nonfinite_gemv_simple)

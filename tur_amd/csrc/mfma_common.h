@@ -128,7 +128,47 @@ __device__ inline uint16_t turq_f2bf(float f) {  // round to nearest even, NaN k
     u += 0x7FFFu + ((u >> 16) & 1u);
     return (uint16_t)(u >> 16);
 }
+// Results that are no finite numbers.  The matrix kernels compute on f16 activations: a finite f32 or bf16 input of magnitude
+// 65520 or more becomes an infinity there, and what it is multiplied into comes out as an infinity or a NaN - as do inputs that
+// were infinities or NaNs to begin with.  Every kernel that stores results counts the elements it stores that are not finite
+// (for an f16 output: that do not fit f16) in a word of device memory, so that a host can tell that it happened
+// (turq_ctx_nonfinite_count).  The word is this translation unit's own copy, one per GPU; it stops counting at 2^20.
+static __device__ uint32_t turq_nonfinite_word;
+template <int YT> __device__ inline void turq_note_result(float v) {
+    const float lim = YT == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
+    if (__builtin_expect(!(__builtin_fabsf(v) < lim), 0)) {
+        if (__hip_atomic_load(&turq_nonfinite_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (1u << 20))
+            __hip_atomic_fetch_add(&turq_nonfinite_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+// the same for a run of stores: one flag per lane, one test at the end
+__device__ inline void turq_note_accum(float v, float lim, uint32_t &bad) { bad |= __builtin_fabsf(v) < lim ? 0u : 1u; }
+__device__ inline void turq_note_flush(uint32_t bad) {
+    if (__builtin_expect(bad != 0, 0)) {
+        if (__hip_atomic_load(&turq_nonfinite_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (1u << 20))
+            __hip_atomic_fetch_add(&turq_nonfinite_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+// host side of it, once per translation unit whose kernels store results: adds the current device's word to *sum (and clears it)
+#define TURQ_NONFINITE_READER(fn)                                                                      \
+    hipError_t fn(unsigned long long *sum, int reset) {                                                \
+        uint32_t v = 0;                                                                                \
+        hipError_t e = hipMemcpyFromSymbol(&v, HIP_SYMBOL(turq_nonfinite_word), sizeof v);             \
+        if (e != hipSuccess) return e;                                                                 \
+        *sum += v;                                                                                     \
+        if (reset && v) {                                                                              \
+            const uint32_t zero = 0;                                                                   \
+            e = hipMemcpyToSymbol(HIP_SYMBOL(turq_nonfinite_word), &zero, sizeof zero);                \
+        }                                                                                              \
+        return e;                                                                                      \
+    }
+template <int YT> __device__ inline void turq_store_out_raw(void *y, int64_t i, float v);
 template <int YT> __device__ inline void turq_store_out(void *y, int64_t i, float v) {
+    turq_note_result<YT>(v);
+    turq_store_out_raw<YT>(y, i, v);
+}
+// (without the count: for kernels that keep one flag for a run of stores)
+template <int YT> __device__ inline void turq_store_out_raw(void *y, int64_t i, float v) {
     if (YT == TURQ_ACT_F32) ((float *)y)[i] = v;
     else if (YT == TURQ_ACT_BF16) ((uint16_t *)y)[i] = turq_f2bf(v);
     else {
@@ -148,6 +188,8 @@ __host__ __device__ inline size_t turq_act_prep32_bytes(int64_t m, int64_t k) {
 // launchers (act_prep.hip, gemv_mfma.hip)
 hipError_t turq_launch_act_prep32(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
                                   hipStream_t stream);
+hipError_t turq_launch_silu_mul_prep32(int dtype, const float *gate, const float *up, int64_t m, int64_t n, void *frags,
+                                       hipStream_t stream);
 hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
                                 hipStream_t stream);
 hipError_t turq_launch_gemv_mfma(int dtype, const void *w_tiled, int64_t n, int64_t k, const void *xin, int x_dtype,

@@ -332,6 +332,55 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
     return TURQ_OK;
 }
 
+// the prefill GEMM of one weight on fragments that already sit in ctx->act_prep
+static int gemm_on_frags(turq_ctx *ctx, const turq_weight *w, int64_t m, void *y, int yt, int64_t ldy, const float *bias, float wscale) {
+    GemmSplit sp;
+    int rc = gemm_split_reserve(ctx, 1, &w, m, &sp);
+    if (rc != TURQ_OK) return rc;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
+    TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, wscale, ctx->compute_units,
+                                        ctx->stream, ev0, ev1, sp.counters[0], sp.partials[0], sp.bytes[0]));
+    return TURQ_OK;
+}
+
+// `Qwen3MLP::forward` (src/models/qwen3.rs:161-167) on a prompt chunk.  The separate calls write the two products (f32), read
+// them back for SiLU(gate) * up, write that as f16, read it back for down_proj's fragment preparation: here one kernel reads
+// the two products and writes the fragments (the same f16 values, so the results are those of the separate calls bit for bit),
+// which saves a launch and a round trip of the intermediate per MLP.
+int turq_mlp_prefill(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt,
+                     int64_t m, int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up,
+                     const float *bias_down, bool *taken) {
+    *taken = false;
+    static const bool off = [] { const char *e = getenv("TURQ_MLP_PREFILL"); return e && atoi(e) == 0; }();
+    const turq_weight *gu[2] = {gate, up};
+    float ws_down = 1.0f, ws_tmp = 1.0f;
+    if (off || m <= TURQ_GEMV_MAX_M || ctx->fixed_scratch) return TURQ_OK;
+    for (const turq_weight *w : {gate, up, down})
+        if (w->device != ctx->device || w->layout != TURQ_LAYOUT_TILED || w->n <= 0 || w->k <= 0 || !gemm_takes(w, &ws_tmp)) return TURQ_OK;
+    if (!gemm_takes(down, &ws_down) || down->k != gate->n || gate->n != up->n || gate->k != up->k) return TURQ_OK;
+    if (ldx < gate->k || ldy < down->n || !turq_act_bytes(xt) || !turq_act_bytes(yt)) return TURQ_OK;
+    if (turq_rows_in_chunks(ctx, 2, gu, x, xt, ldx, m)) return TURQ_OK;  // gate / up through the kernels of up to 32 rows
+    const int64_t n_ff = gate->n;
+    const size_t half = (size_t)m * (size_t)n_ff;
+    int rc = turq_ctx_reserve(ctx, &ctx->gate_up, &ctx->gate_up_cap, 2 * half * sizeof(float) + 16);
+    if (rc != TURQ_OK) return rc;
+    // one fragment buffer serves both preparations: sized for the larger before anything is queued
+    rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, std::max(turq_act_prep32_bytes(m, gate->k), turq_act_prep32_bytes(m, n_ff)));
+    if (rc != TURQ_OK) return rc;
+    void *ys[2] = {ctx->gate_up, (float *)ctx->gate_up + half};
+    const int64_t ldys[2] = {n_ff, n_ff};
+    const float *biases[2] = {bias_gate, bias_up};
+    bool gu_taken = false;
+    rc = turq_qmatmul_multi_gemm(ctx, 2, gu, x, xt, m, ldx, ys, TURQ_ACT_F32, ldys, biases, &gu_taken);
+    if (rc != TURQ_OK || !gu_taken) return rc;
+    TURQ_HIP(ctx, turq_launch_silu_mul_prep32(down->dtype, (const float *)ys[0], (const float *)ys[1], m, n_ff, ctx->act_prep, ctx->stream));
+    rc = gemm_on_frags(ctx, down, m, y, yt, ldy, bias_down, ws_down);
+    if (rc != TURQ_OK) return rc;
+    *taken = true;
+    return TURQ_OK;
+}
+
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
                       int yt, int64_t ldy, const float *bias, int algo) {
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);

@@ -80,3 +80,5 @@ hipError_t turq_launch_rms_norm(const void *x, int x_dtype, int64_t m, int64_t k
     default: return hipErrorInvalidValue;
     }
 }
+
+TURQ_NONFINITE_READER(turq_nonfinite_norm)

@@ -84,3 +84,5 @@ hipError_t turq_launch_wide_rescale(const float *y32, int64_t ld32, int64_t m, i
     }
     return hipGetLastError();
 }
+
+TURQ_NONFINITE_READER(turq_nonfinite_wide)
