@@ -37,15 +37,27 @@ from tur_amd import capi, synth  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, vendor figure
 MFMA_F16_PEAK_TFLOPS = 2500.0   # dense f16 / bf16 MFMA, vendor figure
-# HBM bytes per launch of the timed kernels (average over the launches of a step) from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE, scaled by the same counters on a copy kernel of known size (summaries under profiles/); keyed by
-# (workload, m, activations, one call per matrix?)
-TRAFFIC = {
-    ("q4k_mlp_8b", 1, "f32", False): 42_858_500,    # gate + up in one launch 56 920 900, down 28 796 200
-    ("q4k_mlp_8b", 1, "f32", True): 28_680_000,
-    ("q4k_prefill_up_8b", 512, "bf16", False): 76_833_700,   # every XCD's L2 fetches the activation fragments once
-    ("q4k_prefill_up_8b", 512, "bf16", True): 76_833_700,
-}
+TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "hbm_traffic_per_launch.md")
+
+
+def load_traffic():
+    """HBM bytes per launch of the timed kernels (average over the launches of a step), measured with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE and scaled by the same counters on a copy kernel of known size: the rows of the table in
+    profiles/hbm_traffic_per_launch.md, which names the commands and the commit they ran on.  Keyed by (workload, m,
+    activations, calls); a leg that has no row reports null."""
+    table = {}
+    try:
+        with open(TRAFFIC_TABLE) as f:
+            for line in f:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) >= 5 and cells[1].isdigit() and cells[4].replace(" ", "").isdigit():
+                    table[(cells[0].strip("`"), int(cells[1]), cells[2], cells[3])] = int(cells[4].replace(" ", ""))
+    except OSError:
+        pass
+    return table
+
+
+TRAFFIC = load_traffic()
 
 WORKLOADS = {
     # name: (description, [(label, ggml dtype, n, k), ...] per layer)
@@ -125,6 +137,10 @@ class Bench:
         L, ctx, layers = self.L, self.ctx, self.args.layers
         for p in list(self.x_dev.values()) + list(self.y_dev):
             capi.check(L.turq_dev_free(ctx, p), ctx)
+        if getattr(self, "glue", None):
+            for key in ("xres", "xn", "nw", "tmp"):
+                capi.check(L.turq_dev_free(ctx, self.glue[key]), ctx)
+            self.glue = None
         self.m = m
         self.calls = []
         self.x_host = {}
@@ -181,13 +197,136 @@ class Bench:
             self.step_bytes -= layers * sum(self.m * k * self.xbytes for lb, _, n, k in self.mats if lb == "down")
         self.step_flops = layers * sum(2 * self.m * n * k for _, _, n, k in self.mats)
 
+    def calls_label(self):
+        a = self.args
+        if getattr(a, "glue", None):
+            return ("turq_norm_qmatmul_multi + turq_qmatmul (accumulate) + turq_norm_mlp (accumulate)" if a.glue == "fused"
+                    else "turq_rms_norm + turq_qmatmul_multi + turq_qmatmul + turq_rms_norm + turq_mlp")
+        return ("turq_qmatmul" if a.single_calls else "turq_mlp + turq_qmatmul_multi" if self.use_mlp()
+                else "turq_qmatmul_gate_up + turq_qmatmul_multi" if a.gate_up else "turq_qmatmul_multi")
+
+    def reconfigure(self, m, act=None, out=None, mlp=None, glue=None):
+        """another leg on the same resident weights: activation / output types, turq_mlp per layer or not, m rows"""
+        if act is not None:
+            self.args.act = act
+            self.xt, self.xbytes, self.xnp = ACT[act]
+        if out is not None:
+            self.args.out = out
+            self.yt, self.ybytes = OUT[out]
+        if mlp is not None:
+            self.args.mlp = mlp
+        self.args.glue = glue
+        self.set_m(m)
+
     def use_mlp(self):
         """gate / up / down as one turq_mlp call per layer (--mlp)"""
         labels = [mt[0] for mt in self.mats]
         has = any(labels[i:i + 3] == ["gate", "up", "down"] for i in range(len(labels)))
         return has and bool(getattr(self.args, "mlp", False)) and not self.args.single_calls and not self.args.gate_up
 
+    def setup_glue(self):
+        """buffers of the decoder layer's linear path with its glue (--glue): the residual stream, the attention block's output
+        (random: attention itself is not part of this path), the normalised rows of the separate form, the norm weight"""
+        if getattr(self, "glue", None) and self.glue["m"] == self.m:
+            return
+        L, ctx, m = self.L, self.ctx, self.m
+        labels = [mt[0] for mt in self.mats]
+        if labels != ["q", "k", "v", "o", "gate", "up", "down"] or self.args.act != self.args.out:
+            raise SystemExit("--glue needs the decoder-layer workload (q4km_layer_8b) and --act equal to --out")
+        k = self.mats[0][3]
+        g = {"m": m, "k": k}
+        x0 = synth.random_activation(m, k, seed=7, bf16=(self.args.act == "bf16"))
+        g["x0"] = synth.to_bf16_bits(x0).reshape(m, k) if self.args.act == "bf16" else x0
+        g["x0_f32"] = x0
+        g["xres"] = self.dev_alloc(g["x0"].nbytes)
+        g["xn"] = self.dev_alloc(g["x0"].nbytes)
+        g["attn"] = self.x_dev[k]
+        # a norm weight of 2^-7: the synthetic weights give products of a few hundred at unit activations, and
+        # act(gate) * up of such rows would leave the f16 range that down_proj rounds its input to
+        nw = np.full(k, 2.0 ** -7, np.float32)
+        g["nw_host"] = nw
+        g["nw"] = self.dev_alloc(nw.nbytes)
+        capi.check(L.turq_memcpy_h2d(ctx, g["nw"], capi.ptr(nw), nw.nbytes), ctx)
+        g["tmp"] = self.dev_alloc(m * k * self.ybytes)
+        self.glue = g
+        self.reset_glue()
+
+    def reset_glue(self):
+        g = self.glue
+        capi.check(self.L.turq_memcpy_h2d(self.ctx, g["xres"], capi.ptr(g["x0"]), g["x0"].nbytes), self.ctx)
+
+    def step_glue(self, layers=None):
+        """the reference's decoder layer without its attention block (src/models/qwen3.rs:633-640): ln1 -> q / k / v, o_proj added
+        to the residual stream, ln2 -> MLP added to it; --glue fused: three calls per layer, --glue separate: the norms as calls
+        of their own and the projections into buffers (the two additions are then the engine's own launches, not made here)"""
+        L, ctx, m, xt, yt, g = self.L, self.ctx, self.m, self.xt, self.yt, self.glue
+        k, eps, acc = g["k"], 1e-6, capi.OUT_ACCUMULATE
+        fused = self.args.glue == "fused"
+        for li, layer in enumerate(self.weights if layers is None else self.weights[:layers]):
+            wq, wk, wv, wo, wg, wu, wd = layer
+            warr = (ctypes.c_void_p * 3)(wq.value, wk.value, wv.value)
+            yarr = (ctypes.c_void_p * 3)(*[y.value for y in self.y_dev[:3]])
+            ldys = (ctypes.c_int64 * 3)(*[mt[2] for mt in self.mats[:3]])
+            if fused:
+                rc = L.turq_norm_qmatmul_multi(ctx, 3, warr, g["xres"], xt, m, k, g["nw"], eps, yarr, yt, ldys, None, capi.MEM_DEVICE)
+                rc = rc or L.turq_qmatmul(ctx, wo, g["attn"], xt, m, k, g["xres"], yt | acc, k, None, capi.MEM_DEVICE, capi.ALGO_AUTO)
+                rc = rc or L.turq_norm_mlp(ctx, wg, wu, wd, g["xres"], xt, m, k, g["nw"], eps, g["xres"], yt | acc, k, None, None, None,
+                                           capi.ACTFN_SILU, capi.MEM_DEVICE)
+            else:
+                rc = L.turq_rms_norm(ctx, g["xres"], xt, m, k, k, g["nw"], eps, g["xn"], xt, k, capi.MEM_DEVICE)
+                rc = rc or L.turq_qmatmul_multi(ctx, 3, warr, g["xn"], xt, m, k, yarr, yt, ldys, None, capi.MEM_DEVICE, capi.ALGO_AUTO)
+                rc = rc or L.turq_qmatmul(ctx, wo, g["attn"], xt, m, k, g["tmp"], yt, k, None, capi.MEM_DEVICE, capi.ALGO_AUTO)
+                rc = rc or L.turq_rms_norm(ctx, g["xres"], xt, m, k, k, g["nw"], eps, g["xn"], xt, k, capi.MEM_DEVICE)
+                rc = rc or L.turq_mlp(ctx, wg, wu, wd, g["xn"], xt, m, k, g["tmp"], yt, k, None, None, None, capi.ACTFN_SILU, capi.MEM_DEVICE)
+            if rc:
+                capi.check(rc, ctx)
+
+    def verify_glue(self):
+        """first layer of the fused form against the oracle: the q projection of the normalised rows, and the residual stream
+        after the layer (first rows only; the chain needs every column)"""
+        from oracle import capi as orc
+        from oracle import oracle_np as onp
+        g, m = self.glue, self.m
+        keep = min(m, 8)
+        self.reset_glue()
+        saved = self.args.glue
+        self.args.glue = "fused"
+        self.step_glue(layers=1)
+        self.args.glue = saved
+        self.sync()
+        k = g["k"]
+        x = g["x0_f32"][:keep].astype(np.float64)
+        xn = (x / np.sqrt((x * x).mean(axis=1, keepdims=True) + 1e-6) * g["nw_host"]).astype(np.float32)
+        by = {mt[0]: mt for mt in self.mats}
+
+        def fetch(ptr, n):
+            a = np.empty((m, n), np.float32 if self.yt == capi.ACT_F32 else np.uint16)
+            capi.check(self.L.turq_memcpy_d2h(self.ctx, capi.ptr(a), ptr, a.nbytes), self.ctx)
+            return (a if self.yt == capi.ACT_F32 else synth.from_bf16_bits(a).reshape(m, n))[:keep]
+
+        def rnd(a):
+            return a if self.yt == capi.ACT_F32 else synth.from_bf16_bits(synth.to_bf16_bits(np.asarray(a, np.float32))).reshape(np.shape(a))
+
+        _, dq, nq, _ = by["q"]
+        want_q = orc.matmul_dequant(dq, xn, self.host_raw["q"], nq, k)
+        rel_q = float(np.linalg.norm(fetch(self.y_dev[0], nq) - rnd(want_q)) / np.linalg.norm(want_q))
+        attn = self.x_host[k][:keep]
+        x1 = g["x0_f32"][:keep] + orc.matmul_dequant(by["o"][1], attn, self.host_raw["o"], k, k)
+        x1 = rnd(x1).astype(np.float64)
+        xn2 = (x1 / np.sqrt((x1 * x1).mean(axis=1, keepdims=True) + 1e-6) * g["nw_host"]).astype(np.float32)
+        h = onp.silu_mul(orc.matmul_dequant(by["gate"][1], xn2, self.host_raw["gate"], by["gate"][2], k),
+                         orc.matmul_dequant(by["up"][1], xn2, self.host_raw["up"], by["up"][2], k))
+        want = x1 + orc.matmul_dequant(by["down"][1], h, self.host_raw["down"], by["down"][2], by["down"][3])
+        rel_x = float(np.linalg.norm(fetch(g["xres"], k) - rnd(want)) / np.linalg.norm(want))
+        bar = 1e-3 if self.yt == capi.ACT_F32 else 3e-3
+        if rel_q > bar or rel_x > 2 * bar:
+            raise SystemExit(f"bench: --glue differs from the oracle (q {rel_q:.3e}, residual stream {rel_x:.3e}; bar {bar})")
+        self.reset_glue()
+        return max(rel_q, rel_x)
+
     def step_eager(self):
+        if getattr(self.args, "glue", None):
+            return self.step_glue()
         L, ctx, m, xt = self.L, self.ctx, self.m, self.xt
         ahead = int(getattr(self.args, "prefetch", 0) or 0)
         if not self.args.single_calls:
@@ -259,9 +398,14 @@ class Bench:
                 from oracle import oracle_np as onp
                 sub_up = self.host_raw["up"].reshape(n, -1)[rows].reshape(-1)
                 want = onp.silu_mul(want, orc.matmul_dequant(dt, self.x_host[k], sub_up, len(rows), k))
+            if self.yt != capi.ACT_F32:
+                # a bf16 store alone costs about 1.6e-3: the oracle's result is rounded the same way, so that what is left is
+                # the kernel's own error (and the elements it tips into the neighbouring bf16 value)
+                want = synth.from_bf16_bits(synth.to_bf16_bits(np.asarray(want, np.float32))).reshape(np.shape(want))
             rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
             worst = max(worst, rel)
-        bar = 1e-3 if self.yt == capi.ACT_F32 else 4e-3      # a bf16 store alone costs about 1.6e-3
+        # (the MLP is two matmuls in a row, each inside its own bar)
+        bar = (1e-3 if self.yt == capi.ACT_F32 else 2e-3) * (2 if mlp and self.m > 32 else 1)
         if worst > bar:
             raise SystemExit(f"bench: output differs from the oracle (rel-L2 {worst:.3e} > {bar})")
         return worst
@@ -270,7 +414,14 @@ class Bench:
         """verify against the oracle, time `steps` steps (whole step), then time the matmul kernels alone"""
         a = self.args
         L, ctx = self.L, self.ctx
-        rel = self.verify()
+        if getattr(a, "glue", None):
+            self.setup_glue()
+            rel = self.verify_glue()
+            self.step_eager()      # (scratch buffers reach their size outside the capture)
+            self.sync()
+            self.reset_glue()
+        else:
+            rel = self.verify()
         graph = None
         if not a.eager:
             capi.check(L.turq_graph_begin(ctx), ctx)
@@ -304,7 +455,7 @@ class Bench:
         achieved = bytes_per_launch / (avg_us * 1e-6) / 1e9
         if graph:
             L.turq_graph_destroy(graph)
-        traffic = None if (a.gate_up or self.use_mlp()) else TRAFFIC.get((a.workload, self.m, a.act, bool(a.single_calls)))
+        traffic = TRAFFIC.get((a.workload, self.m, a.act, self.calls_label()))
         if self.m > 32:
             flops_per_launch = self.step_flops * prof_steps / max(1, n_launch.value)
             tfl = flops_per_launch / (avg_us * 1e-6) / 1e12
@@ -340,7 +491,7 @@ class Bench:
             "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": f"{a.workload}: {self.desc}", "m": self.m, "layers": a.layers,
                        "activations": a.act, "outputs": a.out, "launch": "eager" if a.eager else "hip-graph",
-                       "calls": "turq_qmatmul" if a.single_calls else "turq_mlp + turq_qmatmul_multi" if self.use_mlp() else ("turq_qmatmul_gate_up + turq_qmatmul_multi" if a.gate_up else "turq_qmatmul_multi"),
+                       "calls": self.calls_label(),
                        "step_bytes": int(self.step_bytes), "device": self.device, "compute_units": self.cus,
                        "max_rel_l2_vs_oracle": float(f"{r['rel']:.3e}")},
             "whole_step_gbps": round(r["gbps"], 1), "pct_of_hbm_peak": round(100 * r["gbps"] / HBM_PEAK_GBPS, 2),
@@ -466,6 +617,10 @@ def main():
     ap.add_argument("--mlp", action="store_true",
                     help="the whole MLP through turq_mlp (down_proj takes act(gate) * up; the activations are scaled by 2^-7 so that the "
                          "synthetic intermediate stays in the f16 range) instead of gate / up and down on independent activations")
+    ap.add_argument("--glue", choices=["fused", "separate"], default=None,
+                    help="decoder-layer workload: the layer's linear path WITH its norms and residual additions (no attention): 'fused' = "
+                         "turq_norm_qmatmul_multi, turq_qmatmul and turq_norm_mlp with TURQ_OUT_ACCUMULATE (three calls per layer), "
+                         "'separate' = turq_rms_norm calls and plain projections (five calls, the two additions left to the engine)")
     ap.add_argument("--gate-up", action="store_true",
                     help="gate_proj / up_proj through turq_qmatmul_gate_up (SiLU and the product applied in the call, one output)")
     ap.add_argument("--embedding", action="store_true",
@@ -482,41 +637,41 @@ def main():
         per_layer = sum(synth.weight_nbytes(dt, n, k) for _, dt, n, k in WORKLOADS[args.workload][1])
         args.layers = default_layers(per_layer)
     headline = all(getattr(args, f) == ap.get_default(f) for f in ("workload", "m", "act", "out")) and not (
-        args.eager or args.single_calls or args.gate_up or args.mlp or args.calibrate_copy)
+        args.eager or args.single_calls or args.gate_up or args.mlp or args.calibrate_copy or args.glue or args.prefetch)
     b = Bench(args)
     try:
         if args.calibrate_copy:
             b.calibrate_copy()
         out = b.run()
+        if headline and not args.no_extra:
+            out.update(other_halves(args, b))
     finally:
         b.close()
-    if headline and not args.no_extra:
-        out.update(other_halves(args))
     print(json.dumps(out), flush=True)
 
 
-def side_leg(base, workload, ms, act, outdt, steps, warmup):
-    """the same measurement on another workload of the metric, in this process: one entry per m"""
+def leg(b, ms, act, outdt, steps, warmup, mlp=False, glue=None):
+    """one leg of the metric on the weights Bench b holds: a row per m, measured like the headline"""
+    rows = []
+    for m in ms:
+        b.reconfigure(m, act, outdt, mlp, glue)
+        r = b.measure(steps, warmup)
+        rf = r["roofline"]
+        rows.append({"m": m, "value": round(r["value"], 1), "unit": r["unit"], "ms_per_step": round(r["ms_per_step"], 4),
+                     "bound": rf["bound"], "kernel_achieved": rf["achieved"], "frac": rf["frac"], "traffic": rf["traffic"],
+                     "avg_launch_us": rf["avg_launch_us"], "launches_timed": rf["launches_timed"],
+                     "max_rel_l2_vs_oracle": float(f"{r['rel']:.3e}")})
+    wl = b.args.workload
+    return {"workload": f"{wl}: {WORKLOADS[wl][0]}", "layers": b.args.layers, "activations": act, "outputs": outdt,
+            "calls": b.calls_label(), "peaks": {"hbm": HBM_PEAK_GBPS, "mfma": MFMA_F16_PEAK_TFLOPS}, "rows": rows}
+
+
+def bench_for(base, workload):
     args = argparse.Namespace(**vars(base))
-    args.workload, args.act, args.out, args.m = workload, act, outdt, ms[0]
+    args.workload, args.mlp = workload, False
     per_layer = sum(synth.weight_nbytes(dt, n, k) for _, dt, n, k in WORKLOADS[workload][1])
     args.layers = default_layers(per_layer)
-    b = Bench(args)
-    rows = []
-    try:
-        for m in ms:
-            if m != b.m:
-                b.set_m(m)
-            r = b.measure(steps, warmup)
-            rf = r["roofline"]
-            rows.append({"m": m, "value": round(r["value"], 1), "unit": r["unit"], "ms_per_step": round(r["ms_per_step"], 4),
-                         "kernel_achieved": rf["achieved"], "frac": rf["frac"], "avg_launch_us": rf["avg_launch_us"],
-                         "launches_timed": rf["launches_timed"], "max_rel_l2_vs_oracle": float(f"{r['rel']:.3e}")})
-    finally:
-        b.close()
-    return {"workload": f"{workload}: {WORKLOADS[workload][0]}", "layers": args.layers, "activations": act, "outputs": outdt,
-            "bound": "mfma" if ms[0] > 32 else "hbm", "peak": MFMA_F16_PEAK_TFLOPS if ms[0] > 32 else HBM_PEAK_GBPS,
-            "rows": rows}
+    return Bench(args)
 
 
 def read_floor():
@@ -566,18 +721,44 @@ def read_floor():
     return {"what": "a launch of the decode kernels' shape that only reads the same bytes (turq_read_yardstick), kernel time", "rows": rows}
 
 
-def other_halves(base):
+def other_halves(base, b_mlp):
     """The rest of the headline metric, measured in the same process with the same method (value = whole step, frac = the
-    matmul kernels alone against the peak): the prefill GEMM (BASELINE config 4), the mixed Q4_K / Q6_K decoder layer at
-    its batch sizes (config 3) and on prompt chunks of 128 and 512 rows, and the Q6_K LM head (config 5)."""
+    matmul kernels alone against the peak of their bound), one entry per configuration of the metric: the MLP shapes at the
+    other batch sizes and with bf16 activations (config 2) and as whole turq_mlp calls on prompt chunks, the prefill GEMM
+    (config 4), the mixed Q4_K / Q6_K decoder layer at its batch sizes (config 3) and on prompt chunks, the Q6_K and Q5_K LM
+    heads (config 5) and the small Q8_0 matrix that runs on the reference's CPU path today (config 1).  b_mlp: the headline's
+    Bench, whose resident weights serve the legs on the same matrices."""
     steps, warmup = 20, 3
-    return {
-        "prefill": side_leg(base, "q4k_prefill_up_8b", [512, 2048], "bf16", "bf16", steps, warmup),
-        "q4km_layer": side_leg(base, "q4km_layer_8b", [1, 8, 32], "f32", "f32", steps, warmup),
-        "q4km_layer_prefill": side_leg(base, "q4km_layer_8b", [128, 512], "bf16", "bf16", 10, 2),
-        "lm_head_q6k": side_leg(base, "lm_head_q6k_8b", [1], "bf16", "f32", steps, warmup),
-        "read_floor": read_floor(),
-    }
+    out = {}
+    out["q4k_mlp_f32"] = leg(b_mlp, [4, 16], "f32", "f32", steps, warmup)
+    out["q4k_mlp_bf16"] = leg(b_mlp, [1, 4, 16], "bf16", "f32", steps, warmup)
+    out["mlp_prefill"] = leg(b_mlp, [128, 512], "bf16", "bf16", 10, 2, mlp=True)
+    plan = [
+        ("q4k_prefill_up_8b", [("prefill", [512, 2048], "bf16", "bf16", steps, warmup)]),
+        ("q4km_layer_8b", [("q4km_layer", [1, 8, 32], "f32", "f32", steps, warmup),
+                           ("q4km_layer_bf16", [8, 32], "bf16", "f32", steps, warmup),
+                           ("q4km_layer_prefill", [128, 512], "bf16", "bf16", 10, 2),
+                           # the same layer with its norms and residual additions: the fused entry points against separate calls
+                           ("q4km_layer_glue_fused", [1, 8], "f32", "f32", steps, warmup, "fused"),
+                           ("q4km_layer_glue_separate", [1, 8], "f32", "f32", steps, warmup, "separate"),
+                           ("q4km_layer_glue_fused_prefill", [128], "bf16", "bf16", 10, 2, "fused"),
+                           ("q4km_layer_glue_separate_prefill", [128], "bf16", "bf16", 10, 2, "separate")]),
+        ("lm_head_q6k_8b", [("lm_head_q6k", [1, 16, 128], "bf16", "f32", steps, warmup)]),
+        ("lm_head_q5k_8b", [("lm_head_q5k", [1, 16, 128], "bf16", "f32", steps, warmup)]),
+        ("q8_0_gate_0p6b", [("q8_0_gate", [1], "f32", "f32", steps, warmup)]),
+    ]
+    for workload, legs in plan:
+        b = bench_for(base, workload)
+        try:
+            for key, ms, act, outdt, st, wu, *glue in legs:
+                out[key] = leg(b, ms, act, outdt, st, wu, glue=glue[0] if glue else None)
+        finally:
+            b.close()
+    for key in ("q4km_layer_glue_separate", "q4km_layer_glue_separate_prefill"):
+        out[key]["note"] = "the two residual additions per layer are the engine's own launches in this form and are NOT made here; the fused form includes them"
+    out["q8_0_gate"]["note"] = "3.3 MB of weights: the launch itself (about 4 us) bounds it, not the bytes"
+    out["read_floor"] = read_floor()
+    return out
 
 
 if __name__ == "__main__":

@@ -47,6 +47,8 @@ pub const TURQ_BF16: c_int = 30;
 pub const TURQ_ACT_F32: c_int = 0;
 pub const TURQ_ACT_BF16: c_int = 1;
 pub const TURQ_ACT_F16: c_int = 2;
+/// OR-ed into the y_dtype of turq_qmatmul / turq_qmatmul_noalloc / turq_mlp / turq_norm_mlp: results are added to y
+pub const TURQ_OUT_ACCUMULATE: c_int = 0x100;
 
 // weight layouts in HBM
 pub const TURQ_LAYOUT_NATIVE: c_int = 0;
@@ -101,6 +103,8 @@ extern "C" {
     pub fn turq_qmatmul_multi(ctx: *mut turq_ctx, count: c_int, weights: *const *const turq_weight, x: *const c_void, x_dtype: c_int, m: i64, ldx: i64, ys: *const *mut c_void, y_dtype: c_int, ldys: *const i64, biases: *const *const f32, mem: c_int, algo: c_int) -> c_int;
     pub fn turq_qmatmul_gate_up(ctx: *mut turq_ctx, gate: *const turq_weight, up: *const turq_weight, x: *const c_void, x_dtype: c_int, m: i64, ldx: i64, y: *mut c_void, y_dtype: c_int, ldy: i64, bias_gate: *const f32, bias_up: *const f32, act: c_int, mem: c_int) -> c_int;
     pub fn turq_mlp(ctx: *mut turq_ctx, gate: *const turq_weight, up: *const turq_weight, down: *const turq_weight, x: *const c_void, x_dtype: c_int, m: i64, ldx: i64, y: *mut c_void, y_dtype: c_int, ldy: i64, bias_gate: *const f32, bias_up: *const f32, bias_down: *const f32, act: c_int, mem: c_int) -> c_int;
+    pub fn turq_norm_qmatmul_multi(ctx: *mut turq_ctx, count: c_int, weights: *const *const turq_weight, x: *const c_void, x_dtype: c_int, m: i64, ldx: i64, norm_weight: *const f32, eps: f32, ys: *const *mut c_void, y_dtype: c_int, ldys: *const i64, biases: *const *const f32, mem: c_int) -> c_int;
+    pub fn turq_norm_mlp(ctx: *mut turq_ctx, gate: *const turq_weight, up: *const turq_weight, down: *const turq_weight, x: *const c_void, x_dtype: c_int, m: i64, ldx: i64, norm_weight: *const f32, eps: f32, y: *mut c_void, y_dtype: c_int, ldy: i64, bias_gate: *const f32, bias_up: *const f32, bias_down: *const f32, act: c_int, mem: c_int) -> c_int;
     pub fn turq_weight_prefetch(ctx: *mut turq_ctx, w: *const turq_weight) -> c_int;
     pub fn turq_quantize_q8_0(ctx: *mut turq_ctx, x: *const f32, m: i64, k: i64, out: *mut c_void, mem: c_int) -> c_int;
     pub fn turq_quantize_q8_k(ctx: *mut turq_ctx, x: *const f32, m: i64, k: i64, out: *mut c_void, mem: c_int) -> c_int;

@@ -54,6 +54,11 @@ enum {
 
 /* element type of activation / output buffers */
 enum { TURQ_ACT_F32 = 0, TURQ_ACT_BF16 = 1, TURQ_ACT_F16 = 2 };
+/* OR-ed into the y_dtype of turq_qmatmul, turq_qmatmul_noalloc or turq_mlp: the results are ADDED to what y holds,
+ * y[m, n] += x * W^T (+ bias), in f32 before the one rounding to y's type.  It is the residual connection of the reference's decoder layer,
+ * `(x + h)` after o_proj and `x + h2` after the MLP (src/models/qwen3.rs:633-640), taken into the matmul kernel's store: y is the
+ * residual stream, and the separate elementwise launch and its round trip of the outputs go away. */
+#define TURQ_OUT_ACCUMULATE 0x100
 
 /* weight layouts in HBM */
 enum {
@@ -187,6 +192,7 @@ int turq_rms_norm(turq_ctx *ctx, const void *x, int x_dtype, int64_t m, int64_t 
  *        stream) or TURQ_MEM_HOST (x, y are host pointers; staged through the context and
  *        synchronous);
  *   algo: TURQ_ALGO_*.
+ * y_dtype | TURQ_OUT_ACCUMULATE adds the results to y instead of overwriting it (see there).
  * Errors instead of panics for m < 0, ld too small, unsupported dtypes.  m == 0 is a no-op.
  * Device calls of 33 - 64 rows on large weights of up to 4096 columns (gate / up of an 8B model) go through the kernels of up
  * to 32 rows in two chunks.  Device calls of more than 32 rows (prompt chunks) whose workgroup tiles would leave most compute units idle - the tall
@@ -271,6 +277,33 @@ int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weig
 int turq_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int x_dtype,
              int64_t m, int64_t ldx, void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up,
              const float *bias_down, int act, int mem);
+
+/* turq_qmatmul_multi on RmsNorm(x): ys[i][m, n_i] = (x / sqrt(mean(x^2) + eps) * norm_weight) * W_i^T (+ biases[i]), for the
+ * weights that the reference applies to a normalised tensor - q / k / v behind `ln1`, the LM head behind the final norm
+ * (count = 1).  norm_weight: f32 [k] in the memory space of x (the `weight` of the norm as turq_dequantize returns it); every
+ * other argument as in turq_qmatmul_multi (the algorithm is chosen by the call).  With device pointers and tiled weights the norm costs no launch of its own where
+ * the kernels can apply it themselves: for ONE activation row the matmul kernel multiplies its columns by norm_weight while it
+ * stages them, adds up their squares, and scales the results by the row's 1 / sqrt(mean + eps) (it rounds x * norm_weight to f16
+ * where the separate calls round the normalised value: within 5e-4 relative L2 of them, inside the 1e-3 bar against an f64 norm
+ * followed by the f32 matmul); for MORE THAN 32 rows the norm writes the fragments of the prefill GEMM directly (the results of turq_rms_norm into f32
+ * followed by turq_qmatmul_multi, bit for bit).  Every other case runs the norm into scratch memory of the context - as f16
+ * where the matmul kernels would round its output to f16 anyway: the same values, half the bytes for them to read - and then
+ * the plain call (also bit-equal to the separate calls).  Range: the one-row route rounds x * norm_weight, not the normalised
+ * value, to f16, so a residual stream with |x * norm_weight| >= 65520 overflows there (turq_ctx_nonfinite_count sees it); with
+ * wide activations on (turq_ctx_set_wide_activations) every case runs the norm into f32 scratch and takes any finite magnitude.
+ * Replaces: `self.ln1.forward(x)` followed by the three projections (src/models/qwen3.rs:633-634, 272-274), `self.norm` followed
+ * by `lm_head` (src/models/qwen3.rs:979-985). */
+int turq_norm_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int x_dtype, int64_t m,
+                            int64_t ldx, const float *norm_weight, float eps, void *const *ys, int y_dtype, const int64_t *ldys,
+                            const float *const *biases, int mem);
+
+/* turq_mlp on RmsNorm(x), the second half of the reference's decoder layer: with y_dtype | TURQ_OUT_ACCUMULATE and y = the
+ * residual stream it is `x + mlp(ln2(x))` in one call (src/models/qwen3.rs:637-640).  norm_weight and eps as above, everything
+ * else as in turq_mlp; the norm is taken into the kernels in the same two cases (one row: into the gate / up kernel; more than
+ * 32 rows: the norm writes the fragments of the gate / up GEMMs) and runs into scratch memory otherwise. */
+int turq_norm_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int x_dtype,
+                  int64_t m, int64_t ldx, const float *norm_weight, float eps, void *y, int y_dtype, int64_t ldy, const float *bias_gate,
+                  const float *bias_up, const float *bias_down, int act, int mem);
 
 /* A hint that `w` is the weight of one of the next forward calls: one read-only pass over its bytes on a stream of the
  * context's own, which starts where the context's stream stands when the call is made (so it runs next to whatever is queued

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libturq.so")
 OK, ERR_INVALID, ERR_SHAPE, ERR_DTYPE, ERR_HIP, ERR_OOM, ERR_IO, ERR_NOT_FOUND = range(8)
 F32, F16, Q8_0, Q4_K, Q5_K, Q6_K, BF16 = 0, 1, 8, 12, 13, 14, 30
 ACT_F32, ACT_BF16, ACT_F16 = 0, 1, 2
+OUT_ACCUMULATE = 0x100
 LAYOUT_NATIVE, LAYOUT_TILED = 0, 1
 MEM_HOST, MEM_DEVICE = 0, 1
 ALGO_AUTO, ALGO_SIMPLE, ALGO_GEMV, ALGO_GEMM = 0, 1, 2, 3
@@ -56,6 +57,10 @@ _SIGS = {
                                      c_void_p, c_void_p, c_int, c_int]),
     "turq_mlp": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_int64,
                          c_void_p, c_void_p, c_void_p, c_int, c_int]),
+    "turq_norm_qmatmul_multi": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_float, c_void_p, c_int,
+                                        c_void_p, c_void_p, c_int]),
+    "turq_norm_mlp": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_float, c_void_p, c_int,
+                              c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int]),
     "turq_weight_prefetch": (c_int, [c_void_p, c_void_p]),
     "turq_quantize_q8_0": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
     "turq_quantize_q8_k": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),

@@ -23,7 +23,7 @@ __global__ void __launch_bounds__(256) silu_mul_kernel(const float *__restrict__
 hipError_t turq_launch_silu_mul(const float *gate, const float *up, int64_t m, int64_t n, void *y, int y_dtype, int64_t ldy,
                                 hipStream_t stream) {
     if (m <= 0 || n <= 0) return hipSuccess;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     const int64_t blocks = (m * n + 255) / 256;
     if (blocks > 0x7FFFFFFF) return hipErrorInvalidValue;
     silu_mul_kernel<<<(unsigned)blocks, 256, 0, stream>>>(gate, up, m, n, y, y_dtype, ldy);

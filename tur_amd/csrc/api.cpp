@@ -167,6 +167,7 @@ void turq_ctx_destroy(turq_ctx *ctx) {
     if (ctx->act_prep) (void)hipFree(ctx->act_prep);
     if (ctx->gate_up) (void)hipFree(ctx->gate_up);
     if (ctx->mlp_h) (void)hipFree(ctx->mlp_h);
+    if (ctx->norm_x) (void)hipFree(ctx->norm_x);
     if (ctx->gemm_split) (void)hipFree(ctx->gemm_split);
     if (ctx->wide_x) (void)hipFree(ctx->wide_x);
     if (ctx->wide_s) (void)hipFree(ctx->wide_s);
@@ -472,7 +473,7 @@ static int qmatmul_device(turq_ctx *ctx, const turq_weight *w, const void *x, in
         else algo = (m <= TURQ_GEMV_MAX_M || turq_rows_in_chunks(ctx, 1, &w, x, xt, ldx, m)) ? TURQ_ALGO_GEMV : TURQ_ALGO_GEMM;
     }
     if (wide && !ctx->fixed_scratch && xt != TURQ_ACT_F16 && (algo == TURQ_ALGO_GEMV || algo == TURQ_ALGO_GEMM) &&
-        w->layout == TURQ_LAYOUT_TILED && m <= 65535) {
+        w->layout == TURQ_LAYOUT_TILED) {
         // rows scaled by powers of two into the f16 range, the plain call on the f16 copy, rows scaled back (+ bias)
         int rc = turq_ctx_reserve(ctx, &ctx->wide_x, &ctx->wide_x_cap, (size_t)m * (size_t)w->k * 2);
         if (rc != TURQ_OK) return rc;
@@ -480,7 +481,7 @@ static int qmatmul_device(turq_ctx *ctx, const turq_weight *w, const void *x, in
         if (rc != TURQ_OK) return rc;
         float *y32 = (float *)y;
         int64_t ld32 = ldy;
-        if (yt != TURQ_ACT_F32) {
+        if (yt != TURQ_ACT_F32) {  // (also an f32 output that is added to: the product must not land on the residual stream)
             rc = turq_ctx_reserve(ctx, &ctx->wide_y, &ctx->wide_y_cap, (size_t)m * (size_t)w->n * sizeof(float));
             if (rc != TURQ_OK) return rc;
             y32 = (float *)ctx->wide_y;
@@ -515,7 +516,7 @@ static int impl_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int 
     if (w->device != ctx->device) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: weight lives on device %d, context on %d", w->device, ctx->device);
     if (!turq_dt_is_quant(w->dtype) && w->dtype != TURQ_F32 && w->dtype != TURQ_F16 && w->dtype != TURQ_BF16)
         return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: unsupported weight dtype %d", w->dtype);
-    const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
+    const int xb = (xt & ~0xFF) ? 0 : turq_act_bytes(xt), yb = turq_yt_ok(yt, true) ? turq_act_bytes(yt) : 0;
     if (!xb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: unsupported activation dtype %d", xt);
     if (!yb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul: unsupported output dtype %d", yt);
     if (m < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul: m=%lld is negative", (long long)m);
@@ -535,6 +536,8 @@ static int impl_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int 
     rc = turq_ctx_reserve(ctx, &ctx->stage_y, &ctx->stage_y_cap, yrow * (size_t)m);
     if (rc != TURQ_OK) return rc;
     TURQ_HIP(ctx, hipMemcpy2DAsync(ctx->stage_x, xrow, x, (size_t)ldx * xb, xrow, (size_t)m, hipMemcpyHostToDevice, ctx->stream));
+    if (yt & TURQ_OUT_ACCUMULATE)  // the rows that the results are added to
+        TURQ_HIP(ctx, hipMemcpy2DAsync(ctx->stage_y, yrow, y, (size_t)ldy * yb, yrow, (size_t)m, hipMemcpyHostToDevice, ctx->stream));
     if (bias) {  // with host pointers the bias is a host array too
         rc = turq_ctx_reserve(ctx, &ctx->stage_b, &ctx->stage_b_cap, (size_t)w->n * sizeof(float));
         if (rc != TURQ_OK) return rc;
@@ -563,7 +566,8 @@ static int impl_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const
         one_launch = w && ys[i] && w->device == ctx->device && turq_dt_is_quant(w->dtype) && w->layout == TURQ_LAYOUT_TILED &&
                      w->k == weights[0]->k && w->k > 0 && w->n > 0 && ldys[i] >= w->n;
     }
-    const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
+    if (yt & ~0xFF) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul_multi: output dtype %d (TURQ_OUT_ACCUMULATE is for turq_qmatmul and turq_mlp)", yt);
+    const int xb = (xt & ~0xFF) ? 0 : turq_act_bytes(xt), yb = turq_act_bytes(yt);
     one_launch = one_launch && xb && yb && ldx >= weights[0]->k;
     if (one_launch && many_rows && turq_rows_in_chunks(ctx, count, weights, x, xt, ldx, m)) {
         void *yc[4];
@@ -611,7 +615,7 @@ static int impl_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const tu
         return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul_gate_up: gate is [%lld, %lld], up is [%lld, %lld]", (long long)gate->n,
                          (long long)gate->k, (long long)up->n, (long long)up->k);
     if (mem != TURQ_MEM_DEVICE && mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_gate_up: bad mem %d", mem);
-    const int yb = turq_act_bytes(yt);
+    const int yb = (yt & ~0xFF) ? 0 : turq_act_bytes(yt);
     if (!yb) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_qmatmul_gate_up: output dtype %d", yt);
     if (m < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul_gate_up: m=%lld is negative", (long long)m);
     if (ldy < gate->n) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_qmatmul_gate_up: ldy=%lld is smaller than n=%lld", (long long)ldy, (long long)gate->n);
@@ -663,10 +667,7 @@ static int impl_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const tu
     return TURQ_OK;
 }
 
-static int impl_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt, int64_t m,
-                    int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, const float *bias_down, int act,
-                    int mem) {
-    TURQ_ENTER(ctx);
+static int mlp_check(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, int64_t m, int yt, int act, int mem) {
     if (!gate || !up || !down) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_mlp: null weight");
     if (act != TURQ_ACTFN_SILU) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_mlp: activation %d is not supported", act);
     if (gate->n != up->n || gate->k != up->k)
@@ -675,8 +676,19 @@ static int impl_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *u
     if (down->k != gate->n)
         return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_mlp: down takes %lld columns, gate and up give %lld", (long long)down->k, (long long)gate->n);
     if (mem != TURQ_MEM_DEVICE && mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_mlp: bad mem %d", mem);
-    if (!turq_act_bytes(yt)) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_mlp: output dtype %d", yt);
+    if (!turq_yt_ok(yt, true)) return turq_fail(ctx, TURQ_ERR_DTYPE, "turq_mlp: output dtype %d", yt);
     if (m < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "turq_mlp: m=%lld is negative", (long long)m);
+    return TURQ_OK;
+}
+
+static int impl_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt, int64_t m,
+                    int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, const float *bias_down, int act,
+                    int mem) {
+    TURQ_ENTER(ctx);
+    {
+        const int rc = mlp_check(ctx, gate, up, down, m, yt, act, mem);
+        if (rc != TURQ_OK) return rc;
+    }
     const int64_t n_ff = gate->n;
     const size_t h_elems = (size_t)m * (size_t)n_ff;
     if (mem == TURQ_MEM_HOST) {
@@ -703,6 +715,101 @@ static int impl_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *u
     rc = impl_qmatmul_gate_up(ctx, gate, up, x, xt, m, ldx, ctx->mlp_h, ht, n_ff, bias_gate, bias_up, act, mem);
     if (rc != TURQ_OK) return rc;
     return impl_qmatmul(ctx, down, ctx->mlp_h, ht, m, n_ff, y, yt, ldy, bias_down, mem, TURQ_ALGO_AUTO);
+}
+
+// ---- RmsNorm taken into the forward calls ----
+
+// the normalised rows in scratch memory of the context, for the calls whose kernels do not apply the norm themselves: f16 where
+// the matmul kernels would round them to f16 first thing (the same values, half the bytes), f32 with wide activations
+static int norm_to_scratch(turq_ctx *ctx, const void *x, int xt, int64_t m, int64_t k, int64_t ldx, const float *nw, float eps, int *ht) {
+    *ht = ctx->wide ? TURQ_ACT_F32 : TURQ_ACT_F16;
+    int rc = turq_ctx_reserve(ctx, &ctx->norm_x, &ctx->norm_x_cap, (size_t)m * (size_t)k * (size_t)turq_act_bytes(*ht) + 16);
+    if (rc != TURQ_OK) return rc;
+    TURQ_HIP(ctx, turq_launch_rms_norm(x, xt, m, k, ldx, nw, eps, ctx->norm_x, *ht, k, ctx->stream));
+    return TURQ_OK;
+}
+
+static int norm_args(turq_ctx *ctx, const char *fn, const void *x, int xt, int64_t m, int64_t k, int64_t ldx, const float *nw) {
+    if ((xt & ~0xFF) || !turq_act_bytes(xt)) return turq_fail(ctx, TURQ_ERR_DTYPE, "%s: unsupported activation dtype %d", fn, xt);
+    if (m < 0) return turq_fail(ctx, TURQ_ERR_SHAPE, "%s: m=%lld is negative", fn, (long long)m);
+    if (ldx < k) return turq_fail(ctx, TURQ_ERR_SHAPE, "%s: ldx=%lld is smaller than k=%lld", fn, (long long)ldx, (long long)k);
+    if (m > 0 && k > 0 && (!x || !nw)) return turq_fail(ctx, TURQ_ERR_INVALID, "%s: null activation or norm weight pointer", fn);
+    return TURQ_OK;
+}
+
+static int impl_norm_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int xt, int64_t m, int64_t ldx,
+                                   const float *nw, float eps, void *const *ys, int yt, const int64_t *ldys, const float *const *biases,
+                                   int mem) {
+    TURQ_ENTER(ctx);
+    if (count < 0) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_norm_qmatmul_multi: count=%d is negative", count);
+    if (count == 0) return TURQ_OK;
+    if (!weights || !ys || !ldys || !weights[0]) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_norm_qmatmul_multi: null weight, output or stride array");
+    if (mem != TURQ_MEM_DEVICE && mem != TURQ_MEM_HOST) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_norm_qmatmul_multi: bad mem %d", mem);
+    const int64_t k = weights[0]->k;
+    int rc = norm_args(ctx, "turq_norm_qmatmul_multi", x, xt, m, k, ldx, nw);
+    if (rc != TURQ_OK) return rc;
+    if (m == 0 || k == 0) return impl_qmatmul_multi(ctx, count, weights, x, xt, m, ldx, ys, yt, ldys, biases, mem, TURQ_ALGO_AUTO);
+    if (mem == TURQ_MEM_HOST) {
+        std::vector<float> xn;
+        try { xn.resize((size_t)m * (size_t)k); } catch (...) { return turq_fail(ctx, TURQ_ERR_OOM, "turq_norm_qmatmul_multi: host scratch"); }
+        rc = impl_rms_norm(ctx, x, xt, m, k, ldx, nw, eps, xn.data(), TURQ_ACT_F32, k, mem);
+        if (rc != TURQ_OK) return rc;
+        return impl_qmatmul_multi(ctx, count, weights, xn.data(), TURQ_ACT_F32, m, k, ys, yt, ldys, biases, mem, TURQ_ALGO_AUTO);
+    }
+    bool plain = !(yt & ~0xFF) && turq_act_bytes(yt) && count <= 16;
+    for (int i = 0; i < count && plain; i++) plain = weights[i] && ys[i] && ldys[i] >= weights[i]->n;
+    if (plain && turq_norm_fuses(ctx, count, weights, x, xt, ldx, m)) {
+        const TurqNorm nm{nw, eps};
+        if (m == 1) return turq_qmatmul_multi_mfma(ctx, count, weights, x, xt, m, ldx, ys, yt, ldys, biases, &nm);
+        bool taken = false;
+        rc = turq_qmatmul_multi_gemm(ctx, count, weights, x, xt, m, ldx, ys, yt, ldys, biases, &taken, &nm);
+        if (rc != TURQ_OK || taken) return rc;
+    }
+    int ht = TURQ_ACT_F16;
+    rc = norm_to_scratch(ctx, x, xt, m, k, ldx, nw, eps, &ht);
+    if (rc != TURQ_OK) return rc;
+    return impl_qmatmul_multi(ctx, count, weights, ctx->norm_x, ht, m, k, ys, yt, ldys, biases, mem, TURQ_ALGO_AUTO);
+}
+
+static int impl_norm_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt, int64_t m,
+                         int64_t ldx, const float *nw, float eps, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up,
+                         const float *bias_down, int act, int mem) {
+    TURQ_ENTER(ctx);
+    int rc = mlp_check(ctx, gate, up, down, m, yt, act, mem);
+    if (rc != TURQ_OK) return rc;
+    const int64_t k = gate->k, n_ff = gate->n;
+    rc = norm_args(ctx, "turq_norm_mlp", x, xt, m, k, ldx, nw);
+    if (rc != TURQ_OK) return rc;
+    if (m == 0 || k == 0) return impl_mlp(ctx, gate, up, down, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem);
+    if (mem == TURQ_MEM_HOST) {
+        std::vector<float> xn;
+        try { xn.resize((size_t)m * (size_t)k); } catch (...) { return turq_fail(ctx, TURQ_ERR_OOM, "turq_norm_mlp: host scratch"); }
+        rc = impl_rms_norm(ctx, x, xt, m, k, ldx, nw, eps, xn.data(), TURQ_ACT_F32, k, mem);
+        if (rc != TURQ_OK) return rc;
+        return impl_mlp(ctx, gate, up, down, xn.data(), TURQ_ACT_F32, m, k, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem);
+    }
+    const turq_weight *gu[2] = {gate, up};
+    if (y && ldy >= down->n && turq_norm_fuses(ctx, 2, gu, x, xt, ldx, m)) {
+        const TurqNorm nm{nw, eps};
+        bool taken = false;
+        if (m == 1 && gate->dtype == up->dtype) {
+            // as turq_mlp's one-row route: the f16 intermediate where down_proj rounds its input to f16 anyway
+            const bool h16 = turq_dt_is_quant(down->dtype) && down->layout == TURQ_LAYOUT_TILED && n_ff % 8 == 0;
+            const int ht = h16 ? TURQ_ACT_F16 : TURQ_ACT_F32;
+            rc = turq_ctx_reserve(ctx, &ctx->mlp_h, &ctx->mlp_h_cap, (size_t)m * (size_t)n_ff * (h16 ? sizeof(uint16_t) : sizeof(float)) + 16);
+            if (rc != TURQ_OK) return rc;
+            rc = turq_qmatmul_gate_up_mfma(ctx, gate, up, x, xt, m, ldx, ctx->mlp_h, ht, n_ff, bias_gate, bias_up, &taken, &nm);
+            if (rc != TURQ_OK) return rc;
+            if (taken) return impl_qmatmul(ctx, down, ctx->mlp_h, ht, m, n_ff, y, yt, ldy, bias_down, mem, TURQ_ALGO_AUTO);
+        } else if (m > TURQ_GEMV_MAX_M) {
+            rc = turq_mlp_prefill(ctx, gate, up, down, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, bias_down, &taken, &nm);
+            if (rc != TURQ_OK || taken) return rc;
+        }
+    }
+    int ht = TURQ_ACT_F16;
+    rc = norm_to_scratch(ctx, x, xt, m, k, ldx, nw, eps, &ht);
+    if (rc != TURQ_OK) return rc;
+    return impl_mlp(ctx, gate, up, down, ctx->norm_x, ht, m, k, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem);
 }
 
 // ---- graphs and kernel timing ----
@@ -899,6 +1006,16 @@ int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weig
 int turq_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt, int64_t m,
              int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, const float *bias_down, int act, int mem) {
     return capture_guard(ctx, impl_mlp(ctx, gate, up, down, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem));
+}
+int turq_norm_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int xt, int64_t m, int64_t ldx,
+                            const float *norm_weight, float eps, void *const *ys, int yt, const int64_t *ldys, const float *const *biases,
+                            int mem) {
+    return capture_guard(ctx, impl_norm_qmatmul_multi(ctx, count, weights, x, xt, m, ldx, norm_weight, eps, ys, yt, ldys, biases, mem));
+}
+int turq_norm_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt, int64_t m,
+                  int64_t ldx, const float *norm_weight, float eps, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up,
+                  const float *bias_down, int act, int mem) {
+    return capture_guard(ctx, impl_norm_mlp(ctx, gate, up, down, x, xt, m, ldx, norm_weight, eps, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem));
 }
 int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
     return capture_guard(ctx, impl_quantize_q8_0(ctx, x, m, k, out, mem));

@@ -53,8 +53,14 @@ inline const char *turq_dt_name(int dt) {
 inline bool turq_dt_is_quant(int dt) {
     return dt == TURQ_Q8_0 || dt == TURQ_Q4_K || dt == TURQ_Q5_K || dt == TURQ_Q6_K;
 }
+// an output type may carry TURQ_OUT_ACCUMULATE; its element type is the low byte
+inline int turq_yt_base(int yt) { return yt & 0xFF; }
+inline bool turq_yt_ok(int yt, bool accumulate_allowed) {
+    const int b = yt & 0xFF, flags = yt & ~0xFF;
+    return (b == TURQ_ACT_F32 || b == TURQ_ACT_BF16 || b == TURQ_ACT_F16) && (flags == 0 || (accumulate_allowed && flags == TURQ_OUT_ACCUMULATE));
+}
 inline int turq_act_bytes(int act) {
-    switch (act) {
+    switch (act & 0xFF) {
     case TURQ_ACT_F32: return 4;
     case TURQ_ACT_BF16: case TURQ_ACT_F16: return 2;
     default: return 0;
@@ -87,6 +93,7 @@ struct turq_ctx {
     void *wide_y = nullptr;   size_t wide_y_cap = 0;
     bool wide = false;  // device-pointer calls take that path too (host-pointer calls always do)
     void *mlp_h = nullptr;    size_t mlp_h_cap = 0;  // turq_mlp: the f32 intermediate act(gate) * up
+    void *norm_x = nullptr;   size_t norm_x_cap = 0;  // turq_norm_*: the normalised rows where the kernels do not apply the norm themselves
     // prefill GEMM launches that split their columns over several workgroups: kSplitSlots counter blocks (zero between
     // launches; launch i of a call uses block i), then the partial tiles of the call's launches one after the other
     static constexpr int kSplitSlots = 16;
@@ -197,6 +204,15 @@ hipError_t turq_launch_gemv_simple(int dtype, const void *w, int64_t n, int64_t 
 TURQ_NONFINITE_UNITS(TURQ_DECLARE_NONFINITE)
 #undef TURQ_DECLARE_NONFINITE
 
+// RmsNorm taken into a forward call: x stands for x / sqrt(mean(x^2) + eps) * w (w: f32 [k] in device memory)
+struct TurqNorm {
+    const float *w;
+    float eps;
+};
+// whether the kernels of a call with these weights and rows apply the norm themselves (one row: inside the matmul kernel; more
+// than 32 rows: the norm writes the prefill GEMM's fragments); otherwise the caller normalises into scratch first
+bool turq_norm_fuses(const turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t ldx, int64_t m);
+
 // largest m the skinny MFMA kernel takes; above it the LDS-tiled GEMM runs
 #define TURQ_GEMV_MAX_M 32
 // largest m for which the skinny kernel can prepare the activations itself (no separate launch);
@@ -204,7 +220,7 @@ TURQ_NONFINITE_UNITS(TURQ_DECLARE_NONFINITE)
 #define TURQ_GEMV_FUSED_MAX_M 4
 // MFMA paths on the tiled layout (activation preparation + kernel launch), see mfma_dispatch.cpp
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
-                      int yt, int64_t ldy, const float *bias, int algo);
+                      int yt, int64_t ldy, const float *bias, int algo, const TurqNorm *norm = nullptr);
 // act(gate) * up on two f32 matrices [m, n] of row stride n (act_mul.hip)
 hipError_t turq_launch_read_yardstick(const void *buf, size_t nbytes, int workgroups, hipStream_t stream, hipEvent_t ev_start,
                                       hipEvent_t ev_stop);
@@ -214,15 +230,16 @@ hipError_t turq_launch_silu_mul(const float *gate, const float *up, int64_t m, i
                                 hipStream_t stream);
 // act(gate) * up inside the one-row kernel; *taken = false (and nothing launched) where that kernel does not apply
 int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m,
-                              int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, bool *taken);
+                              int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, bool *taken,
+                              const TurqNorm *norm = nullptr);
 // whether a call of 33 .. 64 rows on these weights goes through the kernels of up to 32 rows in two chunks
 bool turq_rows_in_chunks(const turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t ldx, int64_t m);
 int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m, int64_t ldx,
-                            void *const *y, int yt, const int64_t *ldy, const float *const *bias, bool *taken);
+                            void *const *y, int yt, const int64_t *ldy, const float *const *bias, bool *taken, const TurqNorm *norm = nullptr);
 // The whole MLP of a prompt chunk (more than 32 rows): gate / up GEMMs into f32 scratch, one kernel that turns the two products
 // into down_proj's fragments, down_proj's GEMM on them; *taken = false (nothing launched) where that route does not apply
 int turq_mlp_prefill(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt,
                      int64_t m, int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up,
-                     const float *bias_down, bool *taken);
+                     const float *bias_down, bool *taken, const TurqNorm *norm = nullptr);
 int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m,
-                            int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias);
+                            int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias, const TurqNorm *norm = nullptr);

@@ -457,7 +457,23 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
     int lid = blockIdx.x;
     if ((nwg & 7) == 0) lid = (blockIdx.x & 7) * (nwg >> 3) + (blockIdx.x >> 3);
     // (split: the m-blocks of one n-block and one part are consecutive, they share the part's packed weights)
-    const int mb = lid % nblocks_m, part = SK ? (lid / nblocks_m) % split : 0, nb_all = lid / (nblocks_m * (SK ? split : 1));
+    int mb = lid % nblocks_m, nb_all = lid / (nblocks_m * (SK ? split : 1));
+    const int part = SK ? (lid / nblocks_m) % split : 0;
+    if constexpr (!SK) {
+        // Many m-blocks (prompts of 1024 rows and more): the workgroups that run together on an XCD - consecutive logical ids -
+        // should share activation fragments as well as weights.  With the m-blocks of an n-block all next to each other, 32
+        // neighbours are 2 n-blocks x 16 m-blocks: every m-block's fragments (1.1 MB) are then fetched into the L2 once per PAIR of
+        // n-blocks (measured at m = 2048, n = 12288: 456 MB fetched per launch for 46 MB of weights and fragments).  In chunks of
+        // kChunk m-blocks, 32 neighbours are 8 n-blocks x 4 m-blocks (Q4_K 12288 x 4096: 210 -> 205 us at m = 2048, 421 -> 402 us
+        // at m = 4096, same session).
+        constexpr int kChunk = 4;
+        if (nblocks_m > kChunk) {
+            const int per_chunk = kChunk * nblocks_n, chunk = lid / per_chunk, rem = lid - chunk * per_chunk;
+            const int left = nblocks_m - chunk * kChunk, mc = left < kChunk ? left : kChunk;
+            nb_all = rem / mc;
+            mb = chunk * kChunk + rem - nb_all * mc;
+        }
+    }
     // the weight this n-block belongs to
     const uint8_t *__restrict__ w = grp.w[0];
     void *__restrict__ y = grp.y[0];
@@ -849,6 +865,8 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
     // ---- results ----
     // 32x32 result: lane (n32, g32), register e holds row 8 * (e / 4) + 4 * g32 + e % 4 of column n32
     constexpr int OUT_PITCH = G::OUT_PITCH;
+    const bool accum = (yt & TURQ_OUT_ACCUMULATE) != 0;  // y += results: the residual stream
+    const int ytb = yt & 0xFF;
     const int64_t row0 = (int64_t)mb * G::GBM + wm * (WM * 32);
     const int64_t col0 = (int64_t)nb * G::BN + wn * (WN * 32);
     if (vec_out) {
@@ -868,17 +886,19 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         uint32_t bad = 0;  // results that are no finite numbers, or do not fit an f16 output (turq_ctx_nonfinite_count)
-        const float lim = yt == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
-        if (yt == TURQ_ACT_F32) {
+        const float lim = ytb == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
+        if (ytb == TURQ_ACT_F32) {
             constexpr int CPR = WN * 32 / 4;  // 16-byte pieces per row
 #pragma unroll 4
             for (int it = 0; it < WM * 32 * CPR / 64; it++) {
                 const int c = it * 64 + lane;
                 const int r = c / CPR, cc = c - r * CPR;
-                const float4v v = *(const float4v *)(stage + r * OUT_PITCH + 4 * cc);
+                float4v v = *(const float4v *)(stage + r * OUT_PITCH + 4 * cc);
                 if (row0 + r < m && col0 + 4 * cc < n) {
+                    float4v *dst = (float4v *)((float *)y + (row0 + r) * ldy + col0 + 4 * cc);
+                    if (accum) v += *dst;
                     turq_note_accum(v.x, lim, bad), turq_note_accum(v.y, lim, bad), turq_note_accum(v.z, lim, bad), turq_note_accum(v.w, lim, bad);
-                    *(float4v *)((float *)y + (row0 + r) * ldy + col0 + 4 * cc) = v;
+                    *dst = v;
                 }
             }
         } else {
@@ -889,23 +909,39 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                 const int r = c / CPR, cc = c - r * CPR;
                 const float4v v0 = *(const float4v *)(stage + r * OUT_PITCH + 8 * cc);
                 const float4v v1 = *(const float4v *)(stage + r * OUT_PITCH + 8 * cc + 4);
-                uint4v o;
-                if (yt == TURQ_ACT_BF16)
-                    o = uint4v{pack_bf16x2(v0.x, v0.y), pack_bf16x2(v0.z, v0.w), pack_bf16x2(v1.x, v1.y), pack_bf16x2(v1.z, v1.w)};
-                else
-                    o = uint4v{pack_f16x2(v0.x, v0.y), pack_f16x2(v0.z, v0.w), pack_f16x2(v1.x, v1.y), pack_f16x2(v1.z, v1.w)};
                 if (row0 + r < m && col0 + 8 * cc < n) {
-                    const float vs[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+                    uint4v *dst = (uint4v *)((uint16_t *)y + (row0 + r) * ldy + col0 + 8 * cc);
+                    float vs[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+                    if (accum) {
+                        const uint4v old = *dst;
+                        const uint32_t ow[4] = {old.x, old.y, old.z, old.w};
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            if (ytb == TURQ_ACT_BF16) {
+                                vs[2 * e] += __uint_as_float(ow[e] << 16);
+                                vs[2 * e + 1] += __uint_as_float(ow[e] & 0xFFFF0000u);
+                            } else {
+                                const half2v hh = as_half2(ow[e]);
+                                vs[2 * e] += (float)hh.x;
+                                vs[2 * e + 1] += (float)hh.y;
+                            }
+                        }
+                    }
 #pragma unroll
                     for (int e = 0; e < 8; e++) turq_note_accum(vs[e], lim, bad);
-                    *(uint4v *)((uint16_t *)y + (row0 + r) * ldy + col0 + 8 * cc) = o;
+                    uint4v o;
+                    if (ytb == TURQ_ACT_BF16)
+                        o = uint4v{pack_bf16x2(vs[0], vs[1]), pack_bf16x2(vs[2], vs[3]), pack_bf16x2(vs[4], vs[5]), pack_bf16x2(vs[6], vs[7])};
+                    else
+                        o = uint4v{pack_f16x2(vs[0], vs[1]), pack_f16x2(vs[2], vs[3]), pack_f16x2(vs[4], vs[5]), pack_f16x2(vs[6], vs[7])};
+                    *dst = o;
                 }
             }
         }
         turq_note_flush(bad);
     } else {
         uint32_t bad = 0;
-        const float lim = yt == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
+        const float lim = ytb == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
 #pragma unroll
         for (int j = 0; j < WN; j++) {
             const int64_t col = col0 + 32 * j + n32;
@@ -917,10 +953,13 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                 for (int e = 0; e < 16; e++) {
                     const int64_t row = row0 + 32 * i + 8 * (e >> 2) + 4 * g32 + (e & 3);
                     if (row < m) {
-                        const float v = acc[i][j][e] * inv_ws + bv;
+                        float v = acc[i][j][e] * inv_ws + bv;
+                        if (accum)
+                            v += ytb == TURQ_ACT_F32 ? turq_load_out<TURQ_ACT_F32>(y, row * ldy + col)
+                                 : ytb == TURQ_ACT_BF16 ? turq_load_out<TURQ_ACT_BF16>(y, row * ldy + col) : turq_load_out<TURQ_ACT_F16>(y, row * ldy + col);
                         turq_note_accum(v, lim, bad);
-                        if (yt == TURQ_ACT_F32) turq_store_out_raw<TURQ_ACT_F32>(y, row * ldy + col, v);
-                        else if (yt == TURQ_ACT_BF16) turq_store_out_raw<TURQ_ACT_BF16>(y, row * ldy + col, v);
+                        if (ytb == TURQ_ACT_F32) turq_store_out_raw<TURQ_ACT_F32>(y, row * ldy + col, v);
+                        else if (ytb == TURQ_ACT_BF16) turq_store_out_raw<TURQ_ACT_BF16>(y, row * ldy + col, v);
                         else turq_store_out_raw<TURQ_ACT_F16>(y, row * ldy + col, v);
                     }
                 }
@@ -950,7 +989,7 @@ hipError_t launch_gemm(const TurqGemmWeights &ws, int64_t k, const void *frags, 
     if (attr != hipSuccess) return attr;
     GemmGroup grp{};
     grp.count = ws.count;
-    const int es = y_dtype == TURQ_ACT_F32 ? 4 : 2;
+    const int es = (y_dtype & 0xFF) == TURQ_ACT_F32 ? 4 : 2;
     int nbn = 0, vec_out = 1;
     for (int i = 0; i < ws.count; i++) {
         grp.w[i] = (const uint8_t *)ws.w[i];

@@ -88,11 +88,7 @@ __device__ __forceinline__ void cs_body(const uint8_t *__restrict__ w, int64_t n
         const int64_t col = (rt0 + r) * 16 + nn;
         if (rt0 + r >= nrt || col >= n) continue;
         const float bv = bias ? bias[col] : 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int64_t row = 16 * mt + 4 * g + j;
-            if (row < m) turq_store_any(y, yt, row * ldy + col, s[j] + bv);
-        }
+        turq_store_col4(y, yt, 16 * mt + 4 * g, m, ldy, col, s + float4v{bv, bv, bv, bv});
     }
 }
 
@@ -169,7 +165,7 @@ hipError_t turq_launch_gemv_cs(int dtype, int count, const void *const *w, const
     if (count < 1 || count > kMaxMulti || m < 1 || m > TURQ_GEMV_MAX_M || nwaves < 1 || nwaves > 8 || !turq_gemv_cs_rows_ok(row_tiles))
         return hipErrorInvalidValue;
     if (k <= 0 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     CsLaunch l{};
     int64_t blocks = 0;
     for (int i = 0; i < count; i++) {
@@ -222,7 +218,7 @@ hipError_t turq_launch_gemv_cs_staged(int dtype_a, int dtype_b, int count, int s
     if (count < 1 || count > kMaxMulti || second < 1 || second > count || (second == count) != (dtype_a == dtype_b) ||
         !turq_gemv_cs_staged_takes(dtype_a, dtype_b, k, m, row_tiles))
         return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     switch (x_dtype) {
     case TURQ_ACT_F32: return turq_launch_gemv_cs_staged_f32(TURQ_STAGED_LAUNCH_PASS);
     case TURQ_ACT_BF16: return turq_launch_gemv_cs_staged_bf16(TURQ_STAGED_LAUNCH_PASS);
@@ -251,7 +247,7 @@ hipError_t turq_launch_gemv_cs_staged_gateup(int dtype, const void *w_gate, cons
                                              int64_t ldx, int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate,
                                              const float *bias_up, int tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (!turq_gemv_cs_staged_waves(k) || m < 1 || m > 32 || (tiles != 2 && tiles != 6) || (m > 16 && tiles != 6)) return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     switch (x_dtype) {
     case TURQ_ACT_F32: return turq_launch_gemv_cs_staged_gateup_f32(TURQ_STAGED_GATEUP_PASS);
     case TURQ_ACT_BF16: return turq_launch_gemv_cs_staged_gateup_bf16(TURQ_STAGED_GATEUP_PASS);

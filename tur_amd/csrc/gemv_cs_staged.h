@@ -199,16 +199,16 @@ __device__ __forceinline__ void cs_body_staged(const uint8_t *__restrict__ w, in
         const int64_t col = (rt0 + r) * 16 + nn;
         if (rt0 + r >= nrt || col >= n) continue;
         const float bv = bias ? bias[col] : 0.0f, bv2 = (GU && bias2) ? bias2[col] : 0.0f;
+        if constexpr (GU) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int64_t row = HR * h + 4 * g + j;
-            if (row >= m) continue;
-            if constexpr (GU) {
+            for (int j = 0; j < 4; j++) {
+                const int64_t row = HR * h + 4 * g + j;
+                if (row >= m) continue;
                 const float gate = s[j] + bv, up = s2[j] + bv2;
                 turq_store_any(y, yt, row * ldy + col, gate / (1.0f + expf(-gate)) * up);
-            } else {
-                turq_store_any(y, yt, row * ldy + col, s[j] + bv);
             }
+        } else {
+            turq_store_col4(y, yt, HR * h + 4 * g, m, ldy, col, s + float4v{bv, bv, bv, bv});
         }
     }
 }
@@ -347,16 +347,16 @@ __device__ __forceinline__ void cs_body_staged_two(const uint8_t *__restrict__ w
         const int64_t col = (rt0 + r) * 16 + nn;
         if (rt0 + r >= nrt || col >= n) continue;
         const float bv = bias ? bias[col] : 0.0f, bv2 = (GU && bias2) ? bias2[col] : 0.0f;
+        if constexpr (GU) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int64_t row = 16 * mt + 4 * g + j;
-            if (row >= m) continue;
-            if constexpr (GU) {
+            for (int j = 0; j < 4; j++) {
+                const int64_t row = 16 * mt + 4 * g + j;
+                if (row >= m) continue;
                 const float gate = s[j] + bv, up = s2[j] + bv2;
                 turq_store_any(y, yt, row * ldy + col, gate / (1.0f + expf(-gate)) * up);
-            } else {
-                turq_store_any(y, yt, row * ldy + col, s[j] + bv);
             }
+        } else {
+            turq_store_col4(y, yt, 16 * mt + 4 * g, m, ldy, col, s + float4v{bv, bv, bv, bv});
         }
     }
 }

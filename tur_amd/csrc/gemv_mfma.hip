@@ -201,12 +201,7 @@ __device__ __forceinline__ void gemv_body(const uint8_t *__restrict__ w, int64_t
     if (col >= n) return;
     const float bv = bias ? bias[col] : 0.0f;
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int64_t row = 16 * mt + 4 * g + i;
-            if (row < m) turq_store_any(y, yt, row * ldy + col, acc[mt][i] + bv);
-        }
+    for (int mt = 0; mt < MT; mt++) turq_store_col4(y, yt, 16 * mt + 4 * g, m, ldy, col, acc[mt] + float4v{bv, bv, bv, bv});
 }
 
 template <int DT, int MT, int XT, bool FUSED, int MP, int P, int MAXT>
@@ -323,12 +318,7 @@ __device__ __forceinline__ void gemv_frag_body(const uint8_t *__restrict__ w, in
         if (rt0 + r >= nrt || col >= n) continue;
         const float bv = bias ? bias[col] : 0.0f;
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int64_t row = 16 * mt + 4 * g + i;
-                if (row < m) turq_store_any(y, yt, row * ldy + col, acc[r][mt][i] + bv);
-            }
+        for (int mt = 0; mt < MT; mt++) turq_store_col4(y, yt, 16 * mt + 4 * g, m, ldy, col, acc[r][mt] + float4v{bv, bv, bv, bv});
     }
 }
 
@@ -565,7 +555,7 @@ hipError_t turq_launch_gemv_multi(int dtype, int count, const void *const *w, co
                                   hipEvent_t ev_stop) {
     if (count < 1 || count > kMaxMulti || m < 1 || m > (fused ? TURQ_GEMV_FUSED_MAX_M : TURQ_GEMV_MAX_M) || nwaves < 1 || nwaves > 16)
         return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     if (row_tiles != 1 && !(row_tiles == 2 && !fused && nwaves <= 4)) return hipErrorInvalidValue;
     MultiArgs ma{};
     int64_t blocks = 0;
@@ -613,7 +603,7 @@ hipError_t turq_launch_gemv_multi_mixed(int dtype_a, int dtype_b, int count, int
     if (!turq_gemv_multi_mixed_supports(dtype_a, dtype_b) || count < 2 || count > kMaxMulti || second < 1 || second >= count || m < 1 ||
         m > TURQ_GEMV_MAX_M || nwaves < 1 || nwaves > 16)
         return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     MultiArgs ma{};
     int64_t blocks = 0;
     for (int i = 0; i < count; i++) {
@@ -648,7 +638,7 @@ hipError_t turq_launch_gemv_mfma(int dtype, const void *w, int64_t n, int64_t k,
     if (n == 0 || m == 0) return hipSuccess;
     if (m > TURQ_GEMV_MAX_M || nwaves < 1 || nwaves > 16) return hipErrorInvalidValue;
     if (fused && m > TURQ_GEMV_FUSED_MAX_M) return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     const GemvArgs a{w, n, k, xin, ldx, m, y, y_dtype, ldy, bias, nwaves, stream, ev_start, ev_stop};
     switch (dtype) {
     case TURQ_Q4_K: return launch_x<TURQ_Q4_K>(x_dtype, fused, a);
@@ -696,7 +686,7 @@ hipError_t turq_launch_gemv_gateup_frag(int dtype, const void *w_gate, const voi
                                         int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate, const float *bias_up,
                                         int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
     if (nwaves < 1 || nwaves > 4 || m < 1 || m > TURQ_GEMV_MAX_M || k <= 0 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     if (n == 0) return hipSuccess;
     switch (dtype) {
     case TURQ_Q4_K: return launch_gateup_frag<TURQ_Q4_K>(w_gate, w_up, bias_gate, bias_up, n, k, frags, m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);

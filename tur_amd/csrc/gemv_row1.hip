@@ -378,11 +378,17 @@ struct Row1Args {
 // uses them for R weight tiles); M = activation rows the instantiation holds (rows past m repeat row 0 and are not stored)
 // GU (R = 2): the two "row tiles" are row tile rtb of a gate weight (w) and of an up weight (w2) of the same shape, and
 // what is stored is act(gate) * up (src/models/qwen3.rs:161-167 computes that product from the two projections' outputs)
-template <int DT, int XT, int P, int R, int M, bool GU = false>
+// NORM (M = 1): the activation row is RmsNorm(x) with weight gw (src/models/layers/norm.rs:81-93, applied in front of q / k / v,
+// gate / up and the LM head): a lane multiplies its columns by gw when it stages them and adds up their squares, and the row's
+// 1 / sqrt(mean(x^2) + eps), which is the same for every column, multiplies the results - the separate launch of the norm and
+// the round trip of its output go away.
+template <int DT, int XT, int P, int R, int M, bool GU = false, bool NORM = false>
 __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *__restrict__ y, int64_t ldy, const float *__restrict__ bias,
                                           int64_t n, int64_t rtb, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt,
-                                          const uint8_t *__restrict__ w2 = nullptr, const float *__restrict__ bias2 = nullptr) {
+                                          const uint8_t *__restrict__ w2 = nullptr, const float *__restrict__ bias2 = nullptr,
+                                          const float *__restrict__ gw = nullptr, float eps = 0.0f) {
     static_assert(!GU || R == 2, "gate and up take the places of two row tiles");
+    static_assert(!NORM || M == 1, "the norm is taken into the kernel for one activation row");
     extern __shared__ uint8_t smem[];
     using Fmt = Row1Fmt<DT>;
     constexpr int TB = TiledFmt<DT>::kTileBytes;
@@ -401,6 +407,8 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
     static_assert(!PK || M % 2 == 0, "packed pairs");
     uint8_t *region = smem + (size_t)wave * (P * PSTRIDE);  // [p][activation row] or [p][pair]
     float *red = (float *)(smem + (size_t)nwaves * (P * PSTRIDE));
+    float *red_ss = red + (size_t)nwaves * (R * M * 64);  // NORM: a sum of squares per wave
+    float ss = 0.0f;
 
     // the zeros that the idle A rows read, and start values that no format overwrites
     if constexpr (PK) {
@@ -427,8 +435,23 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
     }
 #pragma unroll
     for (int mm = 0; mm < M; mm++) xrow[mm] = (const uint8_t *)x + (mm < m ? mm : 0) * ldx * ES;
+    // TURQ_OUT_ACCUMULATE: the element this lane will add its first result to, requested now so that it has long arrived when
+    // the sums are done (a load at the end of the kernel is a whole memory round trip on the critical path)
+    float old_first = 0.0f;
+    if constexpr (!GU) {
+        if ((yt & TURQ_OUT_ACCUMULATE) && wave < R * M) {
+            const int r = wave / M, mm = wave - r * M;
+            const int64_t col = (rt0 + r) * 16 + (lane >> 2);
+            if ((lane & 3) == 0 && rt0 + r < nrt && col < n && mm < m) {
+                const int64_t at = (int64_t)mm * ldy + col;
+                const int base = yt & 0xFF;
+                old_first = base == TURQ_ACT_F32 ? turq_load_out<TURQ_ACT_F32>(y, at) : base == TURQ_ACT_BF16 ? turq_load_out<TURQ_ACT_BF16>(y, at) : turq_load_out<TURQ_ACT_F16>(y, at);
+            }
+        }
+    }
     for (int64_t b0 = wave; b0 < ntc; b0 += (int64_t)nwaves * P) {
         X1Regs<XT> xr[P][M];
+        float4v gv[NORM ? P : 1];
         typename Fmt::W wr[P][R];
         go.touch();
 #pragma unroll
@@ -436,6 +459,11 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
             const int64_t b = b0 + (int64_t)p * nwaves;
 #pragma unroll
             for (int mm = 0; mm < M; mm++) xr[p][mm] = load_x1<XT, DT == TURQ_Q8_0>(xrow[mm], k, b < ntc ? b : b0, lane, go);
+            if constexpr (NORM) {
+                const int64_t bb = b < ntc ? b : b0;
+                const bool ok = DT != TURQ_Q8_0 || bb * 256 + 4 * lane < k;  // (Q8_0: k may end inside the tile; the columns are zeros then)
+                gv[p] = *(const float4v *)(gw + (ok ? bb * 256 + 4 * lane : 0));
+            }
         }
 #pragma unroll
         for (int p = 0; p < P; p++) {
@@ -453,6 +481,24 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
                     to_half4<XT>(xr[p][mm], h01, h23);
                     *(uint2v *)(pr + kPX + 512 * (mm & 1) + 8 * lane) = uint2v{as_u32(h01), as_u32(h23)};
                     Fmt::sums_pk(h01, h23, pr, lane, mm & 1);
+                } else if constexpr (NORM) {
+                    float f[4];
+                    if constexpr (XT == TURQ_ACT_F32) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) f[e] = __uint_as_float(xr[p][mm].r[e]);
+                    } else if constexpr (XT == TURQ_ACT_BF16) {
+                        f[0] = __uint_as_float(xr[p][mm].r[0] << 16), f[1] = __uint_as_float(xr[p][mm].r[0] & 0xFFFF0000u);
+                        f[2] = __uint_as_float(xr[p][mm].r[1] << 16), f[3] = __uint_as_float(xr[p][mm].r[1] & 0xFFFF0000u);
+                    } else {
+                        const half2v a = as_half2(xr[p][mm].r[0]), c = as_half2(xr[p][mm].r[1]);
+                        f[0] = (float)a.x, f[1] = (float)a.y, f[2] = (float)c.x, f[3] = (float)c.y;
+                    }
+                    if (b0 + (int64_t)p * nwaves < ntc) ss += (f[0] * f[0] + f[1] * f[1]) + (f[2] * f[2] + f[3] * f[3]);  // (a tile past the end repeats another)
+                    const half2v h01 = __builtin_convertvector(float2v{f[0] * gv[p].x, f[1] * gv[p].y}, half2v);
+                    const half2v h23 = __builtin_convertvector(float2v{f[2] * gv[p].z, f[3] * gv[p].w}, half2v);
+                    uint8_t *rg = region + p * PSTRIDE + mm * kRegion;
+                    *(uint2v *)(rg + kX + 8 * lane) = uint2v{as_u32(h01), as_u32(h23)};
+                    Fmt::sums(h01, h23, rg, lane);
                 } else {
                     stage_x1<DT, XT>(xr[p][mm], region + p * PSTRIDE + mm * kRegion, lane);
                 }
@@ -505,7 +551,18 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
     for (int r = 0; r < R; r++)
 #pragma unroll
         for (int mm = 0; mm < M; mm++) red[((r * M + mm) * nwaves + wave) * 64 + lane] = acc[r][mm];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
+        if (lane == 0) red_ss[wave] = ss;
+    }
     __syncthreads();
+    float inv_rms = 1.0f;
+    if constexpr (NORM) {
+        float tot = 0.0f;
+        for (int wv = 0; wv < nwaves; wv++) tot += red_ss[wv];
+        inv_rms = 1.0f / sqrtf(tot / (float)k + eps);
+    }
     const int n4 = lane >> 2, q = lane & 3;
     if constexpr (GU) {
         for (int mm = wave; mm < M; mm += nwaves) {
@@ -518,12 +575,10 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
             su = sum4(su);
             const int64_t col = rt0 * 16 + n4;
             if (q == 0 && col < n && mm < m) {
-                const float gate = sg + (bias ? bias[col] : 0.0f), up = su + (bias2 ? bias2[col] : 0.0f);
+                const float gate = sg * inv_rms + (bias ? bias[col] : 0.0f), up = su * inv_rms + (bias2 ? bias2[col] : 0.0f);
                 const float out = gate / (1.0f + expf(-gate)) * up;  // SiLU
                 const int64_t at = (int64_t)mm * ldy + col;
-                if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, at, out);
-                else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, at, out);
-                else turq_store_out<TURQ_ACT_F16>(y, at, out);
+                turq_store_any(y, yt, at, out);
             }
         }
         return;
@@ -535,11 +590,10 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
         s = sum4(s);
         const int64_t col = (rt0 + r) * 16 + n4;
         if (q == 0 && rt0 + r < nrt && col < n && mm < m) {
-            const float out = s + (bias ? bias[col] : 0.0f);
+            const float out = s * inv_rms + (bias ? bias[col] : 0.0f);
             const int64_t at = (int64_t)mm * ldy + col;
-            if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, at, out);
-            else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, at, out);
-            else turq_store_out<TURQ_ACT_F16>(y, at, out);
+            if (i == wave) turq_store_any(y, yt & 0xFF, at, out + old_first);  // (what y held was requested before the main loop)
+            else turq_store_any(y, yt, at, out);
         }
     }
 }
@@ -555,31 +609,34 @@ __device__ inline Row1Pick row1_pick(const Row1Args &a, int blk) {
 }
 
 // m <= M activation rows of stride ldx; MAXT = largest workgroup of the instantiation
-template <int DT, int XT, int P, int R, int M, int MAXT>
-__global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt) {
+template <int DT, int XT, int P, int R, int M, int MAXT, bool NORM = false>
+__global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt,
+                                                         const float *__restrict__ gw, float eps) {
     const Row1Pick p = row1_pick(a, (int)blockIdx.x);
-    row1_body<DT, XT, P, R, M>(p.w, p.y, p.ldy, p.bias, p.n, (int64_t)((int)blockIdx.x - p.first), k, x, ldx, m, yt);
+    row1_body<DT, XT, P, R, M, false, NORM>(p.w, p.y, p.ldy, p.bias, p.n, (int64_t)((int)blockIdx.x - p.first), k, x, ldx, m, yt, nullptr,
+                                            nullptr, gw, eps);
 }
 
 // gate_proj and up_proj of one MLP in one launch, the activation and the product applied before the store: workgroup b
 // takes row tile b of both weights
-template <int DT, int XT, int P, int M, int MAXT>
+template <int DT, int XT, int P, int M, int MAXT, bool NORM = false>
 __global__ void __launch_bounds__(MAXT) gemv_row1_gateup_kernel(const uint8_t *__restrict__ wg, const uint8_t *__restrict__ wu,
                                                                  const float *__restrict__ bg, const float *__restrict__ bu, int64_t n,
                                                                  int64_t k, const void *__restrict__ x, int64_t ldx, int m,
-                                                                 void *__restrict__ y, int64_t ldy, int yt) {
-    row1_body<DT, XT, P, 2, M, true>(wg, y, ldy, bg, n, (int64_t)blockIdx.x, k, x, ldx, m, yt, wu, bu);
+                                                                 void *__restrict__ y, int64_t ldy, int yt, const float *__restrict__ gw,
+                                                                 float eps) {
+    row1_body<DT, XT, P, 2, M, true, NORM>(wg, y, ldy, bg, n, (int64_t)blockIdx.x, k, x, ldx, m, yt, wu, bu, gw, eps);
 }
 
 // weights of two formats that share an input (q, k Q4_K and v Q6_K of a Q4_K_M file) in one launch: the workgroup's weight
 // decides which body runs
-template <int DTA, int DTB, int XT, int P, int M, int MAXT>
+template <int DTA, int DTB, int XT, int P, int M, int MAXT, bool NORM = false>
 __global__ void __launch_bounds__(MAXT) gemv_row1_mixed_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int64_t ldx, int m,
-                                                                int yt) {
+                                                                int yt, const float *__restrict__ gw, float eps) {
     const Row1Pick p = row1_pick(a, (int)blockIdx.x);
     const int64_t rtb = (int64_t)((int)blockIdx.x - p.first);
-    if (p.index < a.second) row1_body<DTA, XT, P, 1, M>(p.w, p.y, p.ldy, p.bias, p.n, rtb, k, x, ldx, m, yt);
-    else row1_body<DTB, XT, P, 1, M>(p.w, p.y, p.ldy, p.bias, p.n, rtb, k, x, ldx, m, yt);
+    if (p.index < a.second) row1_body<DTA, XT, P, 1, M, false, NORM>(p.w, p.y, p.ldy, p.bias, p.n, rtb, k, x, ldx, m, yt, nullptr, nullptr, gw, eps);
+    else row1_body<DTB, XT, P, 1, M, false, NORM>(p.w, p.y, p.ldy, p.bias, p.n, rtb, k, x, ldx, m, yt, nullptr, nullptr, gw, eps);
 }
 
 struct Row1Launch {
@@ -591,28 +648,38 @@ struct Row1Launch {
     int m, yt, nwaves, rtiles;
     hipStream_t s;
     hipEvent_t ev0, ev1;
+    const float *gw;  // RmsNorm weight (null: the activations are taken as they are) and eps
+    float eps;
 };
 
 template <int DT, int P, int R, int M> size_t row1_lds(int nwaves) {
     const size_t tile = (Row1Fmt<DT>::kPacked && M > 1) ? (size_t)(M / 2) * kPairRegion : (size_t)M * kRegion;
-    return (size_t)nwaves * P * tile + (size_t)nwaves * R * M * 64 * sizeof(float);
+    return (size_t)nwaves * P * tile + (size_t)nwaves * R * M * 64 * sizeof(float) + 64;  // (+ a sum of squares per wave)
 }
 
-template <int DT, int XT, int P, int R, int M>
-hipError_t launch_final(const Row1Launch &l) {
+template <int DT, int XT, int P, int R, int M, bool NORM>
+hipError_t launch_final_n(const Row1Launch &l) {
     const size_t lds = row1_lds<DT, P, R, M>(l.nwaves);
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
     if (lds > (64u << 10)) {  // 16 waves x two tiles in flight x two pairs of rows: 94 KiB
-        const hipError_t raised = turq_raise_lds_limit((const void *)gemv_row1_kernel<DT, XT, P, R, M, 1024>, 128 << 10);
+        const hipError_t raised = turq_raise_lds_limit((const void *)gemv_row1_kernel<DT, XT, P, R, M, 1024, NORM>, 128 << 10);
         if (raised != hipSuccess) return raised;
     }
     if (l.ev0) {
-        hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, R, M, 1024>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k, l.x,
-                              l.ldx, l.m, l.yt);
+        hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, R, M, 1024, NORM>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k,
+                              l.x, l.ldx, l.m, l.yt, l.gw, l.eps);
         return hipGetLastError();
     }
-    gemv_row1_kernel<DT, XT, P, R, M, 1024><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
+    gemv_row1_kernel<DT, XT, P, R, M, 1024, NORM><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt, l.gw, l.eps);
     return hipGetLastError();
+}
+template <int DT, int XT, int P, int R, int M>
+hipError_t launch_final(const Row1Launch &l) {
+    if constexpr (M == 1) {
+        if (l.gw) return launch_final_n<DT, XT, P, R, M, true>(l);
+    }
+    if (l.gw) return hipErrorInvalidValue;  // (the norm inside the kernel: one activation row)
+    return launch_final_n<DT, XT, P, R, M, false>(l);
 }
 
 // column tiles in flight per wave: up to three for one activation row (four do not fit the registers of every format), up to
@@ -652,17 +719,25 @@ hipError_t launch_x(int xt, const Row1Launch &l) {
     }
 }
 
-template <int DTA, int DTB, int XT, int P, int M>
-hipError_t launch_mixed_final(const Row1Launch &l) {
+template <int DTA, int DTB, int XT, int P, int M, bool NORM>
+hipError_t launch_mixed_final_n(const Row1Launch &l) {
     const size_t lds = std::max(row1_lds<DTA, P, 1, M>(l.nwaves), row1_lds<DTB, P, 1, M>(l.nwaves));
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
     if (l.ev0) {
-        hipExtLaunchKernelGGL((gemv_row1_mixed_kernel<DTA, DTB, XT, P, M, 1024>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a,
-                              l.k, l.x, l.ldx, l.m, l.yt);
+        hipExtLaunchKernelGGL((gemv_row1_mixed_kernel<DTA, DTB, XT, P, M, 1024, NORM>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0,
+                              l.a, l.k, l.x, l.ldx, l.m, l.yt, l.gw, l.eps);
         return hipGetLastError();
     }
-    gemv_row1_mixed_kernel<DTA, DTB, XT, P, M, 1024><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt);
+    gemv_row1_mixed_kernel<DTA, DTB, XT, P, M, 1024, NORM><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt, l.gw, l.eps);
     return hipGetLastError();
+}
+template <int DTA, int DTB, int XT, int P, int M>
+hipError_t launch_mixed_final(const Row1Launch &l) {
+    if constexpr (M == 1) {
+        if (l.gw) return launch_mixed_final_n<DTA, DTB, XT, P, M, true>(l);
+    }
+    if (l.gw) return hipErrorInvalidValue;
+    return launch_mixed_final_n<DTA, DTB, XT, P, M, false>(l);
 }
 
 template <int DTA, int DTB, int XT>
@@ -714,16 +789,17 @@ int turq_gemv_row1_rows(int dtype) {
 // aligned); results to y[i] with row stride ldy[i] (null: n[i]); row_tiles (1 or 2; 2 with one activation row only) per workgroup.
 hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w, const int64_t *n, int64_t k, const void *x, int x_dtype,
                                  int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy, const float *const *bias,
-                                 int nwaves, int row_tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+                                 int nwaves, int row_tiles, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop, const float *norm_weight,
+                                 float norm_eps) {
     if (count < 1 || count > kMaxRow1 || nwaves < 1 || nwaves > 16 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
     if (m < 1 || m > TURQ_ROW1_MAX_M || (row_tiles != 1 && !(row_tiles == 2 && m == 1))) return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     Row1Launch l{};
     if (!row1_args(l, count, w, n, y, ldy, bias, row_tiles)) return hipErrorInvalidValue;
     if (l.blocks == 0) return hipSuccess;
     if (k == 0) return hipErrorInvalidValue;
     l.k = k, l.x = x, l.ldx = ldx, l.m = (int)m, l.yt = y_dtype, l.nwaves = nwaves, l.rtiles = row_tiles;
-    l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop;
+    l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop, l.gw = norm_weight, l.eps = norm_eps;
     switch (dtype) {
     case TURQ_Q4_K: return launch_x<TURQ_Q4_K>(x_dtype, l);
     case TURQ_Q5_K: return launch_x<TURQ_Q5_K>(x_dtype, l);
@@ -743,18 +819,18 @@ bool turq_gemv_row1_mixed_supports(int dtype_a, int dtype_b) {
 hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w, const int64_t *n,
                                        int64_t k, const void *x, int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype,
                                        const int64_t *ldy, const float *const *bias, int nwaves, hipStream_t stream,
-                                       hipEvent_t ev_start, hipEvent_t ev_stop) {
+                                       hipEvent_t ev_start, hipEvent_t ev_stop, const float *norm_weight, float norm_eps) {
     if (!turq_gemv_row1_mixed_supports(dtype_a, dtype_b) || count < 2 || count > kMaxRow1 || second < 1 || second >= count ||
         nwaves < 1 || nwaves > 16 || k % 256 != 0 || m < 1 || m > TURQ_ROW1_MAX_M)
         return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     Row1Launch l{};
     if (!row1_args(l, count, w, n, y, ldy, bias, 1)) return hipErrorInvalidValue;
     l.a.second = second;
     if (l.blocks == 0) return hipSuccess;
     if (k == 0) return hipErrorInvalidValue;
     l.k = k, l.x = x, l.ldx = ldx, l.m = (int)m, l.yt = y_dtype, l.nwaves = nwaves, l.rtiles = 1;
-    l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop;
+    l.s = stream, l.ev0 = ev_start, l.ev1 = ev_stop, l.gw = norm_weight, l.eps = norm_eps;
     if (dtype_a == TURQ_Q5_K) {
         switch (x_dtype) {
         case TURQ_ACT_F32: return launch_mixed_p<TURQ_Q5_K, TURQ_Q6_K, TURQ_ACT_F32>(l);
@@ -772,61 +848,74 @@ hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int 
 }
 
 namespace {
-template <int DT, int XT, int P, int M>
-hipError_t launch_gateup_final(const void *wg, const void *wu, const float *bg, const float *bu, int64_t n, int64_t k, const void *x,
-                               int64_t ldx, int m, void *y, int64_t ldy, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
-                               hipEvent_t ev1) {
-    const size_t lds = row1_lds<DT, P, 2, M>(nwaves);
-    const dim3 grid((unsigned)turq_tile_rows(n)), block((unsigned)(64 * nwaves));
-    if (ev0) {
-        hipExtLaunchKernelGGL((gemv_row1_gateup_kernel<DT, XT, P, M, 1024>), grid, block, (unsigned)lds, s, ev0, ev1, 0,
-                              (const uint8_t *)wg, (const uint8_t *)wu, bg, bu, n, k, x, ldx, m, y, ldy, yt);
+struct GateUpLaunch {
+    const void *wg, *wu;
+    const float *bg, *bu;
+    int64_t n, k;
+    const void *x;
+    int64_t ldx;
+    int m;
+    void *y;
+    int64_t ldy;
+    int yt, nwaves;
+    hipStream_t s;
+    hipEvent_t ev0, ev1;
+    const float *gw;  // RmsNorm weight (null: none) and eps
+    float eps;
+};
+
+template <int DT, int XT, int P, int M, bool NORM>
+hipError_t launch_gateup_final(const GateUpLaunch &l) {
+    const size_t lds = row1_lds<DT, P, 2, M>(l.nwaves);
+    const dim3 grid((unsigned)turq_tile_rows(l.n)), block((unsigned)(64 * l.nwaves));
+    if (l.ev0) {
+        hipExtLaunchKernelGGL((gemv_row1_gateup_kernel<DT, XT, P, M, 1024, NORM>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0,
+                              (const uint8_t *)l.wg, (const uint8_t *)l.wu, l.bg, l.bu, l.n, l.k, l.x, l.ldx, l.m, l.y, l.ldy, l.yt, l.gw, l.eps);
         return hipGetLastError();
     }
-    gemv_row1_gateup_kernel<DT, XT, P, M, 1024><<<grid, block, lds, s>>>((const uint8_t *)wg, (const uint8_t *)wu, bg, bu, n, k, x, ldx,
-                                                                          m, y, ldy, yt);
+    gemv_row1_gateup_kernel<DT, XT, P, M, 1024, NORM><<<grid, block, lds, l.s>>>((const uint8_t *)l.wg, (const uint8_t *)l.wu, l.bg, l.bu, l.n,
+                                                                                l.k, l.x, l.ldx, l.m, l.y, l.ldy, l.yt, l.gw, l.eps);
     return hipGetLastError();
 }
 
 template <int DT, int XT>
-hipError_t launch_gateup_p(const void *wg, const void *wu, const float *bg, const float *bu, int64_t n, int64_t k, const void *x,
-                           int64_t ldx, int m, void *y, int64_t ldy, int yt, int nwaves, hipStream_t s, hipEvent_t ev0, hipEvent_t ev1) {
+hipError_t launch_gateup_p(const GateUpLaunch &l) {
     // two weights double what a wave holds per column tile: at most two column tiles in flight
-    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
-    if (m == 2) {
-        if (per_wave <= 1) return launch_gateup_final<DT, XT, 1, 2>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
-        return launch_gateup_final<DT, XT, 2, 2>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    const int64_t per_wave = (turq_tile_cols(l.k) + l.nwaves - 1) / l.nwaves;
+    if (l.m == 2) {
+        if (l.gw) return hipErrorInvalidValue;  // (the norm inside the kernel: one activation row)
+        return per_wave <= 1 ? launch_gateup_final<DT, XT, 1, 2, false>(l) : launch_gateup_final<DT, XT, 2, 2, false>(l);
     }
-    if (per_wave <= 1) return launch_gateup_final<DT, XT, 1, 1>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
-    return launch_gateup_final<DT, XT, 2, 1>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    if (l.gw) return per_wave <= 1 ? launch_gateup_final<DT, XT, 1, 1, true>(l) : launch_gateup_final<DT, XT, 2, 1, true>(l);
+    return per_wave <= 1 ? launch_gateup_final<DT, XT, 1, 1, false>(l) : launch_gateup_final<DT, XT, 2, 1, false>(l);
 }
 
 template <int DT>
-hipError_t launch_gateup_x(int xt, const void *wg, const void *wu, const float *bg, const float *bu, int64_t n, int64_t k,
-                           const void *x, int64_t ldx, int m, void *y, int64_t ldy, int yt, int nwaves, hipStream_t s, hipEvent_t ev0,
-                           hipEvent_t ev1) {
+hipError_t launch_gateup_x(int xt, const GateUpLaunch &l) {
     switch (xt) {
-    case TURQ_ACT_F32: return launch_gateup_p<DT, TURQ_ACT_F32>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
-    case TURQ_ACT_BF16: return launch_gateup_p<DT, TURQ_ACT_BF16>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
-    case TURQ_ACT_F16: return launch_gateup_p<DT, TURQ_ACT_F16>(wg, wu, bg, bu, n, k, x, ldx, m, y, ldy, yt, nwaves, s, ev0, ev1);
+    case TURQ_ACT_F32: return launch_gateup_p<DT, TURQ_ACT_F32>(l);
+    case TURQ_ACT_BF16: return launch_gateup_p<DT, TURQ_ACT_BF16>(l);
+    case TURQ_ACT_F16: return launch_gateup_p<DT, TURQ_ACT_F16>(l);
     default: return hipErrorInvalidValue;
     }
 }
 }  // namespace
 
 // y[mm][c] = silu(x[mm] . gate[c] + bias_gate[c]) * (x[mm] . up[c] + bias_up[c]) for m = 1 or 2 activation rows: gate and up are
-// two tiled weights of one format and one shape [n, k]; rows of x 16-byte aligned
+// two tiled weights of one format and one shape [n, k]; rows of x 16-byte aligned.  norm_weight (m = 1): x stands for RmsNorm(x)
 hipError_t turq_launch_gemv_row1_gateup(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x,
                                         int x_dtype, int64_t ldx, int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate,
-                                        const float *bias_up, int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop) {
+                                        const float *bias_up, int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop,
+                                        const float *norm_weight, float norm_eps) {
     if (nwaves < 1 || nwaves > 16 || m < 1 || m > 2 || k <= 0 || k % turq_dt_block_elems(dtype) != 0) return hipErrorInvalidValue;
-    if (y_dtype != TURQ_ACT_F32 && y_dtype != TURQ_ACT_BF16 && y_dtype != TURQ_ACT_F16) return hipErrorInvalidValue;
+    if (!turq_yt_ok(y_dtype, true)) return hipErrorInvalidValue;
     if (n == 0) return hipSuccess;
+    const GateUpLaunch l{w_gate, w_up, bias_gate, bias_up, n, k, x, ldx, (int)m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop, norm_weight, norm_eps};
     switch (dtype) {
-    case TURQ_Q4_K: return launch_gateup_x<TURQ_Q4_K>(x_dtype, w_gate, w_up, bias_gate, bias_up, n, k, x, ldx, (int)m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
-    case TURQ_Q5_K: return launch_gateup_x<TURQ_Q5_K>(x_dtype, w_gate, w_up, bias_gate, bias_up, n, k, x, ldx, (int)m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
-    case TURQ_Q6_K: return launch_gateup_x<TURQ_Q6_K>(x_dtype, w_gate, w_up, bias_gate, bias_up, n, k, x, ldx, (int)m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
-    case TURQ_Q8_0: return launch_gateup_x<TURQ_Q8_0>(x_dtype, w_gate, w_up, bias_gate, bias_up, n, k, x, ldx, (int)m, y, ldy, y_dtype, nwaves, stream, ev_start, ev_stop);
+    case TURQ_Q4_K: return launch_gateup_x<TURQ_Q4_K>(x_dtype, l);
+    case TURQ_Q5_K: return launch_gateup_x<TURQ_Q5_K>(x_dtype, l);
+    case TURQ_Q6_K: return launch_gateup_x<TURQ_Q6_K>(x_dtype, l);
+    case TURQ_Q8_0: return launch_gateup_x<TURQ_Q8_0>(x_dtype, l);
     default: return hipErrorInvalidValue;
     }
 }

@@ -40,7 +40,7 @@ template <int DT, int XT, int YT>
 __global__ void __launch_bounds__(256) gemv_simple_kernel(const uint8_t *__restrict__ w, int64_t n, int64_t k,
                                                           int64_t row_bytes, const void *__restrict__ x, int64_t m,
                                                           int64_t ldx, void *__restrict__ y, int64_t ldy,
-                                                          const float *__restrict__ bias) {
+                                                          const float *__restrict__ bias, int accum) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= n) return;  // uniform per wave
@@ -87,27 +87,28 @@ __global__ void __launch_bounds__(256) gemv_simple_kernel(const uint8_t *__restr
             float v = acc[i];
 #pragma unroll
             for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
-            if (lane == 0 && m0 + i < m) store_out<YT>(y, (m0 + i) * ldy + row, v + b);
+            if (lane == 0 && m0 + i < m) store_out<YT>(y, (m0 + i) * ldy + row, v + b + (accum ? turq_load_out<YT>(y, (m0 + i) * ldy + row) : 0.0f));
         }
     }
 }
 
 template <int DT, int XT, int YT>
 hipError_t launch3(const void *w, int64_t n, int64_t k, const void *x, int64_t m, int64_t ldx, void *y, int64_t ldy,
-                   const float *bias, hipStream_t s) {
+                   const float *bias, hipStream_t s, int accum) {
     const int64_t row_bytes = k / turq_dt_block_elems(DT) * turq_dt_block_bytes(DT);
     const unsigned grid = (unsigned)((n + 3) / 4);
-    gemv_simple_kernel<DT, XT, YT><<<grid, 256, 0, s>>>((const uint8_t *)w, n, k, row_bytes, x, m, ldx, y, ldy, bias);
+    gemv_simple_kernel<DT, XT, YT><<<grid, 256, 0, s>>>((const uint8_t *)w, n, k, row_bytes, x, m, ldx, y, ldy, bias, accum);
     return hipGetLastError();
 }
 
 template <int DT, int XT>
 hipError_t launch2(int yt, const void *w, int64_t n, int64_t k, const void *x, int64_t m, int64_t ldx, void *y,
                    int64_t ldy, const float *bias, hipStream_t s) {
-    switch (yt) {
-    case TURQ_ACT_F32: return launch3<DT, XT, TURQ_ACT_F32>(w, n, k, x, m, ldx, y, ldy, bias, s);
-    case TURQ_ACT_BF16: return launch3<DT, XT, TURQ_ACT_BF16>(w, n, k, x, m, ldx, y, ldy, bias, s);
-    case TURQ_ACT_F16: return launch3<DT, XT, TURQ_ACT_F16>(w, n, k, x, m, ldx, y, ldy, bias, s);
+    const int accum = (yt & TURQ_OUT_ACCUMULATE) != 0;
+    switch (yt & 0xFF) {
+    case TURQ_ACT_F32: return launch3<DT, XT, TURQ_ACT_F32>(w, n, k, x, m, ldx, y, ldy, bias, s, accum);
+    case TURQ_ACT_BF16: return launch3<DT, XT, TURQ_ACT_BF16>(w, n, k, x, m, ldx, y, ldy, bias, s, accum);
+    case TURQ_ACT_F16: return launch3<DT, XT, TURQ_ACT_F16>(w, n, k, x, m, ldx, y, ldy, bias, s, accum);
     default: return hipErrorInvalidValue;
     }
 }

@@ -22,11 +22,6 @@ __device__ inline float h2f_bits(uint32_t bits16) {
 }
 
 // ---- weight registers of one tile (everything a lane loads from HBM for it) ----
-__device__ inline void turq_store_any(void *y, int yt, int64_t i, float v) {
-    if (yt == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, i, v);
-    else if (yt == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, i, v);
-    else turq_store_out<TURQ_ACT_F16>(y, i, v);
-}
 
 template <int DT> struct WRegs;
 template <> struct WRegs<TURQ_Q4_K> { uint4v qa, qb, hd; };

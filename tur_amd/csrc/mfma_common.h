@@ -178,6 +178,42 @@ template <int YT> __device__ inline void turq_store_out_raw(void *y, int64_t i, 
         ((uint16_t *)y)[i] = b;
     }
 }
+template <int YT> __device__ inline float turq_load_out(const void *y, int64_t i) {
+    if (YT == TURQ_ACT_F32) return ((const float *)y)[i];
+    if (YT == TURQ_ACT_BF16) return __uint_as_float((uint32_t)((const uint16_t *)y)[i] << 16);
+    const uint16_t b = ((const uint16_t *)y)[i];
+    _Float16 h;
+    __builtin_memcpy(&h, &b, 2);
+    return (float)h;
+}
+// the store of a result element whose type is only known at run time; with TURQ_OUT_ACCUMULATE in yt the value is added to
+// what y holds (the residual stream), in f32, and rounded once
+__device__ inline void turq_store_any(void *y, int yt, int64_t i, float v) {
+    const int base = yt & 0xFF;
+    if (yt & TURQ_OUT_ACCUMULATE)
+        v += base == TURQ_ACT_F32 ? turq_load_out<TURQ_ACT_F32>(y, i) : base == TURQ_ACT_BF16 ? turq_load_out<TURQ_ACT_BF16>(y, i) : turq_load_out<TURQ_ACT_F16>(y, i);
+    if (base == TURQ_ACT_F32) turq_store_out<TURQ_ACT_F32>(y, i, v);
+    else if (base == TURQ_ACT_BF16) turq_store_out<TURQ_ACT_BF16>(y, i, v);
+    else turq_store_out<TURQ_ACT_F16>(y, i, v);
+}
+// four rows of one column, y[(row0 + i) * ldy + col] = v[i] for the rows below m: with TURQ_OUT_ACCUMULATE the four values that
+// y holds are requested together and ahead of the stores (one round trip at the end of the kernel instead of four: the compiler
+// cannot move a load of y across a store to y)
+__device__ inline void turq_store_col4(void *y, int yt, int64_t row0, int64_t m, int64_t ldy, int64_t col, float4v v) {
+    const int base = yt & 0xFF;
+    float old[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (yt & TURQ_OUT_ACCUMULATE) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (row0 + i < m) {
+                const int64_t at = (row0 + i) * ldy + col;
+                old[i] = base == TURQ_ACT_F32 ? turq_load_out<TURQ_ACT_F32>(y, at) : base == TURQ_ACT_BF16 ? turq_load_out<TURQ_ACT_BF16>(y, at) : turq_load_out<TURQ_ACT_F16>(y, at);
+            }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+        if (row0 + i < m) turq_store_any(y, base, (row0 + i) * ldy + col, v[i] + old[i]);
+}
 #endif
 
 // bytes of the prefill GEMM's fragment buffer (32-row m-tiles, 17 steps of 1 KiB per column tile)
@@ -188,6 +224,8 @@ __host__ __device__ inline size_t turq_act_prep32_bytes(int64_t m, int64_t k) {
 // launchers (act_prep.hip, gemv_mfma.hip)
 hipError_t turq_launch_act_prep32(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
                                   hipStream_t stream);
+hipError_t turq_launch_rms_norm_prep32(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, const float *weight,
+                                       float eps, void *frags, hipStream_t stream);
 hipError_t turq_launch_silu_mul_prep32(int dtype, const float *gate, const float *up, int64_t m, int64_t n, void *frags,
                                        hipStream_t stream);
 hipError_t turq_launch_act_prep(int dtype, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, void *frags,
@@ -226,11 +264,12 @@ inline hipError_t turq_raise_lds_limit(const void *kernel, int bytes) {
 bool turq_gemv_row1_supports(int dtype);
 hipError_t turq_launch_gemv_row1_gateup(int dtype, const void *w_gate, const void *w_up, int64_t n, int64_t k, const void *x,
                                         int x_dtype, int64_t ldx, int64_t m, void *y, int y_dtype, int64_t ldy, const float *bias_gate,
-                                        const float *bias_up, int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
+                                        const float *bias_up, int nwaves, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop,
+                                        const float *norm_weight = nullptr, float norm_eps = 0.0f);
 hipError_t turq_launch_gemv_row1(int dtype, int count, const void *const *w_tiled, const int64_t *n, int64_t k, const void *x,
                                  int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy,
                                  const float *const *bias, int waves_per_group, int row_tiles_per_group, hipStream_t stream,
-                                 hipEvent_t ev_start, hipEvent_t ev_stop);
+                                 hipEvent_t ev_start, hipEvent_t ev_stop, const float *norm_weight = nullptr, float norm_eps = 0.0f);
 bool turq_gemv_cs_rows_ok(int row_tiles_per_group);
 hipError_t turq_launch_gemv_cs(int dtype, int count, const void *const *w_tiled, const int64_t *n, int64_t k, const void *x, int x_dtype,
                                int64_t ldx, int64_t m, void *const *y, int y_dtype, const int64_t *ldy, const float *const *bias,
@@ -255,7 +294,7 @@ bool turq_gemv_row1_mixed_supports(int dtype_a, int dtype_b);
 hipError_t turq_launch_gemv_row1_mixed(int dtype_a, int dtype_b, int count, int second, const void *const *w_tiled, const int64_t *n,
                                        int64_t k, const void *x, int x_dtype, int64_t ldx, int64_t m, void *const *y, int y_dtype,
                                        const int64_t *ldy, const float *const *bias, int waves_per_group, hipStream_t stream,
-                                       hipEvent_t ev_start, hipEvent_t ev_stop);
+                                       hipEvent_t ev_start, hipEvent_t ev_stop, const float *norm_weight = nullptr, float norm_eps = 0.0f);
 // split_counters, split_partials (may be null: no launch splits its columns): TURQ_GEMM_SPLIT_COUNTER_BYTES of counters that were
 // zero before the first launch that used them (every launch leaves them at zero), and turq_gemm_split_scratch(...) bytes for the
 // partial tiles; launches that share either must not overlap

@@ -223,10 +223,11 @@ static int64_t gemm_cus_taken(const turq_ctx *ctx, const turq_weight *w, int64_t
 }
 
 int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m, int64_t ldx,
-                            void *const *y, int yt, const int64_t *ldy, const float *const *bias, bool *taken) {
+                            void *const *y, int yt, const int64_t *ldy, const float *const *bias, bool *taken, const TurqNorm *norm) {
     *taken = false;
     float ws[16];
     if (count > 16) return TURQ_OK;
+    if (norm && (w[0]->k % 256 != 0 || w[0]->k > 16384)) return TURQ_OK;  // (the kernel that writes normalised fragments)
     for (int i = 0; i < count; i++)
         if (!gemm_takes(w[i], &ws[i])) return TURQ_OK;
     int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep32_bytes(m, w[0]->k));
@@ -258,7 +259,8 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
     for (int i = 0; i < count && e == hipSuccess; i++) {
         const int order = w[i]->dtype == TURQ_Q8_0 ? 2 : 1;
         if (order != prepared) {
-            e = turq_launch_act_prep32(w[i]->dtype, x, xt, m, w[i]->k, ldx, ctx->act_prep, ctx->stream);
+            e = norm ? turq_launch_rms_norm_prep32(w[i]->dtype, x, xt, m, w[i]->k, ldx, norm->w, norm->eps, ctx->act_prep, ctx->stream)
+                     : turq_launch_act_prep32(w[i]->dtype, x, xt, m, w[i]->k, ldx, ctx->act_prep, ctx->stream);
             if (e != hipSuccess) break;
             prepared = order;
         }
@@ -332,6 +334,28 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
     return TURQ_OK;
 }
 
+bool turq_norm_fuses(const turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t ldx, int64_t m) {
+    static const bool off = [] { const char *e = getenv("TURQ_NORM_FUSED"); return e && atoi(e) == 0; }();
+    static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
+    if (off || count < 1 || ctx->wide || ctx->fixed_scratch || !turq_act_bytes(xt)) return false;
+    float ws = 1.0f;
+    for (int i = 0; i < count; i++)
+        if (!w[i] || w[i]->device != ctx->device || !turq_dt_is_quant(w[i]->dtype) || w[i]->layout != TURQ_LAYOUT_TILED || w[i]->k != w[0]->k ||
+            w[i]->k <= 0 || w[i]->n <= 0)
+            return false;
+    const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
+    if (m == 1) {  // the one-row kernels (every quantized format has one), on rows they can load 16 bytes at a time
+        for (int i = 0; i < count; i++)
+            if (!use_row1(w[i]->dtype)) return false;
+        return aligned && !no_fuse;
+    }
+    if (m <= TURQ_GEMV_MAX_M) return false;
+    if (w[0]->k % 256 != 0 || w[0]->k > 16384 || turq_rows_in_chunks(ctx, count, w, x, xt, ldx, m)) return false;
+    for (int i = 0; i < count; i++)
+        if (!gemm_takes(w[i], &ws)) return false;
+    return true;
+}
+
 // the prefill GEMM of one weight on fragments that already sit in ctx->act_prep
 static int gemm_on_frags(turq_ctx *ctx, const turq_weight *w, int64_t m, void *y, int yt, int64_t ldy, const float *bias, float wscale) {
     GemmSplit sp;
@@ -350,7 +374,7 @@ static int gemm_on_frags(turq_ctx *ctx, const turq_weight *w, int64_t m, void *y
 // which saves a launch and a round trip of the intermediate per MLP.
 int turq_mlp_prefill(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt,
                      int64_t m, int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up,
-                     const float *bias_down, bool *taken) {
+                     const float *bias_down, bool *taken, const TurqNorm *norm) {
     *taken = false;
     static const bool off = [] { const char *e = getenv("TURQ_MLP_PREFILL"); return e && atoi(e) == 0; }();
     const turq_weight *gu[2] = {gate, up};
@@ -372,7 +396,7 @@ int turq_mlp_prefill(turq_ctx *ctx, const turq_weight *gate, const turq_weight *
     const int64_t ldys[2] = {n_ff, n_ff};
     const float *biases[2] = {bias_gate, bias_up};
     bool gu_taken = false;
-    rc = turq_qmatmul_multi_gemm(ctx, 2, gu, x, xt, m, ldx, ys, TURQ_ACT_F32, ldys, biases, &gu_taken);
+    rc = turq_qmatmul_multi_gemm(ctx, 2, gu, x, xt, m, ldx, ys, TURQ_ACT_F32, ldys, biases, &gu_taken, norm);
     if (rc != TURQ_OK || !gu_taken) return rc;
     TURQ_HIP(ctx, turq_launch_silu_mul_prep32(down->dtype, (const float *)ys[0], (const float *)ys[1], m, n_ff, ctx->act_prep, ctx->stream));
     rc = gemm_on_frags(ctx, down, m, y, yt, ldy, bias_down, ws_down);
@@ -382,8 +406,10 @@ int turq_mlp_prefill(turq_ctx *ctx, const turq_weight *gate, const turq_weight *
 }
 
 int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y,
-                      int yt, int64_t ldy, const float *bias, int algo) {
+                      int yt, int64_t ldy, const float *bias, int algo, const TurqNorm *norm) {
     const int xb = turq_act_bytes(xt), yb = turq_act_bytes(yt);
+    if (norm && !turq_norm_fuses(ctx, 1, &w, x, xt, ldx, m))
+        return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul: no kernel applies the norm for this call (internal)");
     // prefill chunks: LDS-tiled MFMA GEMM.  Its weights are packed f16 values (base + q) * d * sc (base 1024 for the nibbles of
     // Q4_K / Q5_K, 256 for the 6-bit values of Q6_K; q * d for Q8_0), the scales multiplied by a power of two that puts the
     // largest of them near 2^15 (small scales would otherwise lose bits in the f16 subnormals); a tensor whose largest value
@@ -399,7 +425,8 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
         rc = gemm_split_reserve(ctx, 1, &w, m, &sp);
         if (rc != TURQ_OK) return rc;
         hipEvent_t ev0 = nullptr, ev1 = nullptr;
-        TURQ_HIP(ctx, turq_launch_act_prep32(w->dtype, x, xt, m, w->k, ldx, ctx->act_prep, ctx->stream));
+        if (norm) TURQ_HIP(ctx, turq_launch_rms_norm_prep32(w->dtype, x, xt, m, w->k, ldx, norm->w, norm->eps, ctx->act_prep, ctx->stream));
+        else TURQ_HIP(ctx, turq_launch_act_prep32(w->dtype, x, xt, m, w->k, ldx, ctx->act_prep, ctx->stream));
         TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
         TURQ_HIP(ctx, turq_launch_gemm_mfma(w->dtype, w->dev, w->n, w->k, ctx->act_prep, m, y, yt, ldy, bias, wscale, ctx->compute_units,
                                             ctx->stream, ev0, ev1, sp.counters[0], sp.partials[0], sp.bytes[0]));
@@ -420,7 +447,7 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
             void *yv = yc;
             TURQ_HIP(ctx, turq_launch_gemv_row1(w->dtype, 1, &wp, &w->n, w->k, xc, xt, ldx, mc, &yv, yt, &ldy, bias ? &bias : nullptr,
                                                 pick_waves_row1(w->k), mc == 1 ? pick_rows_row1(ctx, turq_tile_rows(w->n)) : 1,
-                                                ctx->stream, ev0, ev1));
+                                                ctx->stream, ev0, ev1, norm ? norm->w : nullptr, norm ? norm->eps : 0.0f));
             continue;
         }
         if (use_fused(ctx, mc, turq_tile_rows(w->n), w->dev_bytes) && aligned && !no_fuse) {
@@ -462,9 +489,11 @@ bool turq_rows_in_chunks(const turq_ctx *ctx, int count, const turq_weight *cons
 }
 
 int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m,
-                              int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, bool *taken) {
+                              int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, bool *taken,
+                              const TurqNorm *norm) {
     static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
     *taken = false;
+    if (norm && m != 1) return TURQ_OK;  // (the caller normalises into scratch first)
     {
         const turq_weight *pair[2] = {gate, up};
         if (m > TURQ_GEMV_MAX_M && gate->n == up->n && turq_rows_in_chunks(ctx, 2, pair, x, xt, ldx, m) &&
@@ -501,6 +530,7 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
             return TURQ_OK;
         }
     }
+    if (norm && (no_fuse || !aligned || !use_row1(gate->dtype))) return TURQ_OK;
     if (no_fuse || !aligned || m > 2 || !use_row1(gate->dtype) || !row1_takes(m, gate->dev_bytes + up->dev_bytes, gate->dtype)) {
         // up to 32 rows: fragments prepared once, then one launch whose workgroups take row tile b of both weights (the shape
         // of the two-row-tile kernel: at most four waves) and store the product
@@ -523,7 +553,7 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
     int nwaves = pick_waves_row1(gate->k);
     if (!forced) nwaves = (int)std::min<int64_t>({2 * (int64_t)nwaves, 16, turq_tile_cols(gate->k)});
     TURQ_HIP(ctx, turq_launch_gemv_row1_gateup(gate->dtype, gate->dev, up->dev, gate->n, gate->k, x, xt, ldx, m, y, yt, ldy, bias_gate,
-                                               bias_up, nwaves, ctx->stream, ev0, ev1));
+                                               bias_up, nwaves, ctx->stream, ev0, ev1, norm ? norm->w : nullptr, norm ? norm->eps : 0.0f));
     *taken = true;
     return TURQ_OK;
 }
@@ -533,8 +563,10 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
 // TURQ_GEMV_FUSED_MAX_M rows with 16-byte aligned activation rows the kernel converts the activations itself; otherwise
 // the activation fragments are prepared once per fragment order (K-quants / Q8_0) and shared by all the weights.
 int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m,
-                            int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias) {
+                            int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias, const TurqNorm *norm) {
     static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
+    if (norm && !(m == 1 && turq_norm_fuses(ctx, count, w, x, xt, ldx, m)))
+        return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_multi: no kernel applies the norm for this call (internal)");
     const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
     int64_t all_tiles = 0;
     size_t all_bytes = 0;
@@ -599,7 +631,7 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
                 TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
                 TURQ_HIP(ctx, turq_launch_gemv_row1_mixed(w[i]->dtype, w[j]->dtype, j2 - i, j - i, wp, nn, w[i]->k, x, xt, ldx, m, y + i,
                                                           yt, ldy + i, bias ? bias + i : nullptr, pick_waves_row1(w[i]->k), ctx->stream,
-                                                          ev0, ev1));
+                                                          ev0, ev1, norm ? norm->w : nullptr, norm ? norm->eps : 0.0f));
                 i = j2;
                 continue;
             }
@@ -639,7 +671,8 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
             TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
             TURQ_HIP(ctx, turq_launch_gemv_row1(w[i]->dtype, j - i, wp, nn, w[i]->k, x, xt, ldx, m, y + i, yt, ldy + i,
                                                 bias ? bias + i : nullptr, pick_waves_row1(w[i]->k),
-                                                m == 1 ? pick_rows_row1(ctx, turq_tile_rows(rows)) : 1, ctx->stream, ev0, ev1));
+                                                m == 1 ? pick_rows_row1(ctx, turq_tile_rows(rows)) : 1, ctx->stream, ev0, ev1,
+                                                norm ? norm->w : nullptr, norm ? norm->eps : 0.0f));
             i = j;
             continue;
         }

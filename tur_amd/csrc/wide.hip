@@ -52,12 +52,15 @@ __global__ void __launch_bounds__(256) wide_scale_kernel(const void *__restrict_
 // y[r][c] = y32[r][c] * inv[r] + bias[c]
 template <int YT>
 __global__ void __launch_bounds__(256) wide_rescale_kernel(const float *__restrict__ y32, int64_t ld32, int64_t n, const float *__restrict__ inv,
-                                                           const float *__restrict__ bias, void *__restrict__ y, int64_t ldy) {
-    const int64_t row = blockIdx.y;
+                                                           const float *__restrict__ bias, void *__restrict__ y, int64_t ldy, int64_t m,
+                                                           int accum) {
     const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (c >= n) return;
-    const float v = y32[row * ld32 + c] * inv[row] + (bias ? bias[c] : 0.0f);
-    turq_store_out<YT>(y, row * ldy + c, v);
+    const float b = bias ? bias[c] : 0.0f;
+    for (int64_t row = blockIdx.y; row < m; row += gridDim.y) {  // (a grid has at most 65535 rows of workgroups)
+        const float v = y32[row * ld32 + c] * inv[row] + b + (accum ? turq_load_out<YT>(y, row * ldy + c) : 0.0f);
+        turq_store_out<YT>(y, row * ldy + c, v);
+    }
 }
 
 }  // namespace
@@ -74,12 +77,12 @@ hipError_t turq_launch_wide_scale(const void *x, int x_dtype, int64_t m, int64_t
 hipError_t turq_launch_wide_rescale(const float *y32, int64_t ld32, int64_t m, int64_t n, const float *inv, const float *bias, void *y,
                                     int y_dtype, int64_t ldy, hipStream_t stream) {
     if (m == 0 || n == 0) return hipSuccess;
-    if (m > 65535) return hipErrorInvalidValue;
-    const dim3 grid((unsigned)((n + 255) / 256), (unsigned)m);
-    switch (y_dtype) {
-    case TURQ_ACT_F32: wide_rescale_kernel<TURQ_ACT_F32><<<grid, 256, 0, stream>>>(y32, ld32, n, inv, bias, y, ldy); break;
-    case TURQ_ACT_BF16: wide_rescale_kernel<TURQ_ACT_BF16><<<grid, 256, 0, stream>>>(y32, ld32, n, inv, bias, y, ldy); break;
-    case TURQ_ACT_F16: wide_rescale_kernel<TURQ_ACT_F16><<<grid, 256, 0, stream>>>(y32, ld32, n, inv, bias, y, ldy); break;
+    const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(m < 65535 ? m : 65535));
+    const int accum = (y_dtype & TURQ_OUT_ACCUMULATE) != 0;
+    switch (y_dtype & 0xFF) {
+    case TURQ_ACT_F32: wide_rescale_kernel<TURQ_ACT_F32><<<grid, 256, 0, stream>>>(y32, ld32, n, inv, bias, y, ldy, m, accum); break;
+    case TURQ_ACT_BF16: wide_rescale_kernel<TURQ_ACT_BF16><<<grid, 256, 0, stream>>>(y32, ld32, n, inv, bias, y, ldy, m, accum); break;
+    case TURQ_ACT_F16: wide_rescale_kernel<TURQ_ACT_F16><<<grid, 256, 0, stream>>>(y32, ld32, n, inv, bias, y, ldy, m, accum); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
