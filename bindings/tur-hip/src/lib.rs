@@ -10,13 +10,16 @@
 //!
 //! Errors are `candle_core::Error::Msg` with the text of `turq_last_error`, so they surface as `TurError::CandleError`
 //! (src/shared/errors.rs:5-6); nothing here unwraps, expects or panics (the project's lints deny them, Cargo.toml:80-86).
-//! Threading: a `HipDevice` is one context = one stream; calls on it must be serialised by the owner, as tur does by owning the
-//! model on one worker thread (src/server/worker.rs:69-100).  Weights are immutable after upload and reference counted.
+//! Threading: a `HipDevice` is one context = one stream, and libturq contexts are thread-compatible, not thread-safe (a call may
+//! grow or swap the context's scratch buffers under another call's feet).  The context therefore sits behind a `Mutex`: clones
+//! of a `HipDevice` may live on several threads, as candle's `Device` may, and every call holds the lock for its duration.  tur
+//! itself drives a model from one worker thread (src/server/worker.rs:69-100), so the lock is uncontended there.  Weights are
+//! immutable after upload and reference counted.
 
 use std::ffi::{CStr, CString};
 use std::os::raw::{c_int, c_void};
 use std::ptr;
-use std::sync::Arc;
+use std::sync::{Arc, Mutex, MutexGuard};
 
 use candle_core::{Device, Error, Result, Tensor};
 use turq_sys::*;
@@ -36,9 +39,9 @@ fn check(ctx: *const turq_ctx, rc: c_int) -> Result<()> {
 }
 
 struct Ctx(*mut turq_ctx);
-// SAFETY: a context may be created on one thread and used on another; callers serialise calls on it (see the module comment)
+// SAFETY: a context may be created on one thread and used on another, one thread at a time: it is only reachable through the
+// Mutex of HipDevice (Send, deliberately NOT Sync: nothing in libturq locks a context)
 unsafe impl Send for Ctx {}
-unsafe impl Sync for Ctx {}
 impl Drop for Ctx {
     fn drop(&mut self) {
         // SAFETY: the pointer came from turq_ctx_create and is dropped once
@@ -46,9 +49,9 @@ impl Drop for Ctx {
     }
 }
 
-/// One GPU context: device ordinal, stream, scratch.  Cheap to clone.
+/// One GPU context: device ordinal, stream, scratch.  Cheap to clone; calls through any clone are serialised by the lock.
 #[derive(Clone)]
-pub struct HipDevice(Arc<Ctx>);
+pub struct HipDevice(Arc<Mutex<Ctx>>);
 
 impl HipDevice {
     /// the device picked where src/main.rs:188 / src/bin/server.rs:112 pick Metal or CPU today
@@ -56,14 +59,30 @@ impl HipDevice {
         let mut ctx = ptr::null_mut();
         // SAFETY: `ctx` is a valid out pointer
         check(ptr::null(), unsafe { turq_ctx_create(ordinal as c_int, &mut ctx) })?;
-        Ok(Self(Arc::new(Ctx(ctx))))
+        Ok(Self(Arc::new(Mutex::new(Ctx(ctx)))))
     }
-    fn ctx(&self) -> *mut turq_ctx {
-        self.0 .0
+    /// the context, locked for the caller's scope (`guard.0` is the raw pointer)
+    fn lock(&self) -> Result<MutexGuard<'_, Ctx>> {
+        self.0.lock().map_err(|_| Error::Msg("the turq context's lock is poisoned (a call panicked while holding it)".into()))
     }
     pub fn synchronize(&self) -> Result<()> {
+        let guard = self.lock()?;
         // SAFETY: the context is alive as long as `self`
-        check(self.ctx(), unsafe { turq_sync(self.ctx()) })
+        check(guard.0, unsafe { turq_sync(guard.0) })
+    }
+    /// Activations of any finite f32 magnitude on device pointers (host tensors always get them): see turq.h
+    pub fn set_wide_activations(&self, on: bool) -> Result<()> {
+        let guard = self.lock()?;
+        // SAFETY: the context is alive
+        check(guard.0, unsafe { turq_ctx_set_wide_activations(guard.0, on as c_int) })
+    }
+    /// Results stored since the last reset that were no finite numbers (an input left the f16 range, or was an infinity / NaN)
+    pub fn nonfinite_count(&self, reset: bool) -> Result<u64> {
+        let guard = self.lock()?;
+        let mut n = 0u64;
+        // SAFETY: `n` is a valid out pointer
+        check(guard.0, unsafe { turq_ctx_nonfinite_count(guard.0, &mut n, reset as c_int) })?;
+        Ok(n)
     }
 }
 
@@ -97,8 +116,8 @@ impl Drop for HipQTensor {
 impl HipQTensor {
     fn from_handle(dev: &HipDevice, w: *mut turq_weight, one_dim: bool) -> Result<Self> {
         let (mut dtype, mut n, mut k) = (0 as c_int, 0i64, 0i64);
-        // SAFETY: out pointers are valid; unused ones may be null
-        check(dev.ctx(), unsafe { turq_weight_info(w, &mut dtype, &mut n, &mut k, ptr::null_mut(), ptr::null_mut()) })?;
+        // SAFETY: out pointers are valid; unused ones may be null (no context is involved: the error text is the thread's)
+        check(ptr::null(), unsafe { turq_weight_info(w, &mut dtype, &mut n, &mut k, ptr::null_mut(), ptr::null_mut()) })?;
         Ok(Self { dev: dev.clone(), w, dtype, n: n as usize, k: k as usize, one_dim })
     }
     /// raw GGUF block bytes of a tensor of shape (n, k); quantized tensors go to the tiled layout the matmul kernels read
@@ -107,10 +126,13 @@ impl HipQTensor {
         let quant = matches!(dt, TURQ_Q8_0 | TURQ_Q4_K | TURQ_Q5_K | TURQ_Q6_K);
         let layout = if quant { TURQ_LAYOUT_TILED } else { TURQ_LAYOUT_NATIVE };
         let mut w = ptr::null_mut();
-        // SAFETY: `bytes` outlives the call, which copies them
-        check(dev.ctx(), unsafe {
-            turq_weight_upload(dev.ctx(), dt, n as i64, k as i64, bytes.as_ptr().cast(), bytes.len(), layout, &mut w)
-        })?;
+        {
+            let guard = dev.lock()?;
+            // SAFETY: `bytes` outlives the call, which copies them
+            check(guard.0, unsafe {
+                turq_weight_upload(guard.0, dt, n as i64, k as i64, bytes.as_ptr().cast(), bytes.len(), layout, &mut w)
+            })?;
+        }
         Self::from_handle(dev, w, false)
     }
     pub fn shape(&self) -> Vec<usize> {
@@ -126,9 +148,19 @@ impl HipQTensor {
     /// `QTensor::dequantize(device)`: the f32 tensor, bit-exact with candle's `to_float`
     pub fn dequantize(&self, device: &Device) -> Result<Tensor> {
         let mut out = vec![0f32; self.n * self.k];
-        // SAFETY: `out` holds n * k floats
-        check(self.dev.ctx(), unsafe { turq_dequantize(self.dev.ctx(), self.w, out.as_mut_ptr(), TURQ_MEM_HOST) })?;
+        {
+            let guard = self.dev.lock()?;
+            // SAFETY: `out` holds n * k floats
+            check(guard.0, unsafe { turq_dequantize(guard.0, self.w, out.as_mut_ptr(), TURQ_MEM_HOST) })?;
+        }
         Tensor::from_vec(out, self.shape(), device)
+    }
+    /// A hint that this weight belongs to one of the next forward calls (see turq_weight_prefetch: a read-only pass next to
+    /// whatever the device runs; results are unaffected)
+    pub fn prefetch(&self) -> Result<()> {
+        let guard = self.dev.lock()?;
+        // SAFETY: the weight and the context are alive
+        check(guard.0, unsafe { turq_weight_prefetch(guard.0, self.w) })
     }
 }
 
@@ -161,12 +193,15 @@ impl HipQMatMul {
             // the dense arm reads GGUF byte order: export the tiled copy and upload it once more as it is in the file
             let nbytes = unsafe { turq_weight_nbytes(t.dtype, t.n as i64, t.k as i64) };
             let mut raw = vec![0u8; nbytes];
-            // SAFETY: `raw` holds the tensor's GGUF size
-            check(t.dev.ctx(), unsafe { turq_weight_export(t.dev.ctx(), t.w, raw.as_mut_ptr().cast(), nbytes) })?;
             let mut w = ptr::null_mut();
-            check(t.dev.ctx(), unsafe {
-                turq_weight_upload(t.dev.ctx(), t.dtype, t.n as i64, t.k as i64, raw.as_ptr().cast(), nbytes, TURQ_LAYOUT_NATIVE, &mut w)
-            })?;
+            {
+                let guard = t.dev.lock()?;
+                // SAFETY: `raw` holds the tensor's GGUF size
+                check(guard.0, unsafe { turq_weight_export(guard.0, t.w, raw.as_mut_ptr().cast(), nbytes) })?;
+                check(guard.0, unsafe {
+                    turq_weight_upload(guard.0, t.dtype, t.n as i64, t.k as i64, raw.as_ptr().cast(), nbytes, TURQ_LAYOUT_NATIVE, &mut w)
+                })?;
+            }
             return Ok(Self { t: HipQTensor::from_handle(&t.dev, w, false)?, dense: true });
         }
         Ok(Self { t, dense: !quant })
@@ -179,11 +214,36 @@ impl HipQMatMul {
         let x: Vec<f32> = xs.flatten_all()?.to_vec1()?;
         let mut y = vec![0f32; m * n];
         let algo = if self.dense { TURQ_ALGO_SIMPLE } else { TURQ_ALGO_AUTO };
-        let ctx = self.t.dev.ctx();
+        let guard = self.t.dev.lock()?;
+        let ctx = guard.0;
         // SAFETY: x holds m * k floats, y m * n
         check(ctx, unsafe {
             turq_qmatmul(ctx, self.t.w, x.as_ptr().cast(), TURQ_ACT_F32, m as i64, k as i64, y.as_mut_ptr().cast(), TURQ_ACT_F32, n as i64,
                          ptr::null(), TURQ_MEM_HOST, algo)
+        })?;
+        if let Some(last) = dims.last_mut() {
+            *last = n;
+        }
+        Tensor::from_vec(y, dims, xs.device())
+    }
+
+    /// `residual + forward(xs)`: the residual connection (`x + h`, src/models/qwen3.rs:635) taken into the matmul's store
+    /// (TURQ_OUT_ACCUMULATE); `residual` has the output's shape.
+    pub fn forward_add(&self, xs: &Tensor, residual: &Tensor) -> Result<Tensor> {
+        let (n, k) = (self.t.n, self.t.k);
+        let (m, mut dims) = rows_of(xs, k)?;
+        let x: Vec<f32> = xs.flatten_all()?.to_vec1()?;
+        let mut y: Vec<f32> = residual.flatten_all()?.to_vec1()?;
+        if y.len() != m * n {
+            candle_core::bail!("shape mismatch in matmul: the residual has {} elements, the output {}", y.len(), m * n)
+        }
+        let algo = if self.dense { TURQ_ALGO_SIMPLE } else { TURQ_ALGO_AUTO };
+        let guard = self.t.dev.lock()?;
+        let ctx = guard.0;
+        // SAFETY: x holds m * k floats, y m * n
+        check(ctx, unsafe {
+            turq_qmatmul(ctx, self.t.w, x.as_ptr().cast(), TURQ_ACT_F32, m as i64, k as i64, y.as_mut_ptr().cast(),
+                         TURQ_ACT_F32 | TURQ_OUT_ACCUMULATE, n as i64, ptr::null(), TURQ_MEM_HOST, algo)
         })?;
         if let Some(last) = dims.last_mut() {
             *last = n;
@@ -205,7 +265,8 @@ impl HipQMatMul {
         let ws: Vec<*const turq_weight> = layers.iter().map(|l| l.t.w as *const turq_weight).collect();
         let yp: Vec<*mut c_void> = ys.iter_mut().map(|y| y.as_mut_ptr().cast()).collect();
         let ld: Vec<i64> = layers.iter().map(|l| l.t.n as i64).collect();
-        let ctx = first.t.dev.ctx();
+        let guard = first.t.dev.lock()?;
+        let ctx = guard.0;
         // SAFETY: the arrays have one entry per layer and every buffer its full size
         check(ctx, unsafe {
             turq_qmatmul_multi(ctx, ws.len() as c_int, ws.as_ptr(), x.as_ptr().cast(), TURQ_ACT_F32, m as i64, k as i64, yp.as_ptr(),
@@ -229,7 +290,8 @@ impl HipQMatMul {
         let (m, mut dims) = rows_of(xs, k)?;
         let x: Vec<f32> = xs.flatten_all()?.to_vec1()?;
         let mut y = vec![0f32; m * n];
-        let ctx = gate.t.dev.ctx();
+        let guard = gate.t.dev.lock()?;
+        let ctx = guard.0;
         // SAFETY: x holds m * k floats, y m * n
         check(ctx, unsafe {
             turq_qmatmul_gate_up(ctx, gate.t.w, up.t.w, x.as_ptr().cast(), TURQ_ACT_F32, m as i64, k as i64, y.as_mut_ptr().cast(),
@@ -247,7 +309,8 @@ impl HipQMatMul {
         let (m, mut dims) = rows_of(xs, k)?;
         let x: Vec<f32> = xs.flatten_all()?.to_vec1()?;
         let mut y = vec![0f32; m * n_out];
-        let ctx = gate.t.dev.ctx();
+        let guard = gate.t.dev.lock()?;
+        let ctx = guard.0;
         // SAFETY: x holds m * k floats, y m * n_out
         check(ctx, unsafe {
             turq_mlp(ctx, gate.t.w, up.t.w, down.t.w, x.as_ptr().cast(), TURQ_ACT_F32, m as i64, k as i64, y.as_mut_ptr().cast(),
@@ -276,6 +339,65 @@ impl HipRmsNorm {
         }
         Ok(Self { dev: dev.clone(), weight: Arc::new(w), eps: eps as f32 })
     }
+    /// `forward_multi(layers, self.forward(xs))` in one call: ln1 -> q / k / v (src/models/qwen3.rs:633-634, 272-274), the
+    /// final norm -> lm_head; the norm is applied inside the matmul kernels where they can (turq_norm_qmatmul_multi)
+    pub fn forward_then(&self, layers: &[&HipQMatMul], xs: &Tensor) -> Result<Vec<Tensor>> {
+        let Some(first) = layers.first() else { return Ok(Vec::new()) };
+        let k = first.t.k;
+        let (m, dims) = rows_of(xs, k)?;
+        if k != self.weight.len() || layers.iter().any(|l| l.t.k != k || l.dense) {
+            let xn = self.forward(xs)?;
+            return layers.iter().map(|l| l.forward(&xn)).collect();
+        }
+        let x: Vec<f32> = xs.flatten_all()?.to_vec1()?;
+        let mut ys: Vec<Vec<f32>> = layers.iter().map(|l| vec![0f32; m * l.t.n]).collect();
+        let ws: Vec<*const turq_weight> = layers.iter().map(|l| l.t.w as *const turq_weight).collect();
+        let yp: Vec<*mut c_void> = ys.iter_mut().map(|y| y.as_mut_ptr().cast()).collect();
+        let ld: Vec<i64> = layers.iter().map(|l| l.t.n as i64).collect();
+        {
+            let guard = self.dev.lock()?;
+            let ctx = guard.0;
+            // SAFETY: the arrays have one entry per layer and every buffer its full size; the norm weight holds k floats
+            check(ctx, unsafe {
+                turq_norm_qmatmul_multi(ctx, ws.len() as c_int, ws.as_ptr(), x.as_ptr().cast(), TURQ_ACT_F32, m as i64, k as i64,
+                                        self.weight.as_ptr(), self.eps, yp.as_ptr(), TURQ_ACT_F32, ld.as_ptr(), ptr::null(), TURQ_MEM_HOST)
+            })?;
+        }
+        ys.into_iter()
+            .zip(layers)
+            .map(|(y, l)| {
+                let mut d = dims.clone();
+                if let Some(last) = d.last_mut() {
+                    *last = l.t.n;
+                }
+                Tensor::from_vec(y, d, xs.device())
+            })
+            .collect()
+    }
+
+    /// `xs + mlp(self.forward(xs))`, the second half of the decoder layer (src/models/qwen3.rs:637-640), in one call
+    /// (turq_norm_mlp with TURQ_OUT_ACCUMULATE); the MLP's output width must be the input's
+    pub fn forward_mlp_residual(&self, gate: &HipQMatMul, up: &HipQMatMul, down: &HipQMatMul, xs: &Tensor) -> Result<Tensor> {
+        let (k, n_out) = (gate.t.k, down.t.n);
+        let (m, dims) = rows_of(xs, k)?;
+        if n_out != k || k != self.weight.len() {
+            candle_core::bail!("shape mismatch: a residual MLP maps {} features to {}, the norm has {}", k, n_out, self.weight.len())
+        }
+        let x: Vec<f32> = xs.flatten_all()?.to_vec1()?;
+        let mut y = x.clone();
+        {
+            let guard = self.dev.lock()?;
+            let ctx = guard.0;
+            // SAFETY: x and y hold m * k floats, the norm weight k
+            check(ctx, unsafe {
+                turq_norm_mlp(ctx, gate.t.w, up.t.w, down.t.w, x.as_ptr().cast(), TURQ_ACT_F32, m as i64, k as i64, self.weight.as_ptr(),
+                              self.eps, y.as_mut_ptr().cast(), TURQ_ACT_F32 | TURQ_OUT_ACCUMULATE, n_out as i64, ptr::null(), ptr::null(),
+                              ptr::null(), TURQ_ACTFN_SILU, TURQ_MEM_HOST)
+            })?;
+        }
+        Tensor::from_vec(y, dims, xs.device())
+    }
+
     pub fn forward(&self, xs: &Tensor) -> Result<Tensor> {
         let k = self.weight.len();
         let dims = xs.dims().to_vec();
@@ -285,7 +407,8 @@ impl HipRmsNorm {
         let x: Vec<f32> = xs.flatten_all()?.to_vec1()?;
         let m = if k == 0 { 0 } else { x.len() / k };
         let mut y = vec![0f32; x.len()];
-        let ctx = self.dev.ctx();
+        let guard = self.dev.lock()?;
+        let ctx = guard.0;
         // SAFETY: x and y hold m * k floats, the weight k
         check(ctx, unsafe {
             turq_rms_norm(ctx, x.as_ptr().cast(), TURQ_ACT_F32, m as i64, k as i64, k as i64, self.weight.as_ptr(), self.eps,
@@ -368,8 +491,11 @@ impl HipQVarBuilder {
         // matrices the matmul kernels read go to the tiled layout; vectors and dense tensors stay in GGUF order
         let layout = if quant && !one_dim { TURQ_LAYOUT_TILED } else { TURQ_LAYOUT_NATIVE };
         let mut w = ptr::null_mut();
-        // SAFETY: `w` is a valid out pointer
-        check(self.dev.ctx(), unsafe { turq_gguf_load_weight(self.dev.ctx(), self.gguf.0, c.as_ptr(), n, k, layout, &mut w) })?;
+        {
+            let guard = self.dev.lock()?;
+            // SAFETY: `w` is a valid out pointer
+            check(guard.0, unsafe { turq_gguf_load_weight(guard.0, self.gguf.0, c.as_ptr(), n, k, layout, &mut w) })?;
+        }
         HipQTensor::from_handle(&self.dev, w, one_dim)
     }
 }

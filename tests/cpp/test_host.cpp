@@ -144,6 +144,35 @@ int main(int argc, char **argv) {
                 }
             }
         }
+        // the decoder layer's glue on device tensors: norm -> projection in one call (three rows: the norm runs into scratch, the
+        // results are those of the two calls bit for bit; one row: the kernel applies the norm, within 5e-4) and y += x W^T
+        {
+            turq::NormX nx = turq::rms_norm(k, 1e-6, b0.pp("attn_norm"));
+            for (int64_t rows : {(int64_t)3, (int64_t)1}) {
+                turq::DeviceBuffer xn(dev, (size_t)rows * k * 4), y1(dev, (size_t)rows * n * 4), y2(dev, (size_t)rows * n * 4);
+                nx.forward(xd.ptr(), TURQ_ACT_F32, rows, k, xn.ptr(), TURQ_ACT_F32, k);
+                copy.qmatmul().forward(xn.ptr(), TURQ_ACT_F32, rows, k, y1.ptr(), TURQ_ACT_F32, n);
+                nx.forward_then({&copy.qmatmul()}, xd.ptr(), TURQ_ACT_F32, rows, k, {y2.ptr()}, TURQ_ACT_F32);
+                dev.synchronize();
+                std::vector<float> a((size_t)rows * n), b((size_t)rows * n);
+                y1.download(a.data(), a.size() * 4);
+                y2.download(b.data(), b.size() * 4);
+                double num = 0.0, den = 0.0;
+                for (size_t i = 0; i < a.size(); i++) {
+                    num += ((double)a[i] - b[i]) * ((double)a[i] - b[i]);
+                    den += (double)a[i] * a[i];
+                }
+                if (rows > 1 && std::memcmp(a.data(), b.data(), a.size() * 4) != 0) return fail("forward_then differs from norm + forward");
+                if (std::sqrt(num / den) > 5e-4) return fail("forward_then (one row) is not within 5e-4 of norm + forward");
+                // y2 += x W^T on top of what it holds
+                copy.qmatmul().forward_add(xn.ptr(), TURQ_ACT_F32, rows, k, y2.ptr(), TURQ_ACT_F32, n);
+                dev.synchronize();
+                std::vector<float> c((size_t)rows * n);
+                y2.download(c.data(), c.size() * 4);
+                for (size_t i = 0; i < c.size(); i++)
+                    if (c[i] != b[i] + a[i]) return fail("forward_add is not the sum of what y held and forward");
+            }
+        }
     } catch (const std::exception &e) {
         std::fprintf(stderr, "FAIL: exception: %s\n", e.what());
         return 1;

@@ -134,6 +134,11 @@ public:
                                        t_.rows(), bias, TURQ_MEM_HOST, dense_ ? TURQ_ALGO_SIMPLE : TURQ_ALGO_AUTO));
         return y;
     }
+    // y += x W^T on device tensors: the residual connection taken into the matmul's store (`x + h`, src/models/qwen3.rs:635)
+    void forward_add(const void *x_dev, int x_dtype, int64_t m, int64_t ldx, void *y_dev, int y_dtype, int64_t ldy,
+                     const float *bias_dev = nullptr) const {
+        forward(x_dev, x_dtype, m, ldx, y_dev, y_dtype | TURQ_OUT_ACCUMULATE, ldy, bias_dev);
+    }
     // device tensors: asynchronous on the device's stream
     void forward(const void *x_dev, int x_dtype, int64_t m, int64_t ldx, void *y_dev, int y_dtype, int64_t ldy,
                  const float *bias_dev = nullptr) const {
@@ -215,6 +220,29 @@ public:
     void forward(const void *x_dev, int x_dtype, int64_t m, int64_t ldx, void *y_dev, int y_dtype, int64_t ldy) const {
         dev_.check(turq_rms_norm(dev_.ctx(), x_dev, x_dtype, m, (int64_t)w_.size(), ldx, (const float *)wdev_->ptr(), eps_, y_dev, y_dtype, ldy,
                                  TURQ_MEM_DEVICE));
+    }
+    // forward_multi(layers, forward(x)) on a device tensor in one call: ln1 -> q / k / v (src/models/qwen3.rs:633-634, 272-274),
+    // the final norm -> lm_head; the norm is applied inside the matmul kernels where they can (turq_norm_qmatmul_multi)
+    void forward_then(const std::vector<const QMatMul *> &layers, const void *x_dev, int x_dtype, int64_t m, int64_t ldx,
+                      const std::vector<void *> &ys_dev, int y_dtype) const {
+        if (layers.empty()) return;
+        if (layers.size() != ys_dev.size()) throw Error(TURQ_ERR_SHAPE, "forward_then: one output per layer");
+        std::vector<const turq_weight *> w;
+        std::vector<int64_t> ldy;
+        for (const QMatMul *l : layers) {
+            w.push_back(l->qtensor().handle());
+            ldy.push_back(l->qtensor().rows());
+        }
+        dev_.check(turq_norm_qmatmul_multi(dev_.ctx(), (int)w.size(), w.data(), x_dev, x_dtype, m, ldx, (const float *)wdev_->ptr(), eps_,
+                                           ys_dev.data(), y_dtype, ldy.data(), nullptr, TURQ_MEM_DEVICE));
+    }
+    // y += mlp(forward(x)) on device tensors, the second half of the decoder layer (src/models/qwen3.rs:637-640): y is the residual
+    // stream (it may be x); accumulate = false writes the MLP's output instead
+    void forward_mlp(const QMatMul &gate, const QMatMul &up, const QMatMul &down, const void *x_dev, int x_dtype, int64_t m, int64_t ldx,
+                     void *y_dev, int y_dtype, int64_t ldy, bool accumulate = true) const {
+        dev_.check(turq_norm_mlp(dev_.ctx(), gate.qtensor().handle(), up.qtensor().handle(), down.qtensor().handle(), x_dev, x_dtype, m, ldx,
+                                 (const float *)wdev_->ptr(), eps_, y_dev, y_dtype | (accumulate ? TURQ_OUT_ACCUMULATE : 0), ldy, nullptr,
+                                 nullptr, nullptr, TURQ_ACTFN_SILU, TURQ_MEM_DEVICE));
     }
     const std::vector<float> &weight() const { return w_; }
     static const char *name() { return "RmsNorm"; }

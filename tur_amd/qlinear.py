@@ -40,6 +40,14 @@ class Device:
     def new_hip(ordinal: int = 0) -> "Device":
         return Device(ordinal)
 
+    def nonfinite_count(self, reset: bool = True) -> int:
+        """results stored since the last reset that were no finite numbers (``turq_ctx_nonfinite_count``)"""
+        import ctypes
+
+        n = ctypes.c_uint64()
+        capi.check(self.L.turq_ctx_nonfinite_count(self.ctx, ctypes.byref(n), 1 if reset else 0), self.ctx)
+        return n.value
+
     def synchronize(self) -> None:
         capi.check(self.L.turq_sync(self.ctx), self.ctx)
 
@@ -249,6 +257,26 @@ class LinearX:
     def forward(self, x: np.ndarray) -> np.ndarray:
         return self.qmatmul.forward(x, bias=self.bias)
 
+    def forward_add(self, x: np.ndarray, residual: np.ndarray) -> np.ndarray:
+        """``residual + forward(x)``: the residual connection of the decoder layer (``x + h``, src/models/qwen3.rs:635) taken
+        into the matmul's store (``TURQ_OUT_ACCUMULATE``)."""
+        q = self.qmatmul.qtensor
+        n, k = q._n, q._k
+        x = np.ascontiguousarray(x, np.float32)
+        if x.ndim < 2 or x.shape[-1] != k:
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch in matmul: input {x.shape}, weight needs last dim {k}")
+        lead = x.shape[:-1]
+        m = int(np.prod(lead)) if lead else 1
+        y = np.array(residual, np.float32, copy=True).reshape(-1)
+        if y.size != m * n:
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch in matmul: the residual has {y.size} elements, the output {m * n}")
+        b = None if self.bias is None else np.ascontiguousarray(self.bias, np.float32)
+        dev = q.device
+        algo = capi.ALGO_SIMPLE if self.qmatmul.dense else capi.ALGO_AUTO
+        capi.check(dev.L.turq_qmatmul(dev.ctx, q.handle, capi.ptr(x), capi.ACT_F32, m, k, capi.ptr(y), capi.ACT_F32 | capi.OUT_ACCUMULATE,
+                                      n, capi.ptr(b), capi.MEM_HOST, algo), dev.ctx)
+        return y.reshape(lead + (n,))
+
     def __repr__(self) -> str:
         return "LinearX::Quantized"     # candle keeps dense GGUF tensors inside QMatMul too (QMatMul::Tensor)
 
@@ -367,6 +395,47 @@ class NormX:
         dev = self.device
         capi.check(dev.L.turq_rms_norm(dev.ctx, capi.ptr(xs), xt, m, k, k, capi.ptr(self.weight), self.eps, capi.ptr(y), xt, k,
                                        capi.MEM_HOST), dev.ctx)
+        return y
+
+    def forward_then(self, layers: "list[QMatMul]", xs: np.ndarray) -> "list[np.ndarray]":
+        """``QMatMul.forward_multi(layers, self.forward(xs))`` in one call (``turq_norm_qmatmul_multi``): ln1 -> q / k / v
+        (src/models/qwen3.rs:633-634, 272-274), the final norm -> lm_head."""
+        import ctypes
+
+        if not layers:
+            return []
+        xs = np.ascontiguousarray(xs, np.float32)
+        k = self.weight.size
+        if xs.ndim < 2 or xs.shape[-1] != k or any(l.qtensor._k != k for l in layers):
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch in matmul: input {xs.shape}, norm and layers need last dim {k}")
+        if any(l.dense for l in layers):
+            xn = self.forward(xs)
+            return [l.forward(xn) for l in layers]
+        lead = xs.shape[:-1]
+        m = int(np.prod(lead)) if lead else 1
+        cnt = len(layers)
+        ys = [np.empty((m, l.qtensor._n), np.float32) for l in layers]
+        warr = (ctypes.c_void_p * cnt)(*[l.qtensor.handle.value for l in layers])
+        yarr = (ctypes.c_void_p * cnt)(*[y.ctypes.data for y in ys])
+        ldys = (ctypes.c_int64 * cnt)(*[l.qtensor._n for l in layers])
+        dev = self.device
+        capi.check(dev.L.turq_norm_qmatmul_multi(dev.ctx, cnt, warr, capi.ptr(xs), capi.ACT_F32, m, k, capi.ptr(self.weight), self.eps, yarr,
+                                                 capi.ACT_F32, ldys, None, capi.MEM_HOST), dev.ctx)
+        return [y.reshape(lead + (y.shape[1],)) for y in ys]
+
+    def forward_mlp_residual(self, gate: QMatMul, up: QMatMul, down: QMatMul, xs: np.ndarray) -> np.ndarray:
+        """``xs + mlp(self.forward(xs))``, the second half of the decoder layer (src/models/qwen3.rs:637-640), in one call
+        (``turq_norm_mlp`` with ``TURQ_OUT_ACCUMULATE``)."""
+        xs = np.ascontiguousarray(xs, np.float32)
+        k, n_out = gate.qtensor._k, down.qtensor._n
+        if xs.ndim < 2 or xs.shape[-1] != k or n_out != k or self.weight.size != k:
+            raise TurqError(capi.ERR_SHAPE, f"shape mismatch: input {xs.shape}, the MLP maps {k} features to {n_out}, the norm has {self.weight.size}")
+        m = xs.size // k
+        y = xs.copy()
+        dev = self.device
+        capi.check(dev.L.turq_norm_mlp(dev.ctx, gate.qtensor.handle, up.qtensor.handle, down.qtensor.handle, capi.ptr(xs), capi.ACT_F32, m, k,
+                                       capi.ptr(self.weight), self.eps, capi.ptr(y), capi.ACT_F32 | capi.OUT_ACCUMULATE, n_out, None, None,
+                                       None, capi.ACTFN_SILU, capi.MEM_HOST), dev.ctx)
         return y
 
     def __repr__(self) -> str:
