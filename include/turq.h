@@ -106,9 +106,10 @@ void *turq_ctx_stream(turq_ctx *ctx);
  * small kernels: rows multiplied by the power of two that puts their largest magnitude into [2^9, 2^10) and written as f16,
  * output rows multiplied back (both exact) - any finite f32 row then stays within the 1e-3 bar, infinities and NaNs
  * propagate.  It costs two launches per call and the grouped launches of turq_qmatmul_multi / turq_qmatmul_gate_up.  Default:
- * off, for engines whose activations are known to be bounded (after an RmsNorm, say).  Calls on HOST pointers always take the
- * wide path: they are the reference's own contract, and the staging copies dominate them anyway.  turq_qmatmul_noalloc never
- * takes it. */
+ * off, for engines whose activations are known to be bounded (after an RmsNorm, say); turq_ctx_nonfinite_count tells a host
+ * that left it off whether a call overflowed.  Calls on HOST pointers always take the wide path: they are the reference's own
+ * contract, and the staging copies dominate them anyway.  turq_qmatmul_noalloc cannot take it (it has no scratch for the
+ * scaled rows) and refuses f32 / bf16 activations with TURQ_ERR_INVALID while the switch is on. */
 int turq_ctx_set_wide_activations(turq_ctx *ctx, int on);
 /* Whether a forward call left the number range of its kernels.  Every kernel that stores results (the matmuls, turq_rms_norm,
  * the fragment preparation of calls with more than 32 rows, the f16 intermediate of turq_mlp) counts the elements it stores
@@ -365,6 +366,11 @@ int turq_read_yardstick(turq_ctx *ctx, const void *dev_ptr, size_t nbytes);
  * wave_groups: 2 where the 64 x 128 tile runs eight waves as two groups on alternate super-blocks.  Not part of the path, no
  * counterpart in the reference: for tests of the rules and for tuning them on another device. */
 int turq_prefill_plan(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int *tile, int *split, int *wave_groups);
+/* ... and whether turq_qmatmul_multi sends `count` (1 .. 4) neighbouring weights of that format and shape - gate_proj and up_proj -
+ * out as ONE launch over the rows of all of them (merged = 1) or as a launch each (0).  The rule compares how well the two
+ * choices fill their rounds over the device's CUs, so the answer depends on compute_units; the kernels give the same products
+ * either way (another order of the f32 sums where a tile's waves split k: within 2e-6). */
+int turq_prefill_plan_multi(int dtype, int64_t n, int64_t k, int64_t m, int count, int compute_units, int *merged);
 
 /* ---- GGUF files ---- */
 /* Parse the header (magic, version 1..3, metadata, tensor infos, alignment).

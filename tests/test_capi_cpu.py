@@ -251,8 +251,24 @@ def test_prefill_launch_rules_on_a_256_cu_device():
     assert plan(Q4_K, 24576, 4096, 1024) == (3, 1, 1)
     # the LM head: more workgroups than CUs, four waves
     assert plan(Q6_K, 151936, 4096, 64) == (4, 1, 1)
+    # gate_proj and up_proj (2 x 12288 x 4096) through turq_qmatmul_multi: one launch where that fills the rounds better, which the
+    # timings behind the rule show at 128, 256 and 1024 rows and not at 384 and 512; k_proj and v_proj are too small to merge
+    def merged(n, m, cus, count=2):
+        g = ctypes.c_int(-1)
+        capi.check(L.turq_prefill_plan_multi(Q4_K, n, 4096, m, count, cus, ctypes.byref(g)))
+        return g.value
+
+    assert [merged(12288, m, 256) for m in (64, 128, 256, 384, 512, 1024, 2048)] == [0, 1, 1, 0, 0, 1, 0]
+    assert [merged(1024, m, 256) for m in (64, 256, 2048)] == [0, 0, 0]
+    assert merged(12288, 256, 256, count=1) == 0
+    # the rule counts rounds over the CUs, so a device of half the size decides differently at the same shapes
+    assert [merged(12288, m, 128) for m in (64, 128, 256, 384, 512, 1024, 2048)] == [0, 1, 0, 1, 1, 0, 0]
+    assert merged(1024, 2048, 128) == 1
     # arguments
     t = ctypes.c_int()
+    assert L.turq_prefill_plan_multi(Q4_K, 12288, 4096, 8, 2, 256, ctypes.byref(t)) == capi.ERR_SHAPE
+    assert L.turq_prefill_plan_multi(Q4_K, 12288, 4096, 64, 5, 256, ctypes.byref(t)) == capi.ERR_SHAPE
+    assert L.turq_prefill_plan_multi(capi.F32, 12288, 4096, 64, 2, 256, ctypes.byref(t)) == capi.ERR_DTYPE
     assert L.turq_prefill_plan(Q4_K, 4096, 4096, 8, 256, ctypes.byref(t), None, None) == capi.ERR_SHAPE
     assert L.turq_prefill_plan(capi.F32, 4096, 4096, 64, 256, ctypes.byref(t), None, None) == capi.ERR_DTYPE
 

@@ -77,6 +77,31 @@ def test_device_calls_after_the_switch(x_dtype, y_dtype):
         g.close()
 
 
+def test_more_rows_than_a_grid_has_rows_of_workgroups():
+    # 70 000 rows on device pointers under the switch: the kernel that takes the row factors out again walks the rows in a
+    # loop (a grid's second dimension ends at 65 535), so the rows past that are results too, not what the buffer held before
+    g = Gpu()
+    try:
+        L, ctx = g.L, g.ctx
+        dt, n, k, m = Q4_K, 128, 1024, 70000
+        raw = synth.random_weight(dt, n, k, seed=6)
+        w = g.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+        x = np.random.default_rng(8).standard_normal((m, k)).astype(np.float32)
+        rows = np.array([0, 1, 65534, 65535, 65536, 65537, 69998, 69999])
+        x[rows[::2]] *= 1e6
+        capi.check(L.turq_ctx_set_wide_activations(ctx, 1), ctx)
+        y = g.qmatmul(w, x, n, k, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_F32)
+        assert np.all(np.isfinite(y))
+        assert per_row_rel(y[rows], orc.matmul_dequant(dt, x[rows], raw, n, k)).max() <= 1e-3
+        # every 1000th row as well, and no row left at zero
+        some = np.arange(0, m, 1000)
+        assert per_row_rel(y[some], orc.matmul_dequant(dt, x[some], raw, n, k)).max() <= 1e-3
+        assert np.all(np.abs(y).max(axis=1) > 0)
+        g.release(w)
+    finally:
+        g.close()
+
+
 def test_grouped_calls_and_gate_up_under_the_switch():
     from oracle import oracle_np as onp
     g = Gpu()

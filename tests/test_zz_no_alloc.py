@@ -90,6 +90,36 @@ def test_noalloc_refuses_what_does_not_fit(gpu):
         gpu.release(w)
 
 
+def test_noalloc_refuses_f32_rows_while_wide_activations_are_on():
+    # wide activations need scratch of their own (the scaled f16 copy of the rows and a factor per row); the call that
+    # allocates nothing says so instead of rounding f32 rows to f16 unscaled.  f16 rows need no scaling and still pass.
+    g2 = Gpu()
+    try:
+        L, ctx = g2.L, g2.ctx
+        dt, n, k, m = capi.Q4_K, 256, 1024, 8
+        raw = synth.random_weight(dt, n, k, seed=4)
+        w = g2.upload(dt, n, k, raw, capi.LAYOUT_TILED)
+        x = synth.random_activation(m, k, seed=2, bf16=True)
+        before = g2.qmatmul_device(w, x, n, k, x_dtype=capi.ACT_BF16, noalloc=True)
+        capi.check(L.turq_ctx_set_wide_activations(ctx, 1), ctx)
+        xd = g2.dev_buffer(nbytes=m * k * 4)
+        yd = g2.dev_buffer(nbytes=m * n * 4)
+        for xt in (capi.ACT_F32, capi.ACT_BF16):
+            assert L.turq_qmatmul_noalloc(ctx, w, xd, xt, m, k, yd, capi.ACT_F32, n, None) == capi.ERR_INVALID
+            assert "wide activations" in capi.last_error(ctx)
+        x16 = x.astype(np.float16)
+        y16 = g2.qmatmul_device(w, x16, n, k, x_dtype=capi.ACT_F16, noalloc=True)
+        assert rel_l2(y16, orc.matmul_dequant(dt, x16.astype(np.float32), raw, n, k)) <= 2e-5
+        capi.check(L.turq_ctx_set_wide_activations(ctx, 0), ctx)
+        after = g2.qmatmul_device(w, x, n, k, x_dtype=capi.ACT_BF16, noalloc=True)
+        assert np.array_equal(before.view(np.uint32), after.view(np.uint32))
+        g2.dev_free(xd)
+        g2.dev_free(yd)
+        g2.release(w)
+    finally:
+        g2.close()
+
+
 def test_noalloc_leaves_the_context_scratch_alone(gpu):
     # a fresh context: after calls through the no-allocation entry point its own fragment buffer is still unallocated
     g2 = Gpu()

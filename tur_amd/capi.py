@@ -66,6 +66,7 @@ _SIGS = {
     "turq_quantize_q8_k": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int]),
     "turq_read_yardstick": (c_int, [c_void_p, c_void_p, c_size_t]),
     "turq_prefill_plan": (c_int, [c_int, c_int64, c_int64, c_int64, c_int, POINTER(c_int), POINTER(c_int), POINTER(c_int)]),
+    "turq_prefill_plan_multi": (c_int, [c_int, c_int64, c_int64, c_int64, c_int, c_int, POINTER(c_int)]),
     "turq_graph_begin": (c_int, [c_void_p]),
     "turq_graph_end": (c_int, [c_void_p, POINTER(c_void_p)]),
     "turq_graph_launch": (c_int, [c_void_p, c_void_p]),

@@ -972,7 +972,8 @@ static int impl_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t 
 // ---- the entry points a graph capture may hold ----
 // A call that fails while the context's stream is capturing ends the capture and discards what was recorded, so that the stream
 // and the context are usable again (turq_graph_end then reports that no capture is running).
-static int capture_guard(turq_ctx *ctx, int rc) {
+}  // extern "C"
+int turq_capture_guard(turq_ctx *ctx, int rc) {
     if (rc != TURQ_OK && ctx && ctx->capturing) {
         hipGraph_t dead = nullptr;
         (void)hipStreamEndCapture(ctx->stream, &dead);
@@ -983,52 +984,53 @@ static int capture_guard(turq_ctx *ctx, int rc) {
     }
     return rc;
 }
+extern "C" {
 
 int turq_dequantize(turq_ctx *ctx, const turq_weight *w, float *out, int out_mem) {
-    return capture_guard(ctx, impl_dequantize(ctx, w, out, out_mem));
+    return turq_capture_guard(ctx, impl_dequantize(ctx, w, out, out_mem));
 }
 int turq_embedding_lookup(turq_ctx *ctx, const turq_weight *w, const uint32_t *ids, int64_t count, void *out, int out_dtype,
                           int64_t ldo, int mem) {
-    return capture_guard(ctx, impl_embedding_lookup(ctx, w, ids, count, out, out_dtype, ldo, mem));
+    return turq_capture_guard(ctx, impl_embedding_lookup(ctx, w, ids, count, out, out_dtype, ldo, mem));
 }
 int turq_qmatmul(turq_ctx *ctx, const turq_weight *w, const void *x, int xt, int64_t m, int64_t ldx, void *y, int yt,
                  int64_t ldy, const float *bias, int mem, int algo) {
-    return capture_guard(ctx, impl_qmatmul(ctx, w, x, xt, m, ldx, y, yt, ldy, bias, mem, algo));
+    return turq_capture_guard(ctx, impl_qmatmul(ctx, w, x, xt, m, ldx, y, yt, ldy, bias, mem, algo));
 }
 int turq_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int xt, int64_t m,
                        int64_t ldx, void *const *ys, int yt, const int64_t *ldys, const float *const *biases, int mem, int algo) {
-    return capture_guard(ctx, impl_qmatmul_multi(ctx, count, weights, x, xt, m, ldx, ys, yt, ldys, biases, mem, algo));
+    return turq_capture_guard(ctx, impl_qmatmul_multi(ctx, count, weights, x, xt, m, ldx, ys, yt, ldys, biases, mem, algo));
 }
 int turq_qmatmul_gate_up(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m, int64_t ldx,
                          void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, int act, int mem) {
-    return capture_guard(ctx, impl_qmatmul_gate_up(ctx, gate, up, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, act, mem));
+    return turq_capture_guard(ctx, impl_qmatmul_gate_up(ctx, gate, up, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, act, mem));
 }
 int turq_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt, int64_t m,
              int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, const float *bias_down, int act, int mem) {
-    return capture_guard(ctx, impl_mlp(ctx, gate, up, down, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem));
+    return turq_capture_guard(ctx, impl_mlp(ctx, gate, up, down, x, xt, m, ldx, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem));
 }
 int turq_norm_qmatmul_multi(turq_ctx *ctx, int count, const turq_weight *const *weights, const void *x, int xt, int64_t m, int64_t ldx,
                             const float *norm_weight, float eps, void *const *ys, int yt, const int64_t *ldys, const float *const *biases,
                             int mem) {
-    return capture_guard(ctx, impl_norm_qmatmul_multi(ctx, count, weights, x, xt, m, ldx, norm_weight, eps, ys, yt, ldys, biases, mem));
+    return turq_capture_guard(ctx, impl_norm_qmatmul_multi(ctx, count, weights, x, xt, m, ldx, norm_weight, eps, ys, yt, ldys, biases, mem));
 }
 int turq_norm_mlp(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const turq_weight *down, const void *x, int xt, int64_t m,
                   int64_t ldx, const float *norm_weight, float eps, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up,
                   const float *bias_down, int act, int mem) {
-    return capture_guard(ctx, impl_norm_mlp(ctx, gate, up, down, x, xt, m, ldx, norm_weight, eps, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem));
+    return turq_capture_guard(ctx, impl_norm_mlp(ctx, gate, up, down, x, xt, m, ldx, norm_weight, eps, y, yt, ldy, bias_gate, bias_up, bias_down, act, mem));
 }
 int turq_quantize_q8_0(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
-    return capture_guard(ctx, impl_quantize_q8_0(ctx, x, m, k, out, mem));
+    return turq_capture_guard(ctx, impl_quantize_q8_0(ctx, x, m, k, out, mem));
 }
 int turq_quantize_q8_k(turq_ctx *ctx, const float *x, int64_t m, int64_t k, void *out, int mem) {
-    return capture_guard(ctx, impl_quantize_q8_k(ctx, x, m, k, out, mem));
+    return turq_capture_guard(ctx, impl_quantize_q8_k(ctx, x, m, k, out, mem));
 }
 
-int turq_weight_prefetch(turq_ctx *ctx, const turq_weight *w) { return capture_guard(ctx, impl_weight_prefetch(ctx, w)); }
+int turq_weight_prefetch(turq_ctx *ctx, const turq_weight *w) { return turq_capture_guard(ctx, impl_weight_prefetch(ctx, w)); }
 
 int turq_rms_norm(turq_ctx *ctx, const void *x, int x_dtype, int64_t m, int64_t k, int64_t ldx, const float *weight, float eps, void *y,
                   int y_dtype, int64_t ldy, int mem) {
-    return capture_guard(ctx, impl_rms_norm(ctx, x, x_dtype, m, k, ldx, weight, eps, y, y_dtype, ldy, mem));
+    return turq_capture_guard(ctx, impl_rms_norm(ctx, x, x_dtype, m, k, ldx, weight, eps, y, y_dtype, ldy, mem));
 }
 
 int turq_ctx_set_wide_activations(turq_ctx *ctx, int on) {

@@ -173,6 +173,8 @@ inline int turq_fail(turq_ctx *ctx, int code, const char *fmt, ...) {
                              "%s failed: %s", #call, hipGetErrorString(e_));                     \
     } while (0)
 
+// A forward call that fails while the context's stream is capturing ends the capture and discards what was recorded (api.cpp)
+int turq_capture_guard(turq_ctx *ctx, int rc);
 // grow-only scratch on the context's device
 int turq_ctx_reserve(turq_ctx *ctx, void **buf, size_t *cap, size_t need);
 // The static scratch array of the current device (noalloc.hip): its device address and size.  The device must be current.

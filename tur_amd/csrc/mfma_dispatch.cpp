@@ -208,18 +208,34 @@ static int gemm_split_reserve(turq_ctx *ctx, int count, const turq_weight *const
 // CUs that the GEMM launch for [m, n] takes: its workgroups, by the launcher's choice between the 64-row tile (two of those
 // workgroups share a CU) and the 128-row tiles (one per CU; wide tiles counted as two).  Measured on the Q4_K_M layer: launches
 // of 192 workgroups next to each other help with the 64-row tile (m = 128: +4.8 %) and hurt with the 128-row tile (m = 256: -2.7 %).
-static int64_t gemm_cus_taken(const turq_ctx *ctx, const turq_weight *w, int64_t m, bool may_split) {
+static int64_t gemm_cus_taken_shape(int compute_units, int dtype, int64_t n, int64_t k, int64_t m, bool may_split) {
     int form = 0, split = 1;
-    if (may_split && turq_gemm_split_scratch(w->dtype, w->n, w->k, m, ctx->compute_units, &form, &split) != 0) {
-        const int64_t tiles = form == 4 ? ((w->n + 127) / 128) * ((m + 63) / 64) : ((w->n + 255) / 256) * ((m + 127) / 128);
-        const bool whole = form != 4 || turq_gemm_low_two_groups(w->n, w->k, m, split, ctx->compute_units);
+    if (may_split && turq_gemm_split_scratch(dtype, n, k, m, compute_units, &form, &split) != 0) {
+        const int64_t tiles = form == 4 ? ((n + 127) / 128) * ((m + 63) / 64) : ((n + 255) / 256) * ((m + 127) / 128);
+        const bool whole = form != 4 || turq_gemm_low_two_groups(n, k, m, split, compute_units);
         return whole ? tiles * split : (tiles * split + 1) / 2;
     }
-    const int64_t nt = (w->n + 127) / 128, wgs128 = ((m + 127) / 128) * nt;
-    const bool low = m <= 64 || 2 * wgs128 <= ctx->compute_units;
+    const int64_t nt = (n + 127) / 128, wgs128 = ((m + 127) / 128) * nt;
+    const bool low = m <= 64 || 2 * wgs128 <= compute_units;
     if (!low) return wgs128;
     const int64_t tiles = ((m + 63) / 64) * nt;
-    return turq_gemm_low_two_groups(w->n, w->k, m, 1, ctx->compute_units) ? tiles : (tiles + 1) / 2;
+    return turq_gemm_low_two_groups(n, k, m, 1, compute_units) ? tiles : (tiles + 1) / 2;
+}
+static int64_t gemm_cus_taken(const turq_ctx *ctx, const turq_weight *w, int64_t m, bool may_split) {
+    return gemm_cus_taken_shape(ctx->compute_units, w->dtype, w->n, w->k, m, may_split);
+}
+
+// Whether `run` (2 .. 4) neighbouring weights of one K-quant format and one shape [n, k] go out as ONE launch of the prefill
+// GEMM over the rows of all of them: each must take more than half of the machine alone, and the launch over all the rows
+// must fill its rounds over the CUs better - each alone leaves CUs idle and all together still fit one round, or the tile
+// chosen for all the rows keeps a larger share of its rounds busy (by 5 % at least).  taken_alone: CUs one of them takes.
+static bool gemm_merge_rule(int dtype, int64_t n, int64_t k, int64_t m, int run, int compute_units, int64_t taken_alone) {
+    const int64_t cus = compute_units;
+    if (run < 2 || 2 * taken_alone <= cus || !turq_dt_is_quant(dtype) || dtype == TURQ_Q8_0 || n % 256 != 0) return false;
+    int64_t wgs_one = 0, wgs_all = 0;
+    const double fill_one = turq_gemm_fill(dtype, n, k, m, compute_units, &wgs_one);
+    const double fill_all = turq_gemm_fill(dtype, n * run, k, m, compute_units, &wgs_all);
+    return (wgs_one < cus && wgs_all <= cus) || fill_all > 1.05 * fill_one;
 }
 
 int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m, int64_t ldx,
@@ -276,10 +292,7 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
             int j = i + 1;
             while (j < count && j - i < 4 && w[j]->dtype == w[i]->dtype && w[j]->n == w[i]->n) j++;
             if (j - i >= 2) {
-                int64_t wgs_one = 0, wgs_all = 0;
-                const double fill_one = turq_gemm_fill(w[i]->dtype, w[i]->n, w[i]->k, m, ctx->compute_units, &wgs_one);
-                const double fill_all = turq_gemm_fill(w[i]->dtype, w[i]->n * (j - i), w[i]->k, m, ctx->compute_units, &wgs_all);
-                if (merge_all || (wgs_one < cus && wgs_all <= cus) || fill_all > 1.05 * fill_one) {
+                if (merge_all || gemm_merge_rule(w[i]->dtype, w[i]->n, w[i]->k, m, j - i, ctx->compute_units, c)) {
                     TurqGemmWeights g{};
                     g.count = j - i;
                     for (int t = i; t < j; t++) {
@@ -731,6 +744,18 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
                                              ldy + i, bias ? bias + i : nullptr, nwaves, rtiles, ctx->stream, ev0, ev1));
         i = j;
     }
+    return TURQ_OK;
+}
+
+// whether turq_qmatmul_multi sends `count` neighbouring weights of this format and shape out as one prefill launch (no GPU needed)
+extern "C" int turq_prefill_plan_multi(int dtype, int64_t n, int64_t k, int64_t m, int count, int compute_units, int *merged) {
+    if (merged) *merged = 0;
+    if (!turq_dt_is_quant(dtype)) return turq_fail(nullptr, TURQ_ERR_DTYPE, "turq_prefill_plan_multi: dtype %d has no prefill kernel", dtype);
+    if (n <= 0 || k <= 0 || k % 256 != 0 || m <= TURQ_GEMV_MAX_M || compute_units <= 0 || count < 1 || count > 4)
+        return turq_fail(nullptr, TURQ_ERR_SHAPE, "turq_prefill_plan_multi: n=%lld k=%lld m=%lld count=%d on %d compute units", (long long)n,
+                         (long long)k, (long long)m, count, compute_units);
+    const int64_t alone = gemm_cus_taken_shape(compute_units, dtype, n, k, m, true);
+    if (merged) *merged = gemm_merge_rule(dtype, n, k, m, count, compute_units, alone) ? 1 : 0;
     return TURQ_OK;
 }
 

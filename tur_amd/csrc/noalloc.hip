@@ -51,13 +51,18 @@ struct FixedScratch {  // the context's fragment buffer is the static array for 
 };
 }  // namespace
 
-extern "C" int turq_qmatmul_noalloc(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype, int64_t m, int64_t ldx, void *y,
-                                    int y_dtype, int64_t ldy, const float *bias) {
-    if (!ctx) return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_qmatmul_noalloc: null context");
+static int noalloc_impl(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype, int64_t m, int64_t ldx, void *y, int y_dtype,
+                        int64_t ldy, const float *bias) {
     if (!w) return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_noalloc: null weight");
     if (!ctx->static_scratch)
         return turq_fail(ctx, TURQ_ERR_HIP, "turq_qmatmul_noalloc: the static scratch array of device %d could not be located: %s", ctx->device,
                          hipGetErrorString((hipError_t)ctx->static_scratch_err));
+    // wide activations need scratch of their own (the scaled copy of the rows, their factors): rather than round f32 / bf16 rows to
+    // f16 behind the back of a host that asked for the full range, the call says so
+    if (ctx->wide && x_dtype != TURQ_ACT_F16 && w->layout == TURQ_LAYOUT_TILED)
+        return turq_fail(ctx, TURQ_ERR_INVALID,
+                         "turq_qmatmul_noalloc: wide activations are switched on for this context, and the call that allocates nothing cannot "
+                         "scale rows; pass f16 activations, or use turq_qmatmul");
     if (m > 0 && w->k > 0) {
         const size_t need = scratch_need(w, m);
         if (need > ctx->static_scratch_cap)
@@ -68,4 +73,11 @@ extern "C" int turq_qmatmul_noalloc(turq_ctx *ctx, const turq_weight *w, const v
     }
     FixedScratch guard(ctx);
     return turq_qmatmul(ctx, w, x, x_dtype, m, ldx, y, y_dtype, ldy, bias, TURQ_MEM_DEVICE, TURQ_ALGO_AUTO);
+}
+
+extern "C" int turq_qmatmul_noalloc(turq_ctx *ctx, const turq_weight *w, const void *x, int x_dtype, int64_t m, int64_t ldx, void *y,
+                                    int y_dtype, int64_t ldy, const float *bias) {
+    if (!ctx) return turq_fail(nullptr, TURQ_ERR_INVALID, "turq_qmatmul_noalloc: null context");
+    // (its own refusals end a running capture like those of every other forward call)
+    return turq_capture_guard(ctx, noalloc_impl(ctx, w, x, x_dtype, m, ldx, y, y_dtype, ldy, bias));
 }
