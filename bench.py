@@ -98,6 +98,9 @@ class Bench:
         self.device = name.value.decode()
         self.cus = cus.value
         self.desc, self.mats = WORKLOADS[args.workload]
+        if getattr(args, "rows", None):
+            self.mats = [(label, dt, args.rows, k) for label, dt, _, k in self.mats]
+            self.desc += f" [weight rows overridden: {args.rows}]"
         self.xt, self.xbytes, self.xnp = ACT[args.act]
         self.yt, self.ybytes = OUT[args.out]
         self.weights = []      # [layer][matrix] -> handle
@@ -604,6 +607,9 @@ def main():
     ap.add_argument("--workload", default="q4k_mlp_8b", choices=sorted(WORKLOADS))
     ap.add_argument("--m", type=int, default=1, help="activation rows (decode batch)")
     ap.add_argument("--layers", type=int, default=None, help="distinct weight copies streamed per step")
+    ap.add_argument("--rows", type=int, default=None,
+                    help="side measurement: every matrix of the workload with this many weight rows instead of its own (how a "
+                         "prefill launch's time depends on the number of workgroups: q4k_prefill_up_8b with 1536 .. 24576 rows)")
     ap.add_argument("--act", default="f32", choices=sorted(ACT))
     ap.add_argument("--out", default="f32", choices=sorted(OUT), help="output element type")
     ap.add_argument("--eager", action="store_true", help="launch every call from the host instead of replaying a HIP graph")
@@ -634,9 +640,9 @@ def main():
     if args.embedding:
         return run_embedding(args)
     if args.layers is None:
-        per_layer = sum(synth.weight_nbytes(dt, n, k) for _, dt, n, k in WORKLOADS[args.workload][1])
+        per_layer = sum(synth.weight_nbytes(dt, args.rows or n, k) for _, dt, n, k in WORKLOADS[args.workload][1])
         args.layers = default_layers(per_layer)
-    headline = all(getattr(args, f) == ap.get_default(f) for f in ("workload", "m", "act", "out")) and not (
+    headline = not args.rows and all(getattr(args, f) == ap.get_default(f) for f in ("workload", "m", "act", "out")) and not (
         args.eager or args.single_calls or args.gate_up or args.mlp or args.calibrate_copy or args.glue or args.prefetch)
     b = Bench(args)
     try:
