@@ -127,6 +127,7 @@ extern "C" {
         wave_groups: *mut c_int,
     ) -> c_int;
     pub fn turq_prefill_plan_multi(dtype: c_int, n: i64, k: i64, m: i64, count: c_int, compute_units: c_int, merged: *mut c_int) -> c_int;
+    pub fn turq_tuning_describe(buf: *mut c_char, cap: usize, needed: *mut usize) -> c_int;
     pub fn turq_gguf_open(path: *const c_char, out: *mut *mut turq_gguf) -> c_int;
     pub fn turq_gguf_close(g: *mut turq_gguf);
     pub fn turq_gguf_last_error(g: *const turq_gguf) -> *const c_char;

@@ -371,6 +371,12 @@ int turq_prefill_plan(int dtype, int64_t n, int64_t k, int64_t m, int compute_un
  * choices fill their rounds over the device's CUs, so the answer depends on compute_units; the kernels give the same products
  * either way (another order of the f32 sums where a tile's waves split k: within 2e-6). */
 int turq_prefill_plan_multi(int dtype, int64_t n, int64_t k, int64_t m, int count, int compute_units, int *merged);
+/* The environment switches that override the library's kernel-selection rules (names TURQ_*; for A/B timing and tests, none
+ * is needed in production), as this process runs with them: one line per switch, "NAME=value  (default | set)  what it
+ * overrides".  The environment is read once, when the first context is created; a process that has any of them set says so in
+ * one line on stderr then.  buf may be null; *needed receives the bytes the whole text takes, terminator included.  (No
+ * counterpart in the reference, whose CPU path has no such rules.) */
+int turq_tuning_describe(char *buf, size_t cap, size_t *needed);
 
 /* ---- GGUF files ---- */
 /* Parse the header (magic, version 1..3, metadata, tensor infos, alignment).

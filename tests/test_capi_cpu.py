@@ -272,3 +272,35 @@ def test_prefill_launch_rules_on_a_256_cu_device():
     assert L.turq_prefill_plan(Q4_K, 4096, 4096, 8, 256, ctypes.byref(t), None, None) == capi.ERR_SHAPE
     assert L.turq_prefill_plan(capi.F32, 4096, 4096, 64, 256, ctypes.byref(t), None, None) == capi.ERR_DTYPE
 
+
+
+def test_tuning_switches_are_listed_and_overrides_are_announced():
+    # every environment switch of the kernel-selection rules lives in one table (tur_amd/csrc/tuning.h); a process lists what it
+    # runs with, and says on stderr when any of them is set
+    import os
+    import re
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    names = re.findall(r'X\(\w+, "(TURQ_\w+)"', open(os.path.join(root, "tur_amd", "csrc", "tuning.h")).read())
+    assert len(names) >= 25 and len(set(names)) == len(names)
+    # no other source file of the library reads the environment for a TURQ_ variable
+    for dirpath, _, files in os.walk(os.path.join(root, "tur_amd", "csrc")):
+        for f in files:
+            if f.endswith((".cpp", ".hip", ".h", ".hpp")) and f not in ("tuning.cpp", "tuning.h"):
+                assert not re.search(r'getenv\("TURQ_', open(os.path.join(dirpath, f)).read()), f
+    code = ("import ctypes\nfrom tur_amd import capi\nL = capi.lib()\nn = ctypes.c_size_t()\n"
+            "capi.check(L.turq_tuning_describe(None, 0, ctypes.byref(n)))\nb = ctypes.create_string_buffer(n.value)\n"
+            "capi.check(L.turq_tuning_describe(b, n.value, None))\nprint(b.value.decode())\n")
+    env = {k: v for k, v in os.environ.items() if not k.startswith("TURQ_")}
+    plain = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, check=True)
+    lines = plain.stdout.strip().splitlines()
+    assert [ln.split("=")[0] for ln in lines] == names
+    assert all("(default)" in ln for ln in lines) and "libturq" not in plain.stderr
+    env.update(TURQ_GEMM_WIDE="0", TURQ_GEMV_NO_ROW1="1")
+    forced = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, check=True)
+    assert "2 kernel-selection override(s) from the environment: TURQ_GEMV_NO_ROW1=1 TURQ_GEMM_WIDE=0" in forced.stderr
+    by = {ln.split("=")[0]: ln for ln in forced.stdout.strip().splitlines()}
+    assert by["TURQ_GEMM_WIDE"].startswith("TURQ_GEMM_WIDE=0  (set)") and by["TURQ_GEMV_NO_ROW1"].startswith("TURQ_GEMV_NO_ROW1=1  (set)")
+    assert by["TURQ_GEMM_LOW"].startswith("TURQ_GEMM_LOW=-1  (default)")

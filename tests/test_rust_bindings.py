@@ -118,7 +118,7 @@ NOT_WRAPPED = {
     "turq_dev_alloc", "turq_dev_free", "turq_memcpy_h2d", "turq_memcpy_d2h", "turq_ctx_stream", "turq_qmatmul_noalloc",
     "turq_graph_begin", "turq_graph_end", "turq_graph_launch", "turq_graph_destroy", "turq_ctx_scratch_info",
     # measurement aids
-    "turq_profile_begin", "turq_profile_end", "turq_read_yardstick", "turq_prefill_plan", "turq_prefill_plan_multi", "turq_ctx_device_info", "turq_version",
+    "turq_profile_begin", "turq_profile_end", "turq_read_yardstick", "turq_prefill_plan", "turq_prefill_plan_multi", "turq_tuning_describe", "turq_ctx_device_info", "turq_version",
     # host-side layout transforms and geometry used by tools, not by the model path
     "turq_tile_host", "turq_untile_host", "turq_tiled_nbytes", "turq_block_elems", "turq_block_bytes",
     # candle's own code keeps the metadata and the name table of the file; the embedding and the quantizers have no caller in

@@ -67,6 +67,7 @@ _SIGS = {
     "turq_read_yardstick": (c_int, [c_void_p, c_void_p, c_size_t]),
     "turq_prefill_plan": (c_int, [c_int, c_int64, c_int64, c_int64, c_int, POINTER(c_int), POINTER(c_int), POINTER(c_int)]),
     "turq_prefill_plan_multi": (c_int, [c_int, c_int64, c_int64, c_int64, c_int, c_int, POINTER(c_int)]),
+    "turq_tuning_describe": (c_int, [c_char_p, c_size_t, POINTER(c_size_t)]),
     "turq_graph_begin": (c_int, [c_void_p]),
     "turq_graph_end": (c_int, [c_void_p, POINTER(c_void_p)]),
     "turq_graph_launch": (c_int, [c_void_p, c_void_p]),

@@ -152,8 +152,9 @@ int turq_ctx_create(int device, turq_ctx **out) {
         return turq_fail(nullptr, TURQ_ERR_HIP, "turq_ctx_create: the prefetch stream could not be made: %s", hipGetErrorString(e));
     }
     ctx->pf_workgroups = ctx->compute_units > 0 ? ctx->compute_units : 256;
-    if (const char *v = getenv("TURQ_PREFETCH_WGS")) { const int x = atoi(v); if (x >= 1 && x <= 4096) ctx->pf_workgroups = x; }
-    if (const char *v = getenv("TURQ_PREFETCH_DEPTH")) { const int x = atoi(v); if (x >= 1 && x <= 4) ctx->pf_depth = x; }
+    const TurqTuning &tune = turq_tuning();  // (the first context of a process reads the environment here)
+    if (tune.prefetch_wgs >= 1 && tune.prefetch_wgs <= 4096) ctx->pf_workgroups = tune.prefetch_wgs;
+    if (tune.prefetch_depth >= 1 && tune.prefetch_depth <= 4) ctx->pf_depth = tune.prefetch_depth;
     *out = ctx.release();
     return TURQ_OK;
 }

@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "../../include/turq.h"
+#include "tuning.h"
 
 #define TURQ_QK_K 256
 #define TURQ_QK8_0 32

@@ -1031,12 +1031,12 @@ hipError_t launch_gemm(const TurqGemmWeights &ws, int64_t k, const void *frags, 
 // 4: low 64 x 128; 0: no kernel for this format.  compute_units: CUs of the device (0: unknown).
 int turq_gemm_form(int dtype, int64_t n, int64_t k, int64_t m, int compute_units) {
     (void)k;
-    static const bool tall = getenv("TURQ_GEMM_GRID_2X2") == nullptr;  // Q5_K / Q6_K: 1 x 4 waves unless told otherwise
+    const bool tall = !turq_tuning().gemm_grid_2x2;  // Q5_K / Q6_K: 1 x 4 waves unless told otherwise
     // The wide tile (128 x 256, Geo<.., 3>) pulls fewer activation bytes through the L2 per flop (Q4_K: + 12 % at m = 2048 and
     // 4096; LM head Q5_K / Q6_K: + 4 .. 21 % from m = 64 to 512) but makes fewer, larger workgroups: it is taken where its
     // gain outweighs what its workgroup count loses in the last round over the CUs, and only where there are workgroups
     // enough to matter.  TURQ_GEMM_WIDE = 0 / 1 overrides the rule.
-    static const int wide_env = [] { const char *e = getenv("TURQ_GEMM_WIDE"); return e ? (atoi(e) != 0 ? 1 : 0) : -1; }();
+    const int wide_env = turq_tuning().gemm_wide;
     const int64_t cus = compute_units > 0 ? compute_units : 256;
     auto fill = [&](int64_t bn, int64_t *count) {  // share of the CU-rounds a launch with this tile width keeps busy
         const int64_t wgs = ((n + bn - 1) / bn) * ((m + BM - 1) / BM), rounds = (wgs + cus - 1) / cus;
@@ -1051,7 +1051,7 @@ int turq_gemm_form(int dtype, int64_t n, int64_t k, int64_t m, int compute_units
     };
     // The low tile (64 x 128, Geo<.., 4>) for launches of up to 64 rows, and for those whose 128 x 128 tiles would leave at
     // least half of the CUs without a workgroup (twice the workgroups).  TURQ_GEMM_LOW = 0 / 1 overrides the rule.
-    static const int low_env = [] { const char *e = getenv("TURQ_GEMM_LOW"); return e ? (atoi(e) != 0 ? 1 : 0) : -1; }();
+    const int low_env = turq_tuning().gemm_low;
     const int64_t wgs128 = ((n + 127) / 128) * ((m + BM - 1) / BM);
     // (up to 64 rows the low tile is the whole problem's height: half the MFMA work and activation traffic of a 128-row tile)
     const bool low = low_env >= 0 ? low_env == 1 : (m <= 64 || 2 * wgs128 <= cus);
@@ -1086,8 +1086,7 @@ int turq_gemm_form(int dtype, int64_t n, int64_t k, int64_t m, int compute_units
 size_t turq_gemm_split_scratch(int dtype, int64_t n, int64_t k, int64_t m, int compute_units, int *form_out, int *split_out) {
     if (form_out) *form_out = 0;
     if (split_out) *split_out = 1;
-    static const int env = [] { const char *e = getenv("TURQ_GEMM_SPLIT"); return e ? atoi(e) : -1; }();
-    static const int env_form = [] { const char *e = getenv("TURQ_GEMM_SPLIT_FORM"); return e ? atoi(e) : 0; }();
+    const int env = turq_tuning().gemm_split, env_form = turq_tuning().gemm_split_form;
     if (env == 0 || compute_units <= 0 || (dtype != TURQ_Q4_K && dtype != TURQ_Q5_K && dtype != TURQ_Q6_K)) return 0;
     const int64_t cus = compute_units, ntc = k / 256;
     const int64_t low_tiles = ((n + 127) / 128) * ((m + 63) / 64), wide_tiles = ((n + 255) / 256) * ((m + 127) / 128);
@@ -1136,7 +1135,7 @@ double turq_gemm_fill(int dtype, int64_t n, int64_t k, int64_t m, int compute_un
 // whether a low-tile launch whose tiles are split over `split` workgroups each takes the eight-wave form (one such workgroup
 // fills a CU's LDS; two of the four-wave form share one)
 bool turq_gemm_low_two_groups(int64_t n, int64_t k, int64_t m, int split, int compute_units) {
-    static const int kgroups = [] { const char *e = getenv("TURQ_GEMM_KGROUPS"); return e ? atoi(e) : 0; }();
+    const int kgroups = turq_tuning().gemm_kgroups;
     if (split < 1 || (k / 256) % split != 0 || (k / 256 / split) % 2 != 0 || kgroups == 1) return false;
     const int64_t wgs = ((n + 127) / 128) * ((m + 63) / 64) * split;
     return kgroups == 2 || wgs <= (compute_units > 0 ? compute_units : 256);

@@ -685,7 +685,7 @@ hipError_t launch_final(const Row1Launch &l) {
 // column tiles in flight per wave: up to three for one activation row (four do not fit the registers of every format), up to
 // two for several rows, whose raw activations are held next to the weights until they are staged
 inline int row1_in_flight(int64_t k, int nwaves, int m) {
-    static const int forced = [] { const char *e = getenv("TURQ_ROW1_P"); return e ? atoi(e) : 0; }();
+    const int forced = turq_tuning().row1_p;
     const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
     const int most = m > 1 ? 2 : 3;
     int p = (int)(per_wave < most ? per_wave : most);

@@ -10,7 +10,7 @@ namespace {
 // Waves per workgroup (= how many ways a row tile's columns are split).  Enough waves to cover the
 // machine a few times over, never more than there are column tiles.
 int pick_waves(const turq_ctx *ctx, int64_t n, int64_t k) {
-    static const int forced = [] { const char *e = getenv("TURQ_GEMV_WAVES"); return e ? atoi(e) : 0; }();
+    const int forced = turq_tuning().gemv_waves;
     if (forced >= 1 && forced <= 16) return (int)std::min<int64_t>(forced, turq_tile_cols(k));
     const int64_t row_tiles = turq_tile_rows(n);
     const int64_t col_tiles = turq_tile_cols(k);
@@ -32,8 +32,7 @@ bool use_fused(const turq_ctx *ctx, int64_t m, int64_t row_tiles, size_t weight_
 
 // one activation row, formats the sub-block-row kernel covers (TURQ_GEMV_NO_ROW1 keeps the general kernel, for comparison)
 bool use_row1(int dtype) {
-    static const bool off = getenv("TURQ_GEMV_NO_ROW1") != nullptr;
-    return !off && turq_gemv_row1_supports(dtype);
+    return !turq_tuning().gemv_no_row1 && turq_gemv_row1_supports(dtype);
 }
 
 // The one-row kernel stages the raw activations itself, once per wave and column tile, and needs no preparation launch.
@@ -43,7 +42,7 @@ bool use_row1(int dtype) {
 // general kernel's preparation launch and its tail still weigh more (Q4_K: + 6 .. 40 % up to 57 MB, - 4 % at 75 MB,
 // - 19 % at 350 MB; Q5_K: + 7 % at 92 MB, - 12 % at 430 MB).  TURQ_ROW1_M lowers the row limit, for comparison.
 bool row1_takes(int64_t m, size_t weight_bytes, int dtype) {
-    static const int most = [] { const char *e = getenv("TURQ_ROW1_M"); const int x = e ? atoi(e) : TURQ_ROW1_MAX_M; return x < 1 ? 1 : x > TURQ_ROW1_MAX_M ? TURQ_ROW1_MAX_M : x; }();
+    const int most = std::min(std::max(turq_tuning().row1_m, 1), TURQ_ROW1_MAX_M);
     const size_t least = (size_t)8 << 20;  // below: the general kernel is level or up to 10 % ahead, for any number of rows
     if (m == 1) return true;
     if (m > most || m > turq_gemv_row1_rows(dtype) || weight_bytes < least) return false;
@@ -54,8 +53,8 @@ bool row1_takes(int64_t m, size_t weight_bytes, int dtype) {
 // Waves per workgroup of the one-row kernel: it is light on registers and on vector work, so what it wants is many waves
 // with few column tiles each (two by default), up to the largest workgroup.
 int pick_waves_row1(int64_t k) {
-    static const int forced = [] { const char *e = getenv("TURQ_GEMV_WAVES"); return e ? atoi(e) : 0; }();
-    static const int tpw_env = [] { const char *e = getenv("TURQ_ROW1_TPW"); return e && atoi(e) > 0 ? atoi(e) : 0; }();
+    const int forced = turq_tuning().gemv_waves;
+    const int tpw_env = std::max(turq_tuning().row1_tpw, 0);
     const int64_t col_tiles = turq_tile_cols(k);
     // (up to four column tiles, K <= 1024: one per wave; the 3072 x 1024 Q8_0 matrix gains 5 %)
     const int tpw = tpw_env ? tpw_env : (col_tiles <= 4 ? 1 : 2);
@@ -65,7 +64,7 @@ int pick_waves_row1(int64_t k) {
 
 // Row tiles per workgroup of the one-row kernel (TURQ_ROW1_R forces it).
 int pick_rows_row1(const turq_ctx *ctx, int64_t row_tiles) {
-    static const int forced = [] { const char *e = getenv("TURQ_ROW1_R"); return e ? atoi(e) : 0; }();
+    const int forced = turq_tuning().row1_r;
     if (forced == 1 || forced == 2) return forced;
     // two row tiles share the staged activations where there are row tiles to spare (the LM head: + 10 %)
     const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
@@ -79,8 +78,7 @@ int pick_rows_row1(const turq_ctx *ctx, int64_t row_tiles) {
 // and loses where there are many (the LM head: - 12 .. - 30 %) or 32 rows (registers).  TURQ_CS = 0 switches it off,
 // TURQ_CS_RG forces the group size (2, 3 or 6).
 int cs_row_tiles(const turq_ctx *ctx, int64_t m, int64_t row_tiles, int dtype, bool aligned) {
-    static const int mode = [] { const char *e = getenv("TURQ_CS"); return e ? atoi(e) : -1; }();
-    static const int forced = [] { const char *e = getenv("TURQ_CS_RG"); return e ? atoi(e) : 0; }();
+    const int mode = turq_tuning().cs, forced = turq_tuning().cs_rg;
     if (mode == 0 || !aligned || m < 2 || m > TURQ_GEMV_MAX_M) return 0;
     const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
     int rg = (m <= 16 && dtype != TURQ_Q8_0 && row_tiles >= 6 * cus && row_tiles <= 12 * cus) ? 6 : 0;
@@ -99,10 +97,8 @@ int cs_row_tiles(const turq_ctx *ctx, int64_t m, int64_t row_tiles, int dtype, b
 // TURQ_CS_RG forces the group size.
 int staged_row_tiles(const turq_ctx *ctx, int dtype_a, int dtype_b, int64_t k, int64_t m, int64_t row_tiles, int64_t row_tiles_b,
                      bool aligned) {
-    static const int mode = [] { const char *e = getenv("TURQ_CS_STAGED"); return e ? atoi(e) : -1; }();
-    static const int forced = [] { const char *e = getenv("TURQ_CS_RG"); return e ? atoi(e) : 0; }();
-    static const int min_m = [] { const char *e = getenv("TURQ_CS_STAGED_MIN_M"); return e ? atoi(e) : 3; }();
-    static const int max_m = [] { const char *e = getenv("TURQ_CS_STAGED_MAX_M"); return e ? atoi(e) : 32; }();
+    const TurqTuning &tune = turq_tuning();
+    const int mode = tune.cs_staged, forced = tune.cs_rg, min_m = tune.cs_staged_min_m, max_m = tune.cs_staged_max_m;
     if (mode == 0 || !aligned || m < min_m || m > max_m || m > TURQ_GEMV_MAX_M) return 0;
     const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
     if (row_tiles > 12 * cus && !forced) return 0;  // many rounds of workgroups (an LM head): the prepared fragments do better
@@ -256,7 +252,7 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
     // others on further streams that start where it starts (an event recorded there; behind the preparation, the only thing
     // they need) and are joined before the call returns.  Only when one preparation serves the whole call (a later
     // preparation would overwrite fragments that another stream still reads).
-    static const bool no_side = getenv("TURQ_GEMM_NO_SIDE") != nullptr;
+    const bool no_side = turq_tuning().gemm_no_side;
     const int64_t cus = ctx->compute_units;
     int n_small = 0;
     bool one_order = true;
@@ -270,7 +266,7 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
     int64_t group_cus = 0;  // CUs they take together
     int prepared = 0;       // 1: K-quant order, 2: Q8_0 order
     hipError_t e = hipSuccess;
-    static const int merge_env = [] { const char *v = getenv("TURQ_GEMM_MERGE"); return v ? atoi(v) : -1; }();  // 0: never, 2: every run
+    const int merge_env = turq_tuning().gemm_merge;  // 0: never, 2: every run
     const bool no_merge = merge_env == 0, merge_all = merge_env == 2;
     for (int i = 0; i < count && e == hipSuccess; i++) {
         const int order = w[i]->dtype == TURQ_Q8_0 ? 2 : 1;
@@ -348,8 +344,7 @@ int turq_qmatmul_multi_gemm(turq_ctx *ctx, int count, const turq_weight *const *
 }
 
 bool turq_norm_fuses(const turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t ldx, int64_t m) {
-    static const bool off = [] { const char *e = getenv("TURQ_NORM_FUSED"); return e && atoi(e) == 0; }();
-    static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
+    const bool off = turq_tuning().norm_fused_off, no_fuse = turq_tuning().gemv_no_fuse;
     if (off || count < 1 || ctx->wide || ctx->fixed_scratch || !turq_act_bytes(xt)) return false;
     float ws = 1.0f;
     for (int i = 0; i < count; i++)
@@ -389,7 +384,7 @@ int turq_mlp_prefill(turq_ctx *ctx, const turq_weight *gate, const turq_weight *
                      int64_t m, int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up,
                      const float *bias_down, bool *taken, const TurqNorm *norm) {
     *taken = false;
-    static const bool off = [] { const char *e = getenv("TURQ_MLP_PREFILL"); return e && atoi(e) == 0; }();
+    const bool off = turq_tuning().mlp_prefill_off;
     const turq_weight *gu[2] = {gate, up};
     float ws_down = 1.0f, ws_tmp = 1.0f;
     if (off || m <= TURQ_GEMV_MAX_M || ctx->fixed_scratch) return TURQ_OK;
@@ -450,7 +445,7 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
         const int64_t mc = std::min<int64_t>(TURQ_GEMV_MAX_M, m - m0);
         const uint8_t *xc = (const uint8_t *)x + (size_t)m0 * (size_t)ldx * xb;
         uint8_t *yc = (uint8_t *)y + (size_t)m0 * (size_t)ldy * yb;
-        static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
+        const bool no_fuse = turq_tuning().gemv_no_fuse;
         // raw activation rows must be 16-byte (f32) / 8-byte (16-bit) aligned for the fused loads
         const bool aligned = ((uintptr_t)xc % 16 == 0) && ((size_t)ldx * xb) % 16 == 0;
         if (aligned && !no_fuse && use_row1(w->dtype) && row1_takes(mc, w->dev_bytes, w->dtype)) {
@@ -486,7 +481,7 @@ int turq_qmatmul_mfma(turq_ctx *ctx, const turq_weight *w, const void *x, int xt
 // two GEMM launches, plus the preparation launch and, fused, the elementwise pass that the staged kernel has in its epilogue).
 // TURQ_ROWS_IN_CHUNKS = 0 switches it off.
 bool turq_rows_in_chunks(const turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t ldx, int64_t m) {
-    static const bool off = [] { const char *e = getenv("TURQ_ROWS_IN_CHUNKS"); return e && atoi(e) == 0; }();
+    const bool off = turq_tuning().rows_in_chunks_off;
     if (off || m <= TURQ_GEMV_MAX_M || m > 2 * TURQ_GEMV_MAX_M || count < 1 || count > 4) return false;
     const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
     const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
@@ -504,7 +499,7 @@ bool turq_rows_in_chunks(const turq_ctx *ctx, int count, const turq_weight *cons
 int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq_weight *up, const void *x, int xt, int64_t m,
                               int64_t ldx, void *y, int yt, int64_t ldy, const float *bias_gate, const float *bias_up, bool *taken,
                               const TurqNorm *norm) {
-    static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
+    const bool no_fuse = turq_tuning().gemv_no_fuse;
     *taken = false;
     if (norm && m != 1) return TURQ_OK;  // (the caller normalises into scratch first)
     {
@@ -531,7 +526,7 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     // 3 .. 16 rows: the kernel that makes its fragments from the rows themselves (no preparation launch), activation in its epilogue
     {
-        static const int staged = [] { const char *e = getenv("TURQ_CS_STAGED"); return e ? atoi(e) : -1; }();
+        const int staged = turq_tuning().cs_staged;
         const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
         const int tiles = (staged != 0 && aligned && m >= 3 && gate->n == up->n && gate->k == up->k)
                               ? turq_gemv_cs_staged_gateup_tiles(gate->dtype, gate->n, gate->k, m, cus) : 0;
@@ -547,7 +542,7 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
     if (no_fuse || !aligned || m > 2 || !use_row1(gate->dtype) || !row1_takes(m, gate->dev_bytes + up->dev_bytes, gate->dtype)) {
         // up to 32 rows: fragments prepared once, then one launch whose workgroups take row tile b of both weights (the shape
         // of the two-row-tile kernel: at most four waves) and store the product
-        static const bool no_frag = getenv("TURQ_GATEUP_NO_FRAG") != nullptr;
+        const bool no_frag = turq_tuning().gateup_no_frag;
         if (no_frag) return TURQ_OK;
         int rc = turq_ctx_reserve(ctx, &ctx->act_prep, &ctx->act_prep_cap, turq_act_prep_bytes(gate->dtype, m, gate->k));
         if (rc != TURQ_OK) return rc;
@@ -562,7 +557,7 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
     TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
     // a wave holds a tile of each weight per column tile: half as many column tiles per wave as in the plain launch, i.e. twice
     // the waves (K = 4096: 16 waves of one column tile; 8 waves of two cost the MLP step 2.7 %)
-    static const bool forced = getenv("TURQ_GEMV_WAVES") != nullptr;
+    const bool forced = turq_tuning().gemv_waves != 0;
     int nwaves = pick_waves_row1(gate->k);
     if (!forced) nwaves = (int)std::min<int64_t>({2 * (int64_t)nwaves, 16, turq_tile_cols(gate->k)});
     TURQ_HIP(ctx, turq_launch_gemv_row1_gateup(gate->dtype, gate->dev, up->dev, gate->n, gate->k, x, xt, ldx, m, y, yt, ldy, bias_gate,
@@ -577,7 +572,7 @@ int turq_qmatmul_gate_up_mfma(turq_ctx *ctx, const turq_weight *gate, const turq
 // the activation fragments are prepared once per fragment order (K-quants / Q8_0) and shared by all the weights.
 int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *w, const void *x, int xt, int64_t m,
                             int64_t ldx, void *const *y, int yt, const int64_t *ldy, const float *const *bias, const TurqNorm *norm) {
-    static const bool no_fuse = getenv("TURQ_GEMV_NO_FUSE") != nullptr;
+    const bool no_fuse = turq_tuning().gemv_no_fuse;
     if (norm && !(m == 1 && turq_norm_fuses(ctx, count, w, x, xt, ldx, m)))
         return turq_fail(ctx, TURQ_ERR_INVALID, "turq_qmatmul_multi: no kernel applies the norm for this call (internal)");
     const bool aligned = ((uintptr_t)x % 16 == 0) && ((size_t)ldx * turq_act_bytes(xt)) % 16 == 0;
@@ -594,7 +589,7 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
         int j = i + 1;
         while (j < count && j - i < 4 && w[j]->dtype == w[i]->dtype) j++;
         // one activation row: a run of a second format joins the launch where the kernel has that pair (q, k Q4_K + v Q6_K)
-        static const bool no_mixed = getenv("TURQ_GEMV_NO_MIXED") != nullptr;
+        const bool no_mixed = turq_tuning().gemv_no_mixed;
         // 5 .. 16 rows: fragments made in the kernel from the rows themselves (staged through the LDS), a second format in the
         // same launch where the kernel has the pair
         {
@@ -661,7 +656,7 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
                     wp[t - i] = w[t]->dev;
                     nn[t - i] = w[t]->n;
                 }
-                static const int cs_waves = [] { const char *e = getenv("TURQ_CS_WAVES"); return e ? atoi(e) : 0; }();
+                const int cs_waves = turq_tuning().cs_waves;
                 const int nw = (int)std::min<int64_t>(cs_waves >= 1 && cs_waves <= 8 ? cs_waves : 8, turq_tile_cols(w[i]->k));
                 hipEvent_t ev0 = nullptr, ev1 = nullptr;
                 TURQ_HIP(ctx, turq_prof_next(ctx, &ev0, &ev1));
@@ -732,7 +727,7 @@ int turq_qmatmul_multi_mfma(turq_ctx *ctx, int count, const turq_weight *const *
         }
         // prepared fragments are the larger stream (9 - 18 KiB per column tile against 2 - 4 KiB per weight tile): with enough
         // row tiles to keep every CU busy a workgroup takes two of them per set of fragments
-        static const int forced_r = [] { const char *e = getenv("TURQ_GEMV_ROWTILES"); return e ? atoi(e) : 0; }();
+        const int forced_r = turq_tuning().gemv_rowtiles;
         const int64_t cus = ctx->compute_units > 0 ? ctx->compute_units : 256;
         int rtiles = (!fused && turq_tile_rows(rows) >= 4 * cus) ? 2 : 1;
         if (!fused && (forced_r == 1 || forced_r == 2)) rtiles = forced_r;
