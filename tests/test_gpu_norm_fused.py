@@ -127,6 +127,27 @@ def test_norm_then_q_k_v(gpu, m, x_dtype):
         gpu.release(w)
 
 
+@pytest.mark.parametrize("fmts", [[(Q6_K, 512)], [(Q4_K, 768), (Q6_K, 256)], [(13, 512), (Q6_K, 256)]], ids=["q6k", "q4k+q6k", "q5k+q6k"])
+def test_one_row_on_a_wide_hidden_size(gpu, fmts):
+    # 12288 columns are 48 column tiles: 3 per wave, where the plain one-row kernels keep three in flight; with the norm weights
+    # next to them the kernels of the fused call keep two (three spill registers) - same sums, same bars
+    k, m = 12288, 1
+    raws = [synth.random_weight(dt, n, k, seed=20 + i) for i, (dt, n) in enumerate(fmts)]
+    ws = [gpu.upload(dt, n, k, raw, capi.LAYOUT_TILED) for (dt, n), raw in zip(fmts, raws)]
+    ns = [n for _, n in fmts]
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((m, k)) * 3).astype(np.float32)
+    nw = (1.0 + 0.3 * rng.standard_normal(k)).astype(np.float32)
+    got = norm_multi(gpu, ws, ns, x, nw)
+    sep, _ = separate(gpu, ws, ns, x, nw)
+    xn = want_norm(x, nw)
+    for (dt, n), raw, y, s in zip(fmts, raws, got, sep):
+        assert rel_l2(y, orc.matmul_dequant(dt, xn, raw, n, k)) <= 1e-3, (dt, n)
+        assert rel_l2(y, s) <= 5e-4, (dt, n, rel_l2(y, s))
+    for w in ws:
+        gpu.release(w)
+
+
 def test_final_norm_then_lm_head_and_host_pointers(gpu):
     n, k = 5000, 1024
     raw = synth.random_weight(Q6_K, n, k, seed=3)

@@ -676,7 +676,8 @@ hipError_t launch_final_n(const Row1Launch &l) {
 template <int DT, int XT, int P, int R, int M>
 hipError_t launch_final(const Row1Launch &l) {
     if constexpr (M == 1) {
-        if (l.gw) return launch_final_n<DT, XT, P, R, M, true>(l);
+        // (with the norm weights held next to the weights, three column tiles in flight spill registers for Q5_K and Q6_K: two)
+        if (l.gw) return launch_final_n<DT, XT, (P > 2 ? 2 : P), R, M, true>(l);
     }
     if (l.gw) return hipErrorInvalidValue;  // (the norm inside the kernel: one activation row)
     return launch_final_n<DT, XT, P, R, M, false>(l);
@@ -734,7 +735,7 @@ hipError_t launch_mixed_final_n(const Row1Launch &l) {
 template <int DTA, int DTB, int XT, int P, int M>
 hipError_t launch_mixed_final(const Row1Launch &l) {
     if constexpr (M == 1) {
-        if (l.gw) return launch_mixed_final_n<DTA, DTB, XT, P, M, true>(l);
+        if (l.gw) return launch_mixed_final_n<DTA, DTB, XT, (P > 2 ? 2 : P), M, true>(l);  // (as in launch_final)
     }
     if (l.gw) return hipErrorInvalidValue;
     return launch_mixed_final_n<DTA, DTB, XT, P, M, false>(l);
