@@ -129,10 +129,16 @@ hipError_t launch_final(const CsLaunch &l) {
 
 template <int DT, int MT, int XT>
 hipError_t launch_rg(int rg, const CsLaunch &l) {
+    // (not instantiated: the group sizes that do not fit the register file - six row tiles with two activation tiles or with
+    // Q8_0's 4352-byte tiles, three with both; cs_row_tiles() in mfma_dispatch.cpp never asks for them)
     switch (rg) {
     case 2: return launch_final<DT, MT, XT, 2, 2>(l);
-    case 3: return launch_final<DT, MT, XT, 3, 3>(l);
-    case 6: return launch_final<DT, MT, XT, 6, 3>(l);
+    case 3:
+        if constexpr (DT == TURQ_Q8_0 && MT == 2) return hipErrorInvalidValue;
+        else return launch_final<DT, MT, XT, 3, 3>(l);
+    case 6:
+        if constexpr (DT == TURQ_Q8_0 || MT == 2) return hipErrorInvalidValue;
+        else return launch_final<DT, MT, XT, 6, 3>(l);
     default: return hipErrorInvalidValue;
     }
 }
