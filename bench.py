@@ -445,6 +445,8 @@ class Bench:
         gbps = self.step_bytes / (dt_s / steps) / 1e9
 
         # dominant kernel alone: event pairs around every matmul kernel launch, same steps, untimed pass
+        self.step_eager()      # (the timed steps were graph replays: one untimed pass from the host first)
+        self.sync()
         capi.check(L.turq_profile_begin(ctx), ctx)
         prof_steps = max(1, min(steps, 10))
         for _ in range(prof_steps):

@@ -382,7 +382,7 @@ struct Row1Args {
 // gate / up and the LM head): a lane multiplies its columns by gw when it stages them and adds up their squares, and the row's
 // 1 / sqrt(mean(x^2) + eps), which is the same for every column, multiplies the results - the separate launch of the norm and
 // the round trip of its output go away.
-template <int DT, int XT, int P, int R, int M, bool GU = false, bool NORM = false>
+template <int DT, int XT, int P, int R, int M, bool GU = false, bool NORM = false, bool ACC = false>
 __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *__restrict__ y, int64_t ldy, const float *__restrict__ bias,
                                           int64_t n, int64_t rtb, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt,
                                           const uint8_t *__restrict__ w2 = nullptr, const float *__restrict__ bias2 = nullptr,
@@ -435,11 +435,12 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
     }
 #pragma unroll
     for (int mm = 0; mm < M; mm++) xrow[mm] = (const uint8_t *)x + (mm < m ? mm : 0) * ldx * ES;
-    // TURQ_OUT_ACCUMULATE: the element this lane will add its first result to, requested now so that it has long arrived when
-    // the sums are done (a load at the end of the kernel is a whole memory round trip on the critical path)
+    // ACC (TURQ_OUT_ACCUMULATE in yt; an instantiation of its own, since even the untaken branch cost the plain launches 2 %):
+    // the element this lane will add its first result to, requested now so that it has long arrived when the sums are done (a
+    // load at the end of the kernel is a whole memory round trip on the critical path)
     float old_first = 0.0f;
-    if constexpr (!GU) {
-        if ((yt & TURQ_OUT_ACCUMULATE) && wave < R * M) {
+    if constexpr (ACC && !GU) {
+        if (wave < R * M) {
             const int r = wave / M, mm = wave - r * M;
             const int64_t col = (rt0 + r) * 16 + (lane >> 2);
             if ((lane & 3) == 0 && rt0 + r < nrt && col < n && mm < m) {
@@ -592,7 +593,7 @@ __device__ __forceinline__ void row1_body(const uint8_t *__restrict__ w, void *_
         if (q == 0 && rt0 + r < nrt && col < n && mm < m) {
             const float out = s * inv_rms + (bias ? bias[col] : 0.0f);
             const int64_t at = (int64_t)mm * ldy + col;
-            if (i == wave) turq_store_any(y, yt & 0xFF, at, out + old_first);  // (what y held was requested before the main loop)
+            if (ACC && i == wave) turq_store_any(y, yt & 0xFF, at, out + old_first);  // (what y held was requested before the main loop)
             else turq_store_any(y, yt, at, out);
         }
     }
@@ -609,11 +610,11 @@ __device__ inline Row1Pick row1_pick(const Row1Args &a, int blk) {
 }
 
 // m <= M activation rows of stride ldx; MAXT = largest workgroup of the instantiation
-template <int DT, int XT, int P, int R, int M, int MAXT, bool NORM = false>
+template <int DT, int XT, int P, int R, int M, int MAXT, bool NORM = false, bool ACC = false>
 __global__ void __launch_bounds__(MAXT) gemv_row1_kernel(Row1Args a, int64_t k, const void *__restrict__ x, int64_t ldx, int m, int yt,
                                                          const float *__restrict__ gw, float eps) {
     const Row1Pick p = row1_pick(a, (int)blockIdx.x);
-    row1_body<DT, XT, P, R, M, false, NORM>(p.w, p.y, p.ldy, p.bias, p.n, (int64_t)((int)blockIdx.x - p.first), k, x, ldx, m, yt, nullptr,
+    row1_body<DT, XT, P, R, M, false, NORM, ACC>(p.w, p.y, p.ldy, p.bias, p.n, (int64_t)((int)blockIdx.x - p.first), k, x, ldx, m, yt, nullptr,
                                             nullptr, gw, eps);
 }
 
@@ -657,30 +658,35 @@ template <int DT, int P, int R, int M> size_t row1_lds(int nwaves) {
     return (size_t)nwaves * P * tile + (size_t)nwaves * R * M * 64 * sizeof(float) + 64;  // (+ a sum of squares per wave)
 }
 
-template <int DT, int XT, int P, int R, int M, bool NORM>
+template <int DT, int XT, int P, int R, int M, bool NORM, bool ACC>
 hipError_t launch_final_n(const Row1Launch &l) {
     const size_t lds = row1_lds<DT, P, R, M>(l.nwaves);
     const dim3 grid((unsigned)l.blocks), block((unsigned)(64 * l.nwaves));
     if (lds > (64u << 10)) {  // 16 waves x two tiles in flight x two pairs of rows: 94 KiB
-        const hipError_t raised = turq_raise_lds_limit((const void *)gemv_row1_kernel<DT, XT, P, R, M, 1024, NORM>, 128 << 10);
+        const hipError_t raised = turq_raise_lds_limit((const void *)gemv_row1_kernel<DT, XT, P, R, M, 1024, NORM, ACC>, 128 << 10);
         if (raised != hipSuccess) return raised;
     }
     if (l.ev0) {
-        hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, R, M, 1024, NORM>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k,
+        hipExtLaunchKernelGGL((gemv_row1_kernel<DT, XT, P, R, M, 1024, NORM, ACC>), grid, block, (unsigned)lds, l.s, l.ev0, l.ev1, 0, l.a, l.k,
                               l.x, l.ldx, l.m, l.yt, l.gw, l.eps);
         return hipGetLastError();
     }
-    gemv_row1_kernel<DT, XT, P, R, M, 1024, NORM><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt, l.gw, l.eps);
+    gemv_row1_kernel<DT, XT, P, R, M, 1024, NORM, ACC><<<grid, block, lds, l.s>>>(l.a, l.k, l.x, l.ldx, l.m, l.yt, l.gw, l.eps);
     return hipGetLastError();
 }
 template <int DT, int XT, int P, int R, int M>
 hipError_t launch_final(const Row1Launch &l) {
     if constexpr (M == 1) {
         // (with the norm weights held next to the weights, three column tiles in flight spill registers for Q5_K and Q6_K: two)
-        if (l.gw) return launch_final_n<DT, XT, (P > 2 ? 2 : P), R, M, true>(l);
+        if (l.gw) return launch_final_n<DT, XT, (P > 2 ? 2 : P), R, M, true, false>(l);
     }
     if (l.gw) return hipErrorInvalidValue;  // (the norm inside the kernel: one activation row)
-    return launch_final_n<DT, XT, P, R, M, false>(l);
+    // the residual additions behind o_proj and down_proj: one row tile per workgroup (the tall matrices that take two are LM
+    // heads; they would add through the store's own load of y)
+    if constexpr (R == 1) {
+        if (l.yt & TURQ_OUT_ACCUMULATE) return launch_final_n<DT, XT, P, R, M, false, true>(l);
+    }
+    return launch_final_n<DT, XT, P, R, M, false, false>(l);
 }
 
 // column tiles in flight per wave: up to three for one activation row (four do not fit the registers of every format), up to
