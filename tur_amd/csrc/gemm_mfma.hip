@@ -75,6 +75,8 @@ constexpr uint32_t kMagic1024 = 0x64006400u;  // 1024.0: a nibble in mantissa bi
 constexpr uint32_t kMagic64 = 0x54005400u;    // 64.0:   a nibble in mantissa bits 4..7 reads as 64 + n
 constexpr uint32_t kMagic256 = 0x5C005C00u;   // 256.0:  a 6-bit value in mantissa bits 2..7 reads as 256 + q
 constexpr int kCoherent = 16;                 // cache policy of buffer loads and stores that other XCDs must see: sc1, as device-scope atomics carry
+// lanes whose value is no finite number, or too large for the output type: one vector compare, the OR runs on the scalar unit
+__device__ inline uint64_t note_mask(float v, float lim) { return __builtin_amdgcn_ballot_w64(!(__builtin_fabsf(v) < lim)); }
 // A workgroup is 4 waves and covers 128 rows of m (4 m-tiles of 32): as 2 x 2 waves with 2 m-tiles each (WGM = 2), or as
 // 1 x 4 waves that all take the 4 m-tiles (WGM = 1: every weight is unpacked by ONE wave instead of two, at twice the
 // activation reads per wave; for the formats whose unpack is long)
@@ -206,7 +208,7 @@ __device__ inline const uint8_t *uniform_ptr(const uint8_t *p) {
 
 template <int I> __device__ inline uint32_t word_of(uint4v v) { return I == 0 ? v.x : I == 1 ? v.y : I == 2 ? v.z : v.w; }
 
-__device__ inline uint32_t pack_bf16x2(float a, float b) { return (uint32_t)turq_f2bf(a) | ((uint32_t)turq_f2bf(b) << 16); }
+__device__ inline uint32_t pack_bf16x2(float a, float b) { return turq_f2bf_x2(a, b); }
 __device__ inline uint32_t pack_f16x2(float a, float b) {
     const half2v h{(_Float16)a, (_Float16)b};
     return as_u32(h);
@@ -885,7 +887,7 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        uint32_t bad = 0;  // results that are no finite numbers, or do not fit an f16 output (turq_ctx_nonfinite_count)
+        uint64_t badm = 0;  // results that are no finite numbers, or do not fit an f16 output (turq_ctx_nonfinite_count)
         const float lim = ytb == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
         if (ytb == TURQ_ACT_F32) {
             constexpr int CPR = WN * 32 / 4;  // 16-byte pieces per row
@@ -897,7 +899,7 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                 if (row0 + r < m && col0 + 4 * cc < n) {
                     float4v *dst = (float4v *)((float *)y + (row0 + r) * ldy + col0 + 4 * cc);
                     if (accum) v += *dst;
-                    turq_note_accum(v.x, lim, bad), turq_note_accum(v.y, lim, bad), turq_note_accum(v.z, lim, bad), turq_note_accum(v.w, lim, bad);
+                    badm |= note_mask(v.x, lim) | note_mask(v.y, lim) | note_mask(v.z, lim) | note_mask(v.w, lim);
                     *dst = v;
                 }
             }
@@ -928,7 +930,7 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                         }
                     }
 #pragma unroll
-                    for (int e = 0; e < 8; e++) turq_note_accum(vs[e], lim, bad);
+                    for (int e = 0; e < 8; e++) badm |= note_mask(vs[e], lim);
                     uint4v o;
                     if (ytb == TURQ_ACT_BF16)
                         o = uint4v{pack_bf16x2(vs[0], vs[1]), pack_bf16x2(vs[2], vs[3]), pack_bf16x2(vs[4], vs[5]), pack_bf16x2(vs[6], vs[7])};
@@ -938,9 +940,9 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                 }
             }
         }
-        turq_note_flush(bad);
+        turq_note_flush(badm != 0 ? 1u : 0u);
     } else {
-        uint32_t bad = 0;
+        uint64_t badm = 0;
         const float lim = ytb == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
 #pragma unroll
         for (int j = 0; j < WN; j++) {
@@ -957,14 +959,14 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                         if (accum)
                             v += ytb == TURQ_ACT_F32 ? turq_load_out<TURQ_ACT_F32>(y, row * ldy + col)
                                  : ytb == TURQ_ACT_BF16 ? turq_load_out<TURQ_ACT_BF16>(y, row * ldy + col) : turq_load_out<TURQ_ACT_F16>(y, row * ldy + col);
-                        turq_note_accum(v, lim, bad);
+                        badm |= note_mask(v, lim);
                         if (ytb == TURQ_ACT_F32) turq_store_out_raw<TURQ_ACT_F32>(y, row * ldy + col, v);
                         else if (ytb == TURQ_ACT_BF16) turq_store_out_raw<TURQ_ACT_BF16>(y, row * ldy + col, v);
                         else turq_store_out_raw<TURQ_ACT_F16>(y, row * ldy + col, v);
                     }
                 }
         }
-        turq_note_flush(bad);
+        turq_note_flush(badm != 0 ? 1u : 0u);
     }
 }
 

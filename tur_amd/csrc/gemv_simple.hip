@@ -15,17 +15,11 @@ template <int XT> __device__ inline float load_act(const void *x, int64_t i) {
     return turq_h2f(((const uint16_t *)x)[i]);
 }
 
-__device__ inline uint16_t f2bf(float f) {  // round to nearest even, NaN kept quiet
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
-    u += 0x7FFFu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
-}
 
 template <int YT> __device__ inline void store_out(void *y, int64_t i, float v) {
     turq_note_result<YT>(v);
     if (YT == TURQ_ACT_F32) ((float *)y)[i] = v;
-    else if (YT == TURQ_ACT_BF16) ((uint16_t *)y)[i] = f2bf(v);
+    else if (YT == TURQ_ACT_BF16) ((uint16_t *)y)[i] = turq_f2bf(v);
     else {
         const _Float16 h = (_Float16)v;
         uint16_t b;

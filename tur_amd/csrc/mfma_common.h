@@ -122,12 +122,18 @@ struct GOff {
 
 __device__ inline uint32_t rotr32(uint32_t v, uint32_t s) { return __builtin_amdgcn_alignbit(v, v, s); }
 
-__device__ inline uint16_t turq_f2bf(float f) {  // round to nearest even, NaN kept quiet
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
-    u += 0x7FFFu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+// f32 -> bf16, round to nearest even, NaN stays a (quiet) NaN: gfx950 converts two values in one instruction
+// (v_cvt_pk_bf16_f32; seven vector instructions per value when written out with integer arithmetic, which was 1 us of a
+// 60 us prefill launch that stores bf16)
+typedef __bf16 turq_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float turq_f32x2 __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t turq_f2bf_x2(float lo, float hi) {  // lo in bits 0..15
+    const turq_bf16x2 b = __builtin_convertvector(turq_f32x2{lo, hi}, turq_bf16x2);
+    uint32_t u;
+    __builtin_memcpy(&u, &b, 4);
+    return u;
 }
+__device__ inline uint16_t turq_f2bf(float f) { return (uint16_t)turq_f2bf_x2(f, 0.0f); }
 // Results that are no finite numbers.  The matrix kernels compute on f16 activations: a finite f32 or bf16 input of magnitude
 // 65520 or more becomes an infinity there, and what it is multiplied into comes out as an infinity or a NaN - as do inputs that
 // were infinities or NaNs to begin with.  Every kernel that stores results counts the elements it stores that are not finite
