@@ -147,6 +147,35 @@ def nonfinite(g, reset=1):
     return n.value
 
 
+@pytest.mark.parametrize("m", [1, 8, 48])
+def test_a_finite_f32_result_that_no_bf16_holds_is_counted(m):
+    # Q8_0 rows of all 127 with block scale 1: y = 127 * sum(x).  The rows are chosen so that y = 3.399e38: a finite f32, but
+    # past the midpoint between the largest bf16 (3.3895e38) and 2^128, so the bf16 store rounds it to an infinity.  With wide
+    # activations on (the rows are far outside f16) the f32 output is finite and nothing is counted; the bf16 output is counted.
+    g = Gpu()
+    try:
+        L, ctx = g.L, g.ctx
+        n, k = 32, 256
+        block = np.concatenate([np.array([1.0], np.float16).view(np.uint8), np.full(32, 127, np.int8).view(np.uint8)])
+        raw = np.tile(block, n * (k // 32))
+        w = g.upload(Q8_0, n, k, raw, capi.LAYOUT_TILED)
+        x = np.full((m, k), 3.399e38 / (127.0 * k), np.float32)
+        capi.check(L.turq_ctx_set_wide_activations(ctx, 1), ctx)
+        nonfinite(g)
+        y32 = g.qmatmul(w, x, n, k, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_F32)
+        assert np.all(np.isfinite(y32)) and np.all(np.abs(y32 / 3.399e38 - 1) < 1e-3)
+        assert nonfinite(g) == 0
+        y16 = g.qmatmul(w, x, n, k, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_BF16)
+        assert np.all(np.isinf(y16))
+        assert nonfinite(g) >= 1
+        # a little lower and the bf16 store is the largest finite bf16: not counted
+        y16 = g.qmatmul(w, x * np.float32(0.99), n, k, x_dtype=capi.ACT_F32, y_dtype=capi.ACT_BF16)
+        assert np.all(np.isfinite(y16)) and nonfinite(g) == 0
+        g.release(w)
+    finally:
+        g.close()
+
+
 @pytest.mark.parametrize("m", [1, 2, 8, 24, 40, 100])     # one-row kernel, two rows, staged rows, prepared fragments, prefill GEMM
 @pytest.mark.parametrize("dt", [Q4_K, Q6_K, Q8_0])
 def test_overflow_on_device_pointers_is_counted(dt, m):

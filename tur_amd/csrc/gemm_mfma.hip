@@ -888,7 +888,7 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         uint64_t badm = 0;  // results that are no finite numbers, or do not fit an f16 output (turq_ctx_nonfinite_count)
-        const float lim = ytb == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
+        const float lim = turq_finite_limit(ytb);
         if (ytb == TURQ_ACT_F32) {
             constexpr int CPR = WN * 32 / 4;  // 16-byte pieces per row
 #pragma unroll 4
@@ -943,7 +943,7 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
         turq_note_flush(badm != 0 ? 1u : 0u);
     } else {
         uint64_t badm = 0;
-        const float lim = ytb == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
+        const float lim = turq_finite_limit(ytb);
 #pragma unroll
         for (int j = 0; j < WN; j++) {
             const int64_t col = col0 + 32 * j + n32;

@@ -140,8 +140,13 @@ __device__ inline uint16_t turq_f2bf(float f) { return (uint16_t)turq_f2bf_x2(f,
 // (for an f16 output: that do not fit f16) in a word of device memory, so that a host can tell that it happened
 // (turq_ctx_nonfinite_count).  The word is this translation unit's own copy, one per GPU; it stops counting at 2^20.
 static __device__ uint32_t turq_nonfinite_word;
+// magnitudes from which a value of the output type is no finite number any more: the midpoint between the type's largest
+// finite value and the next power of two rounds (to even) to an infinity
+__device__ inline float turq_finite_limit(int yt) {
+    return yt == TURQ_ACT_F16 ? 65520.0f : yt == TURQ_ACT_BF16 ? __uint_as_float(0x7F7F8000u) : __builtin_inff();
+}
 template <int YT> __device__ inline void turq_note_result(float v) {
-    const float lim = YT == TURQ_ACT_F16 ? 65520.0f : __builtin_inff();
+    const float lim = turq_finite_limit(YT);
     if (__builtin_expect(!(__builtin_fabsf(v) < lim), 0)) {
         if (__hip_atomic_load(&turq_nonfinite_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (1u << 20))
             __hip_atomic_fetch_add(&turq_nonfinite_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
