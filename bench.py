@@ -445,14 +445,18 @@ class Bench:
         gbps = self.step_bytes / (dt_s / steps) / 1e9
 
         # dominant kernel alone: event pairs around every matmul kernel launch, same steps, untimed pass
-        self.step_eager()      # (the timed steps were graph replays: one untimed pass from the host first)
-        self.sync()
-        capi.check(L.turq_profile_begin(ctx), ctx)
-        prof_steps = max(1, min(steps, 10))
-        for _ in range(prof_steps):
-            self.step_eager()
         n_launch = ctypes.c_int64()
         tot_ms = ctypes.c_double()
+        # (the timed steps were graph replays: one pass from the host first, which also counts the launches of a step)
+        capi.check(L.turq_profile_begin(ctx), ctx)
+        self.step_eager()
+        capi.check(L.turq_profile_end(ctx, ctypes.byref(n_launch), ctypes.byref(tot_ms)), ctx)
+        per_step = max(1, n_launch.value)
+        # at least 100 launches behind the average (an LM head step is two launches), at most 60 steps
+        prof_steps = min(60, max(1, min(steps, 10), -(-100 // per_step)))
+        capi.check(L.turq_profile_begin(ctx), ctx)
+        for _ in range(prof_steps):
+            self.step_eager()
         capi.check(L.turq_profile_end(ctx, ctypes.byref(n_launch), ctypes.byref(tot_ms)), ctx)
         avg_us = tot_ms.value / max(1, n_launch.value) * 1e3
         # all timed launches are the matmul kernel (one per matrix, or one per group of matrices with a common input)
