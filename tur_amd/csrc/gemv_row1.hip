@@ -131,13 +131,14 @@ template <int DT> struct Row1K45 {
     // header group g sits at bit 24 g of the 12 bytes after (d, dmin) = byte 3 g; group 3 is read one byte early so that the
     // load ends with the header
     __device__ static uint32_t aux_off(int r, int g) { return 16u * (uint32_t)r + 4u + 3u * (uint32_t)g - (g == 3 ? 1u : 0u); }
+    // (non-temporal loads for everything that is read once per launch: see load_tile in gemv_tileop.h)
     __device__ static W load(const uint8_t *__restrict__ tile, const GOff &o) {
         W w;
-        w.qa = *(const uint4v *)(tile + F::kQA + o.o16);
-        w.qb = *(const uint4v *)(tile + F::kQB + o.o16);
-        if constexpr (HIGH) w.hh = *(const uint2v *)(tile + F::kQH + o.o8);
+        w.qa = __builtin_nontemporal_load((const uint4v *)(tile + F::kQA + o.o16));
+        w.qb = __builtin_nontemporal_load((const uint4v *)(tile + F::kQB + o.o16));
+        if constexpr (HIGH) w.hh = __builtin_nontemporal_load((const uint2v *)(tile + F::kQH + o.o8));
         else w.hh = uint2v{0u, 0u};
-        w.hd = *(const uint32_t *)(tile + F::kHDR + o.hdr);  // f16 d, f16 dmin
+        w.hd = __builtin_nontemporal_load((const uint32_t *)(tile + F::kHDR + o.hdr));  // f16 d, f16 dmin
         __builtin_memcpy(&w.grp, tile + F::kHDR + o.aux, 4);  // the (unaligned) dword that holds this lane's 24-bit group
         return w;
     }
@@ -251,11 +252,11 @@ template <> struct Row1Fmt<TURQ_Q6_K> {
     __device__ static uint32_t aux_off(int r, int) { return 2u * (uint32_t)r; }  // the row's d
     __device__ static W load(const uint8_t *__restrict__ tile, const GOff &o) {
         W w;
-        w.qla = *(const uint4v *)(tile + F::kQLA + o.o16);
-        w.qlb = *(const uint4v *)(tile + F::kQLB + o.o16);
-        w.qh = *(const uint4v *)(tile + F::kQH + o.o16);
-        w.scw = *(const uint32_t *)(tile + F::kSC + o.o4);
-        w.d16 = *(const uint16_t *)(tile + F::kD + o.aux);
+        w.qla = __builtin_nontemporal_load((const uint4v *)(tile + F::kQLA + o.o16));
+        w.qlb = __builtin_nontemporal_load((const uint4v *)(tile + F::kQLB + o.o16));
+        w.qh = __builtin_nontemporal_load((const uint4v *)(tile + F::kQH + o.o16));
+        w.scw = __builtin_nontemporal_load((const uint32_t *)(tile + F::kSC + o.o4));
+        w.d16 = __builtin_nontemporal_load((const uint16_t *)(tile + F::kD + o.aux));
         return w;
     }
     // every value is built in the mantissa of 256.0 and stands for q - 32: per sub-block (4 lanes) -288 * sum(x)
@@ -320,8 +321,8 @@ template <> struct Row1Fmt<TURQ_Q8_0> {
     __device__ static W load(const uint8_t *__restrict__ tile, const GOff &o) {
         W w;
 #pragma unroll
-        for (int i = 0; i < 4; i++) w.p[i] = *(const uint4v *)(tile + 1024 * i + o.o16);
-        w.dd = *(const uint2v *)(tile + o.aux);
+        for (int i = 0; i < 4; i++) w.p[i] = __builtin_nontemporal_load((const uint4v *)(tile + 1024 * i + o.o16));
+        w.dd = __builtin_nontemporal_load((const uint2v *)(tile + o.aux));
         return w;
     }
     // bytes are stored as q + 128 and unpacked into the mantissa of 1024.0: per block (8 lanes) -1152 * sum(x).

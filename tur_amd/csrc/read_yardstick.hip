@@ -1,5 +1,6 @@
 // A plain streaming read of device memory with the launch shape of the decode kernels: one 16-wave workgroup per compute unit,
-// every wave two 4 KiB chunks in flight, nothing done with the data but an xor.  It is the yardstick for what a decode launch
+// every wave two 4 KiB chunks in flight (non-temporal loads, as the decode kernels read their weights), nothing done with the
+// data but an xor.  It is the yardstick for what a decode launch
 // of a given size could reach at best on the device at hand: launches of a few tens of MB are short enough for the launch
 // itself (thousands of waves to start, the first loads to return, the last ones to drain) to weigh as much as the bytes.
 #include <hip/hip_ext.h>
@@ -19,7 +20,7 @@ __global__ void __launch_bounds__(1024) read_kernel(const uint8_t *__restrict__ 
         const size_t cc = c + d * stride;
         const uint8_t *p = buf + (cc < nchunks ? cc : 0) * 4096 + 16 * lane;
 #pragma unroll
-        for (int i = 0; i < 4; i++) r[d][i] = *(const uint4v *)(p + 1024 * i);
+        for (int i = 0; i < 4; i++) r[d][i] = __builtin_nontemporal_load((const uint4v *)(p + 1024 * i));
     }
     while (c < nchunks) {
 #pragma unroll
@@ -29,7 +30,7 @@ __global__ void __launch_bounds__(1024) read_kernel(const uint8_t *__restrict__ 
             const size_t cn = c + 2 * stride;
             const uint8_t *p = buf + (cn < nchunks ? cn : 0) * 4096 + 16 * lane;
 #pragma unroll
-            for (int i = 0; i < 4; i++) r[d][i] = *(const uint4v *)(p + 1024 * i);
+            for (int i = 0; i < 4; i++) r[d][i] = __builtin_nontemporal_load((const uint4v *)(p + 1024 * i));
             c += stride;
         }
     }
