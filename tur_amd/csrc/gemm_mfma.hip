@@ -900,7 +900,7 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                     float4v *dst = (float4v *)((float *)y + (row0 + r) * ldy + col0 + 4 * cc);
                     if (accum) v += *dst;
                     badm |= note_mask(v.x, lim) | note_mask(v.y, lim) | note_mask(v.z, lim) | note_mask(v.w, lim);
-                    *dst = v;
+                    __builtin_nontemporal_store(v, dst);
                 }
             }
         } else {
@@ -936,7 +936,7 @@ __global__ void __launch_bounds__(256 * KG) gemm_kq_kernel(GemmGroup grp, int64_
                         o = uint4v{pack_bf16x2(vs[0], vs[1]), pack_bf16x2(vs[2], vs[3]), pack_bf16x2(vs[4], vs[5]), pack_bf16x2(vs[6], vs[7])};
                     else
                         o = uint4v{pack_f16x2(vs[0], vs[1]), pack_f16x2(vs[2], vs[3]), pack_f16x2(vs[4], vs[5]), pack_f16x2(vs[6], vs[7])};
-                    *dst = o;
+                    __builtin_nontemporal_store(o, dst);
                 }
             }
         }
