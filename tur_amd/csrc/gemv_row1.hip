@@ -690,15 +690,17 @@ hipError_t launch_final(const Row1Launch &l) {
     return launch_final_n<DT, XT, P, R, M, false, false>(l);
 }
 
-// column tiles in flight per wave: up to three for one activation row (four do not fit the registers of every format), up to
-// two for several rows, whose raw activations are held next to the weights until they are staged
+// Column tiles in flight per wave: ONE.  The kernels exist with up to three for one activation row (four do not fit the
+// registers of every format) and up to two for several rows, and while the weights were read with plain loads two or three
+// were ahead; with the non-temporal loads a wave that takes its tiles one after the other is ahead on every shape measured
+// (down_proj 12288 columns: 8.0 -> 7.5 us; MLP step at 1 / 2 / 3 / 4 rows + 2.5 / 3.6 / 4.9 / 4.1 %; LM head Q6_K / Q5_K + 7 / + 15 %;
+// 4096 columns, two tiles per wave: level): the waves of a workgroup are at different tiles at any moment, which spreads
+// their requests, and a wave holds fewer registers and less LDS.  TURQ_ROW1_P = 2 / 3 asks for the other forms.
 inline int row1_in_flight(int64_t k, int nwaves, int m) {
+    (void)k, (void)nwaves;
     const int forced = turq_tuning().row1_p;
-    const int64_t per_wave = (turq_tile_cols(k) + nwaves - 1) / nwaves;
     const int most = m > 1 ? 2 : 3;
-    int p = (int)(per_wave < most ? per_wave : most);
-    if (forced >= 1 && forced <= most) p = forced;
-    return p;
+    return forced >= 1 && forced <= most ? forced : 1;
 }
 
 template <int DT, int XT>
@@ -888,14 +890,16 @@ hipError_t launch_gateup_final(const GateUpLaunch &l) {
 
 template <int DT, int XT>
 hipError_t launch_gateup_p(const GateUpLaunch &l) {
-    // two weights double what a wave holds per column tile: at most two column tiles in flight
+    // one column tile in flight, as in row1_in_flight (two weights double what a wave holds per column tile: two at most,
+    // on request, where a wave has two tiles to take)
     const int64_t per_wave = (turq_tile_cols(l.k) + l.nwaves - 1) / l.nwaves;
+    const bool one = per_wave <= 1 || turq_tuning().row1_p != 2;
     if (l.m == 2) {
         if (l.gw) return hipErrorInvalidValue;  // (the norm inside the kernel: one activation row)
-        return per_wave <= 1 ? launch_gateup_final<DT, XT, 1, 2, false>(l) : launch_gateup_final<DT, XT, 2, 2, false>(l);
+        return one ? launch_gateup_final<DT, XT, 1, 2, false>(l) : launch_gateup_final<DT, XT, 2, 2, false>(l);
     }
-    if (l.gw) return per_wave <= 1 ? launch_gateup_final<DT, XT, 1, 1, true>(l) : launch_gateup_final<DT, XT, 2, 1, true>(l);
-    return per_wave <= 1 ? launch_gateup_final<DT, XT, 1, 1, false>(l) : launch_gateup_final<DT, XT, 2, 1, false>(l);
+    if (l.gw) return one ? launch_gateup_final<DT, XT, 1, 1, true>(l) : launch_gateup_final<DT, XT, 2, 1, true>(l);
+    return one ? launch_gateup_final<DT, XT, 1, 1, false>(l) : launch_gateup_final<DT, XT, 2, 1, false>(l);
 }
 
 template <int DT>
